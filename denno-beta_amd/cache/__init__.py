@@ -1,0 +1,4 @@
+from .manager import CacheError, CacheManager, GroupLayout, OutOfPages, PAGED, STATE
+from .storage import CacheStorage
+
+__all__ = ["CacheError", "CacheManager", "GroupLayout", "OutOfPages", "PAGED", "STATE", "CacheStorage"]

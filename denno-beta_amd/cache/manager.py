@@ -1,0 +1,160 @@
+"""CacheManager: the Python face of the host core's page and slot bookkeeping
+(csrc/host/cache_manager.h).  It owns no device memory."""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_int, c_int64, c_void_p, POINTER
+from dataclasses import dataclass
+from typing import List, Sequence
+
+import numpy as np
+
+from ..build import load_library
+
+PAGED, STATE = 0, 1
+
+OK, NO_SLOT, DUPLICATE, UNKNOWN, OUT_OF_PAGES, BAD_ARGUMENT, CORRUPT = 0, -1, -2, -3, -4, -5, -6
+_NAMES = {NO_SLOT: "no free request slot", DUPLICATE: "request id is live already",
+          UNKNOWN: "no live request has this id", OUT_OF_PAGES: "out of pages",
+          BAD_ARGUMENT: "bad argument", CORRUPT: "bookkeeping is corrupt"}
+
+
+class CacheError(RuntimeError):
+    def __init__(self, code, what):
+        self.code = code
+        super().__init__(f"{what}: {_NAMES.get(code, code)}")
+
+
+class OutOfPages(CacheError):
+    pass
+
+
+@dataclass(frozen=True)
+class GroupLayout:
+    kind: int            # PAGED or STATE
+    n_pages: int = 0
+    page_size: int = 1
+    window: int = 0      # 0: all keys are kept
+
+
+_host = None
+
+
+def host_library():
+    global _host
+    if _host is None:
+        lib = load_library("host")
+        I, L, P = c_int, c_int64, c_void_p
+        IP = POINTER(c_int)
+        sig = {
+            "dn_cache_create": (P, [I, IP, IP, IP, IP, I]), "dn_cache_destroy": (None, [P]),
+            "dn_cache_add": (I, [P, L]), "dn_cache_release": (I, [P, L]), "dn_cache_reserve": (I, [P, L, I]),
+            "dn_cache_commit": (I, [P, L, I]), "dn_cache_length": (I, [P, L]), "dn_cache_slot": (I, [P, L]),
+            "dn_cache_generation": (L, [P, I]), "dn_cache_block_table": (I, [P, L, I, c_void_p, I]),
+            "dn_cache_blocks": (I, [P, L, I]), "dn_cache_free_pages": (I, [P, I]),
+            "dn_cache_pages_held": (I, [P, L, I]), "dn_cache_pages_needed": (I, [P, L, I, I, I]),
+            "dn_cache_pages_peak": (I, [P, I, I, I]), "dn_cache_live": (I, [P]), "dn_cache_check": (I, [P]),
+            "dn_cache_reuse_count": (L, [P, I]),
+            "dn_sched_create": (P, [P, I, I, I, I, I]), "dn_sched_destroy": (None, [P]),
+            "dn_sched_add": (I, [P, L, I, I]),
+            "dn_sched_schedule": (I, [P, c_void_p, c_void_p, c_void_p, c_void_p, I, c_void_p, IP, I]),
+            "dn_sched_step_done": (I, [P, L, I]), "dn_sched_token_sampled": (I, [P, L]),
+            "dn_sched_finish": (I, [P, L]), "dn_sched_n_waiting": (I, [P]), "dn_sched_n_running": (I, [P]),
+            "dn_sched_known": (I, [P, L]), "dn_sched_computed": (I, [P, L]), "dn_sched_generated": (I, [P, L]),
+        }
+        for name, (res, args) in sig.items():
+            f = getattr(lib, name)
+            f.restype, f.argtypes = res, args
+        _host = lib
+    return _host
+
+
+class CacheManager:
+    def __init__(self, groups: Sequence[GroupLayout], max_requests: int):
+        self.groups = list(groups)
+        self.max_requests = max_requests
+        self._lib = host_library()
+        n = len(self.groups)
+        arr = lambda vals: (c_int * max(n, 1))(*vals)   # noqa: E731
+        self._h = self._lib.dn_cache_create(
+            n, arr([g.kind for g in self.groups]), arr([g.n_pages for g in self.groups]),
+            arr([g.page_size for g in self.groups]), arr([g.window for g in self.groups]), max_requests)
+        if not self._h:
+            raise ValueError(f"cache manager: bad layout {self.groups} for {max_requests} requests")
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.dn_cache_destroy(self._h)
+            self._h = None
+
+    def _chk(self, rc, what):
+        if rc < 0:
+            raise (OutOfPages if rc == OUT_OF_PAGES else CacheError)(rc, what)
+        return rc
+
+    def add(self, rid: int) -> int:
+        """-> the request's slot (index into per-request state tensors)."""
+        return self._chk(self._lib.dn_cache_add(self._h, rid), f"add request {rid}")
+
+    def release(self, rid: int) -> bool:
+        """Gives back the request's pages and slot.  A stale release (unknown id) changes nothing
+        and returns False, as a release with an old lease does in the reference
+        (crates/denno-engine/src/engine.rs:751-754)."""
+        rc = self._lib.dn_cache_release(self._h, rid)
+        if rc == UNKNOWN:
+            return False
+        self._chk(rc, f"release request {rid}")
+        return True
+
+    def reserve(self, rid: int, new_len: int):
+        """Pages for positions up to new_len in every paged group; raises OutOfPages and
+        changes nothing if any pool is short."""
+        self._chk(self._lib.dn_cache_reserve(self._h, rid, new_len), f"reserve {new_len} tokens for request {rid}")
+
+    def try_reserve(self, rid: int, new_len: int) -> bool:
+        rc = self._lib.dn_cache_reserve(self._h, rid, new_len)
+        if rc == OUT_OF_PAGES:
+            return False
+        self._chk(rc, f"reserve {new_len} tokens for request {rid}")
+        return True
+
+    def commit(self, rid: int, new_len: int):
+        self._chk(self._lib.dn_cache_commit(self._h, rid, new_len), f"commit {new_len} tokens of request {rid}")
+
+    def length(self, rid: int) -> int:
+        return self._chk(self._lib.dn_cache_length(self._h, rid), f"length of request {rid}")
+
+    def has(self, rid: int) -> bool:
+        return self._lib.dn_cache_length(self._h, rid) >= 0
+
+    def slot(self, rid: int) -> int:
+        return self._chk(self._lib.dn_cache_slot(self._h, rid), f"slot of request {rid}")
+
+    def generation(self, slot: int) -> int:
+        return self._lib.dn_cache_generation(self._h, slot)
+
+    def block_table(self, rid: int, group: int) -> np.ndarray:
+        n = self._chk(self._lib.dn_cache_blocks(self._h, rid, group), f"block table of request {rid}")
+        out = np.empty(max(n, 1), dtype=np.int32)
+        self._chk(self._lib.dn_cache_block_table(self._h, rid, group, out.ctypes.data, n), "block table")
+        return out[:n]
+
+    def free_pages(self, group: int) -> int:
+        return self._chk(self._lib.dn_cache_free_pages(self._h, group), "free pages")
+
+    def pages_held(self, rid: int, group: int) -> int:
+        return self._chk(self._lib.dn_cache_pages_held(self._h, rid, group), "pages held")
+
+    def pages_peak(self, group: int, total_len: int, chunk: int) -> int:
+        return self._lib.dn_cache_pages_peak(self._h, group, total_len, chunk)
+
+    def live(self) -> int:
+        return self._lib.dn_cache_live(self._h)
+
+    def reuse_count(self, group: int) -> int:
+        """Pages handed out that some request had held before."""
+        return self._lib.dn_cache_reuse_count(self._h, group)
+
+    def check(self):
+        """Raises if a page or slot is lost, held twice, or both free and held."""
+        self._chk(self._lib.dn_cache_check(self._h), "cache check")

@@ -1,0 +1,158 @@
+// Embedding, LayerNorm, cache write, casts: the memory-bound, row-wise kernels.
+// The residual stream is 32-bit in both precisions; LayerNorm's statistics and affine are
+// 32-bit; only what feeds a matrix product is rounded to bfloat16.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------
+// x[t,:] = wte[token_t,:] + wpe[pos_t,:]      (crates/denno-engine/src/model/gpt2.rs:142-150)
+// wpe may be null (an architecture whose positions enter elsewhere).
+// ---------------------------------------------------------------------------------------
+template <typename TW>
+__global__ void embed_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ positions,
+                             const TW* __restrict__ wte, const TW* __restrict__ wpe, float* __restrict__ x,
+                             int T, int E, int vocab, int n_pos) {
+  int t = blockIdx.x;
+  if (t >= T) return;
+  int tok = tokens[t];
+  int pos = positions[t];
+  bool ok = tok >= 0 && tok < vocab && (wpe == nullptr || (pos >= 0 && pos < n_pos));
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    float v = __uint_as_float(0x7fc00000u);   // an id outside the table: NaN, never a neighbour's row
+    if (ok) {
+      v = to_float(wte[static_cast<size_t>(tok) * E + e]);
+      if (wpe != nullptr) v += to_float(wpe[static_cast<size_t>(pos) * E + e]);
+    }
+    x[static_cast<size_t>(t) * E + e] = v;
+  }
+}
+
+extern "C" int dn_embed(const int32_t* tokens, const int32_t* positions, const void* wte, const void* wpe,
+                        float* x, int T, int E, int vocab, int n_pos, int table_dtype, hipStream_t stream) {
+  if (T <= 0) return 0;
+  dim3 grid(T), block(256);
+  if (table_dtype == DN_F32)
+    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, tokens, positions,
+                       static_cast<const float*>(wte), static_cast<const float*>(wpe), x, T, E, vocab, n_pos);
+  else if (table_dtype == DN_BF16)
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, tokens, positions,
+                       static_cast<const bf16_t*>(wte), static_cast<const bf16_t*>(wpe), x, T, E, vocab, n_pos);
+  else
+    return DN_ERR_DTYPE;
+  return dn_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// LayerNorm of selected rows: mean, biased variance of (x - mean), then affine
+// (crates/denno-engine/src/tensor.rs:1101-1112).  One wave per row; the row is read three
+// times (it stays in cache), so any width works.  rows == null: row r of the output is
+// row r of x.
+// ---------------------------------------------------------------------------------------
+template <typename TO>
+__global__ void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
+                                 const float* __restrict__ beta, TO* __restrict__ out,
+                                 const int32_t* __restrict__ rows, int R, int E, float eps) {
+  int wave = threadIdx.x / DN_WAVE, lane = threadIdx.x % DN_WAVE;
+  int r = blockIdx.x * (blockDim.x / DN_WAVE) + wave;
+  if (r >= R) return;
+  int src = rows ? rows[r] : r;
+  const float* xr = x + static_cast<size_t>(src) * E;
+  float s = 0.f;
+  for (int e = lane; e < E; e += DN_WAVE) s += xr[e];
+  float mean = wave_sum(s) / static_cast<float>(E);
+  float v = 0.f;
+  for (int e = lane; e < E; e += DN_WAVE) {
+    float d = xr[e] - mean;
+    v += d * d;
+  }
+  float inv = 1.0f / sqrtf(wave_sum(v) / static_cast<float>(E) + eps);
+  TO* o = out + static_cast<size_t>(r) * E;
+  for (int e = lane; e < E; e += DN_WAVE) {
+    float y = (xr[e] - mean) * inv * gamma[e];
+    if (beta) y += beta[e];
+    o[e] = from_float<TO>(y);
+  }
+}
+
+extern "C" int dn_layernorm(const float* x, const float* gamma, const float* beta, void* out, const int32_t* rows,
+                            int R, int E, float eps, int out_dtype, hipStream_t stream) {
+  if (R <= 0) return 0;
+  const int waves = 4;
+  dim3 grid((R + waves - 1) / waves), block(waves * DN_WAVE);
+  if (out_dtype == DN_F32)
+    hipLaunchKernelGGL(layernorm_kernel<float>, grid, block, 0, stream, x, gamma, beta, static_cast<float*>(out),
+                       rows, R, E, eps);
+  else if (out_dtype == DN_BF16)
+    hipLaunchKernelGGL(layernorm_kernel<bf16_t>, grid, block, 0, stream, x, gamma, beta,
+                       static_cast<bf16_t*>(out), rows, R, E, eps);
+  else
+    return DN_ERR_DTYPE;
+  return dn_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// Keys and values of this step's tokens go to their pages before attention reads them
+// (crates/denno-engine/src/model/gpt2.rs:159-167).  src is [T, ld]; keys are columns
+// k_col .. k_col + Hkv*dh, values v_col .. ; slot_map[t] = page * page_size + offset, or < 0
+// for a row that is padding.  A pool is [n_pages, Hkv, page_size, dh].
+// ---------------------------------------------------------------------------------------
+template <typename TS>
+__global__ void kv_write_kernel(const TS* __restrict__ src, int ld, int k_col, int v_col,
+                                const int32_t* __restrict__ slot_map, TS* __restrict__ k_pool,
+                                TS* __restrict__ v_pool, int T, int Hkv, int dh, int page_size) {
+  int t = blockIdx.x;
+  if (t >= T) return;
+  int slot = slot_map[t];
+  if (slot < 0) return;
+  int page = slot / page_size, off = slot % page_size;
+  int width = Hkv * dh;
+  const TS* row = src + static_cast<size_t>(t) * ld;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    int h = c / dh, d = c % dh;
+    size_t dst = ((static_cast<size_t>(page) * Hkv + h) * page_size + off) * dh + d;
+    k_pool[dst] = row[k_col + c];
+    v_pool[dst] = row[v_col + c];
+  }
+}
+
+extern "C" int dn_kv_write(const void* src, int ld, int k_col, int v_col, const int32_t* slot_map, void* k_pool,
+                           void* v_pool, int T, int Hkv, int dh, int page_size, int dtype, hipStream_t stream) {
+  if (T <= 0) return 0;
+  dim3 grid(T), block(256);
+  if (dtype == DN_F32)
+    hipLaunchKernelGGL(kv_write_kernel<float>, grid, block, 0, stream, static_cast<const float*>(src), ld, k_col,
+                       v_col, slot_map, static_cast<float*>(k_pool), static_cast<float*>(v_pool), T, Hkv, dh,
+                       page_size);
+  else if (dtype == DN_BF16)
+    hipLaunchKernelGGL(kv_write_kernel<bf16_t>, grid, block, 0, stream, static_cast<const bf16_t*>(src), ld,
+                       k_col, v_col, slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), T, Hkv,
+                       dh, page_size);
+  else
+    return DN_ERR_DTYPE;
+  return dn_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// Element-wise conversion between the two precisions (rows of a matrix product whose
+// weight is held in the other precision).
+// ---------------------------------------------------------------------------------------
+template <typename TI, typename TO>
+__global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, size_t n) {
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (; i < n; i += stride) out[i] = from_float<TO>(to_float(in[i]));
+}
+
+extern "C" int dn_cast(const void* in, void* out, long long n, int in_dtype, int out_dtype, hipStream_t stream) {
+  if (n <= 0) return 0;
+  size_t blocks = (static_cast<size_t>(n) + 255) / 256;
+  dim3 grid(static_cast<unsigned>(blocks < 4096 ? blocks : 4096)), block(256);
+  if (in_dtype == DN_BF16 && out_dtype == DN_F32)
+    hipLaunchKernelGGL((cast_kernel<bf16_t, float>), grid, block, 0, stream, static_cast<const bf16_t*>(in),
+                       static_cast<float*>(out), static_cast<size_t>(n));
+  else if (in_dtype == DN_F32 && out_dtype == DN_BF16)
+    hipLaunchKernelGGL((cast_kernel<float, bf16_t>), grid, block, 0, stream, static_cast<const float*>(in),
+                       static_cast<bf16_t*>(out), static_cast<size_t>(n));
+  else
+    return DN_ERR_DTYPE;
+  return dn_launch_status();
+}

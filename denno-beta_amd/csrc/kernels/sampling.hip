@@ -1,0 +1,202 @@
+// Sampling from rows of 32-bit logits, after the reference's sampler
+// (crates/denno-engine/src/sampler.rs): greedy is the first maximum with NaN ignored
+// (:301-331, 350-367); with a temperature, z = logit/T, e_i = exp(z_i - max z), and the
+// token is the first i whose running sum of e reaches u * sum(e), walking i upwards
+// (:440-463); the last index if rounding leaves none.  The uniform number u comes from the
+// request's own generator on the host, so a request's tokens do not depend on the batch.
+//
+// The penalties before sampling (sampler.rs:42-58, 99-118, 150-172, order :164-179) are one
+// kernel over each row's context.  No reduction here uses atomics.
+#include "common.h"
+
+#include <math.h>
+
+namespace sampling {
+constexpr int THREADS = 1024;
+constexpr int WAVES = THREADS / DN_WAVE;
+
+struct Best {
+  float v;
+  int i;
+};
+__device__ __forceinline__ Best better(Best a, Best b) {
+  // the larger value; of equal values the lower index.  NaN never compares greater.
+  if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
+  return a;
+}
+
+__device__ Best block_best(Best x, Best* scratch) {
+#pragma unroll
+  for (int m = DN_WAVE / 2; m >= 1; m >>= 1) {
+    Best o{__shfl_xor(x.v, m, DN_WAVE), __shfl_xor(x.i, m, DN_WAVE)};
+    x = better(x, o);
+  }
+  int wave = threadIdx.x / DN_WAVE, lane = threadIdx.x % DN_WAVE;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = x;
+  __syncthreads();
+  Best r = scratch[0];
+  for (int w = 1; w < WAVES; ++w) r = better(r, scratch[w]);
+  return r;
+}
+
+__device__ float block_max(float x, float* scratch) {
+  x = wave_max(x);
+  int wave = threadIdx.x / DN_WAVE, lane = threadIdx.x % DN_WAVE;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = x;
+  __syncthreads();
+  float r = scratch[0];
+  for (int w = 1; w < WAVES; ++w) r = fmaxf(r, scratch[w]);
+  return r;
+}
+
+__global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict__ logits, int ld, int V,
+                                                          const float* __restrict__ temperature,
+                                                          const float* __restrict__ uniform,
+                                                          int32_t* __restrict__ out) {
+  __shared__ Best best_scratch[WAVES];
+  __shared__ float f_scratch[WAVES];
+  __shared__ float seg_sum[THREADS];
+  __shared__ int winner;
+  __shared__ float winner_base, target_s;
+  const int r = blockIdx.x, t = threadIdx.x;
+  const float* row = logits + static_cast<size_t>(r) * ld;
+  const float T = temperature[r];
+
+  if (!(T > 0.f)) {
+    Best b{-INFINITY, 0x7fffffff};
+    for (int i = t; i < V; i += THREADS) {
+      float v = row[i];
+      if (v > b.v) b = Best{v, i};
+    }
+    b = block_best(b, best_scratch);
+    if (t == 0) out[r] = b.i == 0x7fffffff ? 0 : b.i;
+    return;
+  }
+
+  // contiguous segments, so that the walk goes upwards through the vocabulary
+  const int seg = (V + THREADS - 1) / THREADS;
+  const int lo = min(V, t * seg), hi = min(V, lo + seg);
+  float mx = -INFINITY;
+  for (int i = lo; i < hi; ++i) {
+    float z = row[i] / T;
+    if (z > mx) mx = z;
+  }
+  mx = block_max(mx, f_scratch);
+  float s = 0.f;
+  for (int i = lo; i < hi; ++i) s += expf(row[i] / T - mx);
+  seg_sum[t] = s;
+  __syncthreads();
+  if (t == 0) {
+    float total = 0.f;
+    for (int k = 0; k < THREADS; ++k) total += seg_sum[k];
+    float target = uniform[r] * total;
+    float run = 0.f;
+    int w = -1;
+    float base = 0.f;
+    for (int k = 0; k < THREADS; ++k) {
+      float next = run + seg_sum[k];
+      if (w < 0 && next >= target && min(V, k * seg) < V) {
+        w = k;
+        base = run;
+      }
+      run = next;
+    }
+    winner = w;
+    winner_base = base;
+    target_s = target;
+  }
+  __syncthreads();
+  if (winner < 0) {
+    if (t == 0) out[r] = V - 1;
+    return;
+  }
+  if (t == winner) {
+    float u = target_s - winner_base;
+    int pick = hi - 1;
+    for (int i = lo; i < hi; ++i) {
+      u -= expf(row[i] / T - mx);
+      if (u <= 0.f) {
+        pick = i;
+        break;
+      }
+    }
+    out[r] = pick;
+  }
+}
+
+// One workgroup per row.  ctx holds the rows' contexts (prompt + generated) one after the
+// other; row r's is ctx[ctx_start[r] .. ctx_start[r+1]).  Each distinct token is handled by
+// the thread that holds its first occurrence, so no two threads write one logit in a phase.
+__global__ __launch_bounds__(THREADS) void penalties_kernel(float* __restrict__ logits, int ld, int V,
+                                                             const int32_t* __restrict__ ctx,
+                                                             const int32_t* __restrict__ ctx_start,
+                                                             const float* __restrict__ repetition,
+                                                             const float* __restrict__ frequency,
+                                                             const float* __restrict__ presence,
+                                                             const int32_t* __restrict__ ngram) {
+  const int r = blockIdx.x;
+  float* row = logits + static_cast<size_t>(r) * ld;
+  const int32_t* c = ctx + ctx_start[r];
+  const int n = ctx_start[r + 1] - ctx_start[r];
+  const float rep = repetition[r], fq = frequency[r], pr = presence[r];
+  const int ng = ngram[r];
+  if (rep != 1.0f || fq != 0.f || pr != 0.f) {
+    for (int i = threadIdx.x; i < n; i += THREADS) {
+      int tok = c[i];
+      if (tok < 0 || tok >= V) continue;
+      bool first = true;
+      int count = 0;
+      for (int j = 0; j < n; ++j) {
+        if (c[j] == tok) {
+          if (j < i) {
+            first = false;
+            break;
+          }
+          count += 1;
+        }
+      }
+      if (!first) continue;
+      float l = row[tok];
+      if (rep != 1.0f) l = l > 0.f ? l / rep : l * rep;
+      float sub = 0.f;
+      if (fq != 0.f) sub += fq * static_cast<float>(count);
+      if (pr != 0.f) sub += pr;
+      if (sub != 0.f) l -= sub;
+      row[tok] = l;
+    }
+  }
+  __syncthreads();
+  if (ng > 1 && n >= ng) {
+    const int32_t* prefix = c + n - (ng - 1);
+    for (int i = threadIdx.x; i <= n - ng; i += THREADS) {
+      bool same = true;
+      for (int k = 0; k < ng - 1 && same; ++k) same = c[i + k] == prefix[k];
+      if (same) {
+        int f = c[i + ng - 1];
+        if (f >= 0 && f < V) row[f] = -INFINITY;
+      }
+    }
+  }
+}
+}  // namespace sampling
+
+extern "C" int dn_sample(const float* logits, int ld, int R, int V, const float* temperature, const float* uniform,
+                         int32_t* out, hipStream_t stream) {
+  if (R <= 0) return 0;
+  if (V < 1 || ld < V) return DN_ERR_SHAPE;
+  hipLaunchKernelGGL(sampling::sample_kernel, dim3(R), dim3(sampling::THREADS), 0, stream, logits, ld, V,
+                     temperature, uniform, out);
+  return dn_launch_status();
+}
+
+extern "C" int dn_penalties(float* logits, int ld, int R, int V, const int32_t* ctx, const int32_t* ctx_start,
+                            const float* repetition, const float* frequency, const float* presence,
+                            const int32_t* ngram, hipStream_t stream) {
+  if (R <= 0) return 0;
+  if (V < 1 || ld < V) return DN_ERR_SHAPE;
+  hipLaunchKernelGGL(sampling::penalties_kernel, dim3(R), dim3(sampling::THREADS), 0, stream, logits, ld, V, ctx,
+                     ctx_start, repetition, frequency, presence, ngram);
+  return dn_launch_status();
+}

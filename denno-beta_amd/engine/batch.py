@@ -1,0 +1,153 @@
+"""One step's batch: which tokens of which requests run, where they stand, where their keys
+and values go, and which rows' logits are wanted.
+
+All index tables are built on the host as one int32 array and reach the device in one copy.
+The reference's forward takes one request's tokens and its cache
+(crates/denno-engine/src/model/mod.rs:58-59) and its batched form takes one decoded token per
+session (:60-73); here a step takes any mix of both.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+TILE_ROWS = 16   # rows of one request that one attention workgroup takes
+
+
+@dataclass
+class StepEntry:
+    rid: int
+    tokens: Sequence[int]          # the request's next tokens
+    want: Sequence[int] = ()       # places among these tokens whose logits are wanted
+
+
+@dataclass
+class GroupStep:
+    """What one cache group's mixers need for this step."""
+    page_size: int
+    window: int
+    slot_map: Optional[torch.Tensor]       # int32 [T]: page * page_size + offset of each row's key
+    block_tables: Optional[torch.Tensor]   # int32 [S, max_blocks], -1: page given back
+    tiles: Optional[torch.Tensor]          # int32 [4, n_tiles]: request, first row, rows, first position
+
+
+@dataclass
+class StepContext:
+    T: int
+    S: int
+    R: int
+    tokens: torch.Tensor           # int32 [T]
+    positions: torch.Tensor        # int32 [T]
+    logit_rows: torch.Tensor       # int32 [R]
+    state_slots: torch.Tensor      # int32 [S]: each request's slot in the fixed-size state tensors
+    row_start: torch.Tensor        # int32 [S + 1]: request s owns rows row_start[s] .. row_start[s+1]
+    groups: List[Optional[GroupStep]]
+    # the same on the host, for parts that loop over requests
+    host_row_start: List[int] = field(default_factory=list)
+    host_first_pos: List[int] = field(default_factory=list)
+    host_slots: List[int] = field(default_factory=list)
+    rids: List[int] = field(default_factory=list)
+
+
+class BatchError(ValueError):
+    pass
+
+
+def plan_rows(entries: Sequence[StepEntry], starts: Sequence[int], vocab: int, max_positions: int):
+    """Host arrays of the batch: tokens, positions, logit rows, row starts, tiles."""
+    tokens, positions, logit_rows, row_start, tiles = [], [], [], [0], []
+    seen = set()
+    for s, (e, start) in enumerate(zip(entries, starts)):
+        n = len(e.tokens)
+        if n == 0:
+            raise BatchError(f"request {e.rid}: an entry without tokens")
+        if e.rid in seen:
+            raise BatchError(f"request {e.rid} appears twice in one step")
+        seen.add(e.rid)
+        if start + n > max_positions:
+            raise BatchError(f"request {e.rid}: {start} tokens in the cache + {n} exceed the model's "
+                             f"{max_positions} positions")
+        row0 = len(tokens)
+        for t in e.tokens:
+            if not 0 <= int(t) < vocab:
+                raise BatchError(f"request {e.rid}: token id {t} is outside the vocabulary of {vocab}")
+        tokens.extend(int(t) for t in e.tokens)
+        positions.extend(range(start, start + n))
+        for w in e.want:
+            if not 0 <= w < n:
+                raise BatchError(f"request {e.rid}: wanted place {w} is not among its {n} tokens")
+            logit_rows.append(row0 + w)
+        for i in range(0, n, TILE_ROWS):
+            tiles.append((s, row0 + i, min(TILE_ROWS, n - i), start + i))
+        row_start.append(row0 + n)
+    return tokens, positions, logit_rows, row_start, tiles
+
+
+def build_context(entries: Sequence[StepEntry], cache, vocab: int, max_positions: int, device) -> StepContext:
+    """Reserves pages for the entries' tokens (raising cache.OutOfPages; pages taken for
+    earlier entries stay with their requests) and builds the step's tables."""
+    mgr = cache.manager
+    starts = [mgr.length(e.rid) for e in entries]
+    tokens, positions, logit_rows, row_start, tiles = plan_rows(entries, starts, vocab, max_positions)
+    for e, start in zip(entries, starts):
+        mgr.reserve(e.rid, start + len(e.tokens))
+    T, S, R = len(tokens), len(entries), len(logit_rows)
+    slots = [mgr.slot(e.rid) for e in entries]
+
+    parts = [("tokens", np.asarray(tokens, dtype=np.int32)),
+             ("positions", np.asarray(positions, dtype=np.int32)),
+             ("logit_rows", np.asarray(logit_rows, dtype=np.int32)),
+             ("state_slots", np.asarray(slots, dtype=np.int32)),
+             ("row_start", np.asarray(row_start, dtype=np.int32)),
+             ("tiles", np.ascontiguousarray(np.asarray(tiles, dtype=np.int32).T).reshape(-1))]
+    group_meta = []
+    for g, layout in enumerate(cache.layouts):
+        if layout.kind != 0:
+            group_meta.append(None)
+            continue
+        tables = [mgr.block_table(e.rid, g) for e in entries]
+        max_blocks = max(len(t) for t in tables)
+        bt = np.full((S, max_blocks), -1, dtype=np.int32)
+        slot_map = np.full(T, -1, dtype=np.int32)
+        for s, (e, start, tab) in enumerate(zip(entries, starts, tables)):
+            bt[s, :len(tab)] = tab
+            n = len(e.tokens)
+            pos = np.arange(start, start + n)
+            pages = tab[pos // layout.page_size]
+            if (pages < 0).any():
+                raise BatchError(f"request {e.rid}: a token's page was given back already")
+            slot_map[row_start[s]:row_start[s] + n] = pages * layout.page_size + pos % layout.page_size
+        parts.append((f"bt{g}", bt.reshape(-1)))
+        parts.append((f"sm{g}", slot_map))
+        group_meta.append((layout, max_blocks))
+
+    total = sum(a.size for _, a in parts)
+    on_gpu = torch.device(device).type == "cuda"
+    host = torch.empty(total, dtype=torch.int32, pin_memory=on_gpu)
+    hv = host.numpy()
+    offs, o = {}, 0
+    for name, a in parts:
+        hv[o:o + a.size] = a
+        offs[name] = (o, a.size)
+        o += a.size
+    dev = host.to(device, non_blocking=True) if on_gpu else host
+
+    def view(name):
+        b, n = offs[name]
+        return dev[b:b + n]
+    tiles_dev = view("tiles").view(4, -1)
+    groups = []
+    for g, meta in enumerate(group_meta):
+        if meta is None:
+            groups.append(GroupStep(0, 0, None, None, None))
+            continue
+        layout, max_blocks = meta
+        groups.append(GroupStep(layout.page_size, layout.window, view(f"sm{g}"),
+                                view(f"bt{g}").view(S, max_blocks), tiles_dev))
+    return StepContext(
+        T=T, S=S, R=R, tokens=view("tokens"), positions=view("positions"), logit_rows=view("logit_rows"),
+        state_slots=view("state_slots"), row_start=view("row_start"), groups=groups,
+        host_row_start=row_start, host_first_pos=starts, host_slots=slots, rids=[e.rid for e in entries])

@@ -1,0 +1,257 @@
+"""The kernels' Python face: one function per entry point of the HIP libraries.
+
+Every function checks on the host what its kernel and launch assume (device, dtype,
+shape, strides), then passes raw pointers and the current HIP stream.  There is no other
+implementation behind these names: without a GPU or without the built library they raise.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_longlong, c_void_p
+
+import torch
+
+from ..build import load_library
+
+F32, BF16 = 0, 1
+_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+EPILOGUES = {"none": 0, "gelu_tanh": 1, "gelu_erf": 2}
+
+_libs = {}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _lib(name):
+    lib = _libs.get(name)
+    if lib is None:
+        if not torch.cuda.is_available():
+            raise KernelError("the HIP kernels need a GPU (torch.cuda.is_available() is False); "
+                              "there is no CPU path")
+        lib = load_library(name)
+        _declare(name, lib)
+        _libs[name] = lib
+    return lib
+
+
+def _declare(name, lib):
+    P, I, F = c_void_p, c_int, c_float
+    sigs = {
+        "elementwise": {
+            "dn_embed": [P, P, P, P, P, I, I, I, I, I, P],
+            "dn_layernorm": [P, P, P, P, P, I, I, F, I, P],
+            "dn_kv_write": [P, I, I, I, P, P, P, I, I, I, I, I, P],
+            "dn_cast": [P, P, c_longlong, I, I, P],
+        },
+        "gemm": {
+            "dn_gemm": [P, I, P, P, P, I, P, I, I, I, I, I, I, I, P],
+        },
+        "attention": {
+            "dn_attention": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, I, P],
+        },
+        "sampling": {
+            "dn_sample": [P, I, I, I, P, P, P, P],
+            "dn_penalties": [P, I, I, I, P, P, P, P, P, P, P],
+        },
+    }[name]
+    for fn, args in sigs.items():
+        f = getattr(lib, fn)
+        f.argtypes = args
+        f.restype = c_int
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ok(rc, what):
+    if rc != 0:
+        if rc == -1:
+            raise KernelError(f"{what}: unsupported dtype combination")
+        if rc == -2:
+            raise KernelError(f"{what}: the kernel does not take these sizes")
+        raise KernelError(f"{what}: HIP error {rc} at launch")
+
+
+def _need(cond, msg):
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(t, name, dtypes=None, dims=None):
+    _need(isinstance(t, torch.Tensor) and t.is_cuda, f"{name}: must be a tensor on the GPU")
+    if dtypes is not None:
+        _need(t.dtype in dtypes, f"{name}: dtype {t.dtype}, wanted one of {dtypes}")
+    if dims is not None:
+        _need(t.dim() == dims, f"{name}: {t.dim()} dimensions, wanted {dims}")
+    return t
+
+
+def _rows(t, name):
+    """A 2-D tensor whose rows are contiguous; returns its leading dimension."""
+    _need(t.dim() == 2 and (t.shape[1] == 1 or t.stride(1) == 1), f"{name}: rows must be contiguous")
+    ld = t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+    _need(ld >= t.shape[1], f"{name}: rows overlap")
+    return ld
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+_FLOATS = (torch.float32, torch.bfloat16)
+_I32 = (torch.int32,)
+
+
+def embed(tokens, positions, wte, wpe, out):
+    """out[t,:] = wte[tokens[t],:] + wpe[positions[t],:]; wpe may be None.  out is 32-bit."""
+    T = tokens.shape[0]
+    _dev(tokens, "tokens", _I32, 1), _dev(positions, "positions", _I32, 1)
+    _dev(wte, "wte", _FLOATS, 2), _dev(out, "out", (torch.float32,), 2)
+    _need(tokens.is_contiguous() and positions.is_contiguous() and positions.shape[0] == T, "tokens/positions")
+    E = wte.shape[1]
+    _need(wte.is_contiguous() and out.is_contiguous() and tuple(out.shape) == (T, E), "embed: shapes")
+    n_pos = 0
+    if wpe is not None:
+        _dev(wpe, "wpe", (wte.dtype,), 2)
+        _need(wpe.is_contiguous() and wpe.shape[1] == E, "embed: wpe shape")
+        n_pos = wpe.shape[0]
+    _ok(_lib("elementwise").dn_embed(tokens.data_ptr(), positions.data_ptr(), wte.data_ptr(), _ptr(wpe),
+                                     out.data_ptr(), T, E, wte.shape[0], n_pos, _CODE[wte.dtype], _stream()),
+        "embed")
+    return out
+
+
+def layernorm(x, gamma, beta, eps, out, rows=None):
+    """out[r,:] = LayerNorm(x[rows[r],:]) (rows None: every row).  x, gamma, beta are 32-bit."""
+    _dev(x, "x", (torch.float32,), 2), _dev(gamma, "gamma", (torch.float32,), 1), _dev(out, "out", _FLOATS, 2)
+    E = x.shape[1]
+    _need(x.is_contiguous() and out.is_contiguous() and gamma.is_contiguous() and gamma.shape[0] == E,
+          "layernorm: shapes")
+    if beta is not None:
+        _dev(beta, "beta", (torch.float32,), 1)
+        _need(beta.is_contiguous() and beta.shape[0] == E, "layernorm: beta")
+    R = out.shape[0]
+    if rows is not None:
+        _dev(rows, "rows", _I32, 1)
+        _need(rows.is_contiguous() and rows.shape[0] == R, "layernorm: rows")
+    else:
+        _need(R == x.shape[0], "layernorm: out rows")
+    _need(out.shape[1] == E, "layernorm: out width")
+    _ok(_lib("elementwise").dn_layernorm(x.data_ptr(), gamma.data_ptr(), _ptr(beta), out.data_ptr(), _ptr(rows),
+                                         R, E, float(eps), _CODE[out.dtype], _stream()), "layernorm")
+    return out
+
+
+def kv_write(src, k_col, v_col, slot_map, k_pool, v_pool):
+    """Rows of src ([T, ld]; keys at columns k_col.., values at v_col..) go to the slots
+    slot_map[t] = page * page_size + offset of the pools [n_pages, Hkv, page_size, dh]."""
+    _dev(src, "src", _FLOATS, 2), _dev(slot_map, "slot_map", _I32, 1)
+    _dev(k_pool, "k_pool", (src.dtype,), 4), _dev(v_pool, "v_pool", (src.dtype,), 4)
+    ld = _rows(src, "src")
+    T = src.shape[0]
+    n_pages, Hkv, ps, dh = k_pool.shape
+    _need(k_pool.is_contiguous() and v_pool.is_contiguous() and v_pool.shape == k_pool.shape, "kv_write: pools")
+    _need(slot_map.is_contiguous() and slot_map.shape[0] == T, "kv_write: slot_map")
+    w = Hkv * dh
+    _need(0 <= k_col and k_col + w <= src.shape[1] and 0 <= v_col and v_col + w <= src.shape[1],
+          "kv_write: columns outside src")
+    _ok(_lib("elementwise").dn_kv_write(src.data_ptr(), ld, k_col, v_col, slot_map.data_ptr(), k_pool.data_ptr(),
+                                        v_pool.data_ptr(), T, Hkv, dh, ps, _CODE[src.dtype], _stream()),
+        "kv_write")
+
+
+def cast(x, out):
+    _dev(x, "x", _FLOATS), _dev(out, "out", _FLOATS)
+    _need(x.is_contiguous() and out.is_contiguous() and x.numel() == out.numel() and x.dtype != out.dtype, "cast")
+    _ok(_lib("elementwise").dn_cast(x.data_ptr(), out.data_ptr(), x.numel(), _CODE[x.dtype], _CODE[out.dtype],
+                                    _stream()), "cast")
+    return out
+
+
+def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
+    """out = epilogue(a @ w.T + bias), or residual += a @ w.T + bias (32-bit, in place).
+    a: [M, K] rows contiguous; w: [N, K] held [out, in]; bias: 32-bit [N]."""
+    _dev(a, "a", _FLOATS, 2), _dev(w, "w", (a.dtype,), 2)
+    M, K = a.shape
+    N = w.shape[0]
+    _need(w.is_contiguous() and w.shape[1] == K, f"linear: w {tuple(w.shape)} does not fit a {tuple(a.shape)}")
+    _need(K % 8 == 0, f"linear: the inner size {K} must be a multiple of 8")
+    lda = _rows(a, "a")
+    if bias is not None:
+        _dev(bias, "bias", (torch.float32,), 1)
+        _need(bias.is_contiguous() and bias.shape[0] == N, "linear: bias")
+    epi = EPILOGUES[epilogue]
+    if residual is not None:
+        _dev(residual, "residual", (torch.float32,), 2)
+        _need(tuple(residual.shape) == (M, N) and epi == 0 and out is None, "linear: residual")
+        ldr = _rows(residual, "residual")
+        _ok(_lib("gemm").dn_gemm(a.data_ptr(), lda, w.data_ptr(), _ptr(bias), 0, 0, residual.data_ptr(), ldr,
+                                 M, N, K, _CODE[a.dtype], F32, 0, _stream()), "linear")
+        return residual
+    _dev(out, "out", _FLOATS, 2)
+    _need(tuple(out.shape) == (M, N), "linear: out shape")
+    ldc = _rows(out, "out")
+    _ok(_lib("gemm").dn_gemm(a.data_ptr(), lda, w.data_ptr(), _ptr(bias), out.data_ptr(), ldc, 0, 0, M, N, K,
+                             _CODE[a.dtype], _CODE[out.dtype], epi, _stream()), "linear")
+    return out
+
+
+def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, window=0):
+    """Causal attention of the batch's rows over the paged cache.
+
+    q: [T, >= H*dh] rows contiguous, head h at columns h*dh..; out: [T, H*dh];
+    pools: [n_pages, Hkv, page_size, dh]; block_tables: int32 [S, max_blocks];
+    tiles: int32 [4, n_tiles] = (request, first row, rows <= 16, first position), request < 0: padding."""
+    _dev(q, "q", _FLOATS, 2), _dev(out, "out", (q.dtype,), 2)
+    _dev(k_pool, "k_pool", (q.dtype,), 4), _dev(v_pool, "v_pool", (q.dtype,), 4)
+    _dev(block_tables, "block_tables", _I32, 2), _dev(tiles, "tiles", _I32, 2)
+    n_pages, Hkv, ps, dh = k_pool.shape
+    T = q.shape[0]
+    _need(k_pool.is_contiguous() and v_pool.is_contiguous() and v_pool.shape == k_pool.shape, "attention: pools")
+    _need(q.shape[1] >= n_heads * dh and tuple(out.shape) == (T, n_heads * dh), "attention: q/out shapes")
+    _need(block_tables.is_contiguous() and tiles.is_contiguous() and tiles.shape[0] == 4, "attention: tables")
+    _need(dh % 16 == 0 and 16 <= dh <= 256, f"attention: head size {dh} must be a multiple of 16 up to 256")
+    _need(n_heads % Hkv == 0, f"attention: {n_heads} heads over {Hkv} key heads")
+    ldq, ldo = _rows(q, "q"), _rows(out, "out")
+    n_tiles = tiles.shape[1]
+    base = tiles.data_ptr()
+    _ok(_lib("attention").dn_attention(
+        q.data_ptr(), ldq, out.data_ptr(), ldo, k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(),
+        block_tables.shape[1], base, base + 4 * n_tiles, base + 8 * n_tiles, base + 12 * n_tiles, n_tiles,
+        n_heads, Hkv, dh, ps, float(scale), int(window), _CODE[q.dtype], _stream()), "attention")
+    return out
+
+
+def sample(logits, temperature, uniform, out):
+    """out[r] = token of row r: the first maximum if temperature[r] <= 0, else the walk with
+    uniform[r] in [0,1)."""
+    _dev(logits, "logits", (torch.float32,), 2), _dev(temperature, "temperature", (torch.float32,), 1)
+    _dev(uniform, "uniform", (torch.float32,), 1), _dev(out, "out", _I32, 1)
+    R, V = logits.shape
+    ld = _rows(logits, "logits")
+    _need(temperature.shape[0] == R and uniform.shape[0] == R and out.shape[0] == R, "sample: rows")
+    _ok(_lib("sampling").dn_sample(logits.data_ptr(), ld, R, V, temperature.data_ptr(), uniform.data_ptr(),
+                                   out.data_ptr(), _stream()), "sample")
+    return out
+
+
+def penalties(logits, ctx, ctx_start, repetition, frequency, presence, ngram):
+    """In place on logits [R, V]: repetition, frequency, presence penalties and the n-gram ban,
+    each row over its own context ctx[ctx_start[r]:ctx_start[r+1]]."""
+    _dev(logits, "logits", (torch.float32,), 2)
+    R, V = logits.shape
+    ld = _rows(logits, "logits")
+    _dev(ctx, "ctx", _I32, 1), _dev(ctx_start, "ctx_start", _I32, 1)
+    _need(ctx_start.shape[0] == R + 1, "penalties: ctx_start")
+    for t, n in ((repetition, "repetition"), (frequency, "frequency"), (presence, "presence")):
+        _dev(t, n, (torch.float32,), 1)
+        _need(t.shape[0] == R, f"penalties: {n}")
+    _dev(ngram, "ngram", _I32, 1)
+    _need(ngram.shape[0] == R, "penalties: ngram")
+    _ok(_lib("sampling").dn_penalties(logits.data_ptr(), ld, R, V, ctx.data_ptr(), ctx_start.data_ptr(),
+                                      repetition.data_ptr(), frequency.data_ptr(), presence.data_ptr(),
+                                      ngram.data_ptr(), _stream()), "penalties")
+    return logits

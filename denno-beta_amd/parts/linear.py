@@ -1,0 +1,45 @@
+"""Linear: a weight held [out, in] with an optional 32-bit bias, and the call that picks the
+product for its dtype.  A weight that a checkpoint stores [in, out] (Conv1D,
+crates/denno-engine/src/quant.rs:951-953) is transposed once at load (ParamSpec.transpose)."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+from ..weights.spec import ParamSpec
+
+
+class Linear:
+    def __init__(self, in_features: int, out_features: int, weight_name: str, bias_name: Optional[str],
+                 stored_in_out: bool = False, init_std: float = 0.02):
+        self.in_features, self.out_features = in_features, out_features
+        self.weight_name, self.bias_name = weight_name, bias_name
+        self.stored_in_out = stored_in_out
+        self.init_std = init_std
+        self.weight = None
+        self.bias = None
+
+    def param_specs(self):
+        shape = (self.in_features, self.out_features) if self.stored_in_out else (self.out_features, self.in_features)
+        specs = [ParamSpec(self.weight_name, shape, "matrix", ("normal", 0.0, self.init_std),
+                           transpose=self.stored_in_out)]
+        if self.bias_name:
+            specs.append(ParamSpec(self.bias_name, (self.out_features,), "vector", ("normal", 0.0, 0.01)))
+        return specs
+
+    def bind(self, tensors):
+        self.weight = tensors[self.weight_name]
+        self.bias = tensors[self.bias_name] if self.bias_name else None
+
+    def __call__(self, a, out_dtype=None, epilogue="none", residual=None):
+        """epilogue(a @ W^T + b) as a new [M, out] tensor of out_dtype, or added into
+        `residual` (32-bit) in place.  An input in another precision than the weight is
+        converted to the weight's (exact from bfloat16 to 32-bit)."""
+        if a.dtype != self.weight.dtype:
+            a = ops.cast(a.contiguous(), torch.empty(a.shape, dtype=self.weight.dtype, device=a.device))
+        if residual is not None:
+            return ops.linear(a, self.weight, self.bias, residual=residual)
+        out = torch.empty((a.shape[0], self.out_features), dtype=out_dtype or a.dtype, device=a.device)
+        return ops.linear(a, self.weight, self.bias, out=out, epilogue=epilogue)

@@ -1,0 +1,55 @@
+"""Mixers: the parts that let a token see other tokens."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import MIXERS, PagedKV, Part
+from .linear import Linear
+
+
+@MIXERS.register("causal_attention")
+class CausalSelfAttention(Part):
+    """One fused projection to q | k | v, keys and values to the cache, causal softmax
+    attention over the cache, output projection added into the residual stream
+    (crates/denno-engine/src/model/gpt2.rs:155-208).
+
+    n_kv_heads < n_heads: query head h reads key head h // (n_heads // n_kv_heads).
+    window > 0: a query at position p reads keys p - window + 1 .. p only.
+    scale multiplies the scores before the softmax."""
+
+    def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
+                 qkv_weight: str, qkv_bias, out_weight: str, out_bias, stored_in_out: bool = False,
+                 window: int = 0, out_init_std: float = 0.02):
+        self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
+        self.scale, self.window = float(scale), int(window)
+        if n_heads % n_kv_heads != 0:
+            raise ValueError(f"{n_heads} heads cannot share {n_kv_heads} key heads")
+        if head_dim % 16 != 0 or not 16 <= head_dim <= 256:
+            raise ValueError(f"head size {head_dim}: the attention kernels take multiples of 16 up to 256")
+        self.q_width = n_heads * head_dim
+        self.kv_width = n_kv_heads * head_dim
+        self.qkv = Linear(width, self.q_width + 2 * self.kv_width, qkv_weight, qkv_bias, stored_in_out)
+        self.out = Linear(self.q_width, width, out_weight, out_bias, stored_in_out, out_init_std)
+
+    def param_specs(self):
+        return self.qkv.param_specs() + self.out.param_specs()
+
+    def cache_spec(self):
+        return PagedKV(self.n_kv_heads, self.head_dim, self.window)
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        self.qkv.bind(tensors)
+        self.out.bind(tensors)
+
+    def forward(self, h, ctx, cache, accumulate_into):
+        act = self.runtime.act_dtype
+        qkv = self.qkv(h, out_dtype=act)
+        g = ctx.groups[cache.group]
+        if cache.writes:
+            ops.kv_write(qkv, self.q_width, self.q_width + self.kv_width, g.slot_map, cache.k, cache.v)
+        o = torch.empty((h.shape[0], self.q_width), dtype=act, device=h.device)
+        ops.attention(qkv[:, :self.q_width], o, cache.k, cache.v, g.block_tables, g.tiles, self.n_heads,
+                      self.scale, self.window)
+        self.out(o, residual=accumulate_into)

@@ -1,0 +1,34 @@
+"""Norms."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights.spec import ParamSpec
+from .base import NORMS, Part
+
+
+@NORMS.register("layernorm")
+class LayerNorm(Part):
+    """(x - mean) / sqrt(var + eps) * weight + bias, statistics and affine in 32-bit
+    (crates/denno-engine/src/tensor.rs:1101-1112)."""
+
+    def __init__(self, width: int, eps: float, weight_name: str, bias_name=None):
+        self.width, self.eps = width, eps
+        self.weight_name, self.bias_name = weight_name, bias_name
+
+    def param_specs(self):
+        specs = [ParamSpec(self.weight_name, (self.width,), "vector", ("normal", 1.0, 0.02))]
+        if self.bias_name:
+            specs.append(ParamSpec(self.bias_name, (self.width,), "vector", ("normal", 0.0, 0.01)))
+        return specs
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        self.weight = tensors[self.weight_name]
+        self.bias = tensors[self.bias_name] if self.bias_name else None
+
+    def forward(self, x, out_dtype, rows=None):
+        n = x.shape[0] if rows is None else rows.shape[0]
+        out = torch.empty((n, self.width), dtype=out_dtype, device=x.device)
+        return ops.layernorm(x, self.weight, self.bias, self.eps, out, rows)

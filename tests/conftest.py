@@ -1,0 +1,58 @@
+import json
+import os
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+# Two tiny configurations of the architecture that differ in every size and option.
+TINY_A = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n_embd=64, n_head=4,
+              n_inner=256, vocab_size=512, n_positions=128, layer_norm_epsilon=1e-5,
+              activation_function="gelu_new", scale_attn_by_inverse_layer_idx=False)
+TINY_B = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=3, n_embd=96, n_head=2,
+              n_inner=320, vocab_size=1000, n_positions=256, layer_norm_epsilon=1e-6,
+              activation_function="gelu", scale_attn_by_inverse_layer_idx=True)
+# a third, for long sequences and other head sizes: 3 heads of 32, odd vocabulary
+TINY_C = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n_embd=96, n_head=3,
+              n_inner=200, vocab_size=777, n_positions=640, layer_norm_epsilon=1e-5,
+              activation_function="gelu_new", scale_attn_weights=True)
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a GPU (run on the MI355X box)")
+
+
+def pytest_collection_modifyitems(config, items):
+    if torch.cuda.is_available():
+        return
+    skip = pytest.mark.skip(reason="no GPU here")
+    for item in items:
+        if "gpu" in item.keywords:
+            item.add_marker(skip)
+
+
+@pytest.fixture(scope="session")
+def model_folders(tmp_path_factory):
+    """{(name, storage dtype): folder} of random-weight model folders, made on demand."""
+    from denno_beta_amd.weights import write_model_folder
+    made = {}
+
+    def get(name, dtype="float32"):
+        key = (name, dtype)
+        if key not in made:
+            cfg, seed = TINY[name]
+            d = tmp_path_factory.mktemp(f"tiny{name}_{dtype}")
+            write_model_folder(str(d), cfg, seed, dtype)
+            made[key] = str(d)
+        return made[key]
+    return get
+
+
+def seeded_tokens(seed, n, vocab):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()

@@ -1,0 +1,125 @@
+"""Plain PyTorch references of the kernels, one function per entry of
+`denno_beta_amd.kernels.ops`, with the same arguments.  Computation is 32-bit (inputs in
+bfloat16 are widened first); outputs are rounded to the output tensor's dtype once.
+
+They serve two ends: the GPU tests compare each HIP kernel with its reference here, and the
+CPU tests put them in the kernels' place to run the engine's host logic (batching, cache,
+scheduling) without a GPU.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+
+def embed(tokens, positions, wte, wpe, out):
+    x = wte[tokens.long()].float()
+    if wpe is not None:
+        x = x + wpe[positions.long()].float()
+    out.copy_(x)
+    return out
+
+
+def layernorm(x, gamma, beta, eps, out, rows=None):
+    src = x if rows is None else x[rows.long()]
+    mean = src.mean(dim=-1, keepdim=True)
+    d = src - mean
+    var = (d * d).mean(dim=-1, keepdim=True)
+    y = d / torch.sqrt(var + eps) * gamma
+    if beta is not None:
+        y = y + beta
+    out.copy_(y)
+    return out
+
+
+def kv_write(src, k_col, v_col, slot_map, k_pool, v_pool):
+    n_pages, hkv, ps, dh = k_pool.shape
+    w = hkv * dh
+    for t in range(src.shape[0]):
+        slot = int(slot_map[t])
+        if slot < 0:
+            continue
+        page, off = divmod(slot, ps)
+        k_pool[page, :, off, :] = src[t, k_col:k_col + w].view(hkv, dh)
+        v_pool[page, :, off, :] = src[t, v_col:v_col + w].view(hkv, dh)
+
+
+def cast(x, out):
+    out.copy_(x)
+    return out
+
+
+def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
+    y = a.float() @ w.float().t()
+    if bias is not None:
+        y = y + bias
+    if residual is not None:
+        residual += y
+        return residual
+    if epilogue == "gelu_tanh":
+        y = torch.nn.functional.gelu(y, approximate="tanh")
+    elif epilogue == "gelu_erf":
+        y = torch.nn.functional.gelu(y)
+    elif epilogue != "none":
+        raise ValueError(epilogue)
+    out.copy_(y)
+    return out
+
+
+def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, window=0):
+    n_pages, hkv, ps, dh = k_pool.shape
+    group = n_heads // hkv
+    tl = tiles.cpu().tolist()
+    bt = block_tables.cpu()
+    kf, vf = k_pool.float(), v_pool.float()
+    for seq, row0, nrows, pos0 in zip(*tl):
+        if seq < 0:
+            continue
+        for i in range(nrows):
+            pos = pos0 + i
+            lo = max(0, pos - window + 1) if window > 0 else 0
+            keys = torch.arange(lo, pos + 1)
+            pages = bt[seq][keys // ps].long()
+            offs = keys % ps
+            assert (pages >= 0).all(), "attention reads a page that was given back"
+            for h in range(n_heads):
+                k = kf[pages, h // group, offs, :]                  # [n, dh]
+                v = vf[pages, h // group, offs, :]
+                qv = q[row0 + i, h * dh:(h + 1) * dh].float()
+                p = torch.softmax((k @ qv) * scale, dim=0)
+                out[row0 + i, h * dh:(h + 1) * dh] = (p @ v).to(out.dtype)
+    return out
+
+
+def sample(logits, temperature, uniform, out):
+    for r in range(logits.shape[0]):
+        row = logits[r]
+        t = float(temperature[r])
+        if not t > 0:
+            best, best_v = 0, float("-inf")
+            for i, v in enumerate(row.tolist()):
+                if v > best_v:
+                    best, best_v = i, v
+            out[r] = best
+            continue
+        z = row / t
+        e = torch.exp(z - z.max())
+        c = torch.cumsum(e.double(), 0)
+        target = float(uniform[r]) * float(c[-1])
+        idx = int(torch.searchsorted(c, torch.tensor(target, dtype=torch.float64)))
+        out[r] = min(idx, row.shape[0] - 1)
+    return out
+
+
+def penalties(logits, ctx, ctx_start, repetition, frequency, presence, ngram):
+    from plain import sampler_plain as sp
+    cs = ctx_start.tolist()
+    for r in range(logits.shape[0]):
+        c = ctx[cs[r]:cs[r + 1]].tolist()
+        row = logits[r].tolist()
+        row = sp.repetition_penalty(row, c, float(repetition[r]))
+        row = sp.frequency_presence(row, c, float(frequency[r]), float(presence[r]))
+        row = sp.no_repeat_ngram(row, c, int(ngram[r]))
+        logits[r] = torch.tensor(row, dtype=torch.float32)
+    return logits

@@ -90,6 +90,11 @@ class CacheStorage:
                 st[:, slot].zero_()
         return slot
 
+    def reset_states(self, slot: int):
+        for st in self.state:
+            if st is not None:
+                st[:, slot].zero_()
+
     def bytes_per_token(self) -> int:
         total = 0
         for g, cs in enumerate(self.group_specs):

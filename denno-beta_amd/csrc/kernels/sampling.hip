@@ -180,6 +180,177 @@ __global__ __launch_bounds__(THREADS) void penalties_kernel(float* __restrict__ 
     }
   }
 }
+
+// ---------------------------------------------------------------------------------------
+// top-k / top-p (sampler.rs:372-435, 487-514): the m largest of z = logit/T (ties: the lower
+// index first) in descending order, e_i = exp(z_i - z_0); with top-p the list is cut where
+// the running sum of e_i / sum(e) reaches p; then the walk with u * sum(kept e) in that order.
+// m = min(k, 2048, V); with top-p alone m = min(2048, V), the reference's subset (where the
+// reference falls back to a full sort because the 2048 largest do not reach p, the tail
+// beyond them is dropped here).
+// ---------------------------------------------------------------------------------------
+constexpr int CAND = 2048;
+
+__device__ __forceinline__ uint32_t order_key(float z) {
+  if (z != z) return 0u;   // NaN sorts last
+  uint32_t u = __float_as_uint(z);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_value(uint32_t k) {
+  uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+  return __uint_as_float(u);
+}
+
+__global__ __launch_bounds__(THREADS) void sample_top_kernel(const float* __restrict__ logits, int ld, int V,
+                                                              const int32_t* __restrict__ rows,
+                                                              const float* __restrict__ temperature,
+                                                              const float* __restrict__ uniform,
+                                                              const int32_t* __restrict__ top_k,
+                                                              const float* __restrict__ top_p,
+                                                              int32_t* __restrict__ out) {
+  __shared__ uint32_t cand_key[CAND];
+  __shared__ int32_t cand_idx[CAND];
+  __shared__ float cand_e[CAND];
+  __shared__ int hist[256];
+  __shared__ int cnt_gt[THREADS], cnt_eq[THREADS];
+  __shared__ uint32_t sel_prefix;
+  __shared__ int sel_remaining, eq_quota;
+  const int t = threadIdx.x;
+  const int r = rows[blockIdx.x];
+  const float* row = logits + static_cast<size_t>(r) * ld;
+  const float T = temperature[r];
+  int k = top_k[blockIdx.x];
+  const int m = min(min(k > 0 ? k : CAND, CAND), V);
+
+  // 1. the m-th largest key, by four passes over 8 bits each
+  if (t == 0) {
+    sel_prefix = 0u;
+    sel_remaining = m;
+  }
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    if (t < 256) hist[t] = 0;
+    __syncthreads();
+    const uint32_t prefix = sel_prefix;
+    const uint32_t mask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
+    for (int i = t; i < V; i += THREADS) {
+      uint32_t key = order_key(row[i] / T);
+      if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 0xff], 1);
+    }
+    __syncthreads();
+    if (t == 0) {
+      int remaining = sel_remaining;
+      int b = 255;
+      for (; b > 0; --b) {
+        if (hist[b] >= remaining) break;
+        remaining -= hist[b];
+      }
+      sel_prefix = prefix | (static_cast<uint32_t>(b) << shift);
+      sel_remaining = remaining;
+    }
+    __syncthreads();
+  }
+  const uint32_t thr = sel_prefix;
+  if (t == 0) eq_quota = sel_remaining;   // how many keys equal to thr belong to the m
+  // 2. the candidates, in order of their index
+  const int seg = (V + THREADS - 1) / THREADS;
+  const int lo = min(V, t * seg), hi = min(V, lo + seg);
+  int ngt = 0, neq = 0;
+  for (int i = lo; i < hi; ++i) {
+    uint32_t key = order_key(row[i] / T);
+    ngt += key > thr;
+    neq += key == thr;
+  }
+  cnt_gt[t] = ngt;
+  cnt_eq[t] = neq;
+  for (int i = t; i < CAND; i += THREADS) {
+    cand_key[i] = 0u;
+    cand_idx[i] = 0x7fffffff;
+  }
+  __syncthreads();
+  if (t == 0) {
+    int a = 0, b = 0;
+    for (int i = 0; i < THREADS; ++i) {
+      int g = cnt_gt[i], e = cnt_eq[i];
+      cnt_gt[i] = a;
+      cnt_eq[i] = b;
+      a += g;
+      b += e;
+    }
+  }
+  __syncthreads();
+  {
+    const int quota = eq_quota;
+    int eq_rank = cnt_eq[t];
+    int dst = cnt_gt[t] + min(eq_rank, quota);
+    for (int i = lo; i < hi; ++i) {
+      uint32_t key = order_key(row[i] / T);
+      bool take = key > thr;
+      if (key == thr) {
+        take = eq_rank < quota;
+        eq_rank += 1;
+      }
+      if (take) {
+        cand_key[dst] = key;
+        cand_idx[dst] = i;
+        dst += 1;
+      }
+    }
+  }
+  __syncthreads();
+  // 3. bitonic sort: key descending, equal keys by ascending index
+  for (int size = 2; size <= CAND; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      for (int i = t; i < CAND / 2; i += THREADS) {
+        int a = 2 * i - (i & (stride - 1));
+        int b = a + stride;
+        bool descending = (a & size) == 0;
+        uint32_t ka = cand_key[a], kb = cand_key[b];
+        int ia = cand_idx[a], ib = cand_idx[b];
+        bool a_first = ka > kb || (ka == kb && ia < ib);
+        if (a_first != descending) {
+          cand_key[a] = kb;
+          cand_key[b] = ka;
+          cand_idx[a] = ib;
+          cand_idx[b] = ia;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  // 4. softmax numerators, cut, walk: in the list's order, one thread, as the reference does it
+  const float z0 = key_value(cand_key[0]);
+  for (int i = t; i < m; i += THREADS) cand_e[i] = expf(key_value(cand_key[i]) - z0);
+  __syncthreads();
+  if (t == 0) {
+    int keep = m;
+    const float p = top_p[blockIdx.x];
+    if (p < 1.0f) {
+      float total = 0.f;
+      for (int i = 0; i < m; ++i) total += cand_e[i];
+      float cum = 0.f;
+      for (int i = 0; i < m; ++i) {
+        cum += cand_e[i] / total;
+        if (cum >= p) {
+          keep = i + 1;
+          break;
+        }
+      }
+    }
+    float total = 0.f;
+    for (int i = 0; i < keep; ++i) total += cand_e[i];
+    float u = uniform[r] * total;
+    int pick = cand_idx[keep - 1];
+    for (int i = 0; i < keep; ++i) {
+      u -= cand_e[i];
+      if (u <= 0.f) {
+        pick = cand_idx[i];
+        break;
+      }
+    }
+    out[r] = pick;
+  }
+}
 }  // namespace sampling
 
 extern "C" int dn_sample(const float* logits, int ld, int R, int V, const float* temperature, const float* uniform,
@@ -198,5 +369,15 @@ extern "C" int dn_penalties(float* logits, int ld, int R, int V, const int32_t* 
   if (V < 1 || ld < V) return DN_ERR_SHAPE;
   hipLaunchKernelGGL(sampling::penalties_kernel, dim3(R), dim3(sampling::THREADS), 0, stream, logits, ld, V, ctx,
                      ctx_start, repetition, frequency, presence, ngram);
+  return dn_launch_status();
+}
+
+extern "C" int dn_sample_top(const float* logits, int ld, int n_rows, int V, const int32_t* rows,
+                             const float* temperature, const float* uniform, const int32_t* top_k,
+                             const float* top_p, int32_t* out, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (V < 1 || ld < V) return DN_ERR_SHAPE;
+  hipLaunchKernelGGL(sampling::sample_top_kernel, dim3(n_rows), dim3(sampling::THREADS), 0, stream, logits, ld, V,
+                     rows, temperature, uniform, top_k, top_p, out);
   return dn_launch_status();
 }

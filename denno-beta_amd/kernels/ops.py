@@ -54,6 +54,7 @@ def _declare(name, lib):
         "sampling": {
             "dn_sample": [P, I, I, I, P, P, P, P],
             "dn_penalties": [P, I, I, I, P, P, P, P, P, P, P],
+            "dn_sample_top": [P, I, I, I, P, P, P, P, P, P, P],
         },
     }[name]
     for fn, args in sigs.items():
@@ -235,6 +236,25 @@ def sample(logits, temperature, uniform, out):
     _need(temperature.shape[0] == R and uniform.shape[0] == R and out.shape[0] == R, "sample: rows")
     _ok(_lib("sampling").dn_sample(logits.data_ptr(), ld, R, V, temperature.data_ptr(), uniform.data_ptr(),
                                    out.data_ptr(), _stream()), "sample")
+    return out
+
+
+def sample_top(logits, rows, temperature, uniform, top_k, top_p, out):
+    """For the rows listed in `rows` (each with temperature > 0): top_k[j] largest candidates
+    (0: no limit but the 2048 that the kernel keeps), cut at cumulative probability top_p[j]
+    (1: no cut), then the walk with uniform[row].  temperature, uniform and out are indexed by
+    row, top_k and top_p by the place in `rows`."""
+    _dev(logits, "logits", (torch.float32,), 2), _dev(rows, "rows", _I32, 1)
+    _dev(temperature, "temperature", (torch.float32,), 1), _dev(uniform, "uniform", (torch.float32,), 1)
+    _dev(top_k, "top_k", _I32, 1), _dev(top_p, "top_p", (torch.float32,), 1), _dev(out, "out", _I32, 1)
+    R, V = logits.shape
+    ld = _rows(logits, "logits")
+    n = rows.shape[0]
+    _need(top_k.shape[0] == n and top_p.shape[0] == n, "sample_top: one top_k and top_p per listed row")
+    _need(temperature.shape[0] == R and uniform.shape[0] == R and out.shape[0] == R, "sample_top: rows")
+    _ok(_lib("sampling").dn_sample_top(logits.data_ptr(), ld, n, V, rows.data_ptr(), temperature.data_ptr(),
+                                       uniform.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), out.data_ptr(),
+                                       _stream()), "sample_top")
     return out
 
 

@@ -1,0 +1,59 @@
+"""Sampler: from rows of logits to tokens, on the device.
+
+Order, as the reference fixes it (crates/denno-engine/src/sampler.rs:164-179): repetition
+penalty, frequency, presence, n-gram ban, then temperature, top-k, top-p, sample.  Rows of
+one step are sampled together; each row has its own parameters and its own generator.
+"""
+from __future__ import annotations
+
+from typing import List, Sequence
+
+import torch
+
+from ..kernels import ops
+from .params import SamplingParams
+from .rng import uniform
+
+
+class Sampler:
+    def __init__(self, device):
+        self.device = device
+
+    def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
+               counters: Sequence[int], contexts: Sequence[Sequence[int]]) -> List[int]:
+        """logits: [R, V] 32-bit (changed in place by penalties); row r belongs to a request
+        with params[r], the seed seeds[r], counters[r] tokens sampled so far and the tokens
+        contexts[r] (prompt + generated)."""
+        R = logits.shape[0]
+        if R == 0:
+            return []
+        dev = self.device
+        if any(p.has_penalties for p in params):
+            starts, flat = [0], []
+            for p, c in zip(params, contexts):
+                if p.has_penalties:
+                    flat.extend(int(t) for t in c)
+                starts.append(len(flat))
+            f32 = lambda vals: torch.tensor(vals, dtype=torch.float32, device=dev)   # noqa: E731
+            ops.penalties(
+                logits, torch.tensor(flat or [0], dtype=torch.int32, device=dev),
+                torch.tensor(starts, dtype=torch.int32, device=dev),
+                f32([p.repetition_penalty if p.repetition_penalty is not None else 1.0 for p in params]),
+                f32([p.frequency_penalty or 0.0 for p in params]),
+                f32([p.presence_penalty or 0.0 for p in params]),
+                torch.tensor([p.no_repeat_ngram_size or 0 for p in params], dtype=torch.int32, device=dev))
+        temps = [0.0 if p.greedy else p.effective_temperature for p in params]
+        us = [0.0 if p.greedy else uniform(s, n) for p, s, n in zip(params, seeds, counters)]
+        out = torch.empty(R, dtype=torch.int32, device=dev)
+        t_dev = torch.tensor(temps, dtype=torch.float32, device=dev)
+        u_dev = torch.tensor(us, dtype=torch.float32, device=dev)
+        restricted = [r for r, p in enumerate(params)
+                      if not p.greedy and (p.top_k is not None or p.top_p is not None)]
+        ops.sample(logits, t_dev, u_dev, out)
+        if restricted:
+            rows = torch.tensor(restricted, dtype=torch.int32, device=dev)
+            ks = torch.tensor([params[r].top_k or 0 for r in restricted], dtype=torch.int32, device=dev)
+            ps = torch.tensor([params[r].top_p if params[r].top_p is not None else 1.0 for r in restricted],
+                              dtype=torch.float32, device=dev)
+            ops.sample_top(logits, rows, t_dev, u_dev, ks, ps, out)
+        return out.tolist()

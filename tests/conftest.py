@@ -56,3 +56,19 @@ def model_folders(tmp_path_factory):
 def seeded_tokens(seed, n, vocab):
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+BACKENDS = [pytest.param("host", id="host"), pytest.param("gpu", marks=pytest.mark.gpu, id="gpu")]
+
+
+@pytest.fixture(params=BACKENDS)
+def backend(request):
+    """The device the engine runs on.  "gpu": the HIP kernels.  "host": the same engine code on
+    the CPU with the kernels' plain references in their place, so that cache, batch and
+    scheduling logic is tested where there is no GPU."""
+    if request.param == "host":
+        from emulation import emulated_kernels
+        with emulated_kernels():
+            yield "cpu"
+    else:
+        yield "cuda:0"

@@ -123,3 +123,13 @@ def penalties(logits, ctx, ctx_start, repetition, frequency, presence, ngram):
         row = sp.no_repeat_ngram(row, c, int(ngram[r]))
         logits[r] = torch.tensor(row, dtype=torch.float32)
     return logits
+
+
+def sample_top(logits, rows, temperature, uniform, top_k, top_p, out):
+    from plain import sampler_plain as sp
+    for j, r in enumerate(rows.tolist()):
+        k = int(top_k[j]) or 2048
+        p = float(top_p[j])
+        out[r] = sp.top_k_top_p(logits[r].tolist(), float(temperature[r]), min(k, 2048),
+                                None if p >= 1.0 else p, float(uniform[r]))
+    return out

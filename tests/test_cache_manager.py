@@ -1,0 +1,167 @@
+"""The cache manager: no page lost, held twice or freed twice, under any order of requests.
+Unit vectors after the reference's cache tests (crates/denno-engine/src/kv_cache.rs:371-468),
+turned from rows of one buffer into pages of a pool."""
+import random
+
+import pytest
+
+from denno_beta_amd.cache import PAGED, STATE, CacheError, CacheManager, GroupLayout, OutOfPages
+
+
+def mk(n_pages=8, page=16, window=0, max_requests=4, extra=()):
+    return CacheManager([GroupLayout(PAGED, n_pages, page, window), *extra], max_requests)
+
+
+def test_new_cache_is_empty():
+    m = mk()
+    assert m.free_pages(0) == 8 and m.live() == 0
+    m.check()
+
+
+def test_add_reserve_commit_release():
+    m = mk()
+    slot = m.add(7)
+    assert slot == 0 and m.length(7) == 0 and m.block_table(7, 0).tolist() == []
+    m.reserve(7, 17)
+    assert m.block_table(7, 0).tolist() == [0, 1] and m.free_pages(0) == 6
+    m.commit(7, 17)
+    assert m.length(7) == 17
+    m.reserve(7, 32)            # still inside the second page
+    assert m.free_pages(0) == 6
+    m.reserve(7, 33)
+    assert m.block_table(7, 0).tolist() == [0, 1, 2]
+    assert m.release(7) and m.free_pages(0) == 8 and m.live() == 0
+    m.check()
+
+
+def test_commit_needs_pages_and_cannot_shrink():
+    m = mk()
+    m.add(1)
+    with pytest.raises(CacheError):
+        m.commit(1, 5)          # nothing reserved
+    m.reserve(1, 20)
+    m.commit(1, 20)
+    with pytest.raises(CacheError):
+        m.commit(1, 10)
+    with pytest.raises(CacheError):
+        m.reserve(1, 10)
+
+
+def test_out_of_pages_changes_nothing():
+    m = mk(n_pages=4)
+    m.add(1), m.add(2)
+    m.reserve(1, 48)
+    with pytest.raises(OutOfPages):
+        m.reserve(2, 40)        # wants 3, one is free
+    assert m.free_pages(0) == 1 and m.block_table(2, 0).tolist() == []
+    assert not m.try_reserve(2, 17) and m.try_reserve(2, 16)
+    assert m.free_pages(0) == 0
+    m.check()
+
+
+def test_stale_and_double_release_are_no_ops():
+    # crates/denno-engine/src/engine.rs:3445-3479
+    m = mk()
+    m.add(1)
+    m.reserve(1, 30)
+    assert m.release(1) is True
+    assert m.release(1) is False and m.release(99) is False
+    assert m.free_pages(0) == 8
+    m.check()
+
+
+def test_slots_and_generations():
+    m = mk(max_requests=2)
+    a, b = m.add(10), m.add(11)
+    assert {a, b} == {0, 1}
+    with pytest.raises(CacheError, match="slot"):
+        m.add(12)
+    with pytest.raises(CacheError, match="live already"):
+        m.add(10)
+    g = m.generation(a)
+    m.release(10)
+    assert m.add(12) == a and m.generation(a) == g + 1      # the slot is used again, under a new generation
+
+
+def test_freed_pages_are_used_again():
+    m = mk(n_pages=4)
+    m.add(1)
+    m.reserve(1, 64)
+    first = m.block_table(1, 0).tolist()
+    assert m.reuse_count(0) == 0
+    m.release(1)
+    m.add(2)
+    m.reserve(2, 64)
+    assert sorted(m.block_table(2, 0).tolist()) == sorted(first) and m.reuse_count(0) == 4
+
+
+def test_window_gives_pages_back_as_it_passes():
+    m = mk(n_pages=8, page=4, window=6)
+    m.add(1)
+    m.reserve(1, 8)
+    m.commit(1, 8)              # the next query (position 8) reads keys 3..8: block 0 still holds key 3
+    assert m.block_table(1, 0).tolist() == [0, 1] and m.pages_held(1, 0) == 2
+    m.reserve(1, 10)
+    m.commit(1, 10)             # next query reads keys 5..: block 0 (keys 0-3) has passed
+    assert m.block_table(1, 0).tolist() == [-1, 1, 2] and m.free_pages(0) == 6
+    for n in range(11, 40):
+        m.reserve(1, n)
+        m.commit(1, n)
+        assert m.pages_held(1, 0) <= 3
+        m.check()
+    assert m.block_table(1, 0).tolist()[:8] == [-1] * 8
+    m.release(1)
+    assert m.free_pages(0) == 8
+    m.check()
+
+
+def test_groups_have_pools_of_their_own():
+    m = CacheManager([GroupLayout(PAGED, 8, 16, 0), GroupLayout(PAGED, 3, 16, 16), GroupLayout(STATE)], 2)
+    m.add(1)
+    m.reserve(1, 40)
+    assert m.free_pages(0) == 5 and m.free_pages(1) == 0
+    m.add(2)
+    with pytest.raises(OutOfPages):
+        m.reserve(2, 1)         # the windowed pool is empty, so nothing is taken from the other either
+    assert m.free_pages(0) == 5
+    m.commit(1, 40)             # window 16: keys 25.. are read; blocks 0 (0-15) has passed
+    assert m.block_table(1, 1).tolist() == [-1, 1, 2] and m.block_table(1, 0).tolist() == [0, 1, 2]
+    m.reserve(2, 1)
+    m.check()
+    assert m.pages_peak(0, 100, 32) == 7 and m.pages_peak(1, 100, 32) == 4 and m.pages_peak(2, 100, 32) == 0
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_keep_every_page_accounted(seed):
+    rng = random.Random(seed)
+    window = [0, 0, 24, 5, 0, 40][seed]
+    m = CacheManager([GroupLayout(PAGED, 24, 8, 0), GroupLayout(PAGED, 12, 8, window)], 5)
+    live, next_rid = {}, 0
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.25 and len(live) < 5:
+            m.add(next_rid)
+            live[next_rid] = 0
+            next_rid += 1
+        elif op < 0.8 and live:
+            rid = rng.choice(list(live))
+            n = live[rid] + rng.choice([1, 1, 1, 2, 7, 19])
+            if m.try_reserve(rid, n):
+                m.commit(rid, n)
+                live[rid] = n
+                tab = m.block_table(rid, 0).tolist()
+                assert len(tab) == -(-n // 8) and all(p >= 0 for p in tab)
+        elif op < 0.95 and live:
+            rid = rng.choice(list(live))
+            assert m.release(rid)
+            del live[rid]
+        else:
+            assert m.release(next_rid + 1000) is False
+        m.check()
+        held = sum(m.pages_held(r, 0) for r in live)
+        assert held + m.free_pages(0) == 24
+        assert sum(m.pages_held(r, 1) for r in live) + m.free_pages(1) == 12
+    for rid in list(live):
+        m.release(rid)
+    assert m.free_pages(0) == 24 and m.free_pages(1) == 12
+    m.check()

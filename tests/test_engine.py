@@ -1,0 +1,176 @@
+"""The engine above the step function: generation through the entry points, sampling,
+what happens when pages run out, failure of a step."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from conftest import ROOT, TINY, seeded_tokens
+from plain.gpt2_plain import PlainGPT2
+from plain import sampler_plain as SP
+
+
+def engine_for(folder, dtype, device, **kw):
+    from denno_beta_amd.config import EngineOptions
+    from denno_beta_amd.engine import Engine
+    opts = dict(dtype=dtype, device=device, page_size=16, cache_tokens=1024, max_live=4)
+    opts.update(kw)
+    return Engine.from_folder(folder, EngineOptions(**opts))
+
+
+def test_greedy_generation_matches_plain(backend, model_folders):
+    """Tiny A's workload: prompts of 7, 19 and 33 tokens, 16 greedy tokens each, prompts cut
+    into portions of 5 beside the decoding of earlier requests."""
+    from denno_beta_amd.engine import SamplingParams
+    folder = model_folders("A", "float32")
+    plain = PlainGPT2.from_folder(folder)
+    prompts = [seeded_tokens(i, n, 512) for i, n in enumerate((7, 19, 33))]
+    want = [plain.greedy(p, 16) for p in prompts]
+    e = engine_for(folder, "float32", backend, prefill_chunk=5, max_batch_tokens=12)
+    assert e.generate(prompts, SamplingParams(max_tokens=16, temperature=0.0)) == want
+    assert any(r.decode_rows and r.prefill_rows for r in e.records), "no step mixed decoding with a prompt"
+    assert e.runner.cache.manager.live() == 0
+    assert [e.finish_reason(i) for i in range(3)] == ["length"] * 3
+
+
+@pytest.mark.parametrize("policy,cache_tokens", [("preempt", 96), ("reserve", 128)])
+def test_few_pages(backend, model_folders, policy, cache_tokens):
+    """With too few pages for all requests at once the result is the same: under "preempt" the
+    youngest request is recomputed, under "reserve" requests wait their turn."""
+    from denno_beta_amd.engine import SamplingParams
+    folder = model_folders("A", "float32")
+    plain = PlainGPT2.from_folder(folder)
+    prompts = [seeded_tokens(i, n, 512) for i, n in enumerate((7, 19, 33))]
+    want = [plain.greedy(p, 16) for p in prompts]
+    e = engine_for(folder, "float32", backend, cache_tokens=cache_tokens, kv_policy=policy, prefill_chunk=8)
+    assert e.generate(prompts, SamplingParams(max_tokens=16, temperature=0.0)) == want
+    pre = sum(r.preemptions for r in e.requests.values())
+    assert (pre > 0) if policy == "preempt" else (pre == 0)
+    e.runner.cache.manager.check()
+    assert e.runner.cache.manager.free_pages(0) == cache_tokens // 16
+
+
+def test_temperature_sampling_is_seeded_and_independent_of_the_batch(backend, model_folders):
+    """Tiny B's workload, shortened on the host: temperature 0.8, seeded, prompts admitted into
+    a running batch.  A request's tokens are those it gets alone."""
+    from denno_beta_amd.engine import SamplingParams
+    folder = model_folders("B", "float32")
+    lengths = (1, 50, 120, 200) if backend != "cpu" else (1, 20, 45)
+    prompts = [seeded_tokens(20 + i, n, 1000) for i, n in enumerate(lengths)]
+    params = [SamplingParams(max_tokens=24, temperature=0.8, seed=100 + i) for i in range(len(prompts))]
+    alone = []
+    for p, sp in zip(prompts, params):
+        e = engine_for(folder, "float32", backend, prefill_chunk=32)
+        alone.append(e.generate([p], sp)[0])
+    e = engine_for(folder, "float32", backend, prefill_chunk=32, max_batch_tokens=48)
+    rids = [e.add_request(prompts[0], params[0])]
+    for _ in range(3):
+        e.step()
+    rids += [e.add_request(p, sp) for p, sp in zip(prompts[1:], params[1:])]    # into a running batch
+    while e.has_unfinished():
+        e.step()
+    together = [e.requests[r].generated for r in rids]
+    assert together == alone
+    assert len(set(map(tuple, alone))) > 1 and all(len(t) == 24 for t in alone)
+    # and the tokens are what the plain sampler picks from the plain logits with the same numbers
+    from denno_beta_amd.sampling import uniform
+    plain = PlainGPT2.from_folder(folder)
+    seq = list(prompts[1])
+    for n, tok in enumerate(alone[1][:6]):
+        row = plain.logits(seq)[-1]
+        assert SP.temperature_walk(row.tolist(), 0.8, uniform(101, n)) == tok
+        seq.append(tok)
+
+
+def test_top_k_top_p_and_penalties_follow_the_plain_sampler(backend, model_folders):
+    from denno_beta_amd.engine import SamplingParams
+    from denno_beta_amd.sampling import uniform
+    folder = model_folders("A", "float32")
+    plain = PlainGPT2.from_folder(folder)
+    prompt = seeded_tokens(9, 12, 512)
+    sp = SamplingParams(max_tokens=8, temperature=0.9, top_k=5, top_p=0.8, seed=7, repetition_penalty=1.3,
+                        frequency_penalty=0.2, presence_penalty=0.1, no_repeat_ngram_size=2)
+    got = engine_for(folder, "float32", backend).generate([prompt], sp)[0]
+    seq = list(prompt)
+    for n, tok in enumerate(got):
+        row = plain.logits(seq)[-1].tolist()
+        row = SP.repetition_penalty(row, seq, 1.3)
+        row = SP.frequency_presence(row, seq, 0.2, 0.1)
+        row = SP.no_repeat_ngram(row, seq, 2)
+        assert SP.top_k_top_p(row, 0.9, 5, 0.8, uniform(7, n)) == tok, n
+        seq.append(tok)
+
+
+def test_eos_and_max_tokens(backend, model_folders, tmp_path):
+    from denno_beta_amd.engine import SamplingParams
+    from denno_beta_amd.weights import write_model_folder
+    cfg, seed = TINY["A"]
+    folder = model_folders("A", "float32")
+    prompt = seeded_tokens(1, 10, 512)
+    first = engine_for(folder, "float32", backend).generate([prompt], SamplingParams(max_tokens=4, temperature=0.0))[0]
+    # the same weights with the third generated token declared end-of-sequence
+    d = write_model_folder(str(tmp_path / "eos"), dict(cfg, eos_token_id=first[2]), seed)
+    e = engine_for(d, "float32", backend)
+    out = e.generate([prompt], SamplingParams(max_tokens=10, temperature=0.0))[0]
+    stop = first.index(first[2])
+    assert out == first[:stop + 1] and e.finish_reason(0) == "eos"      # the stop token is kept (engine.rs:1125-1129)
+    e = engine_for(d, "float32", backend)
+    assert len(e.generate([prompt], SamplingParams(max_tokens=10, temperature=0.0, ignore_eos=True))[0]) == 10
+    # max_tokens is clamped to the positions left; 0 computes the prompt only
+    e = engine_for(folder, "float32", backend)
+    long_prompt = seeded_tokens(2, 120, 512)
+    assert len(e.generate([long_prompt], SamplingParams(max_tokens=50, temperature=0.0))[0]) == 8
+    assert e.generate([prompt], SamplingParams(max_tokens=0))[0] == [] and e.finish_reason(1) == "length"
+    assert e.runner.cache.manager.live() == 0
+
+
+def test_refused_requests(backend, model_folders):
+    from denno_beta_amd.engine import SamplingParams, SchedulerError
+    e = engine_for(model_folders("A", "float32"), "float32", backend, cache_tokens=64)
+    with pytest.raises(SchedulerError, match="empty"):
+        e.add_request([])
+    with pytest.raises(SchedulerError, match="longer"):
+        e.add_request([1] * 129)
+    with pytest.raises(ValueError, match="vocabulary"):
+        e.add_request([1, 999])
+    with pytest.raises(SchedulerError, match="even alone"):
+        e.add_request([1] * 60, SamplingParams(max_tokens=30))
+    with pytest.raises(ValueError, match="no_repeat_ngram_size"):
+        e.add_request([1], SamplingParams(no_repeat_ngram_size=1))
+    assert not e.has_unfinished()
+
+
+def test_a_failed_step_gives_everything_back(backend, model_folders):
+    """crates/denno-engine/src/engine.rs:3395-3438: a failed prefill releases what it took and the
+    next request runs as on a clean engine."""
+    from denno_beta_amd.engine import SamplingParams
+    folder = model_folders("A", "float32")
+    prompt = seeded_tokens(4, 20, 512)
+    sp = SamplingParams(max_tokens=6, temperature=0.0)
+    clean = engine_for(folder, "float32", backend).generate([prompt], sp)[0]
+    e = engine_for(folder, "float32", backend)
+    rid = e.add_request(prompt, sp)
+    e.fail_next_step = True
+    with pytest.raises(RuntimeError, match="injected"):
+        e.step()
+    assert e.finish_reason(rid) == "error" and not e.has_unfinished()
+    assert e.runner.cache.manager.live() == 0 and e.runner.cache.manager.free_pages(0) == 64
+    e.runner.cache.manager.check()
+    assert e.generate([prompt], sp)[0] == clean
+
+
+def test_command_line(backend, model_folders):
+    """`denno generate` with the reference's option names; greedy, against the plain implementation."""
+    if backend == "cpu":
+        pytest.skip("the command line runs the HIP kernels")
+    folder = model_folders("A", "float32")
+    prompt = seeded_tokens(6, 9, 512)
+    want = PlainGPT2.from_folder(folder).greedy(prompt, 8)
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "denno"), "generate", folder, "--prompt-ids",
+                          ",".join(map(str, prompt)), "--max-tokens", "8", "--temperature", "0", "--quant", "fp32",
+                          "--raw"], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert [int(t) for t in out.stdout.strip().split(",")] == want

@@ -1,0 +1,253 @@
+"""Each HIP kernel alone against its plain PyTorch reference (kernel_refs.py), at sizes other
+than the engine's tiny models: widths and vocabularies that are no power of two, head sizes
+from 16 to 256, grouped key heads, several page sizes."""
+import math
+
+import pytest
+import torch
+
+import kernel_refs as R
+from plain import sampler_plain as SP
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def ops():
+    from denno_beta_amd.kernels import ops as o
+    return o
+
+
+def rnd(*shape, seed=0, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def i32(v):
+    return torch.tensor(v, dtype=torch.int32, device=DEV)
+
+
+TOL = {torch.float32: dict(atol=2e-5, rtol=2e-5), torch.bfloat16: dict(atol=2e-2, rtol=2e-2)}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("E", [40, 1600])
+def test_embed(dtype, E):
+    wte, wpe = rnd(777, E, seed=1, dtype=dtype), rnd(50, E, seed=2, dtype=dtype)
+    tok, pos = i32([0, 776, 5, 5, 300]), i32([0, 49, 7, 8, 1])
+    out = torch.empty(5, E, device=DEV)
+    ops().embed(tok, pos, wte, wpe, out)
+    assert torch.equal(out, R.embed(tok, pos, wte, wpe, torch.empty_like(out)))
+    ops().embed(tok, pos, wte, None, out)
+    assert torch.equal(out, wte[tok.long()].float())
+
+
+@pytest.mark.parametrize("E", [40, 100, 1600])
+def test_layernorm(E):
+    x = rnd(9, E, seed=3, scale=3.0) + 1.5
+    g, b = rnd(E, seed=4), rnd(E, seed=5)
+    for out_dtype in (torch.float32, torch.bfloat16):
+        for rows in (None, i32([8, 0, 3])):
+            n = 9 if rows is None else 3
+            out = torch.empty(n, E, dtype=out_dtype, device=DEV)
+            ops().layernorm(x, g, b, 1e-6, out, rows)
+            want = R.layernorm(x, g, b, 1e-6, torch.empty(n, E, device=DEV), rows)
+            assert torch.allclose(out.float(), want, **TOL[out_dtype])
+    out = torch.empty(9, E, device=DEV)
+    ops().layernorm(x, g, None, 1e-2, out)
+    assert torch.allclose(out, R.layernorm(x, g, None, 1e-2, torch.empty_like(out)), atol=2e-5)
+    # the reference's vector (crates/denno-engine/src/tensor.rs:1706-1718), widened to a kernel-sized row
+    x2 = torch.tensor([[0.0, 2.0] * 8], device=DEV)
+    ops().layernorm(x2, torch.full((16,), 2.0, device=DEV), torch.ones(16, device=DEV), 0.0, out16 := torch.empty(1, 16, device=DEV))
+    assert torch.allclose(out16, torch.tensor([[-1.0, 3.0] * 8], device=DEV), atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_kv_write(dtype):
+    hkv, dh, ps, n_pages = 3, 32, 8, 6
+    src = rnd(7, 5 * hkv * dh, seed=6, dtype=dtype)
+    slots = i32([0, 9, 47, -1, 10, 23, 40])
+    k = torch.zeros(n_pages, hkv, ps, dh, dtype=dtype, device=DEV)
+    v = torch.zeros_like(k)
+    k2, v2 = torch.zeros_like(k), torch.zeros_like(k)
+    ops().kv_write(src, hkv * dh, 3 * hkv * dh, slots, k, v)
+    R.kv_write(src, hkv * dh, 3 * hkv * dh, slots, k2, v2)
+    assert torch.equal(k, k2) and torch.equal(v, v2) and k.abs().sum() > 0
+
+
+@pytest.mark.parametrize("in_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 1001, 72), (5, 64, 8), (130, 200, 320), (64, 1600, 1600), (33, 50257, 96)])
+def test_linear(in_dtype, M, N, K):
+    a, w, bias = rnd(M, K, seed=7, dtype=in_dtype), rnd(N, K, seed=8, dtype=in_dtype, scale=0.2), rnd(N, seed=9)
+    tol = TOL[in_dtype]
+    for out_dtype in (torch.float32, in_dtype):
+        for epi in ("none", "gelu_tanh", "gelu_erf"):
+            out = torch.empty(M, N, dtype=out_dtype, device=DEV)
+            ops().linear(a, w, bias, out=out, epilogue=epi)
+            want = R.linear(a, w, bias, out=torch.empty(M, N, device=DEV), epilogue=epi)
+            assert torch.allclose(out.float(), want, **(TOL[out_dtype] if in_dtype == torch.float32 else tol)), (out_dtype, epi)
+    res = rnd(M, N, seed=10)
+    want = R.linear(a, w, None, residual=res.clone())
+    ops().linear(a, w, None, residual=res)
+    assert torch.allclose(res, want, **tol)
+    # rows taken out of a wider matrix (a leading dimension larger than K)
+    wide = rnd(M, K + 24, seed=11, dtype=in_dtype)
+    out = torch.empty(M, N, device=DEV)
+    ops().linear(wide[:, 8:8 + K], w, bias, out=out)
+    assert torch.allclose(out, R.linear(wide[:, 8:8 + K], w, bias, out=torch.empty_like(out)), **tol)
+
+
+def test_linear_rows_do_not_depend_on_the_batch():
+    a, w = rnd(150, 96, seed=1), rnd(333, 96, seed=2)
+    full = torch.empty(150, 333, device=DEV)
+    ops().linear(a, w, None, out=full)
+    for rows in ([0], [149], [3, 77, 78]):
+        sub = torch.empty(len(rows), 333, device=DEV)
+        ops().linear(a[rows].contiguous(), w, None, out=sub)
+        assert torch.equal(sub, full[rows])
+
+
+def test_linear_refuses_what_it_cannot_take():
+    o = ops()
+    with pytest.raises(o.KernelError, match="multiple of 8"):
+        o.linear(rnd(2, 12), rnd(4, 12), None, out=torch.empty(2, 4, device=DEV))
+    with pytest.raises(o.KernelError, match="does not fit"):
+        o.linear(rnd(2, 16), rnd(4, 24), None, out=torch.empty(2, 4, device=DEV))
+    with pytest.raises(o.KernelError):
+        o.linear(rnd(2, 16), rnd(4, 16, dtype=torch.bfloat16), None, out=torch.empty(2, 4, device=DEV))
+    with pytest.raises(o.KernelError, match="GPU"):
+        o.linear(torch.zeros(2, 16), rnd(4, 16), None, out=torch.empty(2, 4, device=DEV))
+
+
+def paged_case(seq_lens, new_rows, H, Hkv, dh, ps, dtype, seed=0, q_scale=1.0):
+    """A cache filled with random keys and values for requests of the given lengths, scattered
+    over shuffled pages, and the tables of a step in which request s brings new_rows[s] rows."""
+    g = torch.Generator().manual_seed(seed)
+    blocks = [-(-n // ps) for n in seq_lens]
+    n_pages = sum(blocks) + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    k = (torch.randn(n_pages, Hkv, ps, dh, generator=g)).to(dtype).to(DEV)
+    v = (torch.randn(n_pages, Hkv, ps, dh, generator=g)).to(dtype).to(DEV)
+    bt = torch.full((len(seq_lens), max(blocks)), -1, dtype=torch.int32)
+    tiles, row = [], 0
+    for s, (n, new) in enumerate(zip(seq_lens, new_rows)):
+        for b in range(blocks[s]):
+            bt[s, b] = perm.pop()
+        for i in range(0, new, 16):
+            tiles.append((s, row + i, min(16, new - i), n - new + i))
+        row += new
+    q = (torch.randn(row, 3 * H * dh, generator=g) * q_scale).to(dtype).to(DEV)
+    return q, k, v, bt.to(DEV), i32(tiles).t().contiguous(), row
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,Hkv,dh,ps,window", [(4, 4, 16, 16, 0), (25, 25, 64, 16, 0), (6, 2, 48, 8, 0),
+                                                (2, 1, 128, 64, 0), (3, 3, 256, 16, 0), (4, 2, 32, 16, 20),
+                                                (5, 5, 80, 32, 7)])
+def test_attention(dtype, H, Hkv, dh, ps, window):
+    # four requests: a decoded token far into a long context, a whole prompt, a portion, a first token
+    seq_lens, new_rows = [300, 70, 133, 1], [1, 70, 21, 1]
+    q, k, v, bt, tiles, T = paged_case(seq_lens, new_rows, H, Hkv, dh, ps, dtype, seed=H + dh)
+    scale = 1 / math.sqrt(dh)
+    out = torch.zeros(T, H * dh, dtype=dtype, device=DEV)
+    ops().attention(q[:, H * dh:2 * H * dh], out, k, v, bt, tiles, H, scale, window)
+    want = R.attention(q[:, H * dh:2 * H * dh], torch.zeros(T, H * dh, device=DEV), k, v, bt, tiles, H, scale, window)
+    assert torch.allclose(out.float(), want, **TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_finds_a_far_key(dtype):
+    """One key among hundreds matches the query strongly: the output must be its value, whichever
+    page and tile it lies in (the first key, a page's edge, the last key of a tile, the newest)."""
+    H, dh, ps, n = 2, 64, 16, 700
+    for far in (0, 15, 16, 63, 64, 383, 699):
+        q, k, v, bt, tiles, T = paged_case([n], [1], H, H, dh, ps, dtype, seed=far)
+        page, off = int(bt[0, far // ps]), far % ps
+        qh = q[0, :dh].float()
+        k[page, 0, off] = (qh / qh.norm() * 40).to(dtype)       # score 40 |q| against about |q| for the others
+        out = torch.zeros(1, H * dh, dtype=dtype, device=DEV)
+        ops().attention(q[:, :H * dh] , out, k, v, bt, tiles, H, 1.0)
+        assert torch.allclose(out[0, :dh].float(), v[page, 0, off].float(), atol=1e-2 if dtype == torch.bfloat16 else 1e-4), far
+
+
+def test_attention_window_edges():
+    """With values that encode their position, the window's first and last key are seen exactly."""
+    H, dh, ps, n, window = 1, 16, 16, 200, 37
+    q, k, v, bt, tiles, T = paged_case([n], [n], H, H, dh, ps, torch.float32, seed=1)
+    k.zero_()                       # all scores equal: the output is the mean of the values in the window
+    for pos in range(n):
+        v[int(bt[0, pos // ps]), 0, pos % ps] = float(pos)
+    out = torch.zeros(T, dh, device=DEV)
+    ops().attention(q[:, :dh], out, k, v, bt, tiles, H, 1.0, window)
+    for pos in (0, 1, 36, 37, 38, 100, 199):
+        lo = max(0, pos - window + 1)
+        assert abs(out[pos, 0].item() - (lo + pos) / 2) < 1e-3, pos
+
+
+def test_attention_rows_do_not_depend_on_the_batch():
+    H, dh, ps = 4, 32, 16
+    q, k, v, bt, tiles, T = paged_case([200, 90], [50, 90], H, H, dh, ps, torch.float32, seed=2)
+    out = torch.zeros(T, H * dh, device=DEV)
+    ops().attention(q[:, :H * dh], out, k, v, bt, tiles, H, 0.2)
+    # request 0's last row alone, as a decoded token
+    one = torch.zeros(1, H * dh, device=DEV)
+    ops().attention(q[49:50, :H * dh], one, k, v, bt, i32([[0], [0], [1], [199]]), H, 0.2)
+    assert torch.equal(one[0], out[49])
+
+
+def test_sample_greedy_and_walk():
+    V = 50257
+    logits = rnd(6, V, seed=3, scale=2.0)
+    logits[0, 100] = logits[0, 40000] = 50.0            # two maxima: the first wins (sampler.rs:569-582)
+    logits[1, 7] = float("nan")                         # NaN is ignored (sampler.rs:1222-1224)
+    logits[2, :] = float("-inf")                        # nothing is greater than -inf: index 0
+    temp = torch.tensor([0.0, 0.0, 0.0, 0.8, 1.0, 2.5], device=DEV)
+    u = torch.tensor([0.0, 0.0, 0.0, 0.3, 0.999999, 0.5], device=DEV)
+    out = torch.empty(6, dtype=torch.int32, device=DEV)
+    ops().sample(logits, temp, u, out)
+    got = out.tolist()
+    assert got[0] == 100 and got[1] == int(torch.nan_to_num(logits[1], nan=-1e30).argmax()) and got[2] == 0
+    for r in (3, 4, 5):
+        want = SP.temperature_walk(logits[r].tolist(), float(temp[r]), float(u[r]))
+        assert abs(got[r] - want) <= 1 or abs(float(logits[r, got[r]]) - float(logits[r, want])) < 1e-3, r
+    # u = 0 picks the first token
+    ops().sample(logits[3:4], temp[3:4], torch.zeros(1, device=DEV), out[:1])
+    assert out[0].item() == 0
+
+
+def test_sample_frequencies():
+    # [0, 4] at T = 1: index 1 with probability 0.982 (sampler.rs:686-704), here over a row padded with -inf
+    from denno_beta_amd.sampling import uniform
+    n, V = 4000, 333
+    logits = torch.full((n, V), float("-inf"), device=DEV)
+    logits[:, 17], logits[:, 200] = 0.0, 4.0
+    u = torch.tensor([uniform(5, i) for i in range(n)], device=DEV)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    ops().sample(logits, torch.ones(n, device=DEV), u, out)
+    assert set(out.tolist()) == {17, 200}
+    assert abs((out == 200).float().mean().item() - 0.982) < 0.02
+
+
+def test_sample_top_and_penalties():
+    from denno_beta_amd.sampling import uniform
+    V = 1003
+    logits = rnd(8, V, seed=4, scale=3.0)
+    logits[2, 10] = logits[2, 900] = logits[2].max() + 1      # a tie at the top
+    rows = i32([1, 2, 5, 6, 7])
+    ks, ps = i32([5, 1, 0, 40, 2048]), torch.tensor([1.0, 1.0, 0.7, 0.9, 0.3], device=DEV)
+    temp = torch.full((8,), 0.7, device=DEV)
+    for trial in range(5):
+        u = torch.tensor([uniform(trial, i) for i in range(8)], device=DEV)
+        out = torch.full((8,), -1, dtype=torch.int32, device=DEV)
+        ops().sample_top(logits, rows, temp, u, ks, ps, out)
+        want = R.sample_top(logits.cpu(), rows.cpu(), temp.cpu(), u.cpu(), ks.cpu(), ps.cpu(), torch.full((8,), -1, dtype=torch.int32))
+        assert out.tolist() == want.tolist(), trial
+    assert out[2].item() == 10
+    ctx = i32([3, 4, 3, 9, 4, 3] + [7, 8, 7, 8, 7])
+    start = i32([0, 6, 6, 11])
+    l = rnd(3, V, seed=5)
+    want = R.penalties(l.clone().cpu(), ctx.cpu(), start.cpu(), torch.tensor([1.5, 1.0, 1.0]), torch.tensor([0.3, 0.0, 0.0]),
+                       torch.tensor([0.2, 0.0, 0.5]), torch.tensor([0, 0, 2], dtype=torch.int32))
+    ops().penalties(l, ctx, start, torch.tensor([1.5, 1.0, 1.0], device=DEV), torch.tensor([0.3, 0.0, 0.0], device=DEV),
+                    torch.tensor([0.2, 0.0, 0.5], device=DEV), i32([0, 0, 2]))
+    assert torch.allclose(l.cpu(), want, atol=1e-6) and l[2, 8].item() == float("-inf")

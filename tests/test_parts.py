@@ -1,0 +1,265 @@
+"""The parts alone, and what the assembly allows: a layer named twice, a layer that reads
+another layer's cache, and a mixer with state of its own that is defined here, registered,
+built and stepped without a change to the framework's files."""
+import math
+
+import pytest
+import torch
+
+import replay_util as U
+from conftest import TINY, seeded_tokens
+from plain import gpt2_plain as P
+
+
+def options(device, dtype="float32", **kw):
+    from denno_beta_amd.config import EngineOptions
+    o = dict(dtype=dtype, device=device, page_size=16, cache_tokens=256, max_live=4)
+    o.update(kw)
+    return EngineOptions(**o)
+
+
+def gpt2_spec(name, **changes):
+    from denno_beta_amd.config import GPT2Config
+    from denno_beta_amd.models.gpt2 import build_gpt2
+    cfg = dict(TINY[name][0])
+    cfg.update(changes)
+    return cfg, build_gpt2(GPT2Config.from_dict(cfg))
+
+
+def stored(tensors, spec):
+    """{name: tensor in checkpoint layout, CPU 32-bit} from bound tensors (held [out, in])."""
+    out = {}
+    for s in spec.param_specs():
+        t = tensors[s.name].detach().float().cpu()
+        out[s.name] = t.t().contiguous() if s.transpose else t
+    return out
+
+
+def draw(spec, device, seed=3, dtype="float32"):
+    from denno_beta_amd.weights import draw_all
+    return draw_all(spec.param_specs(), seed, engine_dtype=dtype, device=torch.device(device), stored=dtype)
+
+
+# -- each part alone --------------------------------------------------------------------------
+def test_norm_part(backend):
+    from denno_beta_amd.parts import NORMS, Runtime
+    dev = torch.device(backend)
+    n = NORMS.make(("layernorm", dict(width=96, eps=1e-3, weight_name="g", bias_name="b")))
+    assert [(s.name, s.shape, s.role) for s in n.param_specs()] == [("g", (96,), "vector"), ("b", (96,), "vector")]
+    g, b = torch.randn(96, device=dev), torch.randn(96, device=dev)
+    n.bind({"g": g, "b": b}, Runtime(torch.float32, dev))
+    x = torch.randn(7, 96, device=dev) * 2 + 0.5
+    want = P.layer_norm(x.cpu(), g.cpu(), b.cpu(), 1e-3)
+    assert torch.allclose(n.forward(x, torch.float32).cpu(), want, atol=1e-5)
+    rows = torch.tensor([5, 0], dtype=torch.int32, device=dev)
+    assert torch.allclose(n.forward(x, torch.float32, rows=rows).cpu(), want[[5, 0]], atol=1e-5)
+    assert n.forward(x, torch.bfloat16).dtype == torch.bfloat16
+
+
+@pytest.mark.parametrize("act", ["gelu_tanh", "gelu_erf"])
+def test_feed_forward_part(backend, act):
+    from denno_beta_amd.parts import FEED_FORWARDS, Runtime
+    dev = torch.device(backend)
+    f = FEED_FORWARDS.make(("dense_mlp", dict(width=48, inner=136, activation=act, up_weight="u.w", up_bias="u.b",
+                                              down_weight="d.w", down_bias="d.b", stored_in_out=True)))
+    specs = {s.name: s for s in f.param_specs()}
+    assert specs["u.w"].shape == (48, 136) and specs["u.w"].transpose and specs["d.w"].shape == (136, 48)
+    t = {"u.w": torch.randn(136, 48, device=dev) * 0.2, "u.b": torch.randn(136, device=dev) * 0.1,
+         "d.w": torch.randn(48, 136, device=dev) * 0.2, "d.b": torch.randn(48, device=dev) * 0.1}
+    f.bind(t, Runtime(torch.float32, dev))
+    h = torch.randn(9, 48, device=dev)
+    x = torch.randn(9, 48, device=dev)
+    want = x.cpu() + P.mlp_block(h.cpu(), {"mlp.c_fc.weight": t["u.w"].t().cpu(), "mlp.c_fc.bias": t["u.b"].cpu(),
+                                           "mlp.c_proj.weight": t["d.w"].t().cpu(), "mlp.c_proj.bias": t["d.b"].cpu()},
+                                 P.gelu_tanh if act == "gelu_tanh" else P.gelu_erf)
+    f.forward(h, None, accumulate_into=x)
+    assert torch.allclose(x.cpu(), want, atol=2e-5)
+
+
+@pytest.mark.parametrize("heads,kv_heads,dh,window", [(4, 4, 16, 0), (6, 2, 32, 0), (3, 1, 16, 5)])
+def test_attention_mixer_part(backend, heads, kv_heads, dh, window):
+    """The mixer over a real cache, in two portions, against plain attention; grouped key heads
+    and a window are options of the part although GPT-2 uses neither."""
+    from denno_beta_amd.cache import CacheStorage
+    from denno_beta_amd.engine.batch import StepEntry, build_context
+    from denno_beta_amd.parts import MIXERS, Runtime
+    dev = torch.device(backend)
+    E = 64
+    m = MIXERS.make(("causal_attention", dict(width=E, n_heads=heads, n_kv_heads=kv_heads, head_dim=dh, scale=0.3,
+                                              qkv_weight="qkv.w", qkv_bias="qkv.b", out_weight="o.w", out_bias=None,
+                                              window=window)))
+    qw, kw = heads * dh, kv_heads * dh
+    t = {"qkv.w": torch.randn(qw + 2 * kw, E, device=dev) * 0.3, "qkv.b": torch.randn(qw + 2 * kw, device=dev) * 0.1,
+         "o.w": torch.randn(E, qw, device=dev) * 0.2}
+    m.bind(t, Runtime(torch.float32, dev))
+    cache = CacheStorage([m.cache_spec()], kv_dtype=torch.float32, page_size=16, cache_tokens=64, max_live=2,
+                         device=dev)
+    cache.start_request(0)
+    n = 23
+    h = torch.randn(n, E, device=dev)
+    got = torch.zeros(n, E, device=dev)
+    for a, b in ((0, 14), (14, n)):
+        ctx = build_context([StepEntry(0, [0] * (b - a), [])], cache, 10, 64, dev)
+        m.forward(h[a:b].contiguous(), ctx, cache.view(0, True), accumulate_into=got[a:b])
+        cache.manager.commit(0, b)
+    qkv = h.cpu() @ t["qkv.w"].t().cpu() + t["qkv.b"].cpu()
+    q, k, v = qkv[:, :qw], qkv[:, qw:qw + kw], qkv[:, qw + kw:]
+    rep = heads // kv_heads      # query head i reads key head i // rep
+    kx = k.view(n, kv_heads, dh).repeat_interleave(rep, dim=1).reshape(n, qw)
+    vx = v.view(n, kv_heads, dh).repeat_interleave(rep, dim=1).reshape(n, qw)
+    want = P.causal_attention(q, kx, vx, heads, 0.3, window=window or None) @ t["o.w"].t().cpu()
+    assert torch.allclose(got.cpu(), want, atol=2e-5)
+
+
+# -- the order in which layers run is data -----------------------------------------------------
+def test_a_layer_named_twice(backend):
+    from denno_beta_amd.engine import ModelRunner
+    from denno_beta_amd.parts import LayerCall
+    cfg, spec = gpt2_spec("A", n_layer=1)
+    spec.run_order = [LayerCall(0, 0), LayerCall(0, 1)]      # one layer's weights, run twice, a cache each
+    tensors = draw(spec, backend)
+    r = ModelRunner(spec, tensors, options(backend))
+    st = stored(tensors, spec)
+    twice = dict(st)
+    twice.update({k.replace("h.0.", "h.1."): v for k, v in st.items() if k.startswith("h.0.")})
+    plain = P.PlainGPT2(dict(cfg, n_layer=2), twice)
+    seq = seeded_tokens(1, 40, cfg["vocab_size"])
+    got = U.replay(r, U.chunk_trace([seq], sizes=(7, 2, 13)))["r0"]
+    U.assert_close(got, plain.logits(seq), "float32", "a layer run twice")
+    assert len(r.cache.k[0]) == 2       # two caches although there is one layer
+
+
+def test_a_layer_that_reads_another_layers_cache(backend):
+    from denno_beta_amd.engine import ModelRunner
+    from denno_beta_amd.parts import LayerCall
+    cfg, spec = gpt2_spec("A")
+    spec.run_order = [LayerCall(0, 0), LayerCall(1, 0, writes_cache=False)]
+    tensors = draw(spec, backend)
+    r = ModelRunner(spec, tensors, options(backend))
+    assert len(r.cache.k[0]) == 1
+    st = stored(tensors, spec)
+    seq = seeded_tokens(2, 37, cfg["vocab_size"])
+    # plain: layer 1 attends with its own queries over layer 0's keys and values
+    E, H = cfg["n_embd"], cfg["n_head"]
+    scale = 1 / math.sqrt(E // H)
+    lp = lambda i: {k[len(f"h.{i}."):]: v for k, v in st.items() if k.startswith(f"h.{i}.")}   # noqa: E731
+    x = P.embed(torch.tensor(seq), torch.arange(len(seq)), st["wte.weight"], st["wpe.weight"])
+    p0, p1 = lp(0), lp(1)
+    h = P.layer_norm(x, p0["ln_1.weight"], p0["ln_1.bias"], 1e-5)
+    qkv0 = P.linear_in_out(h, p0["attn.c_attn.weight"], p0["attn.c_attn.bias"])
+    k0, v0 = qkv0[:, E:2 * E], qkv0[:, 2 * E:]
+    x = P.block(x, p0, H, scale, 1e-5, P.gelu_tanh)
+    h = P.layer_norm(x, p1["ln_1.weight"], p1["ln_1.bias"], 1e-5)
+    q1 = P.linear_in_out(h, p1["attn.c_attn.weight"], p1["attn.c_attn.bias"])[:, :E]
+    x = x + P.linear_in_out(P.causal_attention(q1, k0, v0, H, scale), p1["attn.c_proj.weight"], p1["attn.c_proj.bias"])
+    x = x + P.mlp_block(P.layer_norm(x, p1["ln_2.weight"], p1["ln_2.bias"], 1e-5), p1, P.gelu_tanh)
+    want = P.head(x, st["ln_f.weight"], st["ln_f.bias"], 1e-5, st["wte.weight"])
+    got = U.replay(r, U.tail_decode_trace([seq], 9))["r0"]
+    U.assert_close(got, want, "float32", "a layer reading another layer's cache")
+
+
+def test_run_order_is_checked():
+    from denno_beta_amd.parts import LayerCall
+    _, spec = gpt2_spec("A")
+    spec.run_order = [LayerCall(0, 0), LayerCall(1, 1, writes_cache=False)]
+    with pytest.raises(ValueError, match="before any call has written"):
+        spec.instantiate()
+    spec.run_order = [LayerCall(0, 0), LayerCall(1, 0)]
+    with pytest.raises(ValueError, match="writes cache 0"):
+        spec.instantiate()
+    spec.run_order = [LayerCall(0, 0), LayerCall(5, 1)]
+    with pytest.raises(ValueError, match="names layer 5"):
+        spec.instantiate()
+
+
+# -- a toy mixer with state of its own ---------------------------------------------------------
+def toy_model(device, mixers):
+    """A decoder whose layers use the given mixer kinds: 'toy_decay' (defined below) or 'attn'."""
+    from denno_beta_amd.parts import DecoderSpec, LayerCall, LayerSpec
+    E = 32
+    layers = []
+    for i, kind in enumerate(mixers):
+        p = f"L{i}."
+        mixer = ("toy_decay", dict(width=E, decay=0.5 + 0.1 * i, weight_name=p + "mix.w")) if kind == "toy_decay" else \
+            ("causal_attention", dict(width=E, n_heads=2, n_kv_heads=2, head_dim=16, scale=0.25, qkv_weight=p + "qkv.w",
+                                      qkv_bias=None, out_weight=p + "o.w", out_bias=None))
+        layers.append(LayerSpec(
+            "pre_norm", ("layernorm", dict(width=E, eps=1e-5, weight_name=p + "n1.g", bias_name=None)), mixer,
+            ("layernorm", dict(width=E, eps=1e-5, weight_name=p + "n2.g", bias_name=None)),
+            ("dense_mlp", dict(width=E, inner=64, activation="gelu_tanh", up_weight=p + "up.w", up_bias=None,
+                               down_weight=p + "down.w", down_bias=None))))
+    return DecoderSpec(vocab=50, width=E, max_positions=128, token_table="tok", position=("none", {}), layers=layers,
+                       run_order=[LayerCall(i, i) for i in range(len(layers))],
+                       final_norm=("layernorm", dict(width=E, eps=1e-5, weight_name="nf.g", bias_name=None)))
+
+
+def register_toy_mixer():
+    from denno_beta_amd.parts import MIXERS, FixedState, Part
+    from denno_beta_amd.weights import ParamSpec
+    if "toy_decay" in MIXERS:
+        return
+
+    @MIXERS.register("toy_decay")
+    class ToyDecayMixer(Part):
+        """s_t = decay * s_(t-1) + h_t ;  out_t = s_t W^T.  Its state is one vector per request,
+        which a portion of a prompt carries on in token order."""
+
+        def __init__(self, width, decay, weight_name):
+            self.width, self.decay, self.weight_name = width, decay, weight_name
+
+        def param_specs(self):
+            return [ParamSpec(self.weight_name, (self.width, self.width), "matrix", ("normal", 0.0, 0.2))]
+
+        def cache_spec(self):
+            return FixedState((self.width,), "float32")
+
+        def bind(self, tensors, runtime):
+            super().bind(tensors, runtime)
+            self.w = tensors[self.weight_name].float()
+
+        def forward(self, h, ctx, cache, accumulate_into):
+            for s, slot in enumerate(ctx.host_slots):
+                a, b = ctx.host_row_start[s], ctx.host_row_start[s + 1]
+                state = cache.state[slot]
+                for t in range(a, b):
+                    state.mul_(self.decay).add_(h[t].float())
+                    accumulate_into[t] += state @ self.w.t()
+
+
+def toy_plain(spec, st, seq):
+    """The toy model on one whole sequence, written out with the plain functions."""
+    x = st["tok"][torch.tensor(seq)]
+    for i, ls in enumerate(spec.layers):
+        p = f"L{i}."
+        h = P.layer_norm(x, st[p + "n1.g"], 0.0, 1e-5)
+        if ls.mixer[0] == "toy_decay":
+            s, out = torch.zeros(x.shape[1]), []
+            for t in range(len(seq)):
+                s = ls.mixer[1]["decay"] * s + h[t]
+                out.append(s @ st[p + "mix.w"].t())
+            x = x + torch.stack(out)
+        else:
+            qkv = h @ st[p + "qkv.w"].t()
+            a = P.causal_attention(qkv[:, :32], qkv[:, 32:64], qkv[:, 64:], 2, 0.25)
+            x = x + a @ st[p + "o.w"].t()
+        h = P.layer_norm(x, st[p + "n2.g"], 0.0, 1e-5)
+        x = x + P.gelu_tanh(h @ st[p + "up.w"].t()) @ st[p + "down.w"].t()
+    return P.layer_norm(x, st["nf.g"], 0.0, 1e-5) @ st["tok"].t()
+
+
+def test_a_toy_mixer_with_state_is_registered_built_and_stepped(backend):
+    from denno_beta_amd.engine import ModelRunner
+    register_toy_mixer()
+    # different mixers in different layers: state, attention, state
+    spec = toy_model(backend, ["toy_decay", "attn", "toy_decay"])
+    tensors = draw(spec, backend)
+    r = ModelRunner(spec, tensors, options(backend, cache_tokens=192))
+    assert r.cache.n_groups == 2 and r.cache.state[0].shape == (2, 4, 32)     # two state caches, four slots
+    st = {k: v.float().cpu() for k, v in tensors.items()}
+    seqs = [seeded_tokens(i, n, 50) for i, n in enumerate((30, 11, 47, 25, 40))]
+    want = [toy_plain(spec, st, s) for s in seqs]
+    for kind, steps in (("whole", U.whole_trace(seqs)), ("mixed", U.mixed_trace(seqs, seed=3))):
+        got = U.replay(r, steps)       # five requests over four slots: a slot is used again and starts at zero
+        for i in range(len(seqs)):
+            U.assert_close(got[f"r{i}"], want[i], "float32", f"toy model, {kind}, request {i}")
+    r.cache.manager.check()

@@ -1,0 +1,122 @@
+"""The same requests replayed in every way of cutting the work, compared with the plain
+implementation: whole; most in one step and the last 32 tokens one by one; portions of
+changing size down to two tokens; mixed, up to four live requests with so few pages that
+they are used again.  In 32-bit and in bfloat16.
+
+Backend "gpu" runs the HIP kernels; backend "host" runs the same engine code on the CPU with
+the kernels' plain references in their place, so the cache and batch logic is tested where
+there is no GPU.
+"""
+import pytest
+import torch
+
+import replay_util as U
+from conftest import TINY, seeded_tokens
+from plain.gpt2_plain import PlainGPT2
+
+def runner_for(folder, dtype, device, cache_tokens, page_size=16, max_live=4):
+    from denno_beta_amd.config import EngineOptions
+    from denno_beta_amd.engine import ModelRunner
+    return ModelRunner.from_folder(folder, EngineOptions(dtype=dtype, device=device, page_size=page_size,
+                                                         cache_tokens=cache_tokens, max_live=max_live))
+
+
+_plain_cache = {}
+
+
+def plain_logits(folder, seqs):
+    out = []
+    for s in seqs:
+        key = (folder, tuple(s))
+        if key not in _plain_cache:
+            _plain_cache[key] = PlainGPT2.from_folder(folder).logits(s)
+        out.append(_plain_cache[key])
+    return out
+
+
+def sequences(name, lengths, seed=11):
+    vocab = TINY[name][0]["vocab_size"]
+    return [seeded_tokens(seed + i, n, vocab) for i, n in enumerate(lengths)]
+
+
+CASES = [("A", "float32", (7, 19, 33, 100)), ("B", "float32", (1, 50, 120, 200)),
+         ("A", "bfloat16", (7, 19, 33, 100)), ("B", "bfloat16", (1, 50, 120, 200))]
+
+
+@pytest.mark.parametrize("name,dtype,lengths", CASES)
+def test_every_cutting_matches_the_plain_implementation(backend, model_folders, name, dtype, lengths):
+    if backend == "cpu" and (dtype == "bfloat16" or name == "B"):
+        lengths = lengths[:3] if name == "A" else (1, 50, 70)    # the host backend is slow
+    folder = model_folders(name, dtype)
+    seqs = sequences(name, lengths)
+    want = plain_logits(folder, seqs)
+    traces = {"whole": U.whole_trace(seqs), "tail": U.tail_decode_trace(seqs, 32),
+              "chunks": U.chunk_trace(seqs), "mixed": U.mixed_trace(seqs, seed=5)}
+    results = {}
+    for kind, steps in traces.items():
+        tokens = U.max_live_tokens(steps)
+        r = runner_for(folder, dtype, backend, cache_tokens=tokens)
+        got = U.replay(r, steps)
+        r.cache.manager.check()
+        assert r.cache.manager.live() == 0 and r.cache.manager.free_pages(0) == -(-tokens // 16)
+        if kind == "mixed":
+            assert r.cache.manager.reuse_count(0) > 0, "the pool was too large: no page was used again"
+        for i in range(len(seqs)):
+            U.assert_close(got[f"r{i}"], want[i], dtype, f"{name} {dtype} {kind} request {i}")
+        results[kind] = got
+    # the same (request, position) agrees across the cuttings: in 32-bit to the last bit, since a
+    # row's sums have one order whatever else is in the batch
+    for kind in ("tail", "chunks", "mixed"):
+        for i in range(len(seqs)):
+            a, b = results["whole"][f"r{i}"], results[kind][f"r{i}"]
+            if dtype == "float32" and backend != "cpu":
+                assert torch.equal(a, b), f"{name} {kind} request {i}: 32-bit logits depend on the cutting"
+            else:
+                U.assert_close(b, a, dtype, f"{name} {dtype} {kind} vs whole, request {i}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(backend, model_folders, dtype):
+    """A sequence decoded token by token from its first token on, across many pages."""
+    n = 60 if backend == "cpu" else 600
+    folder = model_folders("C", dtype)
+    seq = sequences("C", (n,))[0]
+    want = plain_logits(folder, [seq])[0]
+    steps = [{"step": i, "entries": [{"id": "a", "tokens": [t], "want": [0]}], "end": []} for i, t in enumerate(seq)]
+    r = runner_for(folder, dtype, backend, cache_tokens=-(-n // 64) * 64)
+    got = U.replay(r, steps)["a"]
+    U.assert_close(got[:4], want[:4], dtype, "the first tokens")
+    U.assert_close(got, want, dtype, "long decoding")
+
+
+@pytest.mark.parametrize("page_size", [16, 32, 64])
+def test_page_sizes(backend, model_folders, page_size):
+    folder = model_folders("A", "float32")
+    seqs = sequences("A", (70, 45))
+    want = plain_logits(folder, seqs)
+    steps = U.mixed_trace(seqs, seed=2)
+    r = runner_for(folder, "float32", backend, cache_tokens=U.max_live_tokens(steps), page_size=page_size)
+    got = U.replay(r, steps)
+    for i in range(2):
+        U.assert_close(got[f"r{i}"], want[i], "float32", f"page size {page_size} request {i}")
+
+
+def test_step_refuses_what_it_cannot_run(backend, model_folders):
+    from denno_beta_amd.cache import OutOfPages
+    from denno_beta_amd.engine import BatchError, StepEntry
+    r = runner_for(model_folders("A", "float32"), "float32", backend, cache_tokens=64)
+    r.start_request(0)
+    with pytest.raises(BatchError, match="vocabulary"):
+        r.step([StepEntry(0, [5, 512], [0])])
+    with pytest.raises(BatchError, match="positions"):
+        r.step([StepEntry(0, [1] * 129, [])])
+    with pytest.raises(BatchError, match="twice"):
+        r.step([StepEntry(0, [1], []), StepEntry(0, [2], [])])
+    with pytest.raises(BatchError, match="wanted place"):
+        r.step([StepEntry(0, [1, 2], [2])])
+    with pytest.raises(OutOfPages):
+        r.step([StepEntry(0, [1] * 65, [])])
+    # nothing of the refused steps has stayed: the request is still empty and runs
+    assert r.cache.manager.length(0) == 0
+    assert r.step([StepEntry(0, [1, 2, 3], [2])]).shape == (1, 512)
+    assert r.cache.manager.length(0) == 3

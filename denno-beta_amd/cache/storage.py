@@ -2,7 +2,8 @@
 
 Each cache that the model's run order names has a need (PagedKV or FixedState, from its
 mixer).  Caches with the same need form a group: a paged group has one pool of pages,
-[caches, n_pages, Hkv, page_size, dh] for keys and the same for values, and one block table
+[caches, n_pages, Hkv, page_size, dh] for keys and [caches, n_pages, Hkv, dh, page_size] for
+values (a page's values transposed, as attention's second product reads them), and one block table
 per request, shared by the group's caches; a state group has [caches, slots, *shape] and is
 indexed by the request's slot.  Groups with different needs (all keys, a window of them)
 draw from pools of their own.
@@ -54,11 +55,12 @@ class CacheStorage:
             n = len(self.members[g])
             if isinstance(cs, PagedKV):
                 shape = (n, n_pages, cs.n_kv_heads, page_size, cs.head_dim)
+                vshape = (n, n_pages, cs.n_kv_heads, cs.head_dim, page_size)   # a page's values transposed
                 if allocate:
                     # zeros, not empty: a page's unwritten tail is read (masked) by attention,
                     # and must hold numbers, not whatever bits the allocator left
                     self.k.append(torch.zeros(shape, dtype=kv_dtype, device=device))
-                    self.v.append(torch.zeros(shape, dtype=kv_dtype, device=device))
+                    self.v.append(torch.zeros(vshape, dtype=kv_dtype, device=device))
                 else:
                     self.k.append(None), self.v.append(None)
                 self.state.append(None)

@@ -8,7 +8,8 @@
 // length and the softmax is the running ("online") one in 32-bit, so a row's result does not
 // depend on where its portion was cut or on what else is in the batch.
 //
-// A pool is [n_pages, Hkv, page_size, dh]; query head h reads key head h / (H / Hkv).
+// The key pool is [n_pages, Hkv, page_size, dh], the value pool [n_pages, Hkv, dh, page_size];
+// query head h reads key head h / (H / Hkv).
 #include "common.h"
 
 #include <math.h>
@@ -64,9 +65,10 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
       if (key <= last_pos) {
         int page = bt[key / page_size];
         if (page >= 0) {
-          size_t src = ((static_cast<size_t>(page) * Hkv + hk) * page_size + key % page_size) * dh + d;
-          kv = to_float(k_pool[src]);
-          vv = to_float(v_pool[src]);
+          size_t base = (static_cast<size_t>(page) * Hkv + hk) * page_size * dh;
+          int off = key % page_size;
+          kv = to_float(k_pool[base + static_cast<size_t>(off) * dh + d]);
+          vv = to_float(v_pool[base + static_cast<size_t>(d) * page_size + off]);
         }
       }
       Ks[j * (dh + 1) + d] = kv;
@@ -162,5 +164,384 @@ extern "C" int dn_attention(const void* q, int ldq, void* out, int ldo, const vo
                        tile_nrows, tile_pos0, H, Hkv, dh, page_size, BK, scale, window);
   else
     return DN_ERR_DTYPE;
+  return dn_launch_status();
+}
+
+// =======================================================================================
+// bfloat16 kernels.  Both need page_size % 16 == 0 (a run of 16 keys lies in one page).
+// =======================================================================================
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+
+__device__ __forceinline__ __bf16 to_bf16(float f) {
+  bf16_t b = from_float<bf16_t>(f);
+  return __builtin_bit_cast(__bf16, b.bits);
+}
+
+// ---------------------------------------------------------------------------------------
+// flash: portions of prompts.  A workgroup takes up to 128 consecutive rows of one request
+// and one head; each of its 4 waves owns 32 rows and walks the keys in tiles of 32 with
+// v_mfma_f32_32x32x16_bf16, operands straight from the pages (the waves of a workgroup read
+// the same keys at nearly the same time, so they meet in cache).
+//   S^T[key, q] = K . Q^T : lane (key = lane % 32, half g = lane / 32) gives 8 dims of a key.
+//   The result leaves each lane with 16 keys of ONE query (its column), so the running
+//   softmax is lane-local but for one exchange between the halves.
+//   O^T[d, q] += V^T . P^T : the lane's 16 probabilities are, eight by eight, exactly the
+//   B operand of two MFMAs whose k slots are the keys 16a + 4g + {0..3, 8..11}; the A
+//   operand reads those keys of dim d from the transposed value pages, 8 bytes at a time.
+// ---------------------------------------------------------------------------------------
+namespace flash {
+constexpr int ROWS = 128;
+
+template <int DH16>
+__global__ __launch_bounds__(256) void kernel(const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo,
+                                               const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+                                               const int32_t* __restrict__ block_tables, int max_blocks,
+                                               const int32_t* __restrict__ tile_seq,
+                                               const int32_t* __restrict__ tile_row0,
+                                               const int32_t* __restrict__ tile_nrows,
+                                               const int32_t* __restrict__ tile_pos0, int H, int Hkv, int page_size,
+                                               float scale, int window) {
+  constexpr int DH = DH16 * 16;
+  constexpr int DB = (DH + 31) / 32;
+  const int tile = blockIdx.x, h = blockIdx.y;
+  const int seq = tile_seq[tile];
+  if (seq < 0) return;
+  const int row0 = tile_row0[tile], nrows = tile_nrows[tile], pos0 = tile_pos0[tile];
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int wrow0 = wave * 32;
+  if (wrow0 >= nrows) return;   // no barrier follows: a wave without rows may leave
+  const int qcol = lane % 32, g = lane / 32;
+  const int hk = h / (H / Hkv);
+  const int32_t* bt = block_tables + static_cast<size_t>(seq) * max_blocks;
+  const bool row_ok = wrow0 + qcol < nrows;
+  const int my_row = row_ok ? wrow0 + qcol : nrows - 1;
+  const int my_pos = pos0 + my_row;
+  const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
+  const int lo_w = window > 0 ? max(0, pos0 + wrow0 - window + 1) : 0;
+  const int hi_w = pos0 + min(wrow0 + 31, nrows - 1);
+  const float NEG_INF = -INFINITY;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  bf16x8 qf[DH16];
+  {
+    const bf16_t* qr = q + static_cast<size_t>(row0 + my_row) * ldq + h * DH + g * 8;
+#pragma unroll
+    for (int c = 0; c < DH16; ++c) qf[c] = *reinterpret_cast<const bf16x8*>(qr + c * 16);
+  }
+  floatx16 o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+  float m = NEG_INF, l = 0.f;
+
+  for (int kt = (lo_w / 32) * 32; kt <= hi_w; kt += 32) {
+    floatx16 s;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    {
+      const int key = kt + qcol;      // as A operand the lane's row is a key
+      int page = key <= hi_w ? bt[key / page_size] : -1;
+      const bf16_t* kr = k_pool + ((static_cast<size_t>(max(page, 0)) * Hkv + hk) * page_size + key % page_size) * DH + g * 8;
+#pragma unroll
+      for (int c = 0; c < DH16; ++c) {
+        bf16x8 kf = page >= 0 ? *reinterpret_cast<const bf16x8*>(kr + c * 16) : zero8;
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[c], s, 0, 0, 0);
+      }
+    }
+    // s[i]: key kt + 8*(i/4) + 4*g + i%4, query = this lane's column
+    float tmax = NEG_INF;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      int key = kt + 8 * (i / 4) + 4 * g + (i % 4);
+      bool ok = row_ok && key >= my_lo && key <= my_pos;
+      s[i] = ok ? s[i] * scale : NEG_INF;
+      tmax = fmaxf(tmax, s[i]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, DN_WAVE));
+    float p[16];
+    float psum = 0.f, alpha = 1.f;
+    if (tmax > NEG_INF) {
+      float m_new = fmaxf(m, tmax);
+      alpha = m > NEG_INF ? __expf(m - m_new) : 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        p[i] = s[i] > NEG_INF ? __expf(s[i] - m_new) : 0.f;
+        psum += p[i];
+      }
+      m = m_new;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) p[i] = 0.f;
+    }
+    psum += __shfl_xor(psum, 32, DN_WAVE);
+    l = l * alpha + psum;
+    bf16x8 pb[2];
+#pragma unroll
+    for (int a0 = 0; a0 < 2; ++a0)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pb[a0][j] = to_bf16(p[8 * a0 + j]);
+    // alpha belongs to the lane's query, and so do all of the lane's accumulators
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+#pragma unroll
+    for (int a0 = 0; a0 < 2; ++a0) {
+      const int kb = kt + 16 * a0;    // 16 keys of one page
+      int page = kb <= hi_w ? bt[kb / page_size] : -1;
+      if (page < 0) continue;         // the same for every lane of the wave
+      const bf16_t* vb = v_pool + (static_cast<size_t>(page) * Hkv + hk) * DH * page_size + kb % page_size + 4 * g;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int d = 32 * db + qcol;   // as A operand the lane's row is a dim
+        bf16x8 vf = zero8;
+        if (d < DH) {
+          const bf16_t* vr = vb + static_cast<size_t>(d) * page_size;
+          bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(vr);
+          bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(vr + 8);
+          vf = bf16x8{lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+        }
+        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[a0], o[db], 0, 0, 0);
+      }
+    }
+  }
+  if (row_ok) {
+    const float inv = 1.0f / l;
+    bf16_t* orow = out + static_cast<size_t>(row0 + my_row) * ldo + h * DH;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const int d0 = 32 * db + 8 * a + 4 * g;
+        if (d0 < DH) {
+          bf16x4 w = {to_bf16(o[db][4 * a] * inv), to_bf16(o[db][4 * a + 1] * inv), to_bf16(o[db][4 * a + 2] * inv),
+                      to_bf16(o[db][4 * a + 3] * inv)};
+          *reinterpret_cast<bf16x4*>(orow + d0) = w;
+        }
+      }
+  }
+}
+}  // namespace flash
+
+extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
+                                  const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
+                                  const int32_t* tile_row0, const int32_t* tile_nrows, const int32_t* tile_pos0,
+                                  int n_tiles, int H, int Hkv, int dh, int page_size, float scale, int window,
+                                  hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (Hkv < 1 || H % Hkv != 0 || page_size % 16 != 0 || max_blocks < 1 || ldq % 8 != 0 || ldo % 4 != 0 ||
+      reinterpret_cast<uintptr_t>(q) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 8 != 0)
+    return DN_ERR_SHAPE;
+  dim3 grid(n_tiles, H), block(256);
+#define DN_FLASH(D)                                                                                               \
+  hipLaunchKernelGGL(flash::kernel<D>, grid, block, 0, stream, static_cast<const bf16_t*>(q), ldq,                \
+                     static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),                          \
+                     static_cast<const bf16_t*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0, tile_nrows, \
+                     tile_pos0, H, Hkv, page_size, scale, window)
+  switch (dh) {
+    case 16: DN_FLASH(1); break;
+    case 32: DN_FLASH(2); break;
+    case 48: DN_FLASH(3); break;
+    case 64: DN_FLASH(4); break;
+    case 96: DN_FLASH(6); break;
+    case 128: DN_FLASH(8); break;
+    default: return DN_ERR_SHAPE;
+  }
+#undef DN_FLASH
+  return dn_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// decode: one row per request.  The context is cut into splits of 256 keys; a workgroup
+// (4 waves of 64 keys) makes one split's partial result (running maximum, sum, weighted
+// values), and, if there is more than one split, a second kernel joins the partials in split
+// order (crates/denno-engine/kernels/kernels_elem.cu:577-603 has this two-kernel shape).
+// Scores: dh/8 lanes share a key, 16 bytes each, so one load instruction reads whole keys side
+// by side.  Values: lane = dim, 16 keys (32 bytes) of a transposed page at a time.
+// ---------------------------------------------------------------------------------------
+namespace decode {
+constexpr int SPLIT = 256;
+
+template <int LPK>   // lanes per key = dh / 8
+__global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out,
+                                                       int ldo, const bf16_t* __restrict__ k_pool,
+                                                       const bf16_t* __restrict__ v_pool,
+                                                       const int32_t* __restrict__ block_tables, int max_blocks,
+                                                       const int32_t* __restrict__ tile_seq,
+                                                       const int32_t* __restrict__ tile_row0,
+                                                       const int32_t* __restrict__ tile_pos0,
+                                                       float* __restrict__ part, int n_splits, int H, int Hkv,
+                                                       int page_size, float scale, int window) {
+  constexpr int DH = LPK * 8;
+  constexpr int KPI = 64 / LPK;          // keys per load instruction
+  constexpr int DPL = (DH + 63) / 64;    // dims per lane in the second product
+  __shared__ float q_s[DH];
+  __shared__ float sc[4][64];
+  __shared__ float wm[4], wl[4];
+  __shared__ float wacc[4][DH];
+  const int split = blockIdx.x, h = blockIdx.y, tile = blockIdx.z;
+  const int seq = tile_seq[tile];
+  if (seq < 0) return;
+  const int row = tile_row0[tile], pos = tile_pos0[tile];
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int key0 = split * SPLIT;
+  const float NEG_INF = -INFINITY;
+  float* mypart = part + ((static_cast<size_t>(tile) * H + h) * n_splits + split) * (DH + 2);
+  if (key0 > pos || key0 + SPLIT <= lo) {
+    if (n_splits > 1 && threadIdx.x == 0) {
+      mypart[0] = NEG_INF;     // the join skips it
+      mypart[1] = 0.f;
+    }
+    return;
+  }
+  const int hk = h / (H / Hkv);
+  const int32_t* bt = block_tables + static_cast<size_t>(seq) * max_blocks;
+  for (int d = threadIdx.x; d < DH; d += 256)
+    q_s[d] = to_float(q[static_cast<size_t>(row) * ldq + h * DH + d]) * scale;
+  __syncthreads();
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int kbase = key0 + wave * 64;
+  {
+    const int sub = lane % LPK, grp = lane / LPK;
+    float qr[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qr[i] = q_s[sub * 8 + i];
+#pragma unroll
+    for (int it = 0; it < LPK; ++it) {
+      const int j = it * KPI + grp;
+      const int key = kbase + j;
+      const bool valid = key >= lo && key <= pos;
+      float dot = 0.f;
+      if (valid) {
+        const int page = bt[key / page_size];
+        const bf16_t* kr = k_pool + ((static_cast<size_t>(page) * Hkv + hk) * page_size + key % page_size) * DH + sub * 8;
+        bf16x8 kv = *reinterpret_cast<const bf16x8*>(kr);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dot = fmaf(qr[i], static_cast<float>(kv[i]), dot);
+      }
+#pragma unroll
+      for (int msk = LPK / 2; msk >= 1; msk >>= 1) dot += __shfl_xor(dot, msk, DN_WAVE);
+      if (sub == 0) sc[wave][j] = valid ? dot : NEG_INF;
+    }
+  }
+  __syncthreads();
+  const float s = sc[wave][lane];
+  const float m = wave_max(s);
+  const float p = s > NEG_INF ? __expf(s - m) : 0.f;
+  const float l = wave_sum(p);
+  sc[wave][lane] = p;
+  __syncthreads();
+  float acc[DPL];
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) acc[i] = 0.f;
+#pragma unroll
+  for (int blk = 0; blk < 4; ++blk) {
+    const int kb = kbase + blk * 16;
+    if (kb > pos || kb + 16 <= lo) continue;
+    const int page = bt[kb / page_size];
+    if (page < 0) continue;
+    const float* pr = &sc[wave][blk * 16];
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) {
+      const int d = lane + 64 * i;
+      if (d < DH) {
+        const bf16_t* vr = v_pool + ((static_cast<size_t>(page) * Hkv + hk) * DH + d) * page_size + kb % page_size;
+        bf16x8 v0 = *reinterpret_cast<const bf16x8*>(vr);
+        bf16x8 v1 = *reinterpret_cast<const bf16x8*>(vr + 8);
+        float a = acc[i];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a = fmaf(pr[j], static_cast<float>(v0[j]), a);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a = fmaf(pr[8 + j], static_cast<float>(v1[j]), a);
+        acc[i] = a;
+      }
+    }
+  }
+  if (lane == 0) {
+    wm[wave] = m;
+    wl[wave] = l;
+  }
+#pragma unroll
+  for (int i = 0; i < DPL; ++i)
+    if (lane + 64 * i < DH) wacc[wave][lane + 64 * i] = acc[i];
+  __syncthreads();
+  for (int d = threadIdx.x; d < DH; d += 256) {
+    float M = fmaxf(fmaxf(wm[0], wm[1]), fmaxf(wm[2], wm[3]));
+    float L = 0.f, A = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      if (wm[w] > NEG_INF) {
+        float f = __expf(wm[w] - M);
+        L += wl[w] * f;
+        A += wacc[w][d] * f;
+      }
+    }
+    if (n_splits == 1) {
+      out[static_cast<size_t>(row) * ldo + h * DH + d] = from_float<bf16_t>(A / L);
+    } else {
+      mypart[2 + d] = A;
+      if (d == 0) {
+        mypart[0] = M;
+        mypart[1] = L;
+      }
+    }
+  }
+}
+
+__global__ void join_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, int ldo,
+                            const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_row0, int n_splits,
+                            int H, int DH) {
+  const int tile = blockIdx.x, h = blockIdx.y;
+  if (tile_seq[tile] < 0) return;
+  const float* base = part + (static_cast<size_t>(tile) * H + h) * n_splits * (DH + 2);
+  float M = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, base[static_cast<size_t>(s) * (DH + 2)]);
+  for (int d = threadIdx.x; d < DH; d += blockDim.x) {
+    float L = 0.f, A = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float* ps = base + static_cast<size_t>(s) * (DH + 2);
+      if (ps[0] > -INFINITY) {
+        float f = __expf(ps[0] - M);
+        L += ps[1] * f;
+        A += ps[2 + d] * f;
+      }
+    }
+    out[static_cast<size_t>(tile_row0[tile]) * ldo + h * DH + d] = from_float<bf16_t>(A / L);
+  }
+}
+}  // namespace decode
+
+// part: 32-bit workspace of n_tiles * H * n_splits * (dh + 2) floats (unused when n_splits == 1)
+extern "C" int dn_attention_decode(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
+                                   const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
+                                   const int32_t* tile_row0, const int32_t* tile_pos0, int n_tiles, float* part,
+                                   int n_splits, int H, int Hkv, int dh, int page_size, float scale, int window,
+                                   hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (Hkv < 1 || H % Hkv != 0 || page_size % 16 != 0 || max_blocks < 1 || n_splits < 1 ||
+      reinterpret_cast<uintptr_t>(k_pool) % 16 != 0 || reinterpret_cast<uintptr_t>(v_pool) % 16 != 0)
+    return DN_ERR_SHAPE;
+  if (n_splits * decode::SPLIT > max_blocks * page_size + decode::SPLIT) return DN_ERR_SHAPE;
+  dim3 grid(n_splits, H, n_tiles), block(256);
+#define DN_DECODE(L)                                                                                              \
+  hipLaunchKernelGGL(decode::partial_kernel<L>, grid, block, 0, stream, static_cast<const bf16_t*>(q), ldq,       \
+                     static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),                          \
+                     static_cast<const bf16_t*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0, tile_pos0, \
+                     part, n_splits, H, Hkv, page_size, scale, window)
+  switch (dh) {
+    case 16: DN_DECODE(2); break;
+    case 32: DN_DECODE(4); break;
+    case 64: DN_DECODE(8); break;
+    case 128: DN_DECODE(16); break;
+    case 256: DN_DECODE(32); break;
+    default: return DN_ERR_SHAPE;
+  }
+#undef DN_DECODE
+  if (n_splits > 1)
+    hipLaunchKernelGGL(decode::join_kernel, dim3(n_tiles, H), dim3(64), 0, stream, part, static_cast<bf16_t*>(out),
+                       ldo, tile_seq, tile_row0, n_splits, H, dh);
   return dn_launch_status();
 }

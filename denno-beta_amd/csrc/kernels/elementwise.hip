@@ -93,7 +93,9 @@ extern "C" int dn_layernorm(const float* x, const float* gamma, const float* bet
 // Keys and values of this step's tokens go to their pages before attention reads them
 // (crates/denno-engine/src/model/gpt2.rs:159-167).  src is [T, ld]; keys are columns
 // k_col .. k_col + Hkv*dh, values v_col .. ; slot_map[t] = page * page_size + offset, or < 0
-// for a row that is padding.  A pool is [n_pages, Hkv, page_size, dh].
+// for a row that is padding.  The key pool is [n_pages, Hkv, page_size, dh]; the value pool is
+// [n_pages, Hkv, dh, page_size] (a page's values transposed), which is how attention's second
+// product reads them: for one dim, the keys of a page side by side.
 // ---------------------------------------------------------------------------------------
 template <typename TS>
 __global__ void kv_write_kernel(const TS* __restrict__ src, int ld, int k_col, int v_col,
@@ -108,9 +110,9 @@ __global__ void kv_write_kernel(const TS* __restrict__ src, int ld, int k_col, i
   const TS* row = src + static_cast<size_t>(t) * ld;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     int h = c / dh, d = c % dh;
-    size_t dst = ((static_cast<size_t>(page) * Hkv + h) * page_size + off) * dh + d;
-    k_pool[dst] = row[k_col + c];
-    v_pool[dst] = row[v_col + c];
+    size_t base = (static_cast<size_t>(page) * Hkv + h) * page_size * dh;
+    k_pool[base + static_cast<size_t>(off) * dh + d] = row[k_col + c];
+    v_pool[base + static_cast<size_t>(d) * page_size + off] = row[v_col + c];
   }
 }
 

@@ -14,7 +14,8 @@ from typing import List, Optional, Sequence
 import numpy as np
 import torch
 
-TILE_ROWS = 16   # rows of one request that one attention workgroup takes
+TILE_ROWS = 16         # rows of one request that one workgroup of the plain attention kernel takes
+WIDE_TILE_ROWS = 128   # the same for the MFMA attention kernel
 
 
 @dataclass
@@ -31,7 +32,10 @@ class GroupStep:
     window: int
     slot_map: Optional[torch.Tensor]       # int32 [T]: page * page_size + offset of each row's key
     block_tables: Optional[torch.Tensor]   # int32 [S, max_blocks], -1: page given back
-    tiles: Optional[torch.Tensor]          # int32 [4, n_tiles]: request, first row, rows, first position
+    tiles: Optional[torch.Tensor]          # int32 [4, n_tiles]: request, first row, rows <= 16, first position
+    tiles_wide: Optional[torch.Tensor] = None   # the same rows in tiles of up to 128
+    single_rows: bool = False              # every request brings one row (a pure decode step)
+    max_context: int = 0                   # the longest context after this step
 
 
 @dataclass
@@ -57,8 +61,8 @@ class BatchError(ValueError):
 
 
 def plan_rows(entries: Sequence[StepEntry], starts: Sequence[int], vocab: int, max_positions: int):
-    """Host arrays of the batch: tokens, positions, logit rows, row starts, tiles."""
-    tokens, positions, logit_rows, row_start, tiles = [], [], [], [0], []
+    """Host arrays of the batch: tokens, positions, logit rows, row starts, tiles (narrow and wide)."""
+    tokens, positions, logit_rows, row_start, tiles, wide = [], [], [], [0], [], []
     seen = set()
     for s, (e, start) in enumerate(zip(entries, starts)):
         n = len(e.tokens)
@@ -82,8 +86,10 @@ def plan_rows(entries: Sequence[StepEntry], starts: Sequence[int], vocab: int, m
             logit_rows.append(row0 + w)
         for i in range(0, n, TILE_ROWS):
             tiles.append((s, row0 + i, min(TILE_ROWS, n - i), start + i))
+        for i in range(0, n, WIDE_TILE_ROWS):
+            wide.append((s, row0 + i, min(WIDE_TILE_ROWS, n - i), start + i))
         row_start.append(row0 + n)
-    return tokens, positions, logit_rows, row_start, tiles
+    return tokens, positions, logit_rows, row_start, tiles, wide
 
 
 def build_context(entries: Sequence[StepEntry], cache, vocab: int, max_positions: int, device) -> StepContext:
@@ -91,7 +97,7 @@ def build_context(entries: Sequence[StepEntry], cache, vocab: int, max_positions
     earlier entries stay with their requests) and builds the step's tables."""
     mgr = cache.manager
     starts = [mgr.length(e.rid) for e in entries]
-    tokens, positions, logit_rows, row_start, tiles = plan_rows(entries, starts, vocab, max_positions)
+    tokens, positions, logit_rows, row_start, tiles, wide = plan_rows(entries, starts, vocab, max_positions)
     for e, start in zip(entries, starts):
         mgr.reserve(e.rid, start + len(e.tokens))
     T, S, R = len(tokens), len(entries), len(logit_rows)
@@ -102,7 +108,10 @@ def build_context(entries: Sequence[StepEntry], cache, vocab: int, max_positions
              ("logit_rows", np.asarray(logit_rows, dtype=np.int32)),
              ("state_slots", np.asarray(slots, dtype=np.int32)),
              ("row_start", np.asarray(row_start, dtype=np.int32)),
-             ("tiles", np.ascontiguousarray(np.asarray(tiles, dtype=np.int32).T).reshape(-1))]
+             ("tiles", np.ascontiguousarray(np.asarray(tiles, dtype=np.int32).T).reshape(-1)),
+             ("wide", np.ascontiguousarray(np.asarray(wide, dtype=np.int32).T).reshape(-1))]
+    single = all(len(e.tokens) == 1 for e in entries)
+    max_context = max(start + len(e.tokens) for e, start in zip(entries, starts))
     group_meta = []
     for g, layout in enumerate(cache.layouts):
         if layout.kind != 0:
@@ -139,6 +148,7 @@ def build_context(entries: Sequence[StepEntry], cache, vocab: int, max_positions
         b, n = offs[name]
         return dev[b:b + n]
     tiles_dev = view("tiles").view(4, -1)
+    wide_dev = view("wide").view(4, -1)
     groups = []
     for g, meta in enumerate(group_meta):
         if meta is None:
@@ -146,7 +156,7 @@ def build_context(entries: Sequence[StepEntry], cache, vocab: int, max_positions
             continue
         layout, max_blocks = meta
         groups.append(GroupStep(layout.page_size, layout.window, view(f"sm{g}"),
-                                view(f"bt{g}").view(S, max_blocks), tiles_dev))
+                                view(f"bt{g}").view(S, max_blocks), tiles_dev, wide_dev, single, max_context))
     return StepContext(
         T=T, S=S, R=R, tokens=view("tokens"), positions=view("positions"), logit_rows=view("logit_rows"),
         state_slots=view("state_slots"), row_start=view("row_start"), groups=groups,

@@ -50,6 +50,8 @@ def _declare(name, lib):
         },
         "attention": {
             "dn_attention": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, I, P],
+            "dn_attention_flash": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, P],
+            "dn_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, P, I, I, I, I, I, F, I, P],
         },
         "sampling": {
             "dn_sample": [P, I, I, I, P, P, P, P],
@@ -148,13 +150,15 @@ def layernorm(x, gamma, beta, eps, out, rows=None):
 
 def kv_write(src, k_col, v_col, slot_map, k_pool, v_pool):
     """Rows of src ([T, ld]; keys at columns k_col.., values at v_col..) go to the slots
-    slot_map[t] = page * page_size + offset of the pools [n_pages, Hkv, page_size, dh]."""
+    slot_map[t] = page * page_size + offset; k_pool is [n_pages, Hkv, page_size, dh], v_pool
+    [n_pages, Hkv, dh, page_size]."""
     _dev(src, "src", _FLOATS, 2), _dev(slot_map, "slot_map", _I32, 1)
     _dev(k_pool, "k_pool", (src.dtype,), 4), _dev(v_pool, "v_pool", (src.dtype,), 4)
     ld = _rows(src, "src")
     T = src.shape[0]
     n_pages, Hkv, ps, dh = k_pool.shape
-    _need(k_pool.is_contiguous() and v_pool.is_contiguous() and v_pool.shape == k_pool.shape, "kv_write: pools")
+    _need(k_pool.is_contiguous() and v_pool.is_contiguous() and tuple(v_pool.shape) == (n_pages, Hkv, dh, ps),
+          "kv_write: pools")
     _need(slot_map.is_contiguous() and slot_map.shape[0] == T, "kv_write: slot_map")
     w = Hkv * dh
     _need(0 <= k_col and k_col + w <= src.shape[1] and 0 <= v_col and v_col + w <= src.shape[1],
@@ -200,26 +204,63 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
     return out
 
 
-def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, window=0):
+FLASH_HEAD_DIMS = (16, 32, 48, 64, 96, 128)
+DECODE_HEAD_DIMS = (16, 32, 64, 128, 256)
+DECODE_SPLIT = 256
+
+
+def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, window=0, tiles_wide=None,
+              single_rows=False, max_context=0):
     """Causal attention of the batch's rows over the paged cache.
 
     q: [T, >= H*dh] rows contiguous, head h at columns h*dh..; out: [T, H*dh];
-    pools: [n_pages, Hkv, page_size, dh]; block_tables: int32 [S, max_blocks];
-    tiles: int32 [4, n_tiles] = (request, first row, rows <= 16, first position), request < 0: padding."""
+    k_pool: [n_pages, Hkv, page_size, dh]; v_pool: [n_pages, Hkv, dh, page_size];
+    block_tables: int32 [S, max_blocks];
+    tiles: int32 [4, n_tiles] = (request, first row, rows <= 16, first position), request < 0: padding;
+    tiles_wide: the same rows cut into tiles of up to 128 rows;
+    single_rows: every tile has one row (a pure decode step); max_context: the longest context then.
+
+    Three kernels: 32-bit takes the plain one; bfloat16 takes the MFMA kernel over tiles_wide, or,
+    for a pure decode step, the split kernel; a head size that those do not take falls to the plain one."""
     _dev(q, "q", _FLOATS, 2), _dev(out, "out", (q.dtype,), 2)
     _dev(k_pool, "k_pool", (q.dtype,), 4), _dev(v_pool, "v_pool", (q.dtype,), 4)
     _dev(block_tables, "block_tables", _I32, 2), _dev(tiles, "tiles", _I32, 2)
     n_pages, Hkv, ps, dh = k_pool.shape
     T = q.shape[0]
-    _need(k_pool.is_contiguous() and v_pool.is_contiguous() and v_pool.shape == k_pool.shape, "attention: pools")
+    _need(k_pool.is_contiguous() and v_pool.is_contiguous() and tuple(v_pool.shape) == (n_pages, Hkv, dh, ps),
+          "attention: pools")
     _need(q.shape[1] >= n_heads * dh and tuple(out.shape) == (T, n_heads * dh), "attention: q/out shapes")
     _need(block_tables.is_contiguous() and tiles.is_contiguous() and tiles.shape[0] == 4, "attention: tables")
     _need(dh % 16 == 0 and 16 <= dh <= 256, f"attention: head size {dh} must be a multiple of 16 up to 256")
     _need(n_heads % Hkv == 0, f"attention: {n_heads} heads over {Hkv} key heads")
     ldq, ldo = _rows(q, "q"), _rows(out, "out")
+    lib = _lib("attention")
+    fast = q.dtype == torch.bfloat16 and ps % 16 == 0 and ldq % 8 == 0 and q.data_ptr() % 16 == 0
+    if fast and single_rows and dh in DECODE_HEAD_DIMS and max_context > 0:
+        n_tiles = tiles.shape[1]
+        n_splits = -(-max_context // DECODE_SPLIT)
+        _need(max_context <= block_tables.shape[1] * ps, "attention: max_context exceeds the block tables")
+        part = torch.empty(n_tiles * n_heads * n_splits * (dh + 2) if n_splits > 1 else 1, dtype=torch.float32,
+                           device=q.device)
+        base = tiles.data_ptr()
+        _ok(lib.dn_attention_decode(
+            q.data_ptr(), ldq, out.data_ptr(), ldo, k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(),
+            block_tables.shape[1], base, base + 4 * n_tiles, base + 12 * n_tiles, n_tiles, part.data_ptr(), n_splits,
+            n_heads, Hkv, dh, ps, float(scale), int(window), _stream()), "attention (decode)")
+        return out
+    if fast and tiles_wide is not None and dh in FLASH_HEAD_DIMS:
+        _dev(tiles_wide, "tiles_wide", _I32, 2)
+        _need(tiles_wide.is_contiguous() and tiles_wide.shape[0] == 4, "attention: tiles_wide")
+        n_tiles = tiles_wide.shape[1]
+        base = tiles_wide.data_ptr()
+        _ok(lib.dn_attention_flash(
+            q.data_ptr(), ldq, out.data_ptr(), ldo, k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(),
+            block_tables.shape[1], base, base + 4 * n_tiles, base + 8 * n_tiles, base + 12 * n_tiles, n_tiles,
+            n_heads, Hkv, dh, ps, float(scale), int(window), _stream()), "attention (flash)")
+        return out
     n_tiles = tiles.shape[1]
     base = tiles.data_ptr()
-    _ok(_lib("attention").dn_attention(
+    _ok(lib.dn_attention(
         q.data_ptr(), ldq, out.data_ptr(), ldo, k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(),
         block_tables.shape[1], base, base + 4 * n_tiles, base + 8 * n_tiles, base + 12 * n_tiles, n_tiles,
         n_heads, Hkv, dh, ps, float(scale), int(window), _CODE[q.dtype], _stream()), "attention")

@@ -51,5 +51,6 @@ class CausalSelfAttention(Part):
             ops.kv_write(qkv, self.q_width, self.q_width + self.kv_width, g.slot_map, cache.k, cache.v)
         o = torch.empty((h.shape[0], self.q_width), dtype=act, device=h.device)
         ops.attention(qkv[:, :self.q_width], o, cache.k, cache.v, g.block_tables, g.tiles, self.n_heads,
-                      self.scale, self.window)
+                      self.scale, self.window, tiles_wide=g.tiles_wide, single_rows=g.single_rows,
+                      max_context=g.max_context)
         self.out(o, residual=accumulate_into)

@@ -67,7 +67,7 @@ class CacheView:
     group: int                    # index into ctx.groups
     writes: bool
     k: Optional[torch.Tensor] = None       # paged: [n_pages, Hkv, page_size, dh] of this call's cache
-    v: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None       #        [n_pages, Hkv, dh, page_size]
     state: Optional[torch.Tensor] = None   # fixed state: [n_slots, *shape]
 
 

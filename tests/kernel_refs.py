@@ -42,7 +42,7 @@ def kv_write(src, k_col, v_col, slot_map, k_pool, v_pool):
             continue
         page, off = divmod(slot, ps)
         k_pool[page, :, off, :] = src[t, k_col:k_col + w].view(hkv, dh)
-        v_pool[page, :, off, :] = src[t, v_col:v_col + w].view(hkv, dh)
+        v_pool[page, :, :, off] = src[t, v_col:v_col + w].view(hkv, dh)
 
 
 def cast(x, out):
@@ -67,7 +67,8 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
     return out
 
 
-def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, window=0):
+def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, window=0, tiles_wide=None,
+              single_rows=False, max_context=0):
     n_pages, hkv, ps, dh = k_pool.shape
     group = n_heads // hkv
     tl = tiles.cpu().tolist()
@@ -85,7 +86,7 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
             assert (pages >= 0).all(), "attention reads a page that was given back"
             for h in range(n_heads):
                 k = kf[pages, h // group, offs, :]                  # [n, dh]
-                v = vf[pages, h // group, offs, :]
+                v = vf[pages, h // group, :, offs]
                 qv = q[row0 + i, h * dh:(h + 1) * dh].float()
                 p = torch.softmax((k @ qv) * scale, dim=0)
                 out[row0 + i, h * dh:(h + 1) * dh] = (p @ v).to(out.dtype)

@@ -68,8 +68,8 @@ def test_kv_write(dtype):
     src = rnd(7, 5 * hkv * dh, seed=6, dtype=dtype)
     slots = i32([0, 9, 47, -1, 10, 23, 40])
     k = torch.zeros(n_pages, hkv, ps, dh, dtype=dtype, device=DEV)
-    v = torch.zeros_like(k)
-    k2, v2 = torch.zeros_like(k), torch.zeros_like(k)
+    v = torch.zeros(n_pages, hkv, dh, ps, dtype=dtype, device=DEV)
+    k2, v2 = torch.zeros_like(k), torch.zeros_like(v)
     ops().kv_write(src, hkv * dh, 3 * hkv * dh, slots, k, v)
     R.kv_write(src, hkv * dh, 3 * hkv * dh, slots, k2, v2)
     assert torch.equal(k, k2) and torch.equal(v, v2) and k.abs().sum() > 0
@@ -127,16 +127,19 @@ def paged_case(seq_lens, new_rows, H, Hkv, dh, ps, dtype, seed=0, q_scale=1.0):
     n_pages = sum(blocks) + 3
     perm = torch.randperm(n_pages, generator=g).tolist()
     k = (torch.randn(n_pages, Hkv, ps, dh, generator=g)).to(dtype).to(DEV)
-    v = (torch.randn(n_pages, Hkv, ps, dh, generator=g)).to(dtype).to(DEV)
+    v = (torch.randn(n_pages, Hkv, dh, ps, generator=g)).to(dtype).to(DEV)
     bt = torch.full((len(seq_lens), max(blocks)), -1, dtype=torch.int32)
-    tiles, row = [], 0
+    tiles, wide, row = [], [], 0
     for s, (n, new) in enumerate(zip(seq_lens, new_rows)):
         for b in range(blocks[s]):
             bt[s, b] = perm.pop()
         for i in range(0, new, 16):
             tiles.append((s, row + i, min(16, new - i), n - new + i))
+        for i in range(0, new, 128):
+            wide.append((s, row + i, min(128, new - i), n - new + i))
         row += new
     q = (torch.randn(row, 3 * H * dh, generator=g) * q_scale).to(dtype).to(DEV)
+    paged_case.wide = i32(wide).t().contiguous()
     return q, k, v, bt.to(DEV), i32(tiles).t().contiguous(), row
 
 
@@ -155,6 +158,45 @@ def test_attention(dtype, H, Hkv, dh, ps, window):
     assert torch.allclose(out.float(), want, **TOL[dtype])
 
 
+@pytest.mark.parametrize("H,Hkv,dh,ps,window", [(4, 4, 16, 16, 0), (25, 25, 64, 16, 0), (6, 2, 48, 32, 0),
+                                                (2, 1, 128, 64, 0), (3, 3, 96, 16, 0), (4, 2, 32, 16, 20),
+                                                (5, 5, 64, 32, 7), (2, 2, 64, 16, 150)])
+def test_attention_mfma_kernel_for_portions(H, Hkv, dh, ps, window):
+    """The bfloat16 kernel for portions of prompts (tiles of up to 128 rows): a long portion deep
+    in a context, a whole prompt, a short portion, single rows."""
+    seq_lens, new_rows = [430, 70, 133, 1, 200], [300, 70, 21, 1, 1]
+    q, k, v, bt, tiles, T = paged_case(seq_lens, new_rows, H, Hkv, dh, ps, torch.bfloat16, seed=H + dh)
+    scale = 1 / math.sqrt(dh)
+    out = torch.zeros(T, H * dh, dtype=torch.bfloat16, device=DEV)
+    ops().attention(q[:, :H * dh], out, k, v, bt, tiles, H, scale, window, tiles_wide=paged_case.wide)
+    want = R.attention(q[:, :H * dh], torch.zeros(T, H * dh, device=DEV), k, v, bt, tiles, H, scale, window)
+    assert torch.allclose(out.float(), want, **TOL[torch.bfloat16])
+
+
+@pytest.mark.parametrize("H,Hkv,dh,ps,window", [(4, 4, 16, 16, 0), (25, 25, 64, 16, 0), (6, 2, 32, 32, 0),
+                                                (2, 1, 128, 64, 0), (3, 3, 256, 16, 0), (5, 5, 64, 16, 100),
+                                                (2, 2, 64, 32, 300)])
+def test_attention_split_kernel_for_decoding(H, Hkv, dh, ps, window):
+    """The bfloat16 kernel for steps in which every request brings one row: contexts on both sides
+    of a split's edge (256 keys) and of a page's."""
+    seq_lens = [1, 17, 256, 257, 700, 1024, 512, 64]
+    q, k, v, bt, tiles, T = paged_case(seq_lens, [1] * len(seq_lens), H, Hkv, dh, ps, torch.bfloat16, seed=dh)
+    scale = 1 / math.sqrt(dh)
+    want = R.attention(q[:, :H * dh], torch.zeros(T, H * dh, device=DEV), k, v, bt, tiles, H, scale, window)
+    for max_context in (1024, 1040):         # the second: a launch sized for a longer context than any request's
+        if max_context > bt.shape[1] * ps:
+            continue
+        out = torch.zeros(T, H * dh, dtype=torch.bfloat16, device=DEV)
+        ops().attention(q[:, :H * dh], out, k, v, bt, tiles, H, scale, window, tiles_wide=paged_case.wide,
+                        single_rows=True, max_context=max_context)
+        assert torch.allclose(out.float(), want, **TOL[torch.bfloat16])
+    # one short request alone: a single split, written without the join
+    out = torch.zeros(1, H * dh, dtype=torch.bfloat16, device=DEV)
+    ops().attention(q[1:2, :H * dh], out, k, v, bt, i32([[1], [0], [1], [16]]), H, scale, window, single_rows=True,
+                    max_context=17)
+    assert torch.allclose(out.float(), want[1:2], **TOL[torch.bfloat16])
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_finds_a_far_key(dtype):
     """One key among hundreds matches the query strongly: the output must be its value, whichever
@@ -165,9 +207,11 @@ def test_attention_finds_a_far_key(dtype):
         page, off = int(bt[0, far // ps]), far % ps
         qh = q[0, :dh].float()
         k[page, 0, off] = (qh / qh.norm() * 40).to(dtype)       # score 40 |q| against about |q| for the others
-        out = torch.zeros(1, H * dh, dtype=dtype, device=DEV)
-        ops().attention(q[:, :H * dh] , out, k, v, bt, tiles, H, 1.0)
-        assert torch.allclose(out[0, :dh].float(), v[page, 0, off].float(), atol=1e-2 if dtype == torch.bfloat16 else 1e-4), far
+        tol = 1e-2 if dtype == torch.bfloat16 else 1e-4
+        for kw in (dict(), dict(tiles_wide=paged_case.wide), dict(single_rows=True, max_context=n)):
+            out = torch.zeros(1, H * dh, dtype=dtype, device=DEV)
+            ops().attention(q[:, :H * dh], out, k, v, bt, tiles, H, 1.0, **kw)
+            assert torch.allclose(out[0, :dh].float(), v[page, 0, :, off].float(), atol=tol), (far, kw.keys())
 
 
 def test_attention_window_edges():
@@ -176,7 +220,7 @@ def test_attention_window_edges():
     q, k, v, bt, tiles, T = paged_case([n], [n], H, H, dh, ps, torch.float32, seed=1)
     k.zero_()                       # all scores equal: the output is the mean of the values in the window
     for pos in range(n):
-        v[int(bt[0, pos // ps]), 0, pos % ps] = float(pos)
+        v[int(bt[0, pos // ps]), 0, :, pos % ps] = float(pos)
     out = torch.zeros(T, dh, device=DEV)
     ops().attention(q[:, :dh], out, k, v, bt, tiles, H, 1.0, window)
     for pos in (0, 1, 36, 37, 38, 100, 199):

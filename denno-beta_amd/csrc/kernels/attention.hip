@@ -355,15 +355,18 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
 }
 
 // ---------------------------------------------------------------------------------------
-// decode: one row per request.  The context is cut into splits of 256 keys; a workgroup
-// (4 waves of 64 keys) makes one split's partial result (running maximum, sum, weighted
-// values), and, if there is more than one split, a second kernel joins the partials in split
-// order (crates/denno-engine/kernels/kernels_elem.cu:577-603 has this two-kernel shape).
+// decode: one row per request.  The context is cut into n_splits runs of `chunks` * 256 keys;
+// a workgroup walks its run 256 keys at a time (4 waves of 64 keys, each with a running
+// maximum, sum and weighted values, joined through LDS at the end) and, if there is more than
+// one split, a second kernel joins the splits' results in split order
+// (crates/denno-engine/kernels/kernels_elem.cu:577-603 has this two-kernel shape).
 // Scores: dh/8 lanes share a key, 16 bytes each, so one load instruction reads whole keys side
-// by side.  Values: lane = dim, 16 keys (32 bytes) of a transposed page at a time.
+// by side; all loads of 64 keys are issued before the first is used.  Values: lane = dim,
+// 16 keys (32 bytes) of a transposed page at a time.  Nothing but registers and lane
+// exchanges inside the loop.
 // ---------------------------------------------------------------------------------------
 namespace decode {
-constexpr int SPLIT = 256;
+constexpr int CHUNK = 256;   // keys that a workgroup's 4 waves take at a time, 64 each
 
 template <int LPK>   // lanes per key = dh / 8
 __global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out,
@@ -373,13 +376,12 @@ __global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__
                                                        const int32_t* __restrict__ tile_seq,
                                                        const int32_t* __restrict__ tile_row0,
                                                        const int32_t* __restrict__ tile_pos0,
-                                                       float* __restrict__ part, int n_splits, int H, int Hkv,
-                                                       int page_size, float scale, int window) {
+                                                       float* __restrict__ part, int n_splits, int chunks, int H,
+                                                       int Hkv, int page_size, float scale, int window) {
   constexpr int DH = LPK * 8;
   constexpr int KPI = 64 / LPK;          // keys per load instruction
   constexpr int DPL = (DH + 63) / 64;    // dims per lane in the second product
-  __shared__ float q_s[DH];
-  __shared__ float sc[4][64];
+  constexpr int GROUP = LPK < 8 ? LPK : 8;   // load instructions issued together
   __shared__ float wm[4], wl[4];
   __shared__ float wacc[4][DH];
   const int split = blockIdx.x, h = blockIdx.y, tile = blockIdx.z;
@@ -387,10 +389,10 @@ __global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__
   if (seq < 0) return;
   const int row = tile_row0[tile], pos = tile_pos0[tile];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  const int key0 = split * SPLIT;
+  const int key0 = split * chunks * CHUNK;
   const float NEG_INF = -INFINITY;
   float* mypart = part + ((static_cast<size_t>(tile) * H + h) * n_splits + split) * (DH + 2);
-  if (key0 > pos || key0 + SPLIT <= lo) {
+  if (key0 > pos || key0 + chunks * CHUNK <= lo) {
     if (n_splits > 1 && threadIdx.x == 0) {
       mypart[0] = NEG_INF;     // the join skips it
       mypart[1] = 0.f;
@@ -399,70 +401,92 @@ __global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__
   }
   const int hk = h / (H / Hkv);
   const int32_t* bt = block_tables + static_cast<size_t>(seq) * max_blocks;
-  for (int d = threadIdx.x; d < DH; d += 256)
-    q_s[d] = to_float(q[static_cast<size_t>(row) * ldq + h * DH + d]) * scale;
-  __syncthreads();
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-  const int kbase = key0 + wave * 64;
+  const int sub = lane % LPK, grp = lane / LPK;
+  float qr[8];
   {
-    const int sub = lane % LPK, grp = lane / LPK;
-    float qr[8];
+    bf16x8 qv = *reinterpret_cast<const bf16x8*>(q + static_cast<size_t>(row) * ldq + h * DH + sub * 8);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) qr[i] = q_s[sub * 8 + i];
-#pragma unroll
-    for (int it = 0; it < LPK; ++it) {
-      const int j = it * KPI + grp;
-      const int key = kbase + j;
-      const bool valid = key >= lo && key <= pos;
-      float dot = 0.f;
-      if (valid) {
-        const int page = bt[key / page_size];
-        const bf16_t* kr = k_pool + ((static_cast<size_t>(page) * Hkv + hk) * page_size + key % page_size) * DH + sub * 8;
-        bf16x8 kv = *reinterpret_cast<const bf16x8*>(kr);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) dot = fmaf(qr[i], static_cast<float>(kv[i]), dot);
-      }
-#pragma unroll
-      for (int msk = LPK / 2; msk >= 1; msk >>= 1) dot += __shfl_xor(dot, msk, DN_WAVE);
-      if (sub == 0) sc[wave][j] = valid ? dot : NEG_INF;
-    }
+    for (int i = 0; i < 8; ++i) qr[i] = static_cast<float>(qv[i]) * scale;
   }
-  __syncthreads();
-  const float s = sc[wave][lane];
-  const float m = wave_max(s);
-  const float p = s > NEG_INF ? __expf(s - m) : 0.f;
-  const float l = wave_sum(p);
-  sc[wave][lane] = p;
-  __syncthreads();
+  float m_run = NEG_INF, l_run = 0.f;
   float acc[DPL];
 #pragma unroll
   for (int i = 0; i < DPL; ++i) acc[i] = 0.f;
+
+  for (int c = 0; c < chunks; ++c) {
+    const int kbase = key0 + c * CHUNK + wave * 64;
+    if (kbase > pos || kbase + 64 <= lo) continue;     // the same for the whole wave; no barrier in this loop
+    // scores: lane (key group grp, part sub of the key) ; afterwards lane j holds key kbase + j
+    float s = NEG_INF;
 #pragma unroll
-  for (int blk = 0; blk < 4; ++blk) {
-    const int kb = kbase + blk * 16;
-    if (kb > pos || kb + 16 <= lo) continue;
-    const int page = bt[kb / page_size];
-    if (page < 0) continue;
-    const float* pr = &sc[wave][blk * 16];
+    for (int it0 = 0; it0 < LPK; it0 += GROUP) {
+      bf16x8 kv[GROUP];
+      bool valid[GROUP];
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) {
-      const int d = lane + 64 * i;
-      if (d < DH) {
-        const bf16_t* vr = v_pool + ((static_cast<size_t>(page) * Hkv + hk) * DH + d) * page_size + kb % page_size;
-        bf16x8 v0 = *reinterpret_cast<const bf16x8*>(vr);
-        bf16x8 v1 = *reinterpret_cast<const bf16x8*>(vr + 8);
-        float a = acc[i];
+      for (int u = 0; u < GROUP; ++u) {
+        const int key = kbase + (it0 + u) * KPI + grp;
+        valid[u] = key >= lo && key <= pos;
+        const int kk = valid[u] ? key : pos;            // a key that surely has a page
+        const int page = bt[kk / page_size];
+        kv[u] = *reinterpret_cast<const bf16x8*>(
+            k_pool + ((static_cast<size_t>(page) * Hkv + hk) * page_size + kk % page_size) * DH + sub * 8);
+      }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) a = fmaf(pr[j], static_cast<float>(v0[j]), a);
+      for (int u = 0; u < GROUP; ++u) {
+        float dot = 0.f;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) a = fmaf(pr[8 + j], static_cast<float>(v1[j]), a);
-        acc[i] = a;
+        for (int i = 0; i < 8; ++i) dot = fmaf(qr[i], static_cast<float>(kv[u][i]), dot);
+#pragma unroll
+        for (int msk = LPK / 2; msk >= 1; msk >>= 1) dot += __shfl_xor(dot, msk, DN_WAVE);
+        if (!valid[u]) dot = NEG_INF;
+        // key j = (it0 + u) * KPI + g was made by group g: lane j takes it in its turn
+        float got = __shfl(dot, (lane % KPI) * LPK, DN_WAVE);
+        if (lane / KPI == it0 + u) s = got;
+      }
+    }
+    const float m_c = wave_max(s);
+    if (!(m_c > NEG_INF)) continue;
+    const float m_new = fmaxf(m_run, m_c);
+    const float alpha = m_run > NEG_INF ? __expf(m_run - m_new) : 0.f;
+    const float p = s > NEG_INF ? __expf(s - m_new) : 0.f;
+    l_run = l_run * alpha + wave_sum(p);
+    m_run = m_new;
+    // values: lane = dim; 16 keys of one page at a time, all four loads of the 64 keys first
+    bf16x8 v0[4][DPL], v1[4][DPL];
+    bool live[4];
+#pragma unroll
+    for (int blk = 0; blk < 4; ++blk) {
+      const int kb = kbase + blk * 16;
+      live[blk] = kb <= pos && kb + 16 > lo;
+      const int kk = live[blk] ? kb : (pos / 16) * 16;
+      const int page = bt[kk / page_size];
+      live[blk] = live[blk] && page >= 0;
+      const bf16_t* vb = v_pool + (static_cast<size_t>(max(page, 0)) * Hkv + hk) * DH * page_size + kk % page_size;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        const int d = min(lane + 64 * i, DH - 1);
+        v0[blk][i] = *reinterpret_cast<const bf16x8*>(vb + static_cast<size_t>(d) * page_size);
+        v1[blk][i] = *reinterpret_cast<const bf16x8*>(vb + static_cast<size_t>(d) * page_size + 8);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) acc[i] *= alpha;
+#pragma unroll
+    for (int blk = 0; blk < 4; ++blk) {
+      if (!live[blk]) continue;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const float pj = __shfl(p, blk * 16 + j, DN_WAVE);
+#pragma unroll
+        for (int i = 0; i < DPL; ++i)
+          acc[i] = fmaf(pj, static_cast<float>(j < 8 ? v0[blk][i][j] : v1[blk][i][j - 8]), acc[i]);
       }
     }
   }
   if (lane == 0) {
-    wm[wave] = m;
-    wl[wave] = l;
+    wm[wave] = m_run;
+    wl[wave] = l_run;
   }
 #pragma unroll
   for (int i = 0; i < DPL; ++i)
@@ -514,23 +538,24 @@ __global__ void join_kernel(const float* __restrict__ part, bf16_t* __restrict__
 }
 }  // namespace decode
 
-// part: 32-bit workspace of n_tiles * H * n_splits * (dh + 2) floats (unused when n_splits == 1)
+// part: 32-bit workspace of n_tiles * H * n_splits * (dh + 2) floats (unused when n_splits == 1);
+// the splits cover n_splits * chunks * 256 keys, which must reach the longest context
 extern "C" int dn_attention_decode(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
                                    const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
                                    const int32_t* tile_row0, const int32_t* tile_pos0, int n_tiles, float* part,
-                                   int n_splits, int H, int Hkv, int dh, int page_size, float scale, int window,
-                                   hipStream_t stream) {
+                                   int n_splits, int chunks, int H, int Hkv, int dh, int page_size, float scale,
+                                   int window, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
-  if (Hkv < 1 || H % Hkv != 0 || page_size % 16 != 0 || max_blocks < 1 || n_splits < 1 ||
-      reinterpret_cast<uintptr_t>(k_pool) % 16 != 0 || reinterpret_cast<uintptr_t>(v_pool) % 16 != 0)
+  if (Hkv < 1 || H % Hkv != 0 || page_size % 16 != 0 || max_blocks < 1 || n_splits < 1 || chunks < 1 ||
+      ldq % 8 != 0 || reinterpret_cast<uintptr_t>(q) % 16 != 0 || reinterpret_cast<uintptr_t>(k_pool) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(v_pool) % 16 != 0)
     return DN_ERR_SHAPE;
-  if (n_splits * decode::SPLIT > max_blocks * page_size + decode::SPLIT) return DN_ERR_SHAPE;
   dim3 grid(n_splits, H, n_tiles), block(256);
 #define DN_DECODE(L)                                                                                              \
   hipLaunchKernelGGL(decode::partial_kernel<L>, grid, block, 0, stream, static_cast<const bf16_t*>(q), ldq,       \
                      static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),                          \
                      static_cast<const bf16_t*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0, tile_pos0, \
-                     part, n_splits, H, Hkv, page_size, scale, window)
+                     part, n_splits, chunks, H, Hkv, page_size, scale, window)
   switch (dh) {
     case 16: DN_DECODE(2); break;
     case 32: DN_DECODE(4); break;

@@ -73,17 +73,80 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const float* __res
   }
 }
 
+// The same with one workgroup per row and the row held in registers (one read of x): the
+// kernel for every width up to 256 * 32.  Sums meet in a fixed order: lanes by butterfly, the
+// four waves one after the other.
+__device__ __forceinline__ float block_sum_256(float v, float* scratch) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / DN_WAVE, lane = threadIdx.x % DN_WAVE;
+  __syncthreads();   // scratch may still be read from the call before
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  return ((scratch[0] + scratch[1]) + scratch[2]) + scratch[3];
+}
+
+template <typename TO, int VPT>
+__global__ __launch_bounds__(256) void layernorm_row_kernel(const float* __restrict__ x,
+                                                             const float* __restrict__ gamma,
+                                                             const float* __restrict__ beta, TO* __restrict__ out,
+                                                             const int32_t* __restrict__ rows, int E, float eps) {
+  __shared__ float scratch[4];
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  const float* xr = x + static_cast<size_t>(src) * E;
+  float v[VPT];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    int e = threadIdx.x + i * 256;
+    v[i] = e < E ? xr[e] : 0.f;
+    s += v[i];
+  }
+  const float mean = block_sum_256(s, scratch) / static_cast<float>(E);
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    int e = threadIdx.x + i * 256;
+    float d = e < E ? v[i] - mean : 0.f;
+    q += d * d;
+  }
+  const float inv = 1.0f / sqrtf(block_sum_256(q, scratch) / static_cast<float>(E) + eps);
+  TO* o = out + static_cast<size_t>(r) * E;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    int e = threadIdx.x + i * 256;
+    if (e < E) {
+      float y = (v[i] - mean) * inv * gamma[e];
+      if (beta) y += beta[e];
+      o[e] = from_float<TO>(y);
+    }
+  }
+}
+
+template <typename TO>
+static void launch_layernorm(const float* x, const float* gamma, const float* beta, TO* out, const int32_t* rows,
+                             int R, int E, float eps, hipStream_t stream) {
+  if (E <= 512)
+    hipLaunchKernelGGL((layernorm_row_kernel<TO, 2>), dim3(R), dim3(256), 0, stream, x, gamma, beta, out, rows, E, eps);
+  else if (E <= 2048)
+    hipLaunchKernelGGL((layernorm_row_kernel<TO, 8>), dim3(R), dim3(256), 0, stream, x, gamma, beta, out, rows, E, eps);
+  else if (E <= 8192)
+    hipLaunchKernelGGL((layernorm_row_kernel<TO, 32>), dim3(R), dim3(256), 0, stream, x, gamma, beta, out, rows, E,
+                       eps);
+  else {
+    const int waves = 4;
+    hipLaunchKernelGGL(layernorm_kernel<TO>, dim3((R + waves - 1) / waves), dim3(waves * DN_WAVE), 0, stream, x, gamma,
+                       beta, out, rows, R, E, eps);
+  }
+}
+
 extern "C" int dn_layernorm(const float* x, const float* gamma, const float* beta, void* out, const int32_t* rows,
                             int R, int E, float eps, int out_dtype, hipStream_t stream) {
   if (R <= 0) return 0;
-  const int waves = 4;
-  dim3 grid((R + waves - 1) / waves), block(waves * DN_WAVE);
   if (out_dtype == DN_F32)
-    hipLaunchKernelGGL(layernorm_kernel<float>, grid, block, 0, stream, x, gamma, beta, static_cast<float*>(out),
-                       rows, R, E, eps);
+    launch_layernorm<float>(x, gamma, beta, static_cast<float*>(out), rows, R, E, eps, stream);
   else if (out_dtype == DN_BF16)
-    hipLaunchKernelGGL(layernorm_kernel<bf16_t>, grid, block, 0, stream, x, gamma, beta,
-                       static_cast<bf16_t*>(out), rows, R, E, eps);
+    launch_layernorm<bf16_t>(x, gamma, beta, static_cast<bf16_t*>(out), rows, R, E, eps, stream);
   else
     return DN_ERR_DTYPE;
   return dn_launch_status();

@@ -111,14 +111,24 @@ __global__ __launch_bounds__(256) void gemm_kernel(const TI* __restrict__ A, int
 namespace skinny {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
-constexpr int UNROLL = 4;
+constexpr int UNROLL = 8;
 
-template <int MB, int WAVES, typename TC>
+// Where a fused projection's key and value columns go besides C: columns q_width .. of row m are
+// the keys, then the values, of the token whose slot is slot_map[m] (page * page_size + offset,
+// < 0: none).  Pools as in the cache: keys [page, Hkv, page_size, dh], values [page, Hkv, dh, page_size].
+struct KVScatter {
+  const int32_t* slot_map;
+  bf16_t* k_pool;
+  bf16_t* v_pool;
+  int q_width, kv_width, dh, page_size, Hkv;
+};
+
+template <int MB, int WAVES, typename TC, bool KV>
 __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restrict__ A, int lda,
                                                            const bf16_t* __restrict__ W,
                                                            const float* __restrict__ bias, TC* __restrict__ C,
                                                            int ldc, float* __restrict__ resid, int ldr, int M, int N,
-                                                           int K, int epi) {
+                                                           int K, int epi, KVScatter kv) {
   __shared__ floatx4 red[WAVES][MB][64];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int col = lane % 16, g = lane / 16;
@@ -176,7 +186,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
         float* x = resid + static_cast<size_t>(m) * ldr + nn;
         *x = *x + v;
       } else {
-        C[static_cast<size_t>(m) * ldc + nn] = from_float<TC>(apply_epilogue(v, epi));
+        TC cv = from_float<TC>(apply_epilogue(v, epi));
+        C[static_cast<size_t>(m) * ldc + nn] = cv;
+        if constexpr (KV) {
+          if (nn >= kv.q_width) {
+            int c = nn - kv.q_width;
+            const bool is_value = c >= kv.kv_width;
+            if (is_value) c -= kv.kv_width;
+            const int slot = kv.slot_map[m];
+            if (slot >= 0) {
+              const int page = slot / kv.page_size, off = slot % kv.page_size;
+              const int hh = c / kv.dh, d = c % kv.dh;
+              const size_t base = (static_cast<size_t>(page) * kv.Hkv + hh) * kv.page_size * kv.dh;
+              if (is_value)
+                kv.v_pool[base + static_cast<size_t>(d) * kv.page_size + off] = cv;
+              else
+                kv.k_pool[base + static_cast<size_t>(off) * kv.dh + d] = cv;
+            }
+          }
+        }
       }
     }
   }
@@ -184,25 +212,41 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
 
 template <int MB, int WAVES>
 static void launch(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr,
-                   int M, int N, int K, int out_dtype, int epi, hipStream_t stream) {
+                   int M, int N, int K, int out_dtype, int epi, const KVScatter* kv, hipStream_t stream) {
   dim3 grid((N + 15) / 16), block(WAVES * 64);
-  if (out_dtype == DN_BF16)
-    hipLaunchKernelGGL((gemm_kernel<MB, WAVES, bf16_t>), grid, block, 0, stream, static_cast<const bf16_t*>(A), lda,
-                       static_cast<const bf16_t*>(W), bias, static_cast<bf16_t*>(C), ldc, resid, ldr, M, N, K, epi);
+  KVScatter none{};
+  if (kv != nullptr)
+    hipLaunchKernelGGL((gemm_kernel<MB, WAVES, bf16_t, true>), grid, block, 0, stream,
+                       static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), bias,
+                       static_cast<bf16_t*>(C), ldc, resid, ldr, M, N, K, epi, *kv);
+  else if (out_dtype == DN_BF16)
+    hipLaunchKernelGGL((gemm_kernel<MB, WAVES, bf16_t, false>), grid, block, 0, stream,
+                       static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), bias,
+                       static_cast<bf16_t*>(C), ldc, resid, ldr, M, N, K, epi, none);
   else
-    hipLaunchKernelGGL((gemm_kernel<MB, WAVES, float>), grid, block, 0, stream, static_cast<const bf16_t*>(A), lda,
-                       static_cast<const bf16_t*>(W), bias, static_cast<float*>(C), ldc, resid, ldr, M, N, K, epi);
+    hipLaunchKernelGGL((gemm_kernel<MB, WAVES, float, false>), grid, block, 0, stream,
+                       static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), bias,
+                       static_cast<float*>(C), ldc, resid, ldr, M, N, K, epi, none);
 }
 
 template <int WAVES>
 static void launch_mb(int mb, const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid,
-                      int ldr, int M, int N, int K, int out_dtype, int epi, hipStream_t stream) {
+                      int ldr, int M, int N, int K, int out_dtype, int epi, const KVScatter* kv, hipStream_t stream) {
   switch (mb) {
-    case 1: launch<1, WAVES>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, stream); break;
-    case 2: launch<2, WAVES>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, stream); break;
-    case 3: launch<3, WAVES>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, stream); break;
-    default: launch<4, WAVES>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, stream); break;
+    case 1: launch<1, WAVES>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream); break;
+    case 2: launch<2, WAVES>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream); break;
+    case 3: launch<3, WAVES>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream); break;
+    default: launch<4, WAVES>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream); break;
   }
+}
+
+static void run(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr, int M,
+                int N, int K, int out_dtype, int epi, const KVScatter* kv, hipStream_t stream) {
+  int mb = (M + 15) / 16;
+  if (K >= 1024)
+    launch_mb<8>(mb, A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream);
+  else
+    launch_mb<4>(mb, A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream);
 }
 
 // operands must allow 16-byte loads: K and lda multiples of 8, bases aligned
@@ -212,6 +256,140 @@ static bool takes(const void* A, int lda, const void* W, int M, int K, int in_dt
 }
 }  // namespace skinny
 
+
+// ---------------------------------------------------------------------------------------
+// Many rows, bfloat16: the prefill's products, bound by the matrix cores.
+// A workgroup makes a 128 x 128 tile of C with 4 waves (2 x 2, each 64 x 64 as 2 x 2 tiles of
+// v_mfma_f32_32x32x16_bf16).  K advances 64 at a time: the next 128 x 64 slabs of A and W are
+// fetched into registers while the matrix cores work on the slabs in LDS.  In LDS a row is 8
+// chunks of 16 bytes, stored at chunk ^ (row & 7), so that the 32 rows a lane group reads fall
+// on different banks.  Workgroup ids are remapped so that tiles which share a slab of W run on
+// the same XCD (each XCD has its own L2; ids go round the 8 XCDs).
+// ---------------------------------------------------------------------------------------
+namespace tiled {
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+constexpr int BM = 128, BN = 128, BK = 64, XCDS = 8;
+
+template <typename TC>
+__global__ __launch_bounds__(256) void gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
+                                                    const float* __restrict__ bias, TC* __restrict__ C, int ldc,
+                                                    float* __restrict__ resid, int ldr, int M, int N, int K, int epi,
+                                                    int tiles_m, int tiles_n) {
+  __shared__ u32x4 As[BM * 8];
+  __shared__ u32x4 Ws[BN * 8];
+  // logical tile: consecutive ids on one XCD walk down a column of tiles (same slab of W)
+  const int total = tiles_m * tiles_n;
+  int pid = blockIdx.x;
+  {
+    const int per = (total + XCDS - 1) / XCDS;
+    const int l = (pid % XCDS) * per + pid / XCDS;
+    pid = l < total && (total % XCDS == 0) ? l : pid;   // the remap is a permutation only if total divides
+  }
+  const int tm = pid % tiles_m, tn = pid / tiles_m;
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int t = threadIdx.x, wave = t / 64, lane = t % 64;
+  const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;
+  const int r32 = lane % 32, g = lane / 32;
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  u32x4 pa[4], pw[4];
+  auto fetch = [&](int kt) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = t + u * 256, row = c / 8, ch = c % 8;
+      const int k = kt * BK + ch * 8;
+      const int m = m0 + row, n = n0 + row;
+      pa[u] = (m < M && k < K) ? *reinterpret_cast<const u32x4*>(A + static_cast<size_t>(m) * lda + k) : zero;
+      pw[u] = (n < N && k < K) ? *reinterpret_cast<const u32x4*>(W + static_cast<size_t>(n) * K + k) : zero;
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = t + u * 256, row = c / 8, ch = c % 8;
+      As[row * 8 + (ch ^ (row & 7))] = pa[u];
+      Ws[row * 8 + (ch ^ (row & 7))] = pw[u];
+    }
+  };
+  const int ktiles = (K + BK - 1) / BK;
+  fetch(0);
+  for (int kt = 0; kt < ktiles; ++kt) {
+    __syncthreads();          // the slabs in LDS have been used up
+    stash();
+    __syncthreads();
+    if (kt + 1 < ktiles) fetch(kt + 1);
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      bf16x8 af[2], wf[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int row = wm + i * 32 + r32;
+        af[i] = __builtin_bit_cast(bf16x8, As[row * 8 + ((kk * 2 + g) ^ (row & 7))]);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int row = wn + j * 32 + r32;
+        wf[j] = __builtin_bit_cast(bf16x8, Ws[row * 8 + ((kk * 2 + g) ^ (row & 7))]);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+    }
+  }
+  // acc[i][j][r]: row m0 + wm + 32 i + 8 (r / 4) + 4 g + r % 4, column n0 + wn + 32 j + lane % 32
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int n = n0 + wn + j * 32 + r32;
+    if (n >= N) continue;
+    const float bv = bias ? bias[n] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm + i * 32 + 8 * (r / 4) + 4 * g + (r % 4);
+        if (m >= M) continue;
+        float v = acc[i][j][r] + bv;
+        if (resid) {
+          float* x = resid + static_cast<size_t>(m) * ldr + n;
+          *x = *x + v;
+        } else {
+          C[static_cast<size_t>(m) * ldc + n] = from_float<TC>(apply_epilogue(v, epi));
+        }
+      }
+  }
+}
+
+static bool takes(const void* A, int lda, const void* W, int K, int in_dtype) {
+  return in_dtype == DN_BF16 && K % 8 == 0 && lda % 8 == 0 && reinterpret_cast<uintptr_t>(A) % 16 == 0 &&
+         reinterpret_cast<uintptr_t>(W) % 16 == 0;
+}
+
+static void run(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr, int M,
+                int N, int K, int out_dtype, int epi, hipStream_t stream) {
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  dim3 grid(tiles_m * tiles_n), block(256);
+  if (out_dtype == DN_BF16)
+    hipLaunchKernelGGL(gemm_kernel<bf16_t>, grid, block, 0, stream, static_cast<const bf16_t*>(A), lda,
+                       static_cast<const bf16_t*>(W), bias, static_cast<bf16_t*>(C), ldc, resid, ldr, M, N, K, epi,
+                       tiles_m, tiles_n);
+  else
+    hipLaunchKernelGGL(gemm_kernel<float>, grid, block, 0, stream, static_cast<const bf16_t*>(A), lda,
+                       static_cast<const bf16_t*>(W), bias, static_cast<float*>(C), ldc, resid, ldr, M, N, K, epi,
+                       tiles_m, tiles_n);
+}
+}  // namespace tiled
+
 extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid,
                        int ldr, int M, int N, int K, int in_dtype, int out_dtype, int epilogue,
                        hipStream_t stream) {
@@ -220,11 +398,11 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
   if (epilogue < EPI_NONE || epilogue > EPI_GELU_ERF) return DN_ERR_SHAPE;
   if (resid != nullptr && epilogue != EPI_NONE) return DN_ERR_SHAPE;
   if (skinny::takes(A, lda, W, M, K, in_dtype)) {
-    int mb = (M + 15) / 16;
-    if (K >= 1024)
-      skinny::launch_mb<8>(mb, A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, stream);
-    else
-      skinny::launch_mb<4>(mb, A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, stream);
+    skinny::run(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr, stream);
+    return dn_launch_status();
+  }
+  if (tiled::takes(A, lda, W, K, in_dtype)) {
+    tiled::run(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, stream);
     return dn_launch_status();
   }
   dim3 grid((N + plain::BN - 1) / plain::BN, (M + plain::BM - 1) / plain::BM), block(256);
@@ -242,5 +420,21 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
   else
     return DN_ERR_DTYPE;
 #undef DN_LAUNCH
+  return dn_launch_status();
+}
+
+// The fused projection q | k | v of a decode step: C = A . W^T + bias as above, and the key and
+// value columns also go to their pages (see KVScatter).  Returns 1 (nothing launched) if the
+// sizes are not those of the few-rows kernel: the caller then runs dn_gemm and the separate
+// cache write.
+extern "C" int dn_gemm_qkv(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, int M, int N,
+                           int K, const int32_t* slot_map, void* k_pool, void* v_pool, int q_width, int Hkv, int dh,
+                           int page_size, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (!skinny::takes(A, lda, W, M, K, DN_BF16)) return 1;
+  if (q_width < 0 || q_width + 2 * Hkv * dh != N || page_size < 1) return DN_ERR_SHAPE;
+  skinny::KVScatter kv{slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_width, Hkv * dh, dh,
+                       page_size, Hkv};
+  skinny::run(A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv, stream);
   return dn_launch_status();
 }

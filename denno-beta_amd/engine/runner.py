@@ -32,6 +32,10 @@ class ModelRunner:
                                   max_live=options.max_live, device=self.device)
         self.notes: List[str] = []
         self.steps_run = 0
+        self.graphs = None
+        if options.use_graphs and self.device.type == "cuda":
+            from .graphs import DecodeGraphs
+            self.graphs = DecodeGraphs(self)
 
     # -- construction --------------------------------------------------------------------
     @classmethod
@@ -76,6 +80,9 @@ class ModelRunner:
         entries = list(entries)
         if not entries:
             return torch.empty((0, self.spec.vocab), dtype=torch.float32, device=self.device)
+        if self.graphs is not None and self.graphs.takes(entries):
+            self.steps_run += 1
+            return self.graphs.step(entries)
         ctx = build_context(entries, self.cache, self.spec.vocab, self.spec.max_positions, self.device)
         logits = self.model.forward(ctx, self.cache)
         mgr = self.cache.manager

@@ -47,11 +47,12 @@ def _declare(name, lib):
         },
         "gemm": {
             "dn_gemm": [P, I, P, P, P, I, P, I, I, I, I, I, I, I, P],
+            "dn_gemm_qkv": [P, I, P, P, P, I, I, I, I, P, P, P, I, I, I, I, P],
         },
         "attention": {
             "dn_attention": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, I, P],
             "dn_attention_flash": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, P],
-            "dn_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, P, I, I, I, I, I, F, I, P],
+            "dn_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, F, I, P],
         },
         "sampling": {
             "dn_sample": [P, I, I, I, P, P, P, P],
@@ -204,6 +205,39 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
     return out
 
 
+def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
+    """out = a @ w.T + bias, the fused projection q | k | v; the key columns (q_width ..) and the
+    value columns after them also go to the slots slot_map[t] of the pools, as kv_write does.
+    One kernel where the few-rows product applies (a decode step in bfloat16), else two."""
+    n_pages, Hkv, ps, dh = k_pool.shape
+    kvw = Hkv * dh
+    if (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+            and a.shape[0] <= 64 and a.is_cuda):
+        _dev(a, "a", None, 2), _dev(w, "w", None, 2), _dev(out, "out", None, 2)
+        _dev(slot_map, "slot_map", _I32, 1), _dev(k_pool, "k_pool", (torch.bfloat16,), 4)
+        _dev(v_pool, "v_pool", (torch.bfloat16,), 4)
+        M, K = a.shape
+        N = w.shape[0]
+        _need(w.is_contiguous() and w.shape[1] == K and tuple(out.shape) == (M, N), "linear_qkv: shapes")
+        _need(N == q_width + 2 * kvw, "linear_qkv: columns are not q | k | v")
+        _need(k_pool.is_contiguous() and v_pool.is_contiguous() and tuple(v_pool.shape) == (n_pages, Hkv, dh, ps),
+              "linear_qkv: pools")
+        _need(slot_map.is_contiguous() and slot_map.shape[0] == M, "linear_qkv: slot_map")
+        if bias is not None:
+            _dev(bias, "bias", (torch.float32,), 1)
+            _need(bias.is_contiguous() and bias.shape[0] == N, "linear_qkv: bias")
+        rc = _lib("gemm").dn_gemm_qkv(a.data_ptr(), _rows(a, "a"), w.data_ptr(), _ptr(bias), out.data_ptr(),
+                                      _rows(out, "out"), M, N, K, slot_map.data_ptr(), k_pool.data_ptr(),
+                                      v_pool.data_ptr(), q_width, Hkv, dh, ps, _stream())
+        if rc == 0:
+            return out
+        if rc != 1:
+            _ok(rc, "linear_qkv")
+    linear(a, w, bias, out=out)
+    kv_write(out, q_width, q_width + kvw, slot_map, k_pool, v_pool)
+    return out
+
+
 FLASH_HEAD_DIMS = (16, 32, 48, 64, 96, 128)
 DECODE_HEAD_DIMS = (16, 32, 64, 128, 256)
 DECODE_SPLIT = 256
@@ -238,7 +272,11 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
     fast = q.dtype == torch.bfloat16 and ps % 16 == 0 and ldq % 8 == 0 and q.data_ptr() % 16 == 0
     if fast and single_rows and dh in DECODE_HEAD_DIMS and max_context > 0:
         n_tiles = tiles.shape[1]
-        n_splits = -(-max_context // DECODE_SPLIT)
+        # enough workgroups to fill the chip where the batch alone does not: about 512
+        total_chunks = -(-max_context // DECODE_SPLIT)
+        n_splits = max(1, min(total_chunks, 512 // max(1, n_tiles * n_heads)))
+        chunks = -(-total_chunks // n_splits)
+        n_splits = -(-total_chunks // chunks)
         _need(max_context <= block_tables.shape[1] * ps, "attention: max_context exceeds the block tables")
         part = torch.empty(n_tiles * n_heads * n_splits * (dh + 2) if n_splits > 1 else 1, dtype=torch.float32,
                            device=q.device)
@@ -246,7 +284,7 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
         _ok(lib.dn_attention_decode(
             q.data_ptr(), ldq, out.data_ptr(), ldo, k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(),
             block_tables.shape[1], base, base + 4 * n_tiles, base + 12 * n_tiles, n_tiles, part.data_ptr(), n_splits,
-            n_heads, Hkv, dh, ps, float(scale), int(window), _stream()), "attention (decode)")
+            chunks, n_heads, Hkv, dh, ps, float(scale), int(window), _stream()), "attention (decode)")
         return out
     if fast and tiles_wide is not None and dh in FLASH_HEAD_DIMS:
         _dev(tiles_wide, "tiles_wide", _I32, 2)

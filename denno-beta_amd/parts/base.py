@@ -51,7 +51,12 @@ class Runtime:
 
 
 class Part:
-    """Base of all parts.  `names` maps the part's own tensor names to checkpoint names."""
+    """Base of all parts.
+
+    graph_safe: the part's forward reads the step's tables on the device only (no loop over
+    requests on the host, no size taken from a table's contents), so a decode step with it can be
+    captured once as a HIP graph and replayed over new tables."""
+    graph_safe = False
 
     def param_specs(self) -> List[ParamSpec]:
         return []

@@ -12,6 +12,7 @@ class DenseMLP(Part):
     """act(h W_up + b_up) W_down + b_down, added into the residual stream
     (crates/denno-engine/src/model/gpt2.rs:211-219).  The activation runs in the first
     product's epilogue, in 32-bit, before the rounding to the activation dtype."""
+    graph_safe = True
 
     def __init__(self, width: int, inner: int, activation: str, up_weight: str, up_bias, down_weight: str,
                  down_bias, stored_in_out: bool = False, down_init_std: float = 0.02):

@@ -43,3 +43,14 @@ class Linear:
             return ops.linear(a, self.weight, self.bias, residual=residual)
         out = torch.empty((a.shape[0], self.out_features), dtype=out_dtype or a.dtype, device=a.device)
         return ops.linear(a, self.weight, self.bias, out=out, epilogue=epilogue)
+
+    def project_qkv(self, a, out_dtype, slot_map, k_pool, v_pool, q_width):
+        """The fused projection whose key and value columns also go to the cache's pages."""
+        if a.dtype != self.weight.dtype:
+            a = ops.cast(a.contiguous(), torch.empty(a.shape, dtype=self.weight.dtype, device=a.device))
+        out = torch.empty((a.shape[0], self.out_features), dtype=out_dtype, device=a.device)
+        if out_dtype != a.dtype:
+            ops.linear(a, self.weight, self.bias, out=out)
+            ops.kv_write(out, q_width, q_width + (self.out_features - q_width) // 2, slot_map, k_pool, v_pool)
+            return out
+        return ops.linear_qkv(a, self.weight, self.bias, out, slot_map, k_pool, v_pool, q_width)

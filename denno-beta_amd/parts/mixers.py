@@ -17,6 +17,7 @@ class CausalSelfAttention(Part):
     n_kv_heads < n_heads: query head h reads key head h // (n_heads // n_kv_heads).
     window > 0: a query at position p reads keys p - window + 1 .. p only.
     scale multiplies the scores before the softmax."""
+    graph_safe = True
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                  qkv_weight: str, qkv_bias, out_weight: str, out_bias, stored_in_out: bool = False,
@@ -45,10 +46,11 @@ class CausalSelfAttention(Part):
 
     def forward(self, h, ctx, cache, accumulate_into):
         act = self.runtime.act_dtype
-        qkv = self.qkv(h, out_dtype=act)
         g = ctx.groups[cache.group]
         if cache.writes:
-            ops.kv_write(qkv, self.q_width, self.q_width + self.kv_width, g.slot_map, cache.k, cache.v)
+            qkv = self.qkv.project_qkv(h, act, g.slot_map, cache.k, cache.v, self.q_width)
+        else:
+            qkv = self.qkv(h, out_dtype=act)
         o = torch.empty((h.shape[0], self.q_width), dtype=act, device=h.device)
         ops.attention(qkv[:, :self.q_width], o, cache.k, cache.v, g.block_tables, g.tiles, self.n_heads,
                       self.scale, self.window, tiles_wide=g.tiles_wide, single_rows=g.single_rows,

@@ -86,6 +86,7 @@ class DecoderModel:
         self.head = None if spec.head_weight is None else Linear(spec.width, spec.vocab, spec.head_weight, None)
         self._check_run_order()
         self.runtime = None
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in self.all_parts())
 
     # -- description ---------------------------------------------------------------------
     def _check_run_order(self):

@@ -12,6 +12,7 @@ from .base import NORMS, Part
 class LayerNorm(Part):
     """(x - mean) / sqrt(var + eps) * weight + bias, statistics and affine in 32-bit
     (crates/denno-engine/src/tensor.rs:1101-1112)."""
+    graph_safe = True
 
     def __init__(self, width: int, eps: float, weight_name: str, bias_name=None):
         self.width, self.eps = width, eps

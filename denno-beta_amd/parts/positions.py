@@ -12,6 +12,7 @@ from .base import POSITIONS, Part
 
 class TokenEmbedding(Part):
     """The token table [vocab, width]; also the head's weight when the head is tied."""
+    graph_safe = True
 
     def __init__(self, vocab: int, width: int, name: str):
         self.vocab, self.width, self.name = vocab, width, name
@@ -27,6 +28,7 @@ class TokenEmbedding(Part):
 @POSITIONS.register("learned_absolute")
 class LearnedAbsolutePositions(Part):
     """x[i] += wpe[position_i]                    (crates/denno-engine/src/model/gpt2.rs:142-150)"""
+    graph_safe = True
 
     def __init__(self, n_positions: int, width: int, name: str):
         self.n_positions, self.width, self.name = n_positions, width, name
@@ -47,6 +49,7 @@ class LearnedAbsolutePositions(Part):
 
 @POSITIONS.register("none")
 class NoPositions(Part):
+    graph_safe = True
     def __init__(self):
         pass
 

@@ -51,7 +51,8 @@ def cast(x, out):
 
 
 def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
-    y = a.float() @ w.float().t()
+    wide = torch.float64 if a.dtype == torch.float64 else torch.float32
+    y = a.to(wide) @ w.to(wide).t()
     if bias is not None:
         y = y + bias
     if residual is not None:
@@ -133,4 +134,11 @@ def sample_top(logits, rows, temperature, uniform, top_k, top_p, out):
         p = float(top_p[j])
         out[r] = sp.top_k_top_p(logits[r].tolist(), float(temperature[r]), min(k, 2048),
                                 None if p >= 1.0 else p, float(uniform[r]))
+    return out
+
+
+def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
+    linear(a, w, bias, out=out)
+    kvw = k_pool.shape[1] * k_pool.shape[3]
+    kv_write(out, q_width, q_width + kvw, slot_map, k_pool, v_pool)
     return out

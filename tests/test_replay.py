@@ -120,3 +120,41 @@ def test_step_refuses_what_it_cannot_run(backend, model_folders):
     assert r.cache.manager.length(0) == 0
     assert r.step([StepEntry(0, [1, 2, 3], [2])]).shape == (1, 512)
     assert r.cache.manager.length(0) == 3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_graphs_replay_what_eager_steps_compute(model_folders, dtype):
+    """Decode steps come from captured HIP graphs.  Every replay is checked against the same step
+    run kernel by kernel, over several batch sizes and context lengths, with eager steps (prompts
+    of other requests) and synchronisations between the replays."""
+    from denno_beta_amd.config import EngineOptions
+    from denno_beta_amd.engine import ModelRunner, StepEntry
+    folder = model_folders("C", dtype)
+    vocab = TINY["C"][0]["vocab_size"]
+    mk = lambda graphs: ModelRunner.from_folder(folder, EngineOptions(   # noqa: E731
+        dtype=dtype, page_size=16, cache_tokens=4096, max_live=8, use_graphs=graphs))
+    a, b = mk(True), mk(False)
+    assert a.graphs is not None and b.graphs is None
+    seqs = [seeded_tokens(70 + i, n, vocab) for i, n in enumerate((300, 5, 250, 40, 90))]
+    fed = [0] * len(seqs)
+    live = []
+    for step in range(70):
+        if step % 12 == 0 and len(live) < len(seqs):          # a new request: its prompt runs eagerly in both
+            i = len(live)
+            live.append(i)
+            n = max(1, min(len(seqs[i]) - 60, 260))
+            for r in (a, b):
+                r.start_request(i)
+                r.step([StepEntry(i, seqs[i][:n], [])])
+            fed[i] = n
+        entries = [StepEntry(i, seqs[i][fed[i]:fed[i] + 1], [0]) for i in live if fed[i] < len(seqs[i]) and (step + i) % 5]
+        if not entries:
+            continue
+        la, lb = a.step(entries).cpu(), b.step(entries).cpu()
+        for e in entries:
+            fed[e.rid] += 1
+        assert torch.equal(la, lb), f"step {step}: a replayed graph differs from the eager step"
+        if step % 7 == 0:
+            torch.cuda.synchronize()
+    assert len(a.graphs.graphs) >= 3, "several batch and context buckets were to be captured"

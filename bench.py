@@ -46,6 +46,8 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0: all)")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    ap.add_argument("--only", choices=["decode", "prefill"], default=None,
+                    help="run one workload and print a short line (for profiling)")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
@@ -101,7 +103,14 @@ def main():
                 runner.end_request(1000 + j)
         return sorted(times[1:])[len(times[1:]) // 2]
 
+    if a.only == "prefill":
+        t = prefill_point()
+        print(json.dumps({"prefill_ms": t * 1e3, "tokens": 2048}))
+        return
     step_s, mean_ctx = decode_point(a.batch, a.steps, a.warmup)
+    if a.only == "decode":
+        print(json.dumps({"decode_ms_per_step": step_s * 1e3, "batch": a.batch, "mean_context": mean_ctx}))
+        return
     weight_bytes = runner.model.weight_bytes()
     kv_bytes = a.batch * mean_ctx * runner.cache.bytes_per_token()
     achieved = (weight_bytes + kv_bytes) / step_s / 1e9

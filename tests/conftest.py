@@ -20,7 +20,10 @@ TINY_B = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=3, n
 TINY_C = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n_embd=96, n_head=3,
               n_inner=200, vocab_size=777, n_positions=640, layer_norm_epsilon=1e-5,
               activation_function="gelu_new", scale_attn_weights=True)
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+# a fourth with the head size and context of the large models (4 heads of 64, 1024 positions)
+TINY_D = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n_embd=256, n_head=4,
+              vocab_size=5003, n_positions=1024, layer_norm_epsilon=1e-5, activation_function="gelu_new")
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
 
 
 def pytest_configure(config):

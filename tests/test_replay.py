@@ -158,3 +158,33 @@ def test_decode_graphs_replay_what_eager_steps_compute(model_folders, dtype):
         if step % 7 == 0:
             torch.cuda.synchronize()
     assert len(a.graphs.graphs) >= 3, "several batch and context buckets were to be captured"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_context_with_heads_of_64(model_folders, dtype):
+    """The head size and context length of the large models: a 1,000-token request in portions, with
+    decoding at the end, beside a second request, so that the keys of a row span dozens of pages."""
+    folder = model_folders("D", dtype)
+    seqs = sequences("D", (1000, 300))
+    want = plain_logits(folder, seqs)
+    steps = U.mixed_trace(seqs, seed=4, sizes=(1, 1, 2, 64, 200, 333))
+    r = runner_for(folder, dtype, "cuda:0", cache_tokens=U.max_live_tokens(steps))
+    got = U.replay(r, steps)
+    for i in range(2):
+        U.assert_close(got[f"r{i}"], want[i], dtype, f"long context {dtype} request {i}")
+
+
+def test_weights_stored_in_32_bit_stay_so_in_a_bfloat16_engine(backend, model_folders):
+    """A folder stored in 32-bit, run with --dtype bfloat16: the matrices stay 32-bit and their
+    products run in 32-bit on widened activations; the result is at least as close to the plain
+    implementation as with bfloat16 weights."""
+    folder = model_folders("A", "float32")
+    seqs = sequences("A", (40, 23))
+    want = plain_logits(folder, seqs)
+    steps = U.mixed_trace(seqs, seed=6)
+    r = runner_for(folder, "bfloat16", backend, cache_tokens=U.max_live_tokens(steps))
+    assert r.notes and r.model.blocks[0].mixer.qkv.weight.dtype == torch.float32
+    got = U.replay(r, steps)
+    for i in range(2):
+        U.assert_close(got[f"r{i}"], want[i], "bfloat16", f"32-bit weights in a bfloat16 engine, request {i}")

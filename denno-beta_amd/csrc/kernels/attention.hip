@@ -93,8 +93,7 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
         tmax = fmaxf(tmax, s[c]);
       }
     }
-#pragma unroll
-    for (int mask = 8; mask >= 1; mask >>= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, mask, DN_WAVE));
+    tmax = group_reduce<16>(tmax, MaxOp());
 
     float alpha = 1.f, psum = 0.f;
     if (tmax > NEG_INF) {
@@ -114,8 +113,7 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
       for (int c = 0; c < 4; ++c)
         if (c < nc) Ps[qi * BK + g + 16 * c] = 0.f;
     }
-#pragma unroll
-    for (int mask = 8; mask >= 1; mask >>= 1) psum += __shfl_xor(psum, mask, DN_WAVE);
+    psum = group_reduce<16>(psum, SumOp());
     l = l * alpha + psum;
     __syncthreads();
 
@@ -243,12 +241,18 @@ __global__ __launch_bounds__(256) void kernel(const bf16_t* __restrict__ q, int 
     for (int i = 0; i < 16; ++i) s[i] = 0.f;
     {
       const int key = kt + qcol;      // as A operand the lane's row is a key
-      int page = key <= hi_w ? bt[key / page_size] : -1;
-      const bf16_t* kr = k_pool + ((static_cast<size_t>(max(page, 0)) * Hkv + hk) * page_size + key % page_size) * DH + g * 8;
+      // loads are never conditional: a key outside reads the tile's first key instead and is dropped
+      const int kk = key <= hi_w ? key : hi_w;
+      const int page = bt[kk / page_size];
+      const bool ok = key <= hi_w && page >= 0;
+      const bf16_t* kr = k_pool + ((static_cast<size_t>(max(page, 0)) * Hkv + hk) * page_size + kk % page_size) * DH + g * 8;
+      bf16x8 kf[DH16];
+#pragma unroll
+      for (int c = 0; c < DH16; ++c) kf[c] = *reinterpret_cast<const bf16x8*>(kr + c * 16);
 #pragma unroll
       for (int c = 0; c < DH16; ++c) {
-        bf16x8 kf = page >= 0 ? *reinterpret_cast<const bf16x8*>(kr + c * 16) : zero8;
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[c], s, 0, 0, 0);
+        if (!ok) kf[c] = zero8;
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[c], qf[c], s, 0, 0, 0);
       }
     }
     // s[i]: key kt + 8*(i/4) + 4*g + i%4, query = this lane's column
@@ -260,7 +264,7 @@ __global__ __launch_bounds__(256) void kernel(const bf16_t* __restrict__ q, int 
       s[i] = ok ? s[i] * scale : NEG_INF;
       tmax = fmaxf(tmax, s[i]);
     }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, DN_WAVE));
+    tmax = fmaxf(tmax, other_half(tmax));
     float p[16];
     float psum = 0.f, alpha = 1.f;
     if (tmax > NEG_INF) {
@@ -276,7 +280,7 @@ __global__ __launch_bounds__(256) void kernel(const bf16_t* __restrict__ q, int 
 #pragma unroll
       for (int i = 0; i < 16; ++i) p[i] = 0.f;
     }
-    psum += __shfl_xor(psum, 32, DN_WAVE);
+    psum += other_half(psum);
     l = l * alpha + psum;
     bf16x8 pb[2];
 #pragma unroll
@@ -297,13 +301,11 @@ __global__ __launch_bounds__(256) void kernel(const bf16_t* __restrict__ q, int 
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         const int d = 32 * db + qcol;   // as A operand the lane's row is a dim
-        bf16x8 vf = zero8;
-        if (d < DH) {
-          const bf16_t* vr = vb + static_cast<size_t>(d) * page_size;
-          bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(vr);
-          bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(vr + 8);
-          vf = bf16x8{lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-        }
+        const bf16_t* vr = vb + static_cast<size_t>(min(d, DH - 1)) * page_size;
+        bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(vr);
+        bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(vr + 8);
+        bf16x8 vf = bf16x8{lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+        if (d >= DH) vf = zero8;
         o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[a0], o[db], 0, 0, 0);
       }
     }
@@ -417,42 +419,31 @@ __global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__
   for (int c = 0; c < chunks; ++c) {
     const int kbase = key0 + c * CHUNK + wave * 64;
     if (kbase > pos || kbase + 64 <= lo) continue;     // the same for the whole wave; no barrier in this loop
-    // scores: lane (key group grp, part sub of the key) ; afterwards lane j holds key kbase + j
-    float s = NEG_INF;
+    // scores: lane (key group grp, part sub of the key); after the sum over the key's lanes every
+    // lane of group grp holds, in sc[it], the score of key kbase + it * KPI + grp
+    float sc[LPK];
 #pragma unroll
     for (int it0 = 0; it0 < LPK; it0 += GROUP) {
       bf16x8 kv[GROUP];
-      bool valid[GROUP];
 #pragma unroll
       for (int u = 0; u < GROUP; ++u) {
         const int key = kbase + (it0 + u) * KPI + grp;
-        valid[u] = key >= lo && key <= pos;
-        const int kk = valid[u] ? key : pos;            // a key that surely has a page
+        const int kk = (key >= lo && key <= pos) ? key : pos;     // a key that surely has a page
         const int page = bt[kk / page_size];
         kv[u] = *reinterpret_cast<const bf16x8*>(
             k_pool + ((static_cast<size_t>(page) * Hkv + hk) * page_size + kk % page_size) * DH + sub * 8);
       }
 #pragma unroll
       for (int u = 0; u < GROUP; ++u) {
+        const int key = kbase + (it0 + u) * KPI + grp;
         float dot = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) dot = fmaf(qr[i], static_cast<float>(kv[u][i]), dot);
-#pragma unroll
-        for (int msk = LPK / 2; msk >= 1; msk >>= 1) dot += __shfl_xor(dot, msk, DN_WAVE);
-        if (!valid[u]) dot = NEG_INF;
-        // key j = (it0 + u) * KPI + g was made by group g: lane j takes it in its turn
-        float got = __shfl(dot, (lane % KPI) * LPK, DN_WAVE);
-        if (lane / KPI == it0 + u) s = got;
+        dot = group_reduce<LPK>(dot, SumOp());
+        sc[it0 + u] = (key >= lo && key <= pos) ? dot : NEG_INF;
       }
     }
-    const float m_c = wave_max(s);
-    if (!(m_c > NEG_INF)) continue;
-    const float m_new = fmaxf(m_run, m_c);
-    const float alpha = m_run > NEG_INF ? __expf(m_run - m_new) : 0.f;
-    const float p = s > NEG_INF ? __expf(s - m_new) : 0.f;
-    l_run = l_run * alpha + wave_sum(p);
-    m_run = m_new;
-    // values: lane = dim; 16 keys of one page at a time, all four loads of the 64 keys first
+    // values: lane = dim; 16 keys of one page at a time, all loads of the 64 keys before their use
     bf16x8 v0[4][DPL], v1[4][DPL];
     bool live[4];
 #pragma unroll
@@ -470,6 +461,23 @@ __global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__
         v1[blk][i] = *reinterpret_cast<const bf16x8*>(vb + static_cast<size_t>(d) * page_size + 8);
       }
     }
+    float m_c = NEG_INF;
+#pragma unroll
+    for (int it = 0; it < LPK; ++it) m_c = fmaxf(m_c, sc[it]);
+    m_c = wave_max(m_c);
+    if (!(m_c > NEG_INF)) continue;
+    const float m_new = fmaxf(m_run, m_c);
+    const float alpha = m_run > NEG_INF ? __expf(m_run - m_new) : 0.f;
+    float p[LPK];
+    float psum = 0.f;
+#pragma unroll
+    for (int it = 0; it < LPK; ++it) {
+      p[it] = sc[it] > NEG_INF ? __expf(sc[it] - m_new) : 0.f;
+      psum += p[it];
+    }
+    // each key is held by LPK lanes: its first lane counts it
+    l_run = l_run * alpha + wave_sum(sub == 0 ? psum : 0.f);
+    m_run = m_new;
 #pragma unroll
     for (int i = 0; i < DPL; ++i) acc[i] *= alpha;
 #pragma unroll
@@ -477,7 +485,8 @@ __global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__
       if (!live[blk]) continue;
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
-        const float pj = __shfl(p, blk * 16 + j, DN_WAVE);
+        const int key = blk * 16 + j;      // key = it * KPI + grp: held by lane grp * LPK in p[it]
+        const float pj = lane_value(p[key / KPI], (key % KPI) * LPK);
 #pragma unroll
         for (int i = 0; i < DPL; ++i)
           acc[i] = fmaf(pj, static_cast<float>(j < 8 ? v0[blk][i][j] : v1[blk][i][j - 8]), acc[i]);

@@ -30,21 +30,67 @@ __device__ __forceinline__ float from_float<float>(float f) {
 // round to nearest even; NaN stays NaN
 template <>
 __device__ __forceinline__ bf16_t from_float<bf16_t>(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return bf16_t{static_cast<uint16_t>((u >> 16) | 0x40u)};
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return bf16_t{static_cast<uint16_t>(u >> 16)};
+  const uint32_t u = __float_as_uint(f);
+  const uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  const uint32_t quiet = (u >> 16) | 0x40u;
+  const bool is_nan = (u & 0x7fffffffu) > 0x7f800000u;   // a select, not a branch
+  return bf16_t{static_cast<uint16_t>(is_nan ? quiet : rounded)};
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int m = DN_WAVE / 2; m >= 1; m >>= 1) v += __shfl_xor(v, m, DN_WAVE);
+// Exchanges between lanes without LDS.  A butterfly through ds_bpermute costs a trip to LDS per
+// step; these run in the vector ALU: DPP inside a row of 16 lanes (xor 1, xor 2, then the
+// mirrors of 8 and of 16 lanes, which pair lanes as well as xor 4 and xor 8 do once the quads
+// agree), v_readlane to carry the four rows' results to every lane, and gfx950's
+// v_permlane32_swap where the two halves of a wave exchange a value each.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+#define DN_DPP_XOR1 0xB1          // quad_perm [1,0,3,2]
+#define DN_DPP_XOR2 0x4E          // quad_perm [2,3,0,1]
+#define DN_DPP_HALF_MIRROR 0x141  // lane i <-> 7 - i of each 8
+#define DN_DPP_MIRROR 0x140       // lane i <-> 15 - i of each 16
+
+struct SumOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+struct MaxOp {
+  __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+};
+
+// lane `lane`'s value, the same for every lane (lane is a constant)
+__device__ __forceinline__ float lane_value(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// every lane of each aligned group of N lanes (N = 2, 4, 8, 16, 32, 64) gets the group's result;
+// rows are joined in the order 0, 1, 2, 3
+template <int N, typename Op>
+__device__ __forceinline__ float group_reduce(float v, Op op) {
+  if (N >= 2) v = op(v, dpp_move<DN_DPP_XOR1>(v));
+  if (N >= 4) v = op(v, dpp_move<DN_DPP_XOR2>(v));
+  if (N >= 8) v = op(v, dpp_move<DN_DPP_HALF_MIRROR>(v));
+  if (N >= 16) v = op(v, dpp_move<DN_DPP_MIRROR>(v));
+  if (N >= 32) {
+    const float lower = op(lane_value(v, 0), lane_value(v, 16));
+    const float upper = op(lane_value(v, 32), lane_value(v, 48));
+    v = N >= 64 ? op(lower, upper) : ((threadIdx.x & 32) ? upper : lower);
+  }
   return v;
 }
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int m = DN_WAVE / 2; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, DN_WAVE));
-  return v;
+__device__ __forceinline__ float wave_sum(float v) { return group_reduce<DN_WAVE>(v, SumOp()); }
+__device__ __forceinline__ float wave_max(float v) { return group_reduce<DN_WAVE>(v, MaxOp()); }
+
+// The value that the lane 32 away holds.  v_permlane32_swap exchanges the upper half of its
+// first register with the lower half of its second; it is written as assembly with both
+// registers named as changed (through the compiler's builtin the second result is lost), and
+// with the idle cycles that the instruction wants before and after it, which the compiler does
+// not add around assembly.
+__device__ __forceinline__ float other_half(float v) {
+  unsigned a = __builtin_bit_cast(unsigned, v), b = a;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  // a: the lower half's values in both halves; b: the upper half's
+  return __builtin_bit_cast(float, (threadIdx.x & 32) ? a : b);
 }
 
 static inline int dn_launch_status() { return static_cast<int>(hipGetLastError()); }

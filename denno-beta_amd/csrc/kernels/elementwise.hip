@@ -94,12 +94,19 @@ __global__ __launch_bounds__(256) void layernorm_row_kernel(const float* __restr
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
   const float* xr = x + static_cast<size_t>(src) * E;
-  float v[VPT];
+  // loads are never conditional (a predicated load waits for the one before it)
+  float v[VPT], gm[VPT], bt[VPT];
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    int e = min(static_cast<int>(threadIdx.x) + i * 256, E - 1);
+    v[i] = xr[e];
+    gm[i] = gamma[e];
+    bt[i] = beta ? beta[e] : 0.f;
+  }
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
-    int e = threadIdx.x + i * 256;
-    v[i] = e < E ? xr[e] : 0.f;
+    if (static_cast<int>(threadIdx.x) + i * 256 >= E) v[i] = 0.f;
     s += v[i];
   }
   const float mean = block_sum_256(s, scratch) / static_cast<float>(E);
@@ -116,8 +123,8 @@ __global__ __launch_bounds__(256) void layernorm_row_kernel(const float* __restr
   for (int i = 0; i < VPT; ++i) {
     int e = threadIdx.x + i * 256;
     if (e < E) {
-      float y = (v[i] - mean) * inv * gamma[e];
-      if (beta) y += beta[e];
+      float y = (v[i] - mean) * inv * gm[i];
+      if (beta) y += bt[i];
       o[e] = from_float<TO>(y);
     }
   }

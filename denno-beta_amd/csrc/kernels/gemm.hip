@@ -135,6 +135,37 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   const int n0 = blockIdx.x * 16;
   const int n = min(n0 + col, N - 1);          // a tail tile reads the last row again; its result is not stored
   const bf16_t* wrow = W + static_cast<size_t>(n) * K + g * 8;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int ksteps = (K + 31) / 32;
+
+  // the first round of W is on its way while the prologue works
+  // what the epilogue will read (bias, the residual stream) is asked for first of all: thread o of
+  // the first MB * 64 threads finishes row block o / 64, lane slot o % 64
+  float epi_bias = 0.f;
+  float epi_x[4] = {0.f, 0.f, 0.f, 0.f};
+  if (threadIdx.x < MB * 64) {
+    const int ln = threadIdx.x % 64, emb = threadIdx.x / 64;
+    const int nn = min(n0 + ln % 16, N - 1);
+    if (bias) epi_bias = bias[nn];
+    if (resid) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = min(emb * 16 + (ln / 16) * 4 + r, M - 1);
+        epi_x[r] = resid[static_cast<size_t>(m) * ldr + nn];
+      }
+    }
+  }
+  // Loads are never conditional and nothing uses a loaded value before all loads of a round are
+  // issued (a predicated load, or a use in between, makes each load wait for the one before it).
+  // A step beyond K reads W's first row instead (finite numbers) and meets a zeroed piece of A.
+  bf16x8 b[UNROLL];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    int ks = wave + u * WAVES;
+    bool ok = ks < ksteps && ks * 32 + g * 8 < K;
+    b[u] = *reinterpret_cast<const bf16x8*>(ok ? wrow + ks * 32 : W);
+  }
+
   const bf16_t* arow[MB];
   bool a_ok[MB];
 #pragma unroll
@@ -146,18 +177,24 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   floatx4 acc[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) acc[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  const int ksteps = (K + 31) / 32;
   for (int ks0 = wave; ks0 < ksteps; ks0 += WAVES * UNROLL) {
-    bf16x8 b[UNROLL], a[UNROLL][MB];
+    bf16x8 a[UNROLL][MB];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       int ks = ks0 + u * WAVES;
       bool ok = ks < ksteps && ks * 32 + g * 8 < K;
-      b[u] = ok ? *reinterpret_cast<const bf16x8*>(wrow + ks * 32) : zero;
+      if (ks0 != wave) b[u] = *reinterpret_cast<const bf16x8*>(ok ? wrow + ks * 32 : W);
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
-        a[u][mb] = (ok && a_ok[mb]) ? *reinterpret_cast<const bf16x8*>(arow[mb] + ks * 32) : zero;
+        a[u][mb] = *reinterpret_cast<const bf16x8*>(ok ? arow[mb] + ks * 32 : arow[mb]);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      int ks = ks0 + u * WAVES;
+      bool ok = ks < ksteps && ks * 32 + g * 8 < K;
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+        if (!(ok && a_ok[mb])) a[u][mb] = zero;
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u)
@@ -169,22 +206,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   for (int mb = 0; mb < MB; ++mb) red[wave][mb][lane] = acc[mb];
   __syncthreads();
   // acc[mb][r] of lane (col, g) is row mb*16 + g*4 + r, column n0 + col
-  for (int o = threadIdx.x; o < MB * 64; o += WAVES * 64) {
-    int mb = o / 64, ln = o % 64;
+  if (threadIdx.x < MB * 64) {      // WAVES >= MB: one pass
+    const int mb = threadIdx.x / 64, ln = threadIdx.x % 64;
+    const int nn = n0 + ln % 16;
+    const float bv = epi_bias;
     floatx4 s = red[0][mb][ln];
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) s += red[w][mb][ln];
-    int nn = n0 + ln % 16;
-    if (nn >= N) continue;
-    float bv = bias ? bias[nn] : 0.f;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       int m = mb * 16 + (ln / 16) * 4 + r;
-      if (m >= M) continue;
+      if (m >= M || nn >= N) continue;
       float v = s[r] + bv;
       if (resid) {
-        float* x = resid + static_cast<size_t>(m) * ldr + nn;
-        *x = *x + v;
+        resid[static_cast<size_t>(m) * ldr + nn] = epi_x[r] + v;
       } else {
         TC cv = from_float<TC>(apply_epilogue(v, epi));
         C[static_cast<size_t>(m) * ldc + nn] = cv;
@@ -210,43 +245,43 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   }
 }
 
+struct Call {
+  const void* A; int lda; const void* W; const float* bias; void* C; int ldc; float* resid; int ldr;
+  int M, N, K, out_dtype, epi;
+  const KVScatter* kv;
+};
+
+template <int MB, int WAVES, typename TC, bool KV>
+static void launch_one(const Call& c, hipStream_t stream) {
+  dim3 grid((c.N + 15) / 16), block(WAVES * 64);
+  KVScatter kv = c.kv ? *c.kv : KVScatter{};
+  hipLaunchKernelGGL((gemm_kernel<MB, WAVES, TC, KV>), grid, block, 0, stream, static_cast<const bf16_t*>(c.A), c.lda,
+                     static_cast<const bf16_t*>(c.W), c.bias, static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N,
+                     c.K, c.epi, kv);
+}
+
 template <int MB, int WAVES>
-static void launch(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr,
-                   int M, int N, int K, int out_dtype, int epi, const KVScatter* kv, hipStream_t stream) {
-  dim3 grid((N + 15) / 16), block(WAVES * 64);
-  KVScatter none{};
-  if (kv != nullptr)
-    hipLaunchKernelGGL((gemm_kernel<MB, WAVES, bf16_t, true>), grid, block, 0, stream,
-                       static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), bias,
-                       static_cast<bf16_t*>(C), ldc, resid, ldr, M, N, K, epi, *kv);
-  else if (out_dtype == DN_BF16)
-    hipLaunchKernelGGL((gemm_kernel<MB, WAVES, bf16_t, false>), grid, block, 0, stream,
-                       static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), bias,
-                       static_cast<bf16_t*>(C), ldc, resid, ldr, M, N, K, epi, none);
-  else
-    hipLaunchKernelGGL((gemm_kernel<MB, WAVES, float, false>), grid, block, 0, stream,
-                       static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), bias,
-                       static_cast<float*>(C), ldc, resid, ldr, M, N, K, epi, none);
+static void launch(const Call& c, hipStream_t stream) {
+  if (c.kv) return launch_one<MB, WAVES, bf16_t, true>(c, stream);
+  if (c.out_dtype == DN_BF16) return launch_one<MB, WAVES, bf16_t, false>(c, stream);
+  return launch_one<MB, WAVES, float, false>(c, stream);
 }
 
 template <int WAVES>
-static void launch_mb(int mb, const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid,
-                      int ldr, int M, int N, int K, int out_dtype, int epi, const KVScatter* kv, hipStream_t stream) {
-  switch (mb) {
-    case 1: launch<1, WAVES>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream); break;
-    case 2: launch<2, WAVES>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream); break;
-    case 3: launch<3, WAVES>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream); break;
-    default: launch<4, WAVES>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream); break;
+static void launch_mb(const Call& c, hipStream_t stream) {
+  switch ((c.M + 15) / 16) {
+    case 1: launch<1, WAVES>(c, stream); break;
+    case 2: launch<2, WAVES>(c, stream); break;
+    case 3: launch<3, WAVES>(c, stream); break;
+    default: launch<4, WAVES>(c, stream); break;
   }
 }
 
-static void run(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr, int M,
-                int N, int K, int out_dtype, int epi, const KVScatter* kv, hipStream_t stream) {
-  int mb = (M + 15) / 16;
-  if (K >= 1024)
-    launch_mb<8>(mb, A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream);
+static void run(const Call& c, hipStream_t stream) {
+  if (c.K >= 1024)
+    launch_mb<8>(c, stream);
   else
-    launch_mb<4>(mb, A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream);
+    launch_mb<4>(c, stream);
 }
 
 // operands must allow 16-byte loads: K and lda multiples of 8, bases aligned
@@ -309,8 +344,15 @@ __global__ __launch_bounds__(256) void gemm_kernel(const bf16_t* __restrict__ A,
       const int c = t + u * 256, row = c / 8, ch = c % 8;
       const int k = kt * BK + ch * 8;
       const int m = m0 + row, n = n0 + row;
-      pa[u] = (m < M && k < K) ? *reinterpret_cast<const u32x4*>(A + static_cast<size_t>(m) * lda + k) : zero;
-      pw[u] = (n < N && k < K) ? *reinterpret_cast<const u32x4*>(W + static_cast<size_t>(n) * K + k) : zero;
+      // never a conditional load: an address outside is replaced by one inside, the value dropped
+      const bool ka = k < K, oka = ka && m < M, okw = ka && n < N;
+      pa[u] = *reinterpret_cast<const u32x4*>(A + static_cast<size_t>(oka ? m : 0) * lda + (oka ? k : 0));
+      pw[u] = *reinterpret_cast<const u32x4*>(W + static_cast<size_t>(okw ? n : 0) * K + (okw ? k : 0));
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {      // only A needs zeroing: what lies outside of W meets zeros of A or is not stored
+      const int c = t + u * 256, row = c / 8, ch = c % 8;
+      if (!(kt * BK + ch * 8 < K && m0 + row < M)) pa[u] = zero;
     }
   };
   auto stash = [&]() {
@@ -398,7 +440,8 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
   if (epilogue < EPI_NONE || epilogue > EPI_GELU_ERF) return DN_ERR_SHAPE;
   if (resid != nullptr && epilogue != EPI_NONE) return DN_ERR_SHAPE;
   if (skinny::takes(A, lda, W, M, K, in_dtype)) {
-    skinny::run(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr, stream);
+    skinny::Call c{A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr};
+    skinny::run(c, stream);
     return dn_launch_status();
   }
   if (tiled::takes(A, lda, W, K, in_dtype)) {
@@ -423,10 +466,10 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
   return dn_launch_status();
 }
 
-// The fused projection q | k | v of a decode step: C = A . W^T + bias as above, and the key and
-// value columns also go to their pages (see KVScatter).  Returns 1 (nothing launched) if the
-// sizes are not those of the few-rows kernel: the caller then runs dn_gemm and the separate
-// cache write.
+// The fused projection q | k | v of a decode step: C = A . W^T + bias as dn_gemm computes it, and
+// the key and value columns also go to their pages (see KVScatter).  Returns 1 (nothing
+// launched) if the sizes are not those of the few-rows kernel: the caller then runs dn_gemm and
+// the separate cache write.
 extern "C" int dn_gemm_qkv(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, int M, int N,
                            int K, const int32_t* slot_map, void* k_pool, void* v_pool, int q_width, int Hkv, int dh,
                            int page_size, hipStream_t stream) {
@@ -435,6 +478,7 @@ extern "C" int dn_gemm_qkv(const void* A, int lda, const void* W, const float* b
   if (q_width < 0 || q_width + 2 * Hkv * dh != N || page_size < 1) return DN_ERR_SHAPE;
   skinny::KVScatter kv{slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_width, Hkv * dh, dh,
                        page_size, Hkv};
-  skinny::run(A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv, stream);
+  skinny::Call c{A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv};
+  skinny::run(c, stream);
   return dn_launch_status();
 }

@@ -28,7 +28,7 @@ __device__ __forceinline__ Best better(Best a, Best b) {
 __device__ Best block_best(Best x, Best* scratch) {
 #pragma unroll
   for (int m = DN_WAVE / 2; m >= 1; m >>= 1) {
-    Best o{__shfl_xor(x.v, m, DN_WAVE), __shfl_xor(x.i, m, DN_WAVE)};
+    Best o{__shfl_xor(x.v, m, DN_WAVE), __shfl_xor(x.i, m, DN_WAVE)};   // once per row: the slow exchange will do
     x = better(x, o);
   }
   int wave = threadIdx.x / DN_WAVE, lane = threadIdx.x % DN_WAVE;

@@ -172,16 +172,13 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
-__device__ __forceinline__ __bf16 to_bf16(float f) {
-  bf16_t b = from_float<bf16_t>(f);
-  return __builtin_bit_cast(__bf16, b.bits);
-}
+__device__ __forceinline__ __bf16 to_bf16(float f) { return static_cast<__bf16>(f); }
 
 // ---------------------------------------------------------------------------------------
 // flash: portions of prompts.  A workgroup takes up to 128 consecutive rows of one request
 // and one head; each of its 4 waves owns 32 rows and walks the keys in tiles of 32 with
-// v_mfma_f32_32x32x16_bf16, operands straight from the pages (the waves of a workgroup read
-// the same keys at nearly the same time, so they meet in cache).
+// v_mfma_f32_32x32x16_bf16, operands straight from the pages, one tile ahead of their use (the
+// waves of a workgroup read the same keys at nearly the same time, so they meet in cache).
 //   S^T[key, q] = K . Q^T : lane (key = lane % 32, half g = lane / 32) gives 8 dims of a key.
 //   The result leaves each lane with 16 keys of ONE query (its column), so the running
 //   softmax is lane-local but for one exchange between the halves.
@@ -220,6 +217,7 @@ __global__ __launch_bounds__(256) void kernel(const bf16_t* __restrict__ q, int 
   const int lo_w = window > 0 ? max(0, pos0 + wrow0 - window + 1) : 0;
   const int hi_w = pos0 + min(wrow0 + 31, nrows - 1);
   const float NEG_INF = -INFINITY;
+  const float scale2 = scale * 1.44269504088896340736f;    // log2(e)
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
   bf16x8 qf[DH16];
@@ -235,44 +233,85 @@ __global__ __launch_bounds__(256) void kernel(const bf16_t* __restrict__ q, int 
     for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
   float m = NEG_INF, l = 0.f;
 
-  for (int kt = (lo_w / 32) * 32; kt <= hi_w; kt += 32) {
+  // The keys of the next tile and the values of this one are asked for before this tile's
+  // scores are computed, and the page numbers one tile further ahead still: what a tile needs has
+  // been on its way for a whole tile's arithmetic when it is used.  A tile of 32 keys lies in two
+  // pages (or in one, if pages are longer): pg[0] for keys kt .. kt+15, pg[1] for kt+16 .. kt+31.
+  auto pages_of = [&](int kt_, int* pg) {
+    pg[0] = kt_ <= hi_w ? bt[kt_ / page_size] : -1;
+    pg[1] = kt_ + 16 <= hi_w ? bt[(kt_ + 16) / page_size] : -1;
+  };
+  auto load_keys = [&](int kt_, const int* pg, bf16x8* kf) -> bool {
+    const int key = kt_ + qcol;      // as A operand the lane's row is a key
+    const int page = qcol < 16 ? pg[0] : pg[1];
+    const bool ok = key <= hi_w && page >= 0;
+    // never a conditional load: a key outside reads the pool's first key and is dropped
+    const bf16_t* kr = k_pool + (ok ? ((static_cast<size_t>(page) * Hkv + hk) * page_size + key % page_size) * DH : 0) + g * 8;
+#pragma unroll
+    for (int c = 0; c < DH16; ++c) kf[c] = *reinterpret_cast<const bf16x8*>(kr + c * 16);
+    return ok;
+  };
+  int kt = (lo_w / 32) * 32;
+  int pg[2], pg_next[2];
+  pages_of(kt, pg);
+  bf16x8 kf[DH16];
+  bool k_ok = load_keys(kt, pg, kf);
+  pages_of(kt + 32, pg_next);
+  for (; kt <= hi_w; kt += 32) {
+    // this tile's values: as A operand the lane's row is a dim, its 8 k slots the keys
+    // 16 a0 + 4 g + {0..3, 8..11} of the tile
+    bf16x4 vlo[2][DB], vhi[2][DB];
+#pragma unroll
+    for (int a0 = 0; a0 < 2; ++a0) {
+      const int kb = kt + 16 * a0;
+      const bf16_t* vb = v_pool + (pg[a0] >= 0 ? (static_cast<size_t>(pg[a0]) * Hkv + hk) * DH * page_size + kb % page_size : 0) + 4 * g;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const bf16_t* vr = vb + static_cast<size_t>(min(32 * db + qcol, DH - 1)) * page_size;
+        vlo[a0][db] = *reinterpret_cast<const bf16x4*>(vr);
+        vhi[a0][db] = *reinterpret_cast<const bf16x4*>(vr + 8);
+      }
+    }
+    bf16x8 kf_next[DH16];
+    const bool k_ok_next = load_keys(kt + 32, pg_next, kf_next);
+    int pg_far[2];
+    pages_of(kt + 64, pg_far);
+
     floatx16 s;
 #pragma unroll
     for (int i = 0; i < 16; ++i) s[i] = 0.f;
-    {
-      const int key = kt + qcol;      // as A operand the lane's row is a key
-      // loads are never conditional: a key outside reads the tile's first key instead and is dropped
-      const int kk = key <= hi_w ? key : hi_w;
-      const int page = bt[kk / page_size];
-      const bool ok = key <= hi_w && page >= 0;
-      const bf16_t* kr = k_pool + ((static_cast<size_t>(max(page, 0)) * Hkv + hk) * page_size + kk % page_size) * DH + g * 8;
-      bf16x8 kf[DH16];
 #pragma unroll
-      for (int c = 0; c < DH16; ++c) kf[c] = *reinterpret_cast<const bf16x8*>(kr + c * 16);
-#pragma unroll
-      for (int c = 0; c < DH16; ++c) {
-        if (!ok) kf[c] = zero8;
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[c], qf[c], s, 0, 0, 0);
-      }
-    }
-    // s[i]: key kt + 8*(i/4) + 4*g + i%4, query = this lane's column
+    for (int c = 0; c < DH16; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_ok ? kf[c] : zero8, qf[c], s, 0, 0, 0);
+    // s[i]: key kt + 8*(i/4) + 4*g + i%4, query = this lane's column.  Scores are kept times
+    // log2(e), so that each probability is one multiply-add and one v_exp_f32.  Only a tile that
+    // touches the causal edge (or the window's) of one of the wave's rows needs the mask; the
+    // others skip it, the same for the whole wave.
+    const bool edge = kt + 31 > pos0 + wrow0 || (window > 0 && kt < hi_w - window + 1);
     float tmax = NEG_INF;
+    if (edge) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      int key = kt + 8 * (i / 4) + 4 * g + (i % 4);
-      bool ok = row_ok && key >= my_lo && key <= my_pos;
-      s[i] = ok ? s[i] * scale : NEG_INF;
-      tmax = fmaxf(tmax, s[i]);
+      for (int i = 0; i < 16; ++i) {
+        int key = kt + 8 * (i / 4) + 4 * g + (i % 4);
+        bool ok = key >= my_lo && key <= my_pos;
+        s[i] = ok ? s[i] * scale2 : NEG_INF;
+        tmax = fmaxf(tmax, s[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        s[i] *= scale2;
+        tmax = fmaxf(tmax, s[i]);
+      }
     }
     tmax = fmaxf(tmax, other_half(tmax));
     float p[16];
     float psum = 0.f, alpha = 1.f;
     if (tmax > NEG_INF) {
       float m_new = fmaxf(m, tmax);
-      alpha = m > NEG_INF ? __expf(m - m_new) : 0.f;
+      alpha = __builtin_amdgcn_exp2f(m - m_new);      // m = -inf at first: 2^-inf = 0
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        p[i] = s[i] > NEG_INF ? __expf(s[i] - m_new) : 0.f;
+        p[i] = __builtin_amdgcn_exp2f(s[i] - m_new);  // a masked score is -inf: 0
         psum += p[i];
       }
       m = m_new;
@@ -294,21 +333,20 @@ __global__ __launch_bounds__(256) void kernel(const bf16_t* __restrict__ q, int 
       for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
 #pragma unroll
     for (int a0 = 0; a0 < 2; ++a0) {
-      const int kb = kt + 16 * a0;    // 16 keys of one page
-      int page = kb <= hi_w ? bt[kb / page_size] : -1;
-      if (page < 0) continue;         // the same for every lane of the wave
-      const bf16_t* vb = v_pool + (static_cast<size_t>(page) * Hkv + hk) * DH * page_size + kb % page_size + 4 * g;
+      if (pg[a0] < 0) continue;       // the same for every lane of the wave
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const int d = 32 * db + qcol;   // as A operand the lane's row is a dim
-        const bf16_t* vr = vb + static_cast<size_t>(min(d, DH - 1)) * page_size;
-        bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(vr);
-        bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(vr + 8);
-        bf16x8 vf = bf16x8{lo4[0], lo4[1], lo4[2], lo4[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-        if (d >= DH) vf = zero8;
+        bf16x8 vf = bf16x8{vlo[a0][db][0], vlo[a0][db][1], vlo[a0][db][2], vlo[a0][db][3],
+                           vhi[a0][db][0], vhi[a0][db][1], vhi[a0][db][2], vhi[a0][db][3]};
+        if (32 * db + qcol >= DH) vf = zero8;
         o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[a0], o[db], 0, 0, 0);
       }
     }
+#pragma unroll
+    for (int c = 0; c < DH16; ++c) kf[c] = kf_next[c];
+    k_ok = k_ok_next;
+    pg[0] = pg_next[0], pg[1] = pg_next[1];
+    pg_next[0] = pg_far[0], pg_next[1] = pg_far[1];
   }
   if (row_ok) {
     const float inv = 1.0f / l;

@@ -27,14 +27,11 @@ template <>
 __device__ __forceinline__ float from_float<float>(float f) {
   return f;
 }
-// round to nearest even; NaN stays NaN
+// round to nearest even; NaN stays NaN: gfx950 has the conversion in hardware (v_cvt_pk_bf16_f32),
+// which the compiler picks for a cast to __bf16
 template <>
 __device__ __forceinline__ bf16_t from_float<bf16_t>(float f) {
-  const uint32_t u = __float_as_uint(f);
-  const uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-  const uint32_t quiet = (u >> 16) | 0x40u;
-  const bool is_nan = (u & 0x7fffffffu) > 0x7f800000u;   // a select, not a branch
-  return bf16_t{static_cast<uint16_t>(is_nan ? quiet : rounded)};
+  return bf16_t{__builtin_bit_cast(uint16_t, static_cast<__bf16>(f))};
 }
 
 // Exchanges between lanes without LDS.  A butterfly through ds_bpermute costs a trip to LDS per

@@ -294,109 +294,126 @@ static bool takes(const void* A, int lda, const void* W, int M, int K, int in_dt
 
 // ---------------------------------------------------------------------------------------
 // Many rows, bfloat16: the prefill's products, bound by the matrix cores.
-// A workgroup makes a 128 x 128 tile of C with 4 waves (2 x 2, each 64 x 64 as 2 x 2 tiles of
-// v_mfma_f32_32x32x16_bf16).  K advances 64 at a time: the next 128 x 64 slabs of A and W are
-// fetched into registers while the matrix cores work on the slabs in LDS.  In LDS a row is 8
-// chunks of 16 bytes, stored at chunk ^ (row & 7), so that the 32 rows a lane group reads fall
-// on different banks.  Workgroup ids are remapped so that tiles which share a slab of W run on
-// the same XCD (each XCD has its own L2; ids go round the 8 XCDs).
+// A workgroup of 4 waves (2 x 2) makes a tile of C; each wave makes TM x TN tiles of
+// v_mfma_f32_32x32x16_bf16 (2 x 2: a 128 x 128 tile; 4 x 2 was measured slower: its registers and
+// LDS leave room for one wave per SIMD only, and nothing then hides the latency of LDS).  Two waves
+// per SIMD are asked for.  K advances BK (64 or 32) at a time through two sets of slabs in LDS: while the
+// matrix cores work on one set, the next slabs travel from memory to registers and then into
+// the other set; one barrier per step.  In LDS a row is BK/8 chunks of 16 bytes, chunk c stored
+// at c ^ swz(row), so that the rows a lane group reads fall on different banks.
+// Workgroup ids are remapped so that tiles which share a slab of W run on the same XCD (each
+// XCD has its own L2; ids go round the 8 XCDs).
 // ---------------------------------------------------------------------------------------
 namespace tiled {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
-constexpr int BM = 128, BN = 128, BK = 64, XCDS = 8;
+constexpr int XCDS = 8;
 
-template <typename TC>
-__global__ __launch_bounds__(256) void gemm_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
-                                                    const float* __restrict__ bias, TC* __restrict__ C, int ldc,
-                                                    float* __restrict__ resid, int ldr, int M, int N, int K, int epi,
-                                                    int tiles_m, int tiles_n) {
-  __shared__ u32x4 As[BM * 8];
-  __shared__ u32x4 Ws[BN * 8];
+template <typename TC, int TM, int TN, int BK>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(
+    const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const float* __restrict__ bias,
+    TC* __restrict__ C, int ldc, float* __restrict__ resid, int ldr, int M, int N, int K, int epi, int tiles_m,
+    int tiles_n) {
+  constexpr int BM = 64 * TM, BN = 64 * TN;
+  constexpr int CH = BK / 8;                              // 16-byte chunks in a row of a slab
+  constexpr int UA = BM * CH / 256, UW = BN * CH / 256;   // chunks per thread and slab
+  // a row's chunk c lies at c ^ swz(row): 16 consecutive rows then cover all 16 bank groups
+  auto swz = [](int row) { return (row / (16 / CH)) % CH; };
+  extern __shared__ u32x4 lds[];                          // [2][(BM + BN) * CH]
   // logical tile: consecutive ids on one XCD walk down a column of tiles (same slab of W)
   const int total = tiles_m * tiles_n;
   int pid = blockIdx.x;
-  {
-    const int per = (total + XCDS - 1) / XCDS;
-    const int l = (pid % XCDS) * per + pid / XCDS;
-    pid = l < total && (total % XCDS == 0) ? l : pid;   // the remap is a permutation only if total divides
-  }
+  if (total % XCDS == 0) pid = (pid % XCDS) * (total / XCDS) + pid / XCDS;   // a permutation if 8 divides total
   const int tm = pid % tiles_m, tn = pid / tiles_m;
   const int m0 = tm * BM, n0 = tn * BN;
   const int t = threadIdx.x, wave = t / 64, lane = t % 64;
-  const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;
+  const int wm = (wave / 2) * (BM / 2), wn = (wave % 2) * (BN / 2);
   const int r32 = lane % 32, g = lane / 32;
 
-  floatx16 acc[2][2];
+  floatx16 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   const u32x4 zero = {0u, 0u, 0u, 0u};
-  u32x4 pa[4], pw[4];
+  u32x4 pa[UA], pw[UW];
+  // never a conditional load, and no use between loads: an address outside is replaced by one
+  // inside; what lies outside of A is zeroed afterwards, what lies outside of W meets those zeros
+  // or is not stored
   auto fetch = [&](int kt) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int c = t + u * 256, row = c / 8, ch = c % 8;
-      const int k = kt * BK + ch * 8;
-      const int m = m0 + row, n = n0 + row;
-      // never a conditional load: an address outside is replaced by one inside, the value dropped
-      const bool ka = k < K, oka = ka && m < M, okw = ka && n < N;
-      pa[u] = *reinterpret_cast<const u32x4*>(A + static_cast<size_t>(oka ? m : 0) * lda + (oka ? k : 0));
-      pw[u] = *reinterpret_cast<const u32x4*>(W + static_cast<size_t>(okw ? n : 0) * K + (okw ? k : 0));
+    for (int u = 0; u < UA; ++u) {
+      const int c = t + u * 256, row = c / CH, ch = c % CH;
+      const int k = kt * BK + ch * 8, m = m0 + row;
+      const bool ok = k < K && m < M;
+      pa[u] = *reinterpret_cast<const u32x4*>(A + static_cast<size_t>(ok ? m : 0) * lda + (ok ? k : 0));
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {      // only A needs zeroing: what lies outside of W meets zeros of A or is not stored
-      const int c = t + u * 256, row = c / 8, ch = c % 8;
-      if (!(kt * BK + ch * 8 < K && m0 + row < M)) pa[u] = zero;
+    for (int u = 0; u < UW; ++u) {
+      const int c = t + u * 256, row = c / CH, ch = c % CH;
+      const int k = kt * BK + ch * 8, n = n0 + row;
+      const bool ok = k < K && n < N;
+      pw[u] = *reinterpret_cast<const u32x4*>(W + static_cast<size_t>(ok ? n : 0) * K + (ok ? k : 0));
     }
   };
-  auto stash = [&]() {
+  auto stash = [&](int kt, u32x4* As, u32x4* Ws) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int c = t + u * 256, row = c / 8, ch = c % 8;
-      As[row * 8 + (ch ^ (row & 7))] = pa[u];
-      Ws[row * 8 + (ch ^ (row & 7))] = pw[u];
+    for (int u = 0; u < UA; ++u) {
+      const int c = t + u * 256, row = c / CH, ch = c % CH;
+      const bool ok = kt * BK + ch * 8 < K && m0 + row < M;
+      As[row * CH + (ch ^ swz(row))] = ok ? pa[u] : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < UW; ++u) {
+      const int c = t + u * 256, row = c / CH, ch = c % CH;
+      Ws[row * CH + (ch ^ swz(row))] = pw[u];
     }
   };
   const int ktiles = (K + BK - 1) / BK;
+  constexpr int SET = (BM + BN) * CH;
   fetch(0);
+  stash(0, lds, lds + BM * CH);
+  __syncthreads();
   for (int kt = 0; kt < ktiles; ++kt) {
-    __syncthreads();          // the slabs in LDS have been used up
-    stash();
-    __syncthreads();
+    const u32x4* As = lds + (kt & 1) * SET;
+    const u32x4* Ws = As + BM * CH;
     if (kt + 1 < ktiles) fetch(kt + 1);
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
-      bf16x8 af[2], wf[2];
+      bf16x8 af[TM], wf[TN];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < TM; ++i) {
         const int row = wm + i * 32 + r32;
-        af[i] = __builtin_bit_cast(bf16x8, As[row * 8 + ((kk * 2 + g) ^ (row & 7))]);
+        af[i] = __builtin_bit_cast(bf16x8, As[row * CH + ((kk * 2 + g) ^ swz(row))]);
       }
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < TN; ++j) {
         const int row = wn + j * 32 + r32;
-        wf[j] = __builtin_bit_cast(bf16x8, Ws[row * 8 + ((kk * 2 + g) ^ (row & 7))]);
+        wf[j] = __builtin_bit_cast(bf16x8, Ws[row * CH + ((kk * 2 + g) ^ swz(row))]);
       }
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], wf[j], acc[i][j], 0, 0, 0);
     }
+    if (kt + 1 < ktiles) {
+      u32x4* An = lds + ((kt + 1) & 1) * SET;
+      stash(kt + 1, An, An + BM * CH);
+    }
+    __syncthreads();     // the next set is written and this one has been read by every wave
   }
   // acc[i][j][r]: row m0 + wm + 32 i + 8 (r / 4) + 4 g + r % 4, column n0 + wn + 32 j + lane % 32
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < TN; ++j) {
     const int n = n0 + wn + j * 32 + r32;
     if (n >= N) continue;
     const float bv = bias ? bias[n] : 0.f;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + wm + i * 32 + 8 * (r / 4) + 4 * g + (r % 4);
@@ -417,18 +434,36 @@ static bool takes(const void* A, int lda, const void* W, int K, int in_dtype) {
          reinterpret_cast<uintptr_t>(W) % 16 == 0;
 }
 
-static void run(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr, int M,
-                int N, int K, int out_dtype, int epi, hipStream_t stream) {
+template <typename TC, int TM, int TN, int BK>
+static int launch(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr,
+                  int M, int N, int K, int epi, hipStream_t stream) {
+  constexpr int BM = 64 * TM, BN = 64 * TN;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  dim3 grid(tiles_m * tiles_n), block(256);
-  if (out_dtype == DN_BF16)
-    hipLaunchKernelGGL(gemm_kernel<bf16_t>, grid, block, 0, stream, static_cast<const bf16_t*>(A), lda,
-                       static_cast<const bf16_t*>(W), bias, static_cast<bf16_t*>(C), ldc, resid, ldr, M, N, K, epi,
-                       tiles_m, tiles_n);
-  else
-    hipLaunchKernelGGL(gemm_kernel<float>, grid, block, 0, stream, static_cast<const bf16_t*>(A), lda,
-                       static_cast<const bf16_t*>(W), bias, static_cast<float*>(C), ldc, resid, ldr, M, N, K, epi,
-                       tiles_m, tiles_n);
+  const size_t lds = 2 * static_cast<size_t>(BM + BN) * (BK / 8) * 16;
+  static bool raised = false;      // more than 64 KB of LDS has to be asked for once per kernel
+  if (lds > 65536 && !raised) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<TC, TM, TN, BK>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (e != hipSuccess) return static_cast<int>(e);
+    raised = true;
+  }
+  hipLaunchKernelGGL((gemm_kernel<TC, TM, TN, BK>), dim3(tiles_m * tiles_n), dim3(256), lds, stream,
+                     static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), bias, static_cast<TC*>(C), ldc,
+                     resid, ldr, M, N, K, epi, tiles_m, tiles_n);
+  return 0;
+}
+
+static int run(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr, int M,
+               int N, int K, int out_dtype, int epi, hipStream_t stream) {
+  // many tiles: slabs of 32 along K take half the LDS, so more workgroups share a CU and hide
+  // each other's waits; few tiles: slabs of 64 halve the number of barriers
+  const long tiles = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
+  if (tiles >= 512) {
+    if (out_dtype == DN_BF16) return launch<bf16_t, 2, 2, 32>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, stream);
+    return launch<float, 2, 2, 32>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, stream);
+  }
+  if (out_dtype == DN_BF16) return launch<bf16_t, 2, 2, 64>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, stream);
+  return launch<float, 2, 2, 64>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, stream);
 }
 }  // namespace tiled
 
@@ -445,8 +480,8 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
     return dn_launch_status();
   }
   if (tiled::takes(A, lda, W, K, in_dtype)) {
-    tiled::run(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, stream);
-    return dn_launch_status();
+    int rc = tiled::run(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, stream);
+    return rc != 0 ? rc : dn_launch_status();
   }
   dim3 grid((N + plain::BN - 1) / plain::BN, (M + plain::BM - 1) / plain::BM), block(256);
 #define DN_LAUNCH(TI, TC)                                                                                     \

@@ -395,7 +395,8 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
 }
 
 // ---------------------------------------------------------------------------------------
-// decode: one row per request.  The context is cut into n_splits runs of `chunks` * 256 keys;
+// decode: one row per request, request s being tile s and row s of the step (tile_seq[s] < 0:
+// padding; tile_pos0[s]: its position).  The context is cut into n_splits runs of `chunks` * 256 keys;
 // a workgroup walks its run 256 keys at a time (4 waves of 64 keys, each with a running
 // maximum, sum and weighted values, joined through LDS at the end) and, if there is more than
 // one split, a second kernel joins the splits' results in split order
@@ -424,10 +425,16 @@ __global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__
   constexpr int GROUP = LPK < 8 ? LPK : 8;   // load instructions issued together
   __shared__ float wm[4], wl[4];
   __shared__ float wacc[4][DH];
+  // In a step of single rows request s brings row s and is tile s: the block table and the query
+  // are addressed by the workgroup's index, so their loads do not wait for the tile table's.
   const int split = blockIdx.x, h = blockIdx.y, tile = blockIdx.z;
-  const int seq = tile_seq[tile];
-  if (seq < 0) return;
-  const int row = tile_row0[tile], pos = tile_pos0[tile];
+  const int row = tile;
+  const int32_t* bt = block_tables + static_cast<size_t>(tile) * max_blocks;
+  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int sub = lane % LPK, grp = lane / LPK;
+  const bf16x8 qv = *reinterpret_cast<const bf16x8*>(q + static_cast<size_t>(row) * ldq + h * DH + sub * 8);
+  if (tile_seq[tile] < 0) return;
+  const int pos = tile_pos0[tile];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int key0 = split * chunks * CHUNK;
   const float NEG_INF = -INFINITY;
@@ -440,15 +447,9 @@ __global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__
     return;
   }
   const int hk = h / (H / Hkv);
-  const int32_t* bt = block_tables + static_cast<size_t>(seq) * max_blocks;
-  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-  const int sub = lane % LPK, grp = lane / LPK;
   float qr[8];
-  {
-    bf16x8 qv = *reinterpret_cast<const bf16x8*>(q + static_cast<size_t>(row) * ldq + h * DH + sub * 8);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) qr[i] = static_cast<float>(qv[i]) * scale;
-  }
+  for (int i = 0; i < 8; ++i) qr[i] = static_cast<float>(qv[i]) * scale;
   float m_run = NEG_INF, l_run = 0.f;
   float acc[DPL];
 #pragma unroll
@@ -580,7 +581,7 @@ __global__ void join_kernel(const float* __restrict__ part, bf16_t* __restrict__
         A += ps[2 + d] * f;
       }
     }
-    out[static_cast<size_t>(tile_row0[tile]) * ldo + h * DH + d] = from_float<bf16_t>(A / L);
+    out[static_cast<size_t>(tile) * ldo + h * DH + d] = from_float<bf16_t>(A / L);
   }
 }
 }  // namespace decode

@@ -252,7 +252,8 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
     block_tables: int32 [S, max_blocks];
     tiles: int32 [4, n_tiles] = (request, first row, rows <= 16, first position), request < 0: padding;
     tiles_wide: the same rows cut into tiles of up to 128 rows;
-    single_rows: every tile has one row (a pure decode step); max_context: the longest context then.
+    single_rows: a pure decode step: request s brings row s and is tile s, (s or -1, s, 1, position);
+    max_context: the longest context then.
 
     Three kernels: 32-bit takes the plain one; bfloat16 takes the MFMA kernel over tiles_wide, or,
     for a pure decode step, the split kernel; a head size that those do not take falls to the plain one."""
@@ -272,9 +273,10 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
     fast = q.dtype == torch.bfloat16 and ps % 16 == 0 and ldq % 8 == 0 and q.data_ptr() % 16 == 0
     if fast and single_rows and dh in DECODE_HEAD_DIMS and max_context > 0:
         n_tiles = tiles.shape[1]
-        # enough workgroups to fill the chip where the batch alone does not: about 512
+        # the context is split over workgroups only where the batch alone does not give about one
+        # workgroup per CU: a second kernel has to join the splits
         total_chunks = -(-max_context // DECODE_SPLIT)
-        n_splits = max(1, min(total_chunks, 512 // max(1, n_tiles * n_heads)))
+        n_splits = max(1, min(total_chunks, 256 // max(1, n_tiles * n_heads)))
         chunks = -(-total_chunks // n_splits)
         n_splits = -(-total_chunks // chunks)
         _need(max_context <= block_tables.shape[1] * ps, "attention: max_context exceeds the block tables")

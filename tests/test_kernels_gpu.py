@@ -220,8 +220,8 @@ def test_attention_split_kernel_for_decoding(H, Hkv, dh, ps, window):
         assert torch.allclose(out.float(), want, **TOL[torch.bfloat16])
     # one short request alone: a single split, written without the join
     out = torch.zeros(1, H * dh, dtype=torch.bfloat16, device=DEV)
-    ops().attention(q[1:2, :H * dh], out, k, v, bt, i32([[1], [0], [1], [16]]), H, scale, window, single_rows=True,
-                    max_context=17)
+    ops().attention(q[1:2, :H * dh], out, k, v, bt[1:2].contiguous(), i32([[0], [0], [1], [16]]), H, scale, window,
+                    single_rows=True, max_context=17)
     assert torch.allclose(out.float(), want[1:2], **TOL[torch.bfloat16])
 
 

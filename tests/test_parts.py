@@ -56,6 +56,28 @@ def test_norm_part(backend):
     assert n.forward(x, torch.bfloat16).dtype == torch.bfloat16
 
 
+def test_embedding_and_position_parts(backend):
+    """Token rows plus position rows, by the positions of the step, not by the rows' order."""
+    from denno_beta_amd.kernels import ops
+    from denno_beta_amd.parts import POSITIONS, Runtime
+    from denno_beta_amd.parts.positions import TokenEmbedding
+    dev = torch.device(backend)
+    emb, pos = TokenEmbedding(37, 24, "tok"), POSITIONS.make(("learned_absolute", dict(n_positions=50, width=24, name="pos")))
+    assert [(s.name, s.shape, s.role) for s in emb.param_specs() + pos.param_specs()] == [
+        ("tok", (37, 24), "table"), ("pos", (50, 24), "table")]
+    t = {"tok": torch.randn(37, 24, device=dev), "pos": torch.randn(50, 24, device=dev)}
+    emb.bind(t, Runtime(torch.float32, dev)), pos.bind(t, Runtime(torch.float32, dev))
+    tokens = torch.tensor([5, 5, 36, 0], dtype=torch.int32, device=dev)
+    positions = torch.tensor([49, 0, 7, 7], dtype=torch.int32, device=dev)
+    x = torch.empty(4, 24, device=dev)
+    ops.embed(tokens, positions, emb.weight, pos.table(), x)
+    want = P.embed(tokens.long().cpu(), positions.long().cpu(), t["tok"].cpu(), t["pos"].cpu())
+    assert torch.equal(x.cpu(), want)
+    none = POSITIONS.make(("none", {}))
+    ops.embed(tokens, positions, emb.weight, none.table(), x)
+    assert torch.equal(x.cpu(), t["tok"].cpu()[tokens.long().cpu()])
+
+
 @pytest.mark.parametrize("act", ["gelu_tanh", "gelu_erf"])
 def test_feed_forward_part(backend, act):
     from denno_beta_amd.parts import FEED_FORWARDS, Runtime

@@ -188,3 +188,36 @@ def test_weights_stored_in_32_bit_stay_so_in_a_bfloat16_engine(backend, model_fo
     got = U.replay(r, steps)
     for i in range(2):
         U.assert_close(got[f"r{i}"], want[i], "bfloat16", f"32-bit weights in a bfloat16 engine, request {i}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sharp_attention_shows_a_wrong_key(backend, model_folders, tmp_path, dtype):
+    """Random weights give nearly flat attention, which hides a key read from the wrong place.  With
+    the query and key weights scaled up each row attends to a few keys only, so one misplaced
+    key (a page's edge, a reused page, the start of a portion) changes the logits visibly."""
+    from safetensors.torch import load_file, save_file
+    import shutil
+    src = model_folders("A", dtype)
+    dst = str(tmp_path / "sharp")
+    shutil.copytree(src, dst)
+    t = load_file(dst + "/model.safetensors")
+    for i in range(2):
+        w = t[f"h.{i}.attn.c_attn.weight"].float()
+        w[:, :128] *= 12.0          # the query and key columns of the fused projection
+        t[f"h.{i}.attn.c_attn.weight"] = w.to(t[f"h.{i}.attn.c_attn.weight"].dtype)
+    save_file(t, dst + "/model.safetensors")
+    lengths = (90, 33, 128, 64, 50) if backend != "cpu" else (40, 33, 50)
+    seqs = sequences("A", lengths, seed=31)
+    plain = PlainGPT2.from_folder(dst)
+    want = [plain.logits(s) for s in seqs]
+    # attention is sharp indeed: some row of the first layer puts most of its weight on one key
+    steps = U.mixed_trace(seqs, seed=8)
+    r = runner_for(dst, dtype, backend, cache_tokens=U.max_live_tokens(steps))
+    got = U.replay(r, steps)
+    assert r.cache.manager.reuse_count(0) > 0
+    for i in range(len(seqs)):
+        U.assert_close(got[f"r{i}"], want[i], dtype, f"sharp attention {dtype} request {i}")
+    # and the logits do depend on a far token: changing token 3 changes the last row
+    changed = list(seqs[0])
+    changed[3] = (changed[3] + 1) % 512
+    assert (plain.logits(changed)[-1] - want[0][-1]).abs().max() > 1e-3

@@ -22,6 +22,33 @@ __device__ __forceinline__ float apply_epilogue(float v, int epi) {
   return v;
 }
 
+// Where a fused projection's key and value columns go besides C: columns q_width .. of row m are
+// the keys, then the values, of the token whose slot is slot_map[m] (page * page_size + offset,
+// < 0: none).  Pools as in the cache: keys [page, Hkv, page_size, dh], values [page, Hkv, dh, page_size].
+struct KVScatter {
+  const int32_t* slot_map;
+  bf16_t* k_pool;
+  bf16_t* v_pool;
+  int q_width, kv_width, dh, page_size, Hkv;
+};
+
+
+__device__ __forceinline__ void scatter_kv(const KVScatter& kv, int m, int nn, bf16_t cv) {
+  if (nn < kv.q_width) return;
+  int c = nn - kv.q_width;
+  const bool is_value = c >= kv.kv_width;
+  if (is_value) c -= kv.kv_width;
+  const int slot = kv.slot_map[m];
+  if (slot < 0) return;
+  const int page = slot / kv.page_size, off = slot % kv.page_size;
+  const int hh = c / kv.dh, d = c % kv.dh;
+  const size_t base = (static_cast<size_t>(page) * kv.Hkv + hh) * kv.page_size * kv.dh;
+  if (is_value)
+    kv.v_pool[base + static_cast<size_t>(d) * kv.page_size + off] = cv;
+  else
+    kv.k_pool[base + static_cast<size_t>(off) * kv.dh + d] = cv;
+}
+
 namespace plain {
 constexpr int BM = 64, BN = 64, BK = 16, PAD = 4;
 
@@ -112,16 +139,6 @@ namespace skinny {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 constexpr int UNROLL = 8;
-
-// Where a fused projection's key and value columns go besides C: columns q_width .. of row m are
-// the keys, then the values, of the token whose slot is slot_map[m] (page * page_size + offset,
-// < 0: none).  Pools as in the cache: keys [page, Hkv, page_size, dh], values [page, Hkv, dh, page_size].
-struct KVScatter {
-  const int32_t* slot_map;
-  bf16_t* k_pool;
-  bf16_t* v_pool;
-  int q_width, kv_width, dh, page_size, Hkv;
-};
 
 template <int MB, int WAVES, typename TC, bool KV>
 __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restrict__ A, int lda,
@@ -223,23 +240,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
       } else {
         TC cv = from_float<TC>(apply_epilogue(v, epi));
         C[static_cast<size_t>(m) * ldc + nn] = cv;
-        if constexpr (KV) {
-          if (nn >= kv.q_width) {
-            int c = nn - kv.q_width;
-            const bool is_value = c >= kv.kv_width;
-            if (is_value) c -= kv.kv_width;
-            const int slot = kv.slot_map[m];
-            if (slot >= 0) {
-              const int page = slot / kv.page_size, off = slot % kv.page_size;
-              const int hh = c / kv.dh, d = c % kv.dh;
-              const size_t base = (static_cast<size_t>(page) * kv.Hkv + hh) * kv.page_size * kv.dh;
-              if (is_value)
-                kv.v_pool[base + static_cast<size_t>(d) * kv.page_size + off] = cv;
-              else
-                kv.k_pool[base + static_cast<size_t>(off) * kv.dh + d] = cv;
-            }
-          }
-        }
+        if constexpr (KV) scatter_kv(kv, m, nn, cv);
       }
     }
   }
@@ -294,10 +295,10 @@ static bool takes(const void* A, int lda, const void* W, int M, int K, int in_dt
 
 // ---------------------------------------------------------------------------------------
 // Many rows, bfloat16: the prefill's products, bound by the matrix cores.
-// A workgroup of 4 waves (2 x 2) makes a tile of C; each wave makes TM x TN tiles of
-// v_mfma_f32_32x32x16_bf16 (2 x 2: a 128 x 128 tile; 4 x 2 was measured slower: its registers and
-// LDS leave room for one wave per SIMD only, and nothing then hides the latency of LDS).  Two waves
-// per SIMD are asked for.  K advances BK (64 or 32) at a time through two sets of slabs in LDS: while the
+// A workgroup of WM x 2 waves makes a tile of C; each wave makes 2 x 2 tiles of
+// v_mfma_f32_32x32x16_bf16, a 64 x 64 share (4 x 2 tiles per wave were measured slower: their
+// registers leave room for one wave per SIMD only, and nothing then hides the latency of LDS).
+// Two waves per SIMD are asked for.  K advances BK (64 or 32) at a time through two sets of slabs in LDS: while the
 // matrix cores work on one set, the next slabs travel from memory to registers and then into
 // the other set; one barrier per step.  In LDS a row is BK/8 chunks of 16 bytes, chunk c stored
 // at c ^ swz(row), so that the rows a lane group reads fall on different banks.
@@ -310,14 +311,15 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
 constexpr int XCDS = 8;
 
-template <typename TC, int TM, int TN, int BK>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(
+template <typename TC, int WM, int TM, int TN, int BK, bool KV>
+__global__ __launch_bounds__(WM * 128) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const float* __restrict__ bias,
     TC* __restrict__ C, int ldc, float* __restrict__ resid, int ldr, int M, int N, int K, int epi, int tiles_m,
-    int tiles_n) {
-  constexpr int BM = 64 * TM, BN = 64 * TN;
+    int tiles_n, KVScatter kv) {
+  constexpr int THREADS = WM * 128;                       // WM x 2 waves
+  constexpr int BM = WM * 32 * TM, BN = 64 * TN;
   constexpr int CH = BK / 8;                              // 16-byte chunks in a row of a slab
-  constexpr int UA = BM * CH / 256, UW = BN * CH / 256;   // chunks per thread and slab
+  constexpr int UA = BM * CH / THREADS, UW = BN * CH / THREADS;   // chunks per thread and slab
   // a row's chunk c lies at c ^ swz(row): 16 consecutive rows then cover all 16 bank groups
   auto swz = [](int row) { return (row / (16 / CH)) % CH; };
   extern __shared__ u32x4 lds[];                          // [2][(BM + BN) * CH]
@@ -328,7 +330,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
   const int tm = pid % tiles_m, tn = pid / tiles_m;
   const int m0 = tm * BM, n0 = tn * BN;
   const int t = threadIdx.x, wave = t / 64, lane = t % 64;
-  const int wm = (wave / 2) * (BM / 2), wn = (wave % 2) * (BN / 2);
+  const int wm = (wave / 2) * (BM / WM), wn = (wave % 2) * (BN / 2);
   const int r32 = lane % 32, g = lane / 32;
 
   floatx16 acc[TM][TN];
@@ -347,14 +349,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
   auto fetch = [&](int kt) {
 #pragma unroll
     for (int u = 0; u < UA; ++u) {
-      const int c = t + u * 256, row = c / CH, ch = c % CH;
+      const int c = t + u * THREADS, row = c / CH, ch = c % CH;
       const int k = kt * BK + ch * 8, m = m0 + row;
       const bool ok = k < K && m < M;
       pa[u] = *reinterpret_cast<const u32x4*>(A + static_cast<size_t>(ok ? m : 0) * lda + (ok ? k : 0));
     }
 #pragma unroll
     for (int u = 0; u < UW; ++u) {
-      const int c = t + u * 256, row = c / CH, ch = c % CH;
+      const int c = t + u * THREADS, row = c / CH, ch = c % CH;
       const int k = kt * BK + ch * 8, n = n0 + row;
       const bool ok = k < K && n < N;
       pw[u] = *reinterpret_cast<const u32x4*>(W + static_cast<size_t>(ok ? n : 0) * K + (ok ? k : 0));
@@ -363,13 +365,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
   auto stash = [&](int kt, u32x4* As, u32x4* Ws) {
 #pragma unroll
     for (int u = 0; u < UA; ++u) {
-      const int c = t + u * 256, row = c / CH, ch = c % CH;
+      const int c = t + u * THREADS, row = c / CH, ch = c % CH;
       const bool ok = kt * BK + ch * 8 < K && m0 + row < M;
       As[row * CH + (ch ^ swz(row))] = ok ? pa[u] : zero;
     }
 #pragma unroll
     for (int u = 0; u < UW; ++u) {
-      const int c = t + u * 256, row = c / CH, ch = c % CH;
+      const int c = t + u * THREADS, row = c / CH, ch = c % CH;
       Ws[row * CH + (ch ^ swz(row))] = pw[u];
     }
   };
@@ -423,7 +425,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
           float* x = resid + static_cast<size_t>(m) * ldr + n;
           *x = *x + v;
         } else {
-          C[static_cast<size_t>(m) * ldc + n] = from_float<TC>(apply_epilogue(v, epi));
+          const TC cv = from_float<TC>(apply_epilogue(v, epi));
+          C[static_cast<size_t>(m) * ldc + n] = cv;
+          if constexpr (KV) scatter_kv(kv, m, n, cv);
         }
       }
   }
@@ -434,36 +438,42 @@ static bool takes(const void* A, int lda, const void* W, int K, int in_dtype) {
          reinterpret_cast<uintptr_t>(W) % 16 == 0;
 }
 
-template <typename TC, int TM, int TN, int BK>
+template <typename TC, int WM, int TM, int TN, int BK, bool KV>
 static int launch(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr,
-                  int M, int N, int K, int epi, hipStream_t stream) {
-  constexpr int BM = 64 * TM, BN = 64 * TN;
+                  int M, int N, int K, int epi, const KVScatter* kv, hipStream_t stream) {
+  constexpr int BM = WM * 32 * TM, BN = 64 * TN;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const size_t lds = 2 * static_cast<size_t>(BM + BN) * (BK / 8) * 16;
   static bool raised = false;      // more than 64 KB of LDS has to be asked for once per kernel
   if (lds > 65536 && !raised) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<TC, TM, TN, BK>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<TC, WM, TM, TN, BK, KV>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     if (e != hipSuccess) return static_cast<int>(e);
     raised = true;
   }
-  hipLaunchKernelGGL((gemm_kernel<TC, TM, TN, BK>), dim3(tiles_m * tiles_n), dim3(256), lds, stream,
+  hipLaunchKernelGGL((gemm_kernel<TC, WM, TM, TN, BK, KV>), dim3(tiles_m * tiles_n), dim3(WM * 128), lds, stream,
                      static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), bias, static_cast<TC*>(C), ldc,
-                     resid, ldr, M, N, K, epi, tiles_m, tiles_n);
+                     resid, ldr, M, N, K, epi, tiles_m, tiles_n, kv ? *kv : KVScatter{});
   return 0;
 }
 
+template <int WM, int BK>
+static int launch_bk(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr,
+                     int M, int N, int K, int out_dtype, int epi, const KVScatter* kv, hipStream_t stream) {
+  if (kv) return launch<bf16_t, WM, 2, 2, BK, true>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, kv, stream);
+  if (out_dtype == DN_BF16)
+    return launch<bf16_t, WM, 2, 2, BK, false>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, nullptr, stream);
+  return launch<float, WM, 2, 2, BK, false>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, nullptr, stream);
+}
+
 static int run(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr, int M,
-               int N, int K, int out_dtype, int epi, hipStream_t stream) {
-  // many tiles: slabs of 32 along K take half the LDS, so more workgroups share a CU and hide
-  // each other's waits; few tiles: slabs of 64 halve the number of barriers
+               int N, int K, int out_dtype, int epi, const KVScatter* kv, hipStream_t stream) {
+  // Where 128 x 128 tiles would be many (two or more per CU), a workgroup of 8 waves takes 256 x 128
+  // with slabs of 32 along K: each slab of W serves twice the rows.  Else 4 waves, 128 x 128, slabs
+  // of 64 (half the barriers).  Both measured; see profiles/.
   const long tiles = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
-  if (tiles >= 512) {
-    if (out_dtype == DN_BF16) return launch<bf16_t, 2, 2, 32>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, stream);
-    return launch<float, 2, 2, 32>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, stream);
-  }
-  if (out_dtype == DN_BF16) return launch<bf16_t, 2, 2, 64>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, stream);
-  return launch<float, 2, 2, 64>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, stream);
+  if (tiles >= 512) return launch_bk<4, 32>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream);
+  return launch_bk<2, 64>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream);
 }
 }  // namespace tiled
 
@@ -480,7 +490,7 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
     return dn_launch_status();
   }
   if (tiled::takes(A, lda, W, K, in_dtype)) {
-    int rc = tiled::run(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, stream);
+    int rc = tiled::run(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr, stream);
     return rc != 0 ? rc : dn_launch_status();
   }
   dim3 grid((N + plain::BN - 1) / plain::BN, (M + plain::BM - 1) / plain::BM), block(256);
@@ -501,19 +511,24 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
   return dn_launch_status();
 }
 
-// The fused projection q | k | v of a decode step: C = A . W^T + bias as dn_gemm computes it, and
-// the key and value columns also go to their pages (see KVScatter).  Returns 1 (nothing
-// launched) if the sizes are not those of the few-rows kernel: the caller then runs dn_gemm and
-// the separate cache write.
+// The fused projection q | k | v: C = A . W^T + bias as dn_gemm computes it, and the key and value
+// columns also go to their pages (see KVScatter), from the epilogue of the few-rows or of the
+// tiled kernel.  Returns 1 (nothing launched) if neither takes the operands (32-bit, or not
+// aligned): the caller then runs dn_gemm and the separate cache write.
 extern "C" int dn_gemm_qkv(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, int M, int N,
                            int K, const int32_t* slot_map, void* k_pool, void* v_pool, int q_width, int Hkv, int dh,
                            int page_size, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (!skinny::takes(A, lda, W, M, K, DN_BF16)) return 1;
+  const bool few = skinny::takes(A, lda, W, M, K, DN_BF16);
+  if (!few && !tiled::takes(A, lda, W, K, DN_BF16)) return 1;
   if (q_width < 0 || q_width + 2 * Hkv * dh != N || page_size < 1) return DN_ERR_SHAPE;
-  skinny::KVScatter kv{slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_width, Hkv * dh, dh,
-                       page_size, Hkv};
-  skinny::Call c{A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv};
-  skinny::run(c, stream);
-  return dn_launch_status();
+  KVScatter kv{slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_width, Hkv * dh, dh,
+               page_size, Hkv};
+  if (few) {
+    skinny::Call c{A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv};
+    skinny::run(c, stream);
+    return dn_launch_status();
+  }
+  int rc = tiled::run(A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv, stream);
+  return rc != 0 ? rc : dn_launch_status();
 }

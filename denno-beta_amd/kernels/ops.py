@@ -208,11 +208,10 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
 def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
     """out = a @ w.T + bias, the fused projection q | k | v; the key columns (q_width ..) and the
     value columns after them also go to the slots slot_map[t] of the pools, as kv_write does.
-    One kernel where the few-rows product applies (a decode step in bfloat16), else two."""
+    One kernel in bfloat16 (the cache write is in the product's epilogue), else two."""
     n_pages, Hkv, ps, dh = k_pool.shape
     kvw = Hkv * dh
-    if (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
-            and a.shape[0] <= 64 and a.is_cuda):
+    if (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and a.is_cuda):
         _dev(a, "a", None, 2), _dev(w, "w", None, 2), _dev(out, "out", None, 2)
         _dev(slot_map, "slot_map", _I32, 1), _dev(k_pool, "k_pool", (torch.bfloat16,), 4)
         _dev(v_pool, "v_pool", (torch.bfloat16,), 4)

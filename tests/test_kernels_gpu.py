@@ -101,11 +101,11 @@ def test_linear(in_dtype, M, N, K):
     assert torch.allclose(out, R.linear(wide[:, 8:8 + K], w, bias, out=torch.empty_like(out)), **tol)
 
 
-@pytest.mark.parametrize("M", [1, 8, 20, 64, 70])
+@pytest.mark.parametrize("M", [1, 8, 20, 64, 70, 300])
 def test_linear_qkv_writes_the_cache(M):
-    """The fused projection with the cache write in its epilogue (one kernel up to 64 rows, two
-    beyond) against the product followed by the separate write."""
-    H, Hkv, dh, ps, n_pages, K = 6, 2, 32, 16, 9, 96
+    """The fused projection with the cache write in its epilogue (of the few-rows kernel or of the
+    tiled one) against the product followed by the separate write."""
+    H, Hkv, dh, ps, n_pages, K = 6, 2, 32, 16, 20, 96
     N = (H + 2 * Hkv) * dh
     a, w, bias = rnd(M, K, seed=1, dtype=torch.bfloat16), rnd(N, K, seed=2, dtype=torch.bfloat16, scale=0.2), rnd(N, seed=3)
     g = torch.Generator().manual_seed(M)

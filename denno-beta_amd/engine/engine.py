@@ -8,6 +8,7 @@ request is released when it finishes.
 """
 from __future__ import annotations
 
+import time
 from dataclasses import dataclass, field
 from typing import Dict, Iterable, List, Optional, Sequence
 
@@ -53,6 +54,7 @@ class StepRecord:
     prefill_rows: int
     requests: int
     preempted: int
+    host_ms: float = 0.0     # wall time of Engine.step on the host (it ends with the read of the sampled tokens)
 
 
 class Engine:
@@ -109,6 +111,7 @@ class Engine:
 
     # -- one step ------------------------------------------------------------------------
     def step(self) -> List[StepOutput]:
+        t_begin = time.perf_counter()
         plan, preempted = self.scheduler.schedule()
         for rid in preempted:
             self.requests[rid].preemptions += 1
@@ -149,6 +152,7 @@ class Engine:
             rows=sum(p.count for p in plan), decode_rows=sum(1 for p in plan if p.count == 1 and p.start > 0),
             prefill_rows=sum(p.count for p in plan if not (p.count == 1 and p.start > 0)),
             requests=len(plan), preempted=len(preempted)))
+        record = self.records[-1]
         outputs = []
         by_rid = {r.rid: t for r, t in zip(sampled, tokens)}
         eos = set(self.spec.eos_token_ids)
@@ -169,6 +173,7 @@ class Engine:
                 req.finished = True
                 self.scheduler.finish(p.rid)
             outputs.append(StepOutput(p.rid, None if tok is None else int(tok), req.finished, req.finish_reason))
+        record.host_ms = (time.perf_counter() - t_begin) * 1e3
         return outputs
 
     # -- whole generations ---------------------------------------------------------------

@@ -174,3 +174,34 @@ def test_command_line(backend, model_folders):
                           "--raw"], capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stderr
     assert [int(t) for t in out.stdout.strip().split(",")] == want
+
+
+def test_command_line_with_text(backend, model_folders, tmp_path):
+    """`denno generate <model> --prompt TEXT`: the folder's tokenizer.json, the reference's fallback
+    template for models without one ("user: ..\\n\\nassistant:", crates/denno-engine/src/tokenizer.rs:226-236),
+    and `--raw` without it."""
+    if backend == "cpu":
+        pytest.skip("the command line runs the HIP kernels")
+    import shutil
+    from tokenizers import Tokenizer
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import WhitespaceSplit
+    from denno_beta_amd.cli import fallback_template
+    folder = str(tmp_path / "with_tokenizer")
+    shutil.copytree(model_folders("A", "float32"), folder)
+    words = ["[UNK]", "user:", "assistant:", "system:", "hello", "world", "be", "nice"] + [f"w{i}" for i in range(504)]
+    tok = Tokenizer(WordLevel({w: i for i, w in enumerate(words)}, unk_token="[UNK]"))
+    tok.pre_tokenizer = WhitespaceSplit()
+    tok.save(os.path.join(folder, "tokenizer.json"))
+    plain = PlainGPT2.from_folder(folder)
+    run = lambda *extra: subprocess.run(   # noqa: E731
+        [sys.executable, os.path.join(ROOT, "bin", "denno"), "generate", folder, "--prompt", "hello world",
+         "--max-tokens", "5", "--temperature", "0", "--quant", "fp32", *extra], capture_output=True, text=True, timeout=300)
+    for extra, text in (((), fallback_template(None, "hello world")), (("--raw",), "hello world"),
+                        (("--system", "be nice"), fallback_template("be nice", "hello world"))):
+        out = run(*extra)
+        assert out.returncode == 0, out.stderr
+        ids = tok.encode(text).ids
+        assert out.stdout.strip() == tok.decode(plain.greedy(ids, 5)), extra
+    assert fallback_template(None, "hello") == "user: hello\n\nassistant:"          # tokenizer.rs:319-324
+    assert fallback_template("be nice", "hi") == "system: be nice\n\nuser: hi\n\nassistant:"

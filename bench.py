@@ -46,8 +46,9 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0: all)")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
-    ap.add_argument("--only", choices=["decode", "prefill"], default=None,
-                    help="run one workload and print a short line (for profiling)")
+    ap.add_argument("--only", choices=["decode", "prefill", "serving"], default=None,
+                    help="run one workload and print a short line (decode, prefill: for profiling; serving: "
+                         "BASELINE.json's configs[3], GPT-2 Large shape, 64 requests through the scheduler)")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
@@ -57,6 +58,8 @@ def main():
     from denno_beta_amd.config import EngineOptions
     from denno_beta_amd.engine import Engine, ModelRunner, SamplingParams, StepEntry
 
+    if a.only == "serving":
+        return serving(a)
     cfg, full_layers = xl_config(a.layers)
     V, E, P = cfg["vocab_size"], cfg["n_embd"], cfg["n_positions"]
     if a.context + a.warmup + a.steps + 1 > P:
@@ -135,6 +138,39 @@ def main():
         b64, _ = decode_point(64, min(a.steps, 50), a.warmup)
         out["points"] = {"decode_b1": 1 / b1, "decode_b64": 64 / b64}
     print(json.dumps(out))
+
+
+def serving(a):
+    """GPT-2 Large shape, random weights: 64 requests with prompt lengths uniform in [16, 768], 256
+    generated tokens each, greedy, continuous batching with prompt portions of 512."""
+    import torch
+    from denno_beta_amd.config import EngineOptions
+    from denno_beta_amd.engine import Engine, SamplingParams
+    cfg = dict(architectures=["GPT2LMHeadModel"], n_layer=36, n_embd=1280, n_head=20, n_inner=5120, vocab_size=50257,
+               n_positions=1024, layer_norm_epsilon=1e-5, activation_function="gelu_new")
+    opts = EngineOptions(dtype=a.dtype, page_size=16, cache_tokens=64 * 1024, max_live=64, max_batch_tokens=2048,
+                         prefill_chunk=512, use_graphs=not a.no_graphs, seed=0)
+    eng = Engine.from_random(cfg, 0, opts, stored=a.dtype)
+    gen = torch.Generator().manual_seed(1)
+    lengths = torch.randint(16, 769, (64,), generator=gen).tolist()
+    prompts = [torch.randint(0, 50257, (n,), generator=gen).tolist() for n in lengths]
+    sp = SamplingParams(max_tokens=256, temperature=0.0, ignore_eos=True)
+    eng.generate(prompts[:2], SamplingParams(max_tokens=4, temperature=0.0, ignore_eos=True))   # warm-up
+    eng.records.clear()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = eng.generate(prompts, sp)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert all(len(o) == 256 for o in out)
+    steps = len(eng.records)
+    print(json.dumps({
+        "workload": "GPT-2 Large shape, 64 requests, prompts U[16,768], 256 new tokens, prefill portions of 512",
+        "seconds": dt, "generated_tokens": 64 * 256, "generated_tokens_per_s": 64 * 256 / dt,
+        "prompt_tokens": sum(lengths), "all_tokens_per_s": (64 * 256 + sum(lengths)) / dt, "steps": steps,
+        "mean_rows_per_step": sum(r.rows for r in eng.records) / steps,
+        "mixed_steps": sum(1 for r in eng.records if r.decode_rows and r.prefill_rows),
+        "preemptions": sum(r.preempted for r in eng.records), "dtype": a.dtype}))
 
 
 def _layer_matrices(runner):

@@ -7,6 +7,14 @@
 // path and takes bfloat16 operands too (converted exactly on load).  skinny: bfloat16, up to 64
 // rows, MFMA, bound by reading W once (decode).  tiled: bfloat16, many rows, MFMA through LDS
 // (prefill).
+//
+// The two MFMA kernels take W packed (dn_pack_matrix): blocks of 16 rows x 32 columns, block
+// (n / 16, k / 32) at ((n / 16) * ceil(K / 32) + k / 32) * 512 elements, and inside a block the
+// 8 elements k % 32 / 8 * 8 .. + 7 of row n % 16 at ((k % 32 / 8) * 16 + n % 16) * 8: the 16 bytes
+// that lane (n % 16) + 16 * (k % 32 / 8) feeds to v_mfma_f32_16x16x32_bf16.  A wave then reads 1 KB
+// in one piece per block; from rows of K elements the same load touches 16 cache lines per
+// group of 16 lanes, and the rate of those lookups, not of bytes, bounded the kernel (measured:
+// 8.3 -> 6.7 us for 8 x 1600 . 1600 x 4800).  Rows and columns beyond N and K are zeros.
 #include "common.h"
 
 #define EPI_NONE 0
@@ -129,58 +137,72 @@ __global__ __launch_bounds__(256) void gemm_kernel(const TI* __restrict__ A, int
 
 // ---------------------------------------------------------------------------------------
 // Few rows (M <= 64), bfloat16: the decode step's products, bound by reading W once.
-// A workgroup owns 16 output columns; its waves split K in steps of 32 (wave w takes steps
-// w, w + WAVES, ...), each feeding v_mfma_f32_16x16x32_bf16 with 16 bytes of a W row per lane
-// straight from memory (lane = column + 16 * (k / 8)) and the matching 16 bytes of up to four
-// 16-row blocks of A.  The waves' sums meet in LDS and are added in wave order, so the result
-// has one order of summation whatever M is.  No atomics.
+// A workgroup owns 16, 32 or 64 output columns; its waves split K in steps of 32 (wave w takes
+// steps w, w + WAVES, ...), each feeding v_mfma_f32_16x16x32_bf16 with one packed block of W per
+// 16 columns straight from memory (16 bytes per lane) and the matching 16 bytes of up to four
+// 16-row blocks of A (lane = row + 16 * (k / 8)).  The waves' sums meet in LDS and are added in
+// wave order, so the result has one order of summation whatever M is.  No atomics.
 // ---------------------------------------------------------------------------------------
 namespace skinny {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
-constexpr int UNROLL = 8;
 
-template <int MB, int WAVES, typename TC, bool KV>
+// MB row blocks and NB column blocks of 16 per workgroup; U steps of K in flight per wave.
+template <int MB, int NB, int WAVES, int U, typename TC, bool KV>
 __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restrict__ A, int lda,
                                                            const bf16_t* __restrict__ W,
                                                            const float* __restrict__ bias, TC* __restrict__ C,
                                                            int ldc, float* __restrict__ resid, int ldr, int M, int N,
                                                            int K, int epi, KVScatter kv) {
-  __shared__ floatx4 red[WAVES][MB][64];
+  constexpr int BLOCKS = MB * NB;                          // 16 x 16 blocks of C in this workgroup
+  constexpr int PASSES = (BLOCKS + WAVES - 1) / WAVES;     // wave w finishes blocks w, w + WAVES, ...
+  __shared__ floatx4 red[WAVES][BLOCKS][64];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int col = lane % 16, g = lane / 16;
-  const int n0 = blockIdx.x * 16;
-  const int n = min(n0 + col, N - 1);          // a tail tile reads the last row again; its result is not stored
-  const bf16_t* wrow = W + static_cast<size_t>(n) * K + g * 8;
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  const int ksteps = (K + 31) / 32;
-
-  // the first round of W is on its way while the prologue works
-  // what the epilogue will read (bias, the residual stream) is asked for first of all: thread o of
-  // the first MB * 64 threads finishes row block o / 64, lane slot o % 64
-  float epi_bias = 0.f;
-  float epi_x[4] = {0.f, 0.f, 0.f, 0.f};
-  if (threadIdx.x < MB * 64) {
-    const int ln = threadIdx.x % 64, emb = threadIdx.x / 64;
-    const int nn = min(n0 + ln % 16, N - 1);
-    if (bias) epi_bias = bias[nn];
-    if (resid) {
+  const int n0 = blockIdx.x * (16 * NB);
+  const int ksteps = (K + 31) / 32, nblocks = (N + 15) / 16;
+  const bf16_t* wblk[NB];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int m = min(emb * 16 + (ln / 16) * 4 + r, M - 1);
-        epi_x[r] = resid[static_cast<size_t>(m) * ldr + nn];
+  for (int nb = 0; nb < NB; ++nb) {
+    // a block beyond N reads the last one again; its result is not stored
+    const int blk = min(blockIdx.x * NB + nb, nblocks - 1);
+    wblk[nb] = W + (static_cast<size_t>(blk) * ksteps * 64 + lane) * 8;
+  }
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  // what the epilogue will read (bias, the residual stream) is asked for first of all
+  float epi_bias[PASSES];
+  float epi_x[PASSES][4];
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    const int blk = wave + p * WAVES;
+    epi_bias[p] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) epi_x[p][r] = 0.f;
+    if (blk < BLOCKS) {
+      const int mb = blk / NB, nb = blk % NB;
+      const int nn = min(n0 + nb * 16 + col, N - 1);
+      if (bias) epi_bias[p] = bias[nn];
+      if (resid) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = min(mb * 16 + g * 4 + r, M - 1);
+          epi_x[p][r] = resid[static_cast<size_t>(m) * ldr + nn];
+        }
       }
     }
   }
   // Loads are never conditional and nothing uses a loaded value before all loads of a round are
   // issued (a predicated load, or a use in between, makes each load wait for the one before it).
-  // A step beyond K reads W's first row instead (finite numbers) and meets a zeroed piece of A.
-  bf16x8 b[UNROLL];
+  // A step beyond K reads W's first block instead (finite numbers) and meets a zeroed piece of A.
+  // The first round of W is on its way while the rest of the prologue works.
+  bf16x8 b[U][NB];
 #pragma unroll
-  for (int u = 0; u < UNROLL; ++u) {
-    int ks = wave + u * WAVES;
-    bool ok = ks < ksteps && ks * 32 + g * 8 < K;
-    b[u] = *reinterpret_cast<const bf16x8*>(ok ? wrow + ks * 32 : W);
+  for (int u = 0; u < U; ++u) {
+    const int ks = wave + u * WAVES;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+      b[u][nb] = *reinterpret_cast<const bf16x8*>(ks < ksteps ? wblk[nb] + ks * 512 : W + lane * 8);
   }
 
   const bf16_t* arow[MB];
@@ -191,52 +213,64 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
     a_ok[mb] = row < M;
     arow[mb] = A + static_cast<size_t>(a_ok[mb] ? row : 0) * lda + g * 8;
   }
-  floatx4 acc[MB];
+  floatx4 acc[MB][NB];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) acc[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
-  for (int ks0 = wave; ks0 < ksteps; ks0 += WAVES * UNROLL) {
-    bf16x8 a[UNROLL][MB];
+  for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      int ks = ks0 + u * WAVES;
-      bool ok = ks < ksteps && ks * 32 + g * 8 < K;
-      if (ks0 != wave) b[u] = *reinterpret_cast<const bf16x8*>(ok ? wrow + ks * 32 : W);
+    for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int ks0 = wave; ks0 < ksteps; ks0 += WAVES * U) {
+    bf16x8 a[U][MB];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int ks = ks0 + u * WAVES;
+      const bool ok = ks < ksteps && ks * 32 + g * 8 < K;
+      if (ks0 != wave) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          b[u][nb] = *reinterpret_cast<const bf16x8*>(ks < ksteps ? wblk[nb] + ks * 512 : W + lane * 8);
+      }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
         a[u][mb] = *reinterpret_cast<const bf16x8*>(ok ? arow[mb] + ks * 32 : arow[mb]);
     }
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      int ks = ks0 + u * WAVES;
-      bool ok = ks < ksteps && ks * 32 + g * 8 < K;
+    for (int u = 0; u < U; ++u) {
+      const int ks = ks0 + u * WAVES;
+      const bool ok = ks < ksteps && ks * 32 + g * 8 < K;
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
         if (!(ok && a_ok[mb])) a[u][mb] = zero;
     }
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
+    for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
-        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][mb], b[u], acc[mb], 0, 0, 0);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][mb], b[u][nb], acc[mb][nb], 0, 0, 0);
   }
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) red[wave][mb][lane] = acc[mb];
-  __syncthreads();
-  // acc[mb][r] of lane (col, g) is row mb*16 + g*4 + r, column n0 + col
-  if (threadIdx.x < MB * 64) {      // WAVES >= MB: one pass
-    const int mb = threadIdx.x / 64, ln = threadIdx.x % 64;
-    const int nn = n0 + ln % 16;
-    const float bv = epi_bias;
-    floatx4 s = red[0][mb][ln];
+  for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-    for (int w = 1; w < WAVES; ++w) s += red[w][mb][ln];
+    for (int nb = 0; nb < NB; ++nb) red[wave][mb * NB + nb][lane] = acc[mb][nb];
+  __syncthreads();
+  // acc[mb][nb][r] of lane (col, g) is row mb*16 + g*4 + r, column n0 + nb*16 + col
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    const int blk = wave + p * WAVES;
+    if (blk >= BLOCKS) break;
+    const int mb = blk / NB, nb = blk % NB;
+    const int nn = n0 + nb * 16 + col;
+    floatx4 s = red[0][blk][lane];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) s += red[w][blk][lane];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      int m = mb * 16 + (ln / 16) * 4 + r;
+      int m = mb * 16 + g * 4 + r;
       if (m >= M || nn >= N) continue;
-      float v = s[r] + bv;
+      float v = s[r] + epi_bias[p];
       if (resid) {
-        resid[static_cast<size_t>(m) * ldr + nn] = epi_x[r] + v;
+        resid[static_cast<size_t>(m) * ldr + nn] = epi_x[p][r] + v;
       } else {
         TC cv = from_float<TC>(apply_epilogue(v, epi));
         C[static_cast<size_t>(m) * ldc + nn] = cv;
@@ -252,29 +286,48 @@ struct Call {
   const KVScatter* kv;
 };
 
-template <int MB, int WAVES, typename TC, bool KV>
+template <int MB, int NB, int WAVES, int U, typename TC, bool KV>
 static void launch_one(const Call& c, hipStream_t stream) {
-  dim3 grid((c.N + 15) / 16), block(WAVES * 64);
+  dim3 grid((c.N + 16 * NB - 1) / (16 * NB)), block(WAVES * 64);
   KVScatter kv = c.kv ? *c.kv : KVScatter{};
-  hipLaunchKernelGGL((gemm_kernel<MB, WAVES, TC, KV>), grid, block, 0, stream, static_cast<const bf16_t*>(c.A), c.lda,
-                     static_cast<const bf16_t*>(c.W), c.bias, static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N,
-                     c.K, c.epi, kv);
+  hipLaunchKernelGGL((gemm_kernel<MB, NB, WAVES, U, TC, KV>), grid, block, 0, stream,
+                     static_cast<const bf16_t*>(c.A), c.lda, static_cast<const bf16_t*>(c.W), c.bias,
+                     static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N, c.K, c.epi, kv);
 }
 
-template <int MB, int WAVES>
+template <int MB, int NB, int WAVES, int U>
 static void launch(const Call& c, hipStream_t stream) {
-  if (c.kv) return launch_one<MB, WAVES, bf16_t, true>(c, stream);
-  if (c.out_dtype == DN_BF16) return launch_one<MB, WAVES, bf16_t, false>(c, stream);
-  return launch_one<MB, WAVES, float, false>(c, stream);
+  if (c.kv) return launch_one<MB, NB, WAVES, U, bf16_t, true>(c, stream);
+  if (c.out_dtype == DN_BF16) return launch_one<MB, NB, WAVES, U, bf16_t, false>(c, stream);
+  return launch_one<MB, NB, WAVES, U, float, false>(c, stream);
 }
 
+// With more than 16 rows every workgroup reads all of A (16 cache lines per load and 16 lanes,
+// as A lies in rows), so wider workgroups read less in total, as long as enough of them remain
+// to keep the memory system busy.  Measured at 64 rows: 2 column blocks where N >= 4096 (20 ->
+// 13 us for K = 1600), 4 for a vocabulary, 1 for N = 1600.
 template <int WAVES>
 static void launch_mb(const Call& c, hipStream_t stream) {
-  switch ((c.M + 15) / 16) {
-    case 1: launch<1, WAVES>(c, stream); break;
-    case 2: launch<2, WAVES>(c, stream); break;
-    case 3: launch<3, WAVES>(c, stream); break;
-    default: launch<4, WAVES>(c, stream); break;
+  const int mb = (c.M + 15) / 16;
+  if (mb == 1) return launch<1, 1, WAVES, 8>(c, stream);
+  if (c.N >= 32768) {
+    switch (mb) {
+      case 2: return launch<2, 4, WAVES, 4>(c, stream);
+      case 3: return launch<3, 4, WAVES, 4>(c, stream);
+      default: return launch<4, 4, WAVES, 4>(c, stream);
+    }
+  }
+  if (c.N >= 4096) {
+    switch (mb) {
+      case 2: return launch<2, 2, WAVES, 4>(c, stream);
+      case 3: return launch<3, 2, WAVES, 4>(c, stream);
+      default: return launch<4, 2, WAVES, 4>(c, stream);
+    }
+  }
+  switch (mb) {
+    case 2: return launch<2, 1, WAVES, 8>(c, stream);
+    case 3: return launch<3, 1, WAVES, 8>(c, stream);
+    default: return launch<4, 1, WAVES, 8>(c, stream);
   }
 }
 
@@ -285,10 +338,10 @@ static void run(const Call& c, hipStream_t stream) {
     launch_mb<4>(c, stream);
 }
 
-// operands must allow 16-byte loads: K and lda multiples of 8, bases aligned
-static bool takes(const void* A, int lda, const void* W, int M, int K, int in_dtype) {
-  return in_dtype == DN_BF16 && M <= 64 && K % 8 == 0 && lda % 8 == 0 &&
-         reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0;
+// A must allow 16-byte loads: K and lda multiples of 8, the base aligned; W is packed
+static bool takes(const void* A, int lda, const void* W, int M, int K) {
+  return M <= 64 && K % 8 == 0 && lda % 8 == 0 && reinterpret_cast<uintptr_t>(A) % 16 == 0 &&
+         reinterpret_cast<uintptr_t>(W) % 16 == 0;
 }
 }  // namespace skinny
 
@@ -319,6 +372,8 @@ __global__ __launch_bounds__(WM * 128) __attribute__((amdgpu_waves_per_eu(2))) v
   constexpr int THREADS = WM * 128;                       // WM x 2 waves
   constexpr int BM = WM * 32 * TM, BN = 64 * TN;
   constexpr int CH = BK / 8;                              // 16-byte chunks in a row of a slab
+  constexpr int KS = BK / 32;                             // packed blocks of W along K in a slab
+  const int ksteps = (K + 31) / 32, nblocks = (N + 15) / 16;
   constexpr int UA = BM * CH / THREADS, UW = BN * CH / THREADS;   // chunks per thread and slab
   // a row's chunk c lies at c ^ swz(row): 16 consecutive rows then cover all 16 bank groups
   auto swz = [](int row) { return (row / (16 / CH)) % CH; };
@@ -354,12 +409,13 @@ __global__ __launch_bounds__(WM * 128) __attribute__((amdgpu_waves_per_eu(2))) v
       const bool ok = k < K && m < M;
       pa[u] = *reinterpret_cast<const u32x4*>(A + static_cast<size_t>(ok ? m : 0) * lda + (ok ? k : 0));
     }
+    // W is packed: 64 consecutive threads take one block of 16 rows x 32 columns, 1 KB in one piece
 #pragma unroll
     for (int u = 0; u < UW; ++u) {
-      const int c = t + u * THREADS, row = c / CH, ch = c % CH;
-      const int k = kt * BK + ch * 8, n = n0 + row;
-      const bool ok = k < K && n < N;
-      pw[u] = *reinterpret_cast<const u32x4*>(W + static_cast<size_t>(ok ? n : 0) * K + (ok ? k : 0));
+      const int c = t + u * THREADS, blk = c / 64, in = c % 64;
+      const int ks = kt * KS + blk % KS, nblk = n0 / 16 + blk / KS;
+      const bool ok = ks < ksteps && nblk < nblocks;
+      pw[u] = *reinterpret_cast<const u32x4*>(W + (ok ? (static_cast<size_t>(nblk) * ksteps + ks) * 512 + in * 8 : 0));
     }
   };
   auto stash = [&](int kt, u32x4* As, u32x4* Ws) {
@@ -369,9 +425,11 @@ __global__ __launch_bounds__(WM * 128) __attribute__((amdgpu_waves_per_eu(2))) v
       const bool ok = kt * BK + ch * 8 < K && m0 + row < M;
       As[row * CH + (ch ^ swz(row))] = ok ? pa[u] : zero;
     }
+    // 16 consecutive lanes write the same chunk of 16 consecutive rows: no two on one bank
 #pragma unroll
     for (int u = 0; u < UW; ++u) {
-      const int c = t + u * THREADS, row = c / CH, ch = c % CH;
+      const int c = t + u * THREADS, blk = c / 64, in = c % 64;
+      const int row = (blk / KS) * 16 + in % 16, ch = (blk % KS) * 4 + in / 16;
       Ws[row * CH + (ch ^ swz(row))] = pw[u];
     }
   };
@@ -433,8 +491,8 @@ __global__ __launch_bounds__(WM * 128) __attribute__((amdgpu_waves_per_eu(2))) v
   }
 }
 
-static bool takes(const void* A, int lda, const void* W, int K, int in_dtype) {
-  return in_dtype == DN_BF16 && K % 8 == 0 && lda % 8 == 0 && reinterpret_cast<uintptr_t>(A) % 16 == 0 &&
+static bool takes(const void* A, int lda, const void* W, int K) {
+  return K % 8 == 0 && lda % 8 == 0 && reinterpret_cast<uintptr_t>(A) % 16 == 0 &&
          reinterpret_cast<uintptr_t>(W) % 16 == 0;
 }
 
@@ -477,19 +535,23 @@ static int run(const void* A, int lda, const void* W, const float* bias, void* C
 }
 }  // namespace tiled
 
+// W: rows of K elements (w_packed 0; the plain kernel, any dtype), or packed bfloat16
+// (w_packed 1; the MFMA kernels, which need A in bfloat16 and loadable 16 bytes at a time).
 extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid,
-                       int ldr, int M, int N, int K, int in_dtype, int out_dtype, int epilogue,
+                       int ldr, int M, int N, int K, int in_dtype, int out_dtype, int epilogue, int w_packed,
                        hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || K % 4 != 0 || lda < K) return DN_ERR_SHAPE;
   if (epilogue < EPI_NONE || epilogue > EPI_GELU_ERF) return DN_ERR_SHAPE;
   if (resid != nullptr && epilogue != EPI_NONE) return DN_ERR_SHAPE;
-  if (skinny::takes(A, lda, W, M, K, in_dtype)) {
-    skinny::Call c{A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr};
-    skinny::run(c, stream);
-    return dn_launch_status();
-  }
-  if (tiled::takes(A, lda, W, K, in_dtype)) {
+  if (w_packed) {
+    if (in_dtype != DN_BF16) return DN_ERR_DTYPE;
+    if (skinny::takes(A, lda, W, M, K)) {
+      skinny::Call c{A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr};
+      skinny::run(c, stream);
+      return dn_launch_status();
+    }
+    if (!tiled::takes(A, lda, W, K)) return DN_ERR_SHAPE;
     int rc = tiled::run(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr, stream);
     return rc != 0 ? rc : dn_launch_status();
   }
@@ -511,16 +573,16 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
   return dn_launch_status();
 }
 
-// The fused projection q | k | v: C = A . W^T + bias as dn_gemm computes it, and the key and value
-// columns also go to their pages (see KVScatter), from the epilogue of the few-rows or of the
-// tiled kernel.  Returns 1 (nothing launched) if neither takes the operands (32-bit, or not
-// aligned): the caller then runs dn_gemm and the separate cache write.
+// The fused projection q | k | v with packed W: C = A . W^T + bias as dn_gemm computes it, and the
+// key and value columns also go to their pages (see KVScatter), from the epilogue of the few-rows
+// or of the tiled kernel.
 extern "C" int dn_gemm_qkv(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, int M, int N,
                            int K, const int32_t* slot_map, void* k_pool, void* v_pool, int q_width, int Hkv, int dh,
                            int page_size, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  const bool few = skinny::takes(A, lda, W, M, K, DN_BF16);
-  if (!few && !tiled::takes(A, lda, W, K, DN_BF16)) return 1;
+  if (K <= 0 || lda < K) return DN_ERR_SHAPE;
+  const bool few = skinny::takes(A, lda, W, M, K);
+  if (!few && !tiled::takes(A, lda, W, K)) return DN_ERR_SHAPE;
   if (q_width < 0 || q_width + 2 * Hkv * dh != N || page_size < 1) return DN_ERR_SHAPE;
   KVScatter kv{slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_width, Hkv * dh, dh,
                page_size, Hkv};
@@ -531,4 +593,31 @@ extern "C" int dn_gemm_qkv(const void* A, int lda, const void* W, const float* b
   }
   int rc = tiled::run(A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv, stream);
   return rc != 0 ? rc : dn_launch_status();
+}
+
+// dst (packed, (ceil(N/16) * ceil(K/32) * 512 elements) from src [N, K] in rows.
+__global__ void pack_kernel(const bf16_t* __restrict__ src, bf16_t* __restrict__ dst, int N, int K, int ksteps,
+                            long chunks) {
+  const long c = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;     // one 16-byte chunk each
+  if (c >= chunks) return;
+  const int in = c % 64;
+  const long blk = c / 64;
+  const int ks = blk % ksteps, nblk = blk / ksteps;
+  const int n = nblk * 16 + in % 16, k = ks * 32 + (in / 16) * 8;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    bf16_t v;
+    v.bits = 0;
+    if (n < N && k + j < K) v = src[static_cast<size_t>(n) * K + k + j];
+    dst[c * 8 + j] = v;
+  }
+}
+
+extern "C" int dn_pack_matrix(const void* src, void* dst, int N, int K, hipStream_t stream) {
+  if (N <= 0 || K <= 0) return DN_ERR_SHAPE;
+  const int ksteps = (K + 31) / 32;
+  const long chunks = static_cast<long>((N + 15) / 16) * ksteps * 64;
+  hipLaunchKernelGGL(pack_kernel, dim3((chunks + 255) / 256), dim3(256), 0, stream,
+                     static_cast<const bf16_t*>(src), static_cast<bf16_t*>(dst), N, K, ksteps, chunks);
+  return dn_launch_status();
 }

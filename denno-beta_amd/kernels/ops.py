@@ -46,7 +46,8 @@ def _declare(name, lib):
             "dn_cast": [P, P, c_longlong, I, I, P],
         },
         "gemm": {
-            "dn_gemm": [P, I, P, P, P, I, P, I, I, I, I, I, I, I, P],
+            "dn_gemm": [P, I, P, P, P, I, P, I, I, I, I, I, I, I, I, P],
+            "dn_pack_matrix": [P, P, I, I, P],
             "dn_gemm_qkv": [P, I, P, P, P, I, I, I, I, P, P, P, I, I, I, I, P],
         },
         "attention": {
@@ -177,14 +178,69 @@ def cast(x, out):
     return out
 
 
+class PackedMatrix:
+    """A bfloat16 matrix [N, K] laid out for the matrix cores: blocks of 16 rows x 32 columns, 1 KB
+    each and contiguous, block (n // 16, k // 32) at ((n // 16) * ceil(K / 32) + k // 32) * 512
+    elements; inside it row n % 16, columns (k % 32) // 8 * 8 .. + 7 at (((k % 32) // 8) * 16 + n % 16) * 8.
+    Rows and columns beyond N and K are zeros.  `linear` takes it for the MFMA kernels."""
+    __slots__ = ("data", "shape")
+    dtype = torch.bfloat16
+
+    def __init__(self, data, shape):
+        self.data, self.shape = data, tuple(shape)
+
+    @property
+    def device(self):
+        return self.data.device
+
+    def data_ptr(self):
+        return self.data.data_ptr()
+
+    def numel(self):
+        return self.shape[0] * self.shape[1]
+
+    def element_size(self):
+        return 2
+
+    def rows(self):
+        """The matrix [N, K] again (for tests and tools)."""
+        N, K = self.shape
+        nb, ks = -(-N // 16), -(-K // 32)
+        return self.data.view(nb, ks, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(nb * 16, ks * 32)[:N, :K].contiguous()
+
+
+def pack_matrix(w) -> PackedMatrix:
+    """w: bfloat16 [N, K], rows contiguous, K a multiple of 8."""
+    _dev(w, "w", (torch.bfloat16,), 2)
+    N, K = w.shape
+    _need(w.is_contiguous(), "pack_matrix: w must be contiguous")
+    _need(K % 8 == 0, f"pack_matrix: the inner size {K} must be a multiple of 8")
+    data = torch.empty(-(-N // 16) * -(-K // 32) * 512, dtype=torch.bfloat16, device=w.device)
+    _ok(_lib("gemm").dn_pack_matrix(w.data_ptr(), data.data_ptr(), N, K, _stream()), "pack_matrix")
+    return PackedMatrix(data, (N, K))
+
+
+def _matrix(a, w, what):
+    """(pointer, N, packed flag) of a weight for a [M, K]."""
+    K = a.shape[1]
+    if isinstance(w, PackedMatrix):
+        _need(a.dtype == torch.bfloat16, f"{what}: a packed matrix needs bfloat16 rows, not {a.dtype}")
+        _need(w.device == a.device and w.shape[1] == K, f"{what}: w {w.shape} does not fit a {tuple(a.shape)}")
+        _need(a.data_ptr() % 16 == 0 and a.stride(0) % 8 == 0, f"{what}: the rows of a must be aligned to 16 bytes")
+        return w.data_ptr(), w.shape[0], 1
+    _dev(w, "w", (a.dtype,), 2)
+    _need(w.is_contiguous() and w.shape[1] == K, f"{what}: w {tuple(w.shape)} does not fit a {tuple(a.shape)}")
+    return w.data_ptr(), w.shape[0], 0
+
+
 def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
     """out = epilogue(a @ w.T + bias), or residual += a @ w.T + bias (32-bit, in place).
-    a: [M, K] rows contiguous; w: [N, K] held [out, in]; bias: 32-bit [N]."""
-    _dev(a, "a", _FLOATS, 2), _dev(w, "w", (a.dtype,), 2)
+    a: [M, K] rows contiguous; w: [N, K] held [out, in], in rows (the plain kernel: 32-bit, or a
+    reference for bfloat16) or a PackedMatrix (the MFMA kernels); bias: 32-bit [N]."""
+    _dev(a, "a", _FLOATS, 2)
     M, K = a.shape
-    N = w.shape[0]
-    _need(w.is_contiguous() and w.shape[1] == K, f"linear: w {tuple(w.shape)} does not fit a {tuple(a.shape)}")
     _need(K % 8 == 0, f"linear: the inner size {K} must be a multiple of 8")
+    wp, N, packed = _matrix(a, w, "linear")
     lda = _rows(a, "a")
     if bias is not None:
         _dev(bias, "bias", (torch.float32,), 1)
@@ -194,30 +250,31 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
         _dev(residual, "residual", (torch.float32,), 2)
         _need(tuple(residual.shape) == (M, N) and epi == 0 and out is None, "linear: residual")
         ldr = _rows(residual, "residual")
-        _ok(_lib("gemm").dn_gemm(a.data_ptr(), lda, w.data_ptr(), _ptr(bias), 0, 0, residual.data_ptr(), ldr,
-                                 M, N, K, _CODE[a.dtype], F32, 0, _stream()), "linear")
+        _ok(_lib("gemm").dn_gemm(a.data_ptr(), lda, wp, _ptr(bias), 0, 0, residual.data_ptr(), ldr,
+                                 M, N, K, _CODE[a.dtype], F32, 0, packed, _stream()), "linear")
         return residual
     _dev(out, "out", _FLOATS, 2)
     _need(tuple(out.shape) == (M, N), "linear: out shape")
     ldc = _rows(out, "out")
-    _ok(_lib("gemm").dn_gemm(a.data_ptr(), lda, w.data_ptr(), _ptr(bias), out.data_ptr(), ldc, 0, 0, M, N, K,
-                             _CODE[a.dtype], _CODE[out.dtype], epi, _stream()), "linear")
+    _ok(_lib("gemm").dn_gemm(a.data_ptr(), lda, wp, _ptr(bias), out.data_ptr(), ldc, 0, 0, M, N, K,
+                             _CODE[a.dtype], _CODE[out.dtype], epi, packed, _stream()), "linear")
     return out
 
 
 def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
     """out = a @ w.T + bias, the fused projection q | k | v; the key columns (q_width ..) and the
     value columns after them also go to the slots slot_map[t] of the pools, as kv_write does.
-    One kernel in bfloat16 (the cache write is in the product's epilogue), else two."""
+    One kernel with a PackedMatrix and bfloat16 all through (the cache write is in the product's
+    epilogue), else two."""
     n_pages, Hkv, ps, dh = k_pool.shape
     kvw = Hkv * dh
-    if (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and a.is_cuda):
-        _dev(a, "a", None, 2), _dev(w, "w", None, 2), _dev(out, "out", None, 2)
+    if isinstance(w, PackedMatrix) and out.dtype == torch.bfloat16:
+        _dev(a, "a", (torch.bfloat16,), 2), _dev(out, "out", None, 2)
         _dev(slot_map, "slot_map", _I32, 1), _dev(k_pool, "k_pool", (torch.bfloat16,), 4)
         _dev(v_pool, "v_pool", (torch.bfloat16,), 4)
         M, K = a.shape
-        N = w.shape[0]
-        _need(w.is_contiguous() and w.shape[1] == K and tuple(out.shape) == (M, N), "linear_qkv: shapes")
+        wp, N, _ = _matrix(a, w, "linear_qkv")
+        _need(tuple(out.shape) == (M, N), "linear_qkv: shapes")
         _need(N == q_width + 2 * kvw, "linear_qkv: columns are not q | k | v")
         _need(k_pool.is_contiguous() and v_pool.is_contiguous() and tuple(v_pool.shape) == (n_pages, Hkv, dh, ps),
               "linear_qkv: pools")
@@ -225,13 +282,10 @@ def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
         if bias is not None:
             _dev(bias, "bias", (torch.float32,), 1)
             _need(bias.is_contiguous() and bias.shape[0] == N, "linear_qkv: bias")
-        rc = _lib("gemm").dn_gemm_qkv(a.data_ptr(), _rows(a, "a"), w.data_ptr(), _ptr(bias), out.data_ptr(),
-                                      _rows(out, "out"), M, N, K, slot_map.data_ptr(), k_pool.data_ptr(),
-                                      v_pool.data_ptr(), q_width, Hkv, dh, ps, _stream())
-        if rc == 0:
-            return out
-        if rc != 1:
-            _ok(rc, "linear_qkv")
+        _ok(_lib("gemm").dn_gemm_qkv(a.data_ptr(), _rows(a, "a"), wp, _ptr(bias), out.data_ptr(),
+                                     _rows(out, "out"), M, N, K, slot_map.data_ptr(), k_pool.data_ptr(),
+                                     v_pool.data_ptr(), q_width, Hkv, dh, ps, _stream()), "linear_qkv")
+        return out
     linear(a, w, bias, out=out)
     kv_write(out, q_width, q_width + kvw, slot_map, k_pool, v_pool)
     return out

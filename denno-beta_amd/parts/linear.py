@@ -1,6 +1,8 @@
 """Linear: a weight held [out, in] with an optional 32-bit bias, and the call that picks the
 product for its dtype.  A weight that a checkpoint stores [in, out] (Conv1D,
-crates/denno-engine/src/quant.rs:951-953) is transposed once at load (ParamSpec.transpose)."""
+crates/denno-engine/src/quant.rs:951-953) is transposed once at load (ParamSpec.transpose).
+A bfloat16 weight on the GPU is packed once at bind for the matrix cores (ops.PackedMatrix);
+the rows it came from are not kept, unless another part holds them (a tied table)."""
 from __future__ import annotations
 
 from typing import Optional
@@ -30,7 +32,10 @@ class Linear:
         return specs
 
     def bind(self, tensors):
-        self.weight = tensors[self.weight_name]
+        w = tensors[self.weight_name]
+        if w.dtype == torch.bfloat16 and w.is_cuda and w.shape[1] % 8 == 0:
+            w = ops.pack_matrix(w)
+        self.weight = w
         self.bias = tensors[self.bias_name] if self.bias_name else None
 
     def __call__(self, a, out_dtype=None, epilogue="none", residual=None):
@@ -49,8 +54,4 @@ class Linear:
         if a.dtype != self.weight.dtype:
             a = ops.cast(a.contiguous(), torch.empty(a.shape, dtype=self.weight.dtype, device=a.device))
         out = torch.empty((a.shape[0], self.out_features), dtype=out_dtype, device=a.device)
-        if out_dtype != a.dtype:
-            ops.linear(a, self.weight, self.bias, out=out)
-            ops.kv_write(out, q_width, q_width + (self.out_features - q_width) // 2, slot_map, k_pool, v_pool)
-            return out
         return ops.linear_qkv(a, self.weight, self.bias, out, slot_map, k_pool, v_pool, q_width)

@@ -77,13 +77,20 @@ def test_kv_write(dtype):
 
 @pytest.mark.parametrize("in_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", [(1, 1001, 72), (5, 64, 8), (130, 200, 320), (64, 1600, 1600), (33, 50257, 96),
-                                   (200, 333, 72), (300, 1600, 1600), (257, 129, 200), (2048, 256, 6400)])
+                                   (200, 333, 72), (300, 1600, 1600), (257, 129, 200), (2048, 256, 6400),
+                                   (48, 4800, 1600), (17, 4104, 72), (40, 33000, 40)])
 def test_linear(in_dtype, M, N, K):
     a, w, bias = rnd(M, K, seed=7, dtype=in_dtype), rnd(N, K, seed=8, dtype=in_dtype, scale=0.2), rnd(N, seed=9)
+    if in_dtype == torch.bfloat16:      # the MFMA kernels take the packed matrix; rows go to the plain kernel
+        rows, w = w, ops().pack_matrix(w)
+        assert torch.equal(w.rows(), rows)
+        w_ref = rows
+    else:
+        w_ref = w
     # the reference sums in 64-bit; a 32-bit sum of K terms is off by about sqrt(K) roundings
     tol = dict(TOL[in_dtype])
     tol["atol"] = max(tol["atol"], 4e-6 * math.sqrt(K))
-    exact = lambda epi: R.linear(a.double(), w.double(), bias.double(), out=torch.empty(M, N, dtype=torch.float64, device=DEV),   # noqa: E731
+    exact = lambda epi: R.linear(a.double(), w_ref.double(), bias.double(), out=torch.empty(M, N, dtype=torch.float64, device=DEV),   # noqa: E731
                                  epilogue=epi).float()
     for out_dtype in (torch.float32, in_dtype):
         for epi in ("none", "gelu_tanh", "gelu_erf"):
@@ -91,14 +98,18 @@ def test_linear(in_dtype, M, N, K):
             ops().linear(a, w, bias, out=out, epilogue=epi)
             assert torch.allclose(out.float(), exact(epi), **(tol if out_dtype == in_dtype else dict(tol, rtol=TOL[in_dtype]["rtol"]))), (out_dtype, epi)
     res = rnd(M, N, seed=10)
-    want = (res.double() + a.double() @ w.double().t()).float()
+    want = (res.double() + a.double() @ w_ref.double().t()).float()
     ops().linear(a, w, None, residual=res)
     assert torch.allclose(res, want, **tol)
     # rows taken out of a wider matrix (a leading dimension larger than K)
     wide = rnd(M, K + 24, seed=11, dtype=in_dtype)
     out = torch.empty(M, N, device=DEV)
     ops().linear(wide[:, 8:8 + K], w, bias, out=out)
-    assert torch.allclose(out, R.linear(wide[:, 8:8 + K], w, bias, out=torch.empty_like(out)), **tol)
+    assert torch.allclose(out, R.linear(wide[:, 8:8 + K], w_ref, bias, out=torch.empty_like(out)), **tol)
+    if in_dtype == torch.bfloat16 and M * N * K < 10 ** 8:
+        # bfloat16 rows, not packed: the plain kernel
+        ops().linear(a, w_ref, bias, out=out)
+        assert torch.allclose(out, exact("none"), **tol)
 
 
 @pytest.mark.parametrize("M", [1, 8, 20, 64, 70, 300])
@@ -116,6 +127,7 @@ def test_linear_qkv_writes_the_cache(M):
     pools = [torch.zeros(n_pages, Hkv, ps, dh, dtype=torch.bfloat16, device=DEV),
              torch.zeros(n_pages, Hkv, dh, ps, dtype=torch.bfloat16, device=DEV)]
     want_pools = [torch.zeros_like(p) for p in pools]
+    w = ops().pack_matrix(w)
     out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
     ops().linear_qkv(a, w, bias, out, slots, pools[0], pools[1], H * dh)
     want = torch.empty_like(out)

@@ -552,7 +552,8 @@ __global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__
       }
     }
     if (n_splits == 1) {
-      out[static_cast<size_t>(row) * ldo + h * DH + d] = from_float<bf16_t>(A / L);
+      out[ldo > 0 ? static_cast<size_t>(row) * ldo + h * DH + d : packed_index(row, h * DH + d, H * DH / 32)] =
+          from_float<bf16_t>(A / L);
     } else {
       mypart[2 + d] = A;
       if (d == 0) {
@@ -581,13 +582,15 @@ __global__ void join_kernel(const float* __restrict__ part, bf16_t* __restrict__
         A += ps[2 + d] * f;
       }
     }
-    out[static_cast<size_t>(tile) * ldo + h * DH + d] = from_float<bf16_t>(A / L);
+    out[ldo > 0 ? static_cast<size_t>(tile) * ldo + h * DH + d : packed_index(tile, h * DH + d, H * DH / 32)] =
+        from_float<bf16_t>(A / L);
   }
 }
 }  // namespace decode
 
 // part: 32-bit workspace of n_tiles * H * n_splits * (dh + 2) floats (unused when n_splits == 1);
-// the splits cover n_splits * chunks * 256 keys, which must reach the longest context
+// the splits cover n_splits * chunks * 256 keys, which must reach the longest context.
+// ldo == 0: out is a packed matrix of H * dh columns (a multiple of 32)
 extern "C" int dn_attention_decode(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
                                    const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
                                    const int32_t* tile_row0, const int32_t* tile_pos0, int n_tiles, float* part,
@@ -595,7 +598,7 @@ extern "C" int dn_attention_decode(const void* q, int ldq, void* out, int ldo, c
                                    int window, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (Hkv < 1 || H % Hkv != 0 || page_size % 16 != 0 || max_blocks < 1 || n_splits < 1 || chunks < 1 ||
-      ldq % 8 != 0 || reinterpret_cast<uintptr_t>(q) % 16 != 0 || reinterpret_cast<uintptr_t>(k_pool) % 16 != 0 ||
+      ldq % 8 != 0 || ldo < 0 || (ldo == 0 && (H * dh) % 32 != 0) || reinterpret_cast<uintptr_t>(q) % 16 != 0 || reinterpret_cast<uintptr_t>(k_pool) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(v_pool) % 16 != 0)
     return DN_ERR_SHAPE;
   dim3 grid(n_splits, H, n_tiles), block(256);

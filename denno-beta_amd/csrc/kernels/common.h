@@ -91,3 +91,12 @@ __device__ __forceinline__ float other_half(float v) {
 }
 
 static inline int dn_launch_status() { return static_cast<int>(hipGetLastError()); }
+
+// A packed matrix: blocks of 16 rows x 32 columns, 1 KB each and contiguous, block (r / 16, k / 32)
+// at ((r / 16) * ksteps + k / 32) * 512 elements; inside it the 8 elements from column k % 32 / 8 * 8
+// of row r % 16 lie at ((k % 32 / 8) * 16 + r % 16) * 8: the 16 bytes that lane r % 16 + 16 * (k % 32 / 8)
+// feeds to v_mfma_f32_16x16x32_bf16.  Every weight of the MFMA kernels is held so, and so are the
+// bfloat16 rows that one kernel hands to the next while a step has at most 64 of them.
+__device__ __forceinline__ size_t packed_index(int r, int k, int ksteps) {
+  return ((static_cast<size_t>(r / 16) * ksteps + k / 32) * 64 + ((k % 32) / 8) * 16 + r % 16) * 8 + k % 8;
+}

@@ -50,7 +50,7 @@ extern "C" int dn_embed(const int32_t* tokens, const int32_t* positions, const v
 template <typename TO>
 __global__ void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ gamma,
                                  const float* __restrict__ beta, TO* __restrict__ out,
-                                 const int32_t* __restrict__ rows, int R, int E, float eps) {
+                                 const int32_t* __restrict__ rows, int R, int E, float eps, int packed) {
   int wave = threadIdx.x / DN_WAVE, lane = threadIdx.x % DN_WAVE;
   int r = blockIdx.x * (blockDim.x / DN_WAVE) + wave;
   if (r >= R) return;
@@ -65,11 +65,10 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const float* __res
     v += d * d;
   }
   float inv = 1.0f / sqrtf(wave_sum(v) / static_cast<float>(E) + eps);
-  TO* o = out + static_cast<size_t>(r) * E;
   for (int e = lane; e < E; e += DN_WAVE) {
     float y = (xr[e] - mean) * inv * gamma[e];
     if (beta) y += beta[e];
-    o[e] = from_float<TO>(y);
+    out[packed ? packed_index(r, e, E / 32) : static_cast<size_t>(r) * E + e] = from_float<TO>(y);
   }
 }
 
@@ -89,7 +88,8 @@ template <typename TO, int VPT>
 __global__ __launch_bounds__(256) void layernorm_row_kernel(const float* __restrict__ x,
                                                              const float* __restrict__ gamma,
                                                              const float* __restrict__ beta, TO* __restrict__ out,
-                                                             const int32_t* __restrict__ rows, int E, float eps) {
+                                                             const int32_t* __restrict__ rows, int E, float eps,
+                                                             int packed) {
   __shared__ float scratch[4];
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
@@ -118,42 +118,43 @@ __global__ __launch_bounds__(256) void layernorm_row_kernel(const float* __restr
     q += d * d;
   }
   const float inv = 1.0f / sqrtf(block_sum_256(q, scratch) / static_cast<float>(E) + eps);
-  TO* o = out + static_cast<size_t>(r) * E;
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     int e = threadIdx.x + i * 256;
     if (e < E) {
       float y = (v[i] - mean) * inv * gm[i];
       if (beta) y += bt[i];
-      o[e] = from_float<TO>(y);
+      out[packed ? packed_index(r, e, E / 32) : static_cast<size_t>(r) * E + e] = from_float<TO>(y);
     }
   }
 }
 
 template <typename TO>
 static void launch_layernorm(const float* x, const float* gamma, const float* beta, TO* out, const int32_t* rows,
-                             int R, int E, float eps, hipStream_t stream) {
+                             int R, int E, float eps, int packed, hipStream_t stream) {
   if (E <= 512)
-    hipLaunchKernelGGL((layernorm_row_kernel<TO, 2>), dim3(R), dim3(256), 0, stream, x, gamma, beta, out, rows, E, eps);
+    hipLaunchKernelGGL((layernorm_row_kernel<TO, 2>), dim3(R), dim3(256), 0, stream, x, gamma, beta, out, rows, E, eps, packed);
   else if (E <= 2048)
-    hipLaunchKernelGGL((layernorm_row_kernel<TO, 8>), dim3(R), dim3(256), 0, stream, x, gamma, beta, out, rows, E, eps);
+    hipLaunchKernelGGL((layernorm_row_kernel<TO, 8>), dim3(R), dim3(256), 0, stream, x, gamma, beta, out, rows, E, eps, packed);
   else if (E <= 8192)
     hipLaunchKernelGGL((layernorm_row_kernel<TO, 32>), dim3(R), dim3(256), 0, stream, x, gamma, beta, out, rows, E,
-                       eps);
+                       eps, packed);
   else {
     const int waves = 4;
     hipLaunchKernelGGL(layernorm_kernel<TO>, dim3((R + waves - 1) / waves), dim3(waves * DN_WAVE), 0, stream, x, gamma,
-                       beta, out, rows, R, E, eps);
+                       beta, out, rows, R, E, eps, packed);
   }
 }
 
+// packed: out is a packed matrix of ceil(R / 16) * 16 rows (bfloat16, E a multiple of 32)
 extern "C" int dn_layernorm(const float* x, const float* gamma, const float* beta, void* out, const int32_t* rows,
-                            int R, int E, float eps, int out_dtype, hipStream_t stream) {
+                            int R, int E, float eps, int out_dtype, int packed, hipStream_t stream) {
   if (R <= 0) return 0;
+  if (packed && (out_dtype != DN_BF16 || E % 32 != 0)) return DN_ERR_SHAPE;
   if (out_dtype == DN_F32)
-    launch_layernorm<float>(x, gamma, beta, static_cast<float*>(out), rows, R, E, eps, stream);
+    launch_layernorm<float>(x, gamma, beta, static_cast<float*>(out), rows, R, E, eps, 0, stream);
   else if (out_dtype == DN_BF16)
-    launch_layernorm<bf16_t>(x, gamma, beta, static_cast<bf16_t*>(out), rows, R, E, eps, stream);
+    launch_layernorm<bf16_t>(x, gamma, beta, static_cast<bf16_t*>(out), rows, R, E, eps, packed, stream);
   else
     return DN_ERR_DTYPE;
   return dn_launch_status();

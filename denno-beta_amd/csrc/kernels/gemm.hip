@@ -143,6 +143,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(const TI* __restrict__ A, int
 // 16-row blocks of A (lane = row + 16 * (k / 8)).  The waves' sums meet in LDS and are added in
 // wave order, so the result has one order of summation whatever M is.  No atomics.
 // ---------------------------------------------------------------------------------------
+#define PACKED_W 1
+#define PACKED_A 2
+#define PACKED_C 4
+
 namespace skinny {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
@@ -153,7 +157,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
                                                            const bf16_t* __restrict__ W,
                                                            const float* __restrict__ bias, TC* __restrict__ C,
                                                            int ldc, float* __restrict__ resid, int ldr, int M, int N,
-                                                           int K, int epi, KVScatter kv) {
+                                                           int K, int epi, int packed, KVScatter kv) {
   constexpr int BLOCKS = MB * NB;                          // 16 x 16 blocks of C in this workgroup
   constexpr int PASSES = (BLOCKS + WAVES - 1) / WAVES;     // wave w finishes blocks w, w + WAVES, ...
   __shared__ floatx4 red[WAVES][BLOCKS][64];
@@ -205,13 +209,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
       b[u][nb] = *reinterpret_cast<const bf16x8*>(ks < ksteps ? wblk[nb] + ks * 512 : W + lane * 8);
   }
 
+  // A in rows, or packed like W (PACKED_A): then a wave reads 1 KB in one piece per block
   const bf16_t* arow[MB];
   bool a_ok[MB];
+  const int astep = (packed & PACKED_A) ? 512 : 32;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     int row = mb * 16 + col;
     a_ok[mb] = row < M;
-    arow[mb] = A + static_cast<size_t>(a_ok[mb] ? row : 0) * lda + g * 8;
+    arow[mb] = (packed & PACKED_A) ? A + (static_cast<size_t>(mb) * ksteps * 64 + lane) * 8
+                                   : A + static_cast<size_t>(a_ok[mb] ? row : 0) * lda + g * 8;
   }
   floatx4 acc[MB][NB];
 #pragma unroll
@@ -231,7 +238,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
       }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
-        a[u][mb] = *reinterpret_cast<const bf16x8*>(ok ? arow[mb] + ks * 32 : arow[mb]);
+        a[u][mb] = *reinterpret_cast<const bf16x8*>(ok ? arow[mb] + ks * astep : arow[mb]);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -273,7 +280,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
         resid[static_cast<size_t>(m) * ldr + nn] = epi_x[p][r] + v;
       } else {
         TC cv = from_float<TC>(apply_epilogue(v, epi));
-        C[static_cast<size_t>(m) * ldc + nn] = cv;
+        C[(packed & PACKED_C) ? packed_index(m, nn, N / 32) : static_cast<size_t>(m) * ldc + nn] = cv;
         if constexpr (KV) scatter_kv(kv, m, nn, cv);
       }
     }
@@ -282,7 +289,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
 
 struct Call {
   const void* A; int lda; const void* W; const float* bias; void* C; int ldc; float* resid; int ldr;
-  int M, N, K, out_dtype, epi;
+  int M, N, K, out_dtype, epi, packed;
   const KVScatter* kv;
 };
 
@@ -292,7 +299,7 @@ static void launch_one(const Call& c, hipStream_t stream) {
   KVScatter kv = c.kv ? *c.kv : KVScatter{};
   hipLaunchKernelGGL((gemm_kernel<MB, NB, WAVES, U, TC, KV>), grid, block, 0, stream,
                      static_cast<const bf16_t*>(c.A), c.lda, static_cast<const bf16_t*>(c.W), c.bias,
-                     static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N, c.K, c.epi, kv);
+                     static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N, c.K, c.epi, c.packed, kv);
 }
 
 template <int MB, int NB, int WAVES, int U>
@@ -338,10 +345,11 @@ static void run(const Call& c, hipStream_t stream) {
     launch_mb<4>(c, stream);
 }
 
-// A must allow 16-byte loads: K and lda multiples of 8, the base aligned; W is packed
-static bool takes(const void* A, int lda, const void* W, int M, int K) {
-  return M <= 64 && K % 8 == 0 && lda % 8 == 0 && reinterpret_cast<uintptr_t>(A) % 16 == 0 &&
-         reinterpret_cast<uintptr_t>(W) % 16 == 0;
+// A must allow 16-byte loads: in rows with K and lda multiples of 8 and the base aligned, or packed
+// (K a multiple of 32 then: nothing zeroes a packed block's columns beyond K); W is packed
+static bool takes(const void* A, int lda, const void* W, int M, int K, int packed) {
+  if (M > 64 || reinterpret_cast<uintptr_t>(A) % 16 != 0 || reinterpret_cast<uintptr_t>(W) % 16 != 0) return false;
+  return (packed & PACKED_A) ? K % 32 == 0 : (K % 8 == 0 && lda % 8 == 0);
 }
 }  // namespace skinny
 
@@ -535,22 +543,27 @@ static int run(const void* A, int lda, const void* W, const float* bias, void* C
 }
 }  // namespace tiled
 
-// W: rows of K elements (w_packed 0; the plain kernel, any dtype), or packed bfloat16
-// (w_packed 1; the MFMA kernels, which need A in bfloat16 and loadable 16 bytes at a time).
+// packed: bit flags.  W in rows of K elements (the plain kernel, any dtype), or packed bfloat16
+// (PACKED_W 1: the MFMA kernels, which need A in bfloat16 and loadable 16 bytes at a time).  With
+// at most 64 rows A may be packed too (PACKED_A 2; lda is not read) and so may a bfloat16 C
+// (PACKED_C 4; N a multiple of 32; ldc is not read).
 extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid,
-                       int ldr, int M, int N, int K, int in_dtype, int out_dtype, int epilogue, int w_packed,
+                       int ldr, int M, int N, int K, int in_dtype, int out_dtype, int epilogue, int packed,
                        hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || K % 4 != 0 || lda < K) return DN_ERR_SHAPE;
+  if (K <= 0 || K % 4 != 0 || (lda < K && !(packed & PACKED_A))) return DN_ERR_SHAPE;
   if (epilogue < EPI_NONE || epilogue > EPI_GELU_ERF) return DN_ERR_SHAPE;
   if (resid != nullptr && epilogue != EPI_NONE) return DN_ERR_SHAPE;
-  if (w_packed) {
+  if ((packed & (PACKED_A | PACKED_C)) && (!(packed & PACKED_W) || M > 64)) return DN_ERR_SHAPE;
+  if ((packed & PACKED_C) && (resid != nullptr || out_dtype != DN_BF16 || N % 32 != 0)) return DN_ERR_SHAPE;
+  if (packed & PACKED_W) {
     if (in_dtype != DN_BF16) return DN_ERR_DTYPE;
-    if (skinny::takes(A, lda, W, M, K)) {
-      skinny::Call c{A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr};
+    if (skinny::takes(A, lda, W, M, K, packed)) {
+      skinny::Call c{A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, packed, nullptr};
       skinny::run(c, stream);
       return dn_launch_status();
     }
+    if (packed & (PACKED_A | PACKED_C)) return DN_ERR_SHAPE;
     if (!tiled::takes(A, lda, W, K)) return DN_ERR_SHAPE;
     int rc = tiled::run(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr, stream);
     return rc != 0 ? rc : dn_launch_status();
@@ -575,19 +588,20 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
 
 // The fused projection q | k | v with packed W: C = A . W^T + bias as dn_gemm computes it, and the
 // key and value columns also go to their pages (see KVScatter), from the epilogue of the few-rows
-// or of the tiled kernel.
+// or of the tiled kernel.  a_packed: A is packed (at most 64 rows).
 extern "C" int dn_gemm_qkv(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, int M, int N,
                            int K, const int32_t* slot_map, void* k_pool, void* v_pool, int q_width, int Hkv, int dh,
-                           int page_size, hipStream_t stream) {
+                           int page_size, int a_packed, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || lda < K) return DN_ERR_SHAPE;
-  const bool few = skinny::takes(A, lda, W, M, K);
-  if (!few && !tiled::takes(A, lda, W, K)) return DN_ERR_SHAPE;
+  const int packed = PACKED_W | (a_packed ? PACKED_A : 0);
+  if (K <= 0 || (lda < K && !a_packed)) return DN_ERR_SHAPE;
+  const bool few = skinny::takes(A, lda, W, M, K, packed);
+  if (!few && (a_packed || !tiled::takes(A, lda, W, K))) return DN_ERR_SHAPE;
   if (q_width < 0 || q_width + 2 * Hkv * dh != N || page_size < 1) return DN_ERR_SHAPE;
   KVScatter kv{slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_width, Hkv * dh, dh,
                page_size, Hkv};
   if (few) {
-    skinny::Call c{A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv};
+    skinny::Call c{A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, packed, &kv};
     skinny::run(c, stream);
     return dn_launch_status();
   }

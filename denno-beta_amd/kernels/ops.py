@@ -41,14 +41,14 @@ def _declare(name, lib):
     sigs = {
         "elementwise": {
             "dn_embed": [P, P, P, P, P, I, I, I, I, I, P],
-            "dn_layernorm": [P, P, P, P, P, I, I, F, I, P],
+            "dn_layernorm": [P, P, P, P, P, I, I, F, I, I, P],
             "dn_kv_write": [P, I, I, I, P, P, P, I, I, I, I, I, P],
             "dn_cast": [P, P, c_longlong, I, I, P],
         },
         "gemm": {
             "dn_gemm": [P, I, P, P, P, I, P, I, I, I, I, I, I, I, I, P],
             "dn_pack_matrix": [P, P, I, I, P],
-            "dn_gemm_qkv": [P, I, P, P, P, I, I, I, I, P, P, P, I, I, I, I, P],
+            "dn_gemm_qkv": [P, I, P, P, P, I, I, I, I, P, P, P, I, I, I, I, I, P],
         },
         "attention": {
             "dn_attention": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, I, P],
@@ -129,11 +129,74 @@ def embed(tokens, positions, wte, wpe, out):
     return out
 
 
+class PackedMatrix:
+    """A bfloat16 matrix [N, K] laid out for the matrix cores: blocks of 16 rows x 32 columns, 1 KB
+    each and contiguous, block (n // 16, k // 32) at ((n // 16) * ceil(K / 32) + k // 32) * 512
+    elements; inside it row n % 16, columns (k % 32) // 8 * 8 .. + 7 at (((k % 32) // 8) * 16 + n % 16) * 8.
+    `linear` takes it for the MFMA kernels.  Every bfloat16 weight is held so (rows and columns
+    beyond N and K are zeros), and so are the bfloat16 rows that one kernel hands to the next
+    while a step has at most 64 of them (`packed_rows`; K a multiple of 32, rows beyond N are
+    not written and never read into a result)."""
+    __slots__ = ("data", "shape")
+    dtype = torch.bfloat16
+
+    def __init__(self, data, shape):
+        self.data, self.shape = data, tuple(shape)
+
+    @property
+    def device(self):
+        return self.data.device
+
+    def data_ptr(self):
+        return self.data.data_ptr()
+
+    def numel(self):
+        return self.shape[0] * self.shape[1]
+
+    def element_size(self):
+        return 2
+
+    def rows(self):
+        """The matrix [N, K] again (for tests and tools)."""
+        N, K = self.shape
+        nb, ks = -(-N // 16), -(-K // 32)
+        return self.data.view(nb, ks, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(nb * 16, ks * 32)[:N, :K].contiguous()
+
+
+PACKED_ROWS_MAX = 64     # the few-rows product's limit
+PACKED_ROWS_MIN = 9      # below, rows in the ordinary layout were measured as fast or faster (one row: 10 % faster)
+
+
+def packed_rows(n_rows, width, device) -> PackedMatrix:
+    """An empty packed matrix for n_rows <= 64 rows of activations."""
+    _need(n_rows <= PACKED_ROWS_MAX and width % 32 == 0,
+          f"packed rows: at most {PACKED_ROWS_MAX} rows of a width that is a multiple of 32, not {n_rows} x {width}")
+    data = torch.empty(-(-n_rows // 16) * (width // 32) * 512, dtype=torch.bfloat16, device=device)
+    return PackedMatrix(data, (n_rows, width))
+
+
+def pack_matrix(w) -> PackedMatrix:
+    """w: bfloat16 [N, K], rows contiguous, K a multiple of 8."""
+    _dev(w, "w", (torch.bfloat16,), 2)
+    N, K = w.shape
+    _need(w.is_contiguous(), "pack_matrix: w must be contiguous")
+    _need(K % 8 == 0, f"pack_matrix: the inner size {K} must be a multiple of 8")
+    data = torch.empty(-(-N // 16) * -(-K // 32) * 512, dtype=torch.bfloat16, device=w.device)
+    _ok(_lib("gemm").dn_pack_matrix(w.data_ptr(), data.data_ptr(), N, K, _stream()), "pack_matrix")
+    return PackedMatrix(data, (N, K))
+
+
 def layernorm(x, gamma, beta, eps, out, rows=None):
-    """out[r,:] = LayerNorm(x[rows[r],:]) (rows None: every row).  x, gamma, beta are 32-bit."""
-    _dev(x, "x", (torch.float32,), 2), _dev(gamma, "gamma", (torch.float32,), 1), _dev(out, "out", _FLOATS, 2)
+    """out[r,:] = LayerNorm(x[rows[r],:]) (rows None: every row).  x, gamma, beta are 32-bit;
+    out: a tensor [R, E], or packed rows."""
+    packed = isinstance(out, PackedMatrix)
+    _dev(x, "x", (torch.float32,), 2), _dev(gamma, "gamma", (torch.float32,), 1)
+    if packed:
+        _need(out.device == x.device, "layernorm: out on another device")
+    else:
+        _dev(out, "out", _FLOATS, 2)
     E = x.shape[1]
-    _need(x.is_contiguous() and out.is_contiguous() and gamma.is_contiguous() and gamma.shape[0] == E,
+    _need(x.is_contiguous() and (packed or out.is_contiguous()) and gamma.is_contiguous() and gamma.shape[0] == E,
           "layernorm: shapes")
     if beta is not None:
         _dev(beta, "beta", (torch.float32,), 1)
@@ -146,7 +209,7 @@ def layernorm(x, gamma, beta, eps, out, rows=None):
         _need(R == x.shape[0], "layernorm: out rows")
     _need(out.shape[1] == E, "layernorm: out width")
     _ok(_lib("elementwise").dn_layernorm(x.data_ptr(), gamma.data_ptr(), _ptr(beta), out.data_ptr(), _ptr(rows),
-                                         R, E, float(eps), _CODE[out.dtype], _stream()), "layernorm")
+                                         R, E, float(eps), _CODE[out.dtype], int(packed), _stream()), "layernorm")
     return out
 
 
@@ -178,70 +241,38 @@ def cast(x, out):
     return out
 
 
-class PackedMatrix:
-    """A bfloat16 matrix [N, K] laid out for the matrix cores: blocks of 16 rows x 32 columns, 1 KB
-    each and contiguous, block (n // 16, k // 32) at ((n // 16) * ceil(K / 32) + k // 32) * 512
-    elements; inside it row n % 16, columns (k % 32) // 8 * 8 .. + 7 at (((k % 32) // 8) * 16 + n % 16) * 8.
-    Rows and columns beyond N and K are zeros.  `linear` takes it for the MFMA kernels."""
-    __slots__ = ("data", "shape")
-    dtype = torch.bfloat16
-
-    def __init__(self, data, shape):
-        self.data, self.shape = data, tuple(shape)
-
-    @property
-    def device(self):
-        return self.data.device
-
-    def data_ptr(self):
-        return self.data.data_ptr()
-
-    def numel(self):
-        return self.shape[0] * self.shape[1]
-
-    def element_size(self):
-        return 2
-
-    def rows(self):
-        """The matrix [N, K] again (for tests and tools)."""
-        N, K = self.shape
-        nb, ks = -(-N // 16), -(-K // 32)
-        return self.data.view(nb, ks, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(nb * 16, ks * 32)[:N, :K].contiguous()
+PACKED_W, PACKED_A, PACKED_C = 1, 2, 4
 
 
-def pack_matrix(w) -> PackedMatrix:
-    """w: bfloat16 [N, K], rows contiguous, K a multiple of 8."""
-    _dev(w, "w", (torch.bfloat16,), 2)
-    N, K = w.shape
-    _need(w.is_contiguous(), "pack_matrix: w must be contiguous")
-    _need(K % 8 == 0, f"pack_matrix: the inner size {K} must be a multiple of 8")
-    data = torch.empty(-(-N // 16) * -(-K // 32) * 512, dtype=torch.bfloat16, device=w.device)
-    _ok(_lib("gemm").dn_pack_matrix(w.data_ptr(), data.data_ptr(), N, K, _stream()), "pack_matrix")
-    return PackedMatrix(data, (N, K))
-
-
-def _matrix(a, w, what):
-    """(pointer, N, packed flag) of a weight for a [M, K]."""
-    K = a.shape[1]
+def _operands(a, w, what):
+    """(leading dimension of a, N, packed flags) of the product a [M, K] . w [N, K]^T."""
+    M, K = a.shape
+    if isinstance(a, PackedMatrix):
+        _need(isinstance(w, PackedMatrix), f"{what}: packed rows need a packed matrix")
+        _need(M <= PACKED_ROWS_MAX and K % 32 == 0, f"{what}: packed rows {a.shape}")
+        lda, flags = 0, PACKED_A
+    else:
+        _dev(a, "a", _FLOATS, 2)
+        lda, flags = _rows(a, "a"), 0
     if isinstance(w, PackedMatrix):
         _need(a.dtype == torch.bfloat16, f"{what}: a packed matrix needs bfloat16 rows, not {a.dtype}")
         _need(w.device == a.device and w.shape[1] == K, f"{what}: w {w.shape} does not fit a {tuple(a.shape)}")
-        _need(a.data_ptr() % 16 == 0 and a.stride(0) % 8 == 0, f"{what}: the rows of a must be aligned to 16 bytes")
-        return w.data_ptr(), w.shape[0], 1
+        _need(a.data_ptr() % 16 == 0 and lda % 8 == 0, f"{what}: the rows of a must be aligned to 16 bytes")
+        return lda, w.shape[0], flags | PACKED_W
     _dev(w, "w", (a.dtype,), 2)
     _need(w.is_contiguous() and w.shape[1] == K, f"{what}: w {tuple(w.shape)} does not fit a {tuple(a.shape)}")
-    return w.data_ptr(), w.shape[0], 0
+    return lda, w.shape[0], flags
 
 
 def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
     """out = epilogue(a @ w.T + bias), or residual += a @ w.T + bias (32-bit, in place).
     a: [M, K] rows contiguous; w: [N, K] held [out, in], in rows (the plain kernel: 32-bit, or a
-    reference for bfloat16) or a PackedMatrix (the MFMA kernels); bias: 32-bit [N]."""
-    _dev(a, "a", _FLOATS, 2)
+    reference for bfloat16) or a PackedMatrix (the MFMA kernels); bias: 32-bit [N].  With a packed
+    w and at most 64 rows, a and a bfloat16 out may be packed rows."""
     M, K = a.shape
     _need(K % 8 == 0, f"linear: the inner size {K} must be a multiple of 8")
-    wp, N, packed = _matrix(a, w, "linear")
-    lda = _rows(a, "a")
+    lda, N, packed = _operands(a, w, "linear")
+    wp = w.data_ptr()
     if bias is not None:
         _dev(bias, "bias", (torch.float32,), 1)
         _need(bias.is_contiguous() and bias.shape[0] == N, "linear: bias")
@@ -253,9 +284,14 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
         _ok(_lib("gemm").dn_gemm(a.data_ptr(), lda, wp, _ptr(bias), 0, 0, residual.data_ptr(), ldr,
                                  M, N, K, _CODE[a.dtype], F32, 0, packed, _stream()), "linear")
         return residual
-    _dev(out, "out", _FLOATS, 2)
+    if isinstance(out, PackedMatrix):
+        _need((packed & PACKED_W) and M <= PACKED_ROWS_MAX and N % 32 == 0 and out.device == a.device,
+              f"linear: packed rows as out need a packed w, at most {PACKED_ROWS_MAX} rows and N a multiple of 32")
+        ldc, packed = 0, packed | PACKED_C
+    else:
+        _dev(out, "out", _FLOATS, 2)
+        ldc = _rows(out, "out")
     _need(tuple(out.shape) == (M, N), "linear: out shape")
-    ldc = _rows(out, "out")
     _ok(_lib("gemm").dn_gemm(a.data_ptr(), lda, wp, _ptr(bias), out.data_ptr(), ldc, 0, 0, M, N, K,
                              _CODE[a.dtype], _CODE[out.dtype], epi, packed, _stream()), "linear")
     return out
@@ -269,11 +305,11 @@ def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
     n_pages, Hkv, ps, dh = k_pool.shape
     kvw = Hkv * dh
     if isinstance(w, PackedMatrix) and out.dtype == torch.bfloat16:
-        _dev(a, "a", (torch.bfloat16,), 2), _dev(out, "out", None, 2)
+        _dev(out, "out", None, 2)
         _dev(slot_map, "slot_map", _I32, 1), _dev(k_pool, "k_pool", (torch.bfloat16,), 4)
         _dev(v_pool, "v_pool", (torch.bfloat16,), 4)
         M, K = a.shape
-        wp, N, _ = _matrix(a, w, "linear_qkv")
+        lda, N, packed = _operands(a, w, "linear_qkv")
         _need(tuple(out.shape) == (M, N), "linear_qkv: shapes")
         _need(N == q_width + 2 * kvw, "linear_qkv: columns are not q | k | v")
         _need(k_pool.is_contiguous() and v_pool.is_contiguous() and tuple(v_pool.shape) == (n_pages, Hkv, dh, ps),
@@ -282,9 +318,10 @@ def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
         if bias is not None:
             _dev(bias, "bias", (torch.float32,), 1)
             _need(bias.is_contiguous() and bias.shape[0] == N, "linear_qkv: bias")
-        _ok(_lib("gemm").dn_gemm_qkv(a.data_ptr(), _rows(a, "a"), wp, _ptr(bias), out.data_ptr(),
+        _ok(_lib("gemm").dn_gemm_qkv(a.data_ptr(), lda, w.data_ptr(), _ptr(bias), out.data_ptr(),
                                      _rows(out, "out"), M, N, K, slot_map.data_ptr(), k_pool.data_ptr(),
-                                     v_pool.data_ptr(), q_width, Hkv, dh, ps, _stream()), "linear_qkv")
+                                     v_pool.data_ptr(), q_width, Hkv, dh, ps, int(bool(packed & PACKED_A)),
+                                     _stream()), "linear_qkv")
         return out
     linear(a, w, bias, out=out)
     kv_write(out, q_width, q_width + kvw, slot_map, k_pool, v_pool)
@@ -294,6 +331,12 @@ def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
 FLASH_HEAD_DIMS = (16, 32, 48, 64, 96, 128)
 DECODE_HEAD_DIMS = (16, 32, 64, 128, 256)
 DECODE_SPLIT = 256
+
+
+def decode_attention_applies(dtype, page_size, head_dim, single_rows, max_context):
+    """Whether `attention` takes the split kernel of pure decode steps (which can write packed rows)."""
+    return (dtype == torch.bfloat16 and page_size % 16 == 0 and bool(single_rows) and head_dim in DECODE_HEAD_DIMS
+            and max_context > 0)
 
 
 def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, window=0, tiles_wide=None,
@@ -309,8 +352,12 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
     max_context: the longest context then.
 
     Three kernels: 32-bit takes the plain one; bfloat16 takes the MFMA kernel over tiles_wide, or,
-    for a pure decode step, the split kernel; a head size that those do not take falls to the plain one."""
-    _dev(q, "q", _FLOATS, 2), _dev(out, "out", (q.dtype,), 2)
+    for a pure decode step, the split kernel (out may then be packed rows); a head size that those
+    do not take falls to the plain one."""
+    out_packed = isinstance(out, PackedMatrix)
+    _dev(q, "q", _FLOATS, 2)
+    if not out_packed:
+        _dev(out, "out", (q.dtype,), 2)
     _dev(k_pool, "k_pool", (q.dtype,), 4), _dev(v_pool, "v_pool", (q.dtype,), 4)
     _dev(block_tables, "block_tables", _I32, 2), _dev(tiles, "tiles", _I32, 2)
     n_pages, Hkv, ps, dh = k_pool.shape
@@ -321,10 +368,12 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
     _need(block_tables.is_contiguous() and tiles.is_contiguous() and tiles.shape[0] == 4, "attention: tables")
     _need(dh % 16 == 0 and 16 <= dh <= 256, f"attention: head size {dh} must be a multiple of 16 up to 256")
     _need(n_heads % Hkv == 0, f"attention: {n_heads} heads over {Hkv} key heads")
-    ldq, ldo = _rows(q, "q"), _rows(out, "out")
+    ldq, ldo = _rows(q, "q"), (0 if out_packed else _rows(out, "out"))
     lib = _lib("attention")
     fast = q.dtype == torch.bfloat16 and ps % 16 == 0 and ldq % 8 == 0 and q.data_ptr() % 16 == 0
-    if fast and single_rows and dh in DECODE_HEAD_DIMS and max_context > 0:
+    decode = fast and decode_attention_applies(q.dtype, ps, dh, single_rows, max_context)
+    _need(decode or not out_packed, "attention: packed rows as out are written by the decode kernel only")
+    if decode:
         n_tiles = tiles.shape[1]
         # the context is split over workgroups only where the batch alone does not give about one
         # workgroup per CU: a second kernel has to join the splits

@@ -64,6 +64,12 @@ class Part:
     def bind(self, tensors: Dict[str, torch.Tensor], runtime: Runtime) -> None:
         self.runtime = runtime
 
+    def packed_input(self, n_rows: int) -> bool:
+        """A mixer or feed-forward whose first product takes packed rows (kernels.ops.PackedMatrix)
+        for a step of n_rows rows says so here; the block then asks the norm before it for them.
+        The default, a tensor [rows, width], is always right."""
+        return False
+
     # helpers ---------------------------------------------------------------
     def _take(self, tensors, name):
         return tensors[name]

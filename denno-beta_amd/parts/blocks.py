@@ -15,7 +15,8 @@ class PreNormBlock:
         return [self.norm1, self.mixer, self.norm2, self.ffn]
 
     def forward(self, x, ctx, cache, runtime):
-        h = self.norm1.forward(x, runtime.act_dtype)
+        n = x.shape[0]
+        h = self.norm1.forward(x, runtime.act_dtype, packed=self.mixer.packed_input(n))
         self.mixer.forward(h, ctx, cache, accumulate_into=x)
-        h = self.norm2.forward(x, runtime.act_dtype)
+        h = self.norm2.forward(x, runtime.act_dtype, packed=self.ffn.packed_input(n))
         self.ffn.forward(h, ctx, accumulate_into=x)

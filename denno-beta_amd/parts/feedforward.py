@@ -32,6 +32,11 @@ class DenseMLP(Part):
         self.up.bind(tensors)
         self.down.bind(tensors)
 
+    def packed_input(self, n_rows):
+        return self.up.packed_input(n_rows)
+
     def forward(self, h, ctx, accumulate_into):
-        f = self.up(h, out_dtype=self.runtime.act_dtype, epilogue=ACTIVATION_EPILOGUES[self.activation])
+        n = h.shape[0]
+        f = self.up(h, out_dtype=self.runtime.act_dtype, epilogue=ACTIVATION_EPILOGUES[self.activation],
+                    packed_out=self.up.few_rows(n) and self.down.packed_input(n))
         self.down(f, residual=accumulate_into)

@@ -38,15 +38,30 @@ class Linear:
         self.weight = w
         self.bias = tensors[self.bias_name] if self.bias_name else None
 
-    def __call__(self, a, out_dtype=None, epilogue="none", residual=None):
-        """epilogue(a @ W^T + b) as a new [M, out] tensor of out_dtype, or added into
-        `residual` (32-bit) in place.  An input in another precision than the weight is
-        converted to the weight's (exact from bfloat16 to 32-bit)."""
+    def few_rows(self, n_rows: int) -> bool:
+        """Whether a call with n_rows rows runs the few-rows product, which reads and writes packed rows."""
+        return isinstance(self.weight, ops.PackedMatrix) and n_rows <= ops.PACKED_ROWS_MAX
+
+    def packed_input(self, n_rows: int) -> bool:
+        """Whether the rows for a call with n_rows rows should be made as packed rows
+        (ops.packed_rows): whoever makes them asks here.  It pays from about nine rows on: a wave of
+        the few-rows product then reads 1 KB in one piece where rows of the ordinary layout cost it
+        16 cache lines per 16 lanes."""
+        return self.few_rows(n_rows) and n_rows >= ops.PACKED_ROWS_MIN and self.in_features % 32 == 0
+
+    def __call__(self, a, out_dtype=None, epilogue="none", residual=None, packed_out=False):
+        """epilogue(a @ W^T + b) as a new [M, out] tensor of out_dtype (as packed rows if
+        packed_out, for a Linear whose packed_input said so), or added into `residual` (32-bit) in
+        place.  An input in another precision than the weight is converted to the weight's (exact
+        from bfloat16 to 32-bit)."""
         if a.dtype != self.weight.dtype:
             a = ops.cast(a.contiguous(), torch.empty(a.shape, dtype=self.weight.dtype, device=a.device))
         if residual is not None:
             return ops.linear(a, self.weight, self.bias, residual=residual)
-        out = torch.empty((a.shape[0], self.out_features), dtype=out_dtype or a.dtype, device=a.device)
+        if packed_out:
+            out = ops.packed_rows(a.shape[0], self.out_features, a.device)
+        else:
+            out = torch.empty((a.shape[0], self.out_features), dtype=out_dtype or a.dtype, device=a.device)
         return ops.linear(a, self.weight, self.bias, out=out, epilogue=epilogue)
 
     def project_qkv(self, a, out_dtype, slot_map, k_pool, v_pool, q_width):

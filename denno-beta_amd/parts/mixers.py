@@ -44,6 +44,9 @@ class CausalSelfAttention(Part):
         self.qkv.bind(tensors)
         self.out.bind(tensors)
 
+    def packed_input(self, n_rows):
+        return self.qkv.packed_input(n_rows)
+
     def forward(self, h, ctx, cache, accumulate_into):
         act = self.runtime.act_dtype
         g = ctx.groups[cache.group]
@@ -51,7 +54,12 @@ class CausalSelfAttention(Part):
             qkv = self.qkv.project_qkv(h, act, g.slot_map, cache.k, cache.v, self.q_width)
         else:
             qkv = self.qkv(h, out_dtype=act)
-        o = torch.empty((h.shape[0], self.q_width), dtype=act, device=h.device)
+        # a pure decode step's kernel hands its rows to the output projection packed
+        if self.out.packed_input(h.shape[0]) and ops.decode_attention_applies(
+                act, cache.k.shape[2], self.head_dim, g.single_rows, g.max_context):
+            o = ops.packed_rows(h.shape[0], self.q_width, h.device)
+        else:
+            o = torch.empty((h.shape[0], self.q_width), dtype=act, device=h.device)
         ops.attention(qkv[:, :self.q_width], o, cache.k, cache.v, g.block_tables, g.tiles, self.n_heads,
                       self.scale, self.window, tiles_wide=g.tiles_wide, single_rows=g.single_rows,
                       max_context=g.max_context)

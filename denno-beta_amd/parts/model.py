@@ -174,5 +174,5 @@ class DecoderModel:
             self.blocks[call.layer].forward(x, ctx, cache.view(call.cache, call.writes_cache), rt)
         if ctx.R == 0:
             return torch.empty((0, self.spec.vocab), dtype=torch.float32, device=rt.device)
-        h = self.final_norm.forward(x, rt.act_dtype, rows=ctx.logit_rows)
+        h = self.final_norm.forward(x, rt.act_dtype, rows=ctx.logit_rows, packed=self.head.packed_input(ctx.R))
         return self.head(h, out_dtype=torch.float32)

@@ -29,7 +29,10 @@ class LayerNorm(Part):
         self.weight = tensors[self.weight_name]
         self.bias = tensors[self.bias_name] if self.bias_name else None
 
-    def forward(self, x, out_dtype, rows=None):
+    def forward(self, x, out_dtype, rows=None, packed=False):
         n = x.shape[0] if rows is None else rows.shape[0]
-        out = torch.empty((n, self.width), dtype=out_dtype, device=x.device)
+        if packed:
+            out = ops.packed_rows(n, self.width, x.device)
+        else:
+            out = torch.empty((n, self.width), dtype=out_dtype, device=x.device)
         return ops.layernorm(x, self.weight, self.bias, self.eps, out, rows)

@@ -137,6 +137,50 @@ def test_linear_qkv_writes_the_cache(M):
     assert pools[0].abs().sum() > 0 and pools[1].abs().sum() > 0
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("N,K", [(1600, 1600), (4800, 1600), (96, 6400), (33024, 64)])
+def test_linear_with_packed_rows(M, N, K):
+    """The few-rows product reading packed rows and writing them gives, bit for bit, what it gives
+    with rows in the ordinary layout; so does LayerNorm."""
+    o = ops()
+    a, w, bias = rnd(M, K, seed=M, dtype=torch.bfloat16), o.pack_matrix(rnd(N, K, seed=N, dtype=torch.bfloat16, scale=0.05)), rnd(N, seed=3)
+    ap = o.pack_matrix(a)
+    assert torch.equal(ap.rows(), a)
+    want = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    for epi in ("none", "gelu_tanh"):
+        o.linear(a, w, bias, out=want, epilogue=epi)
+        got = o.packed_rows(M, N, DEV)
+        o.linear(ap, w, bias, out=got, epilogue=epi)
+        assert torch.equal(got.rows(), want)
+        mixed = torch.empty_like(want)
+        o.linear(ap, w, bias, out=mixed, epilogue=epi)
+        assert torch.equal(mixed, want)
+    res, res2 = rnd(M, N, seed=4), rnd(M, N, seed=4)
+    o.linear(a, w, bias, residual=res)
+    o.linear(ap, w, bias, residual=res2)
+    assert torch.equal(res, res2)
+    x, g, b = rnd(M, K, seed=5), rnd(K, seed=6), rnd(K, seed=7)
+    rows = o.layernorm(x, g, b, 1e-5, torch.empty(M, K, dtype=torch.bfloat16, device=DEV))
+    assert torch.equal(o.layernorm(x, g, b, 1e-5, o.packed_rows(M, K, DEV)).rows(), rows)
+    pick = i32(list(range(M - 1, -1, -1)))
+    assert torch.equal(o.layernorm(x, g, b, 1e-5, o.packed_rows(M, K, DEV), pick).rows(), rows.flip(0))
+
+
+def test_packed_rows_are_refused_where_no_kernel_takes_them():
+    o = ops()
+    w = o.pack_matrix(rnd(64, 64, dtype=torch.bfloat16))
+    with pytest.raises(o.KernelError, match="at most 64 rows"):
+        o.packed_rows(65, 64, DEV)
+    with pytest.raises(o.KernelError, match="multiple of 32"):
+        o.packed_rows(4, 48, DEV)
+    with pytest.raises(o.KernelError, match="need a packed matrix"):
+        o.linear(o.packed_rows(4, 64, DEV), rnd(64, 64, dtype=torch.bfloat16), None, out=torch.empty(4, 64, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(o.KernelError, match="packed rows as out"):
+        o.linear(rnd(70, 64, dtype=torch.bfloat16), w, None, out=o.PackedMatrix(torch.empty(5 * 2 * 512, dtype=torch.bfloat16, device=DEV), (70, 64)))
+    with pytest.raises(o.KernelError, match="bfloat16 rows"):
+        o.linear(rnd(4, 64), w, None, out=torch.empty(4, 64, device=DEV))
+
+
 def test_linear_rows_do_not_depend_on_the_batch():
     a, w = rnd(150, 96, seed=1), rnd(333, 96, seed=2)
     full = torch.empty(150, 333, device=DEV)
@@ -230,11 +274,22 @@ def test_attention_split_kernel_for_decoding(H, Hkv, dh, ps, window):
         ops().attention(q[:, :H * dh], out, k, v, bt, tiles, H, scale, window, tiles_wide=paged_case.wide,
                         single_rows=True, max_context=max_context)
         assert torch.allclose(out.float(), want, **TOL[torch.bfloat16])
+        if (H * dh) % 32 == 0:               # the same rows, packed for the product that follows
+            packed = ops().packed_rows(T, H * dh, DEV)
+            ops().attention(q[:, :H * dh], packed, k, v, bt, tiles, H, scale, window, single_rows=True,
+                            max_context=max_context)
+            assert torch.equal(packed.rows(), out)
     # one short request alone: a single split, written without the join
     out = torch.zeros(1, H * dh, dtype=torch.bfloat16, device=DEV)
-    ops().attention(q[1:2, :H * dh], out, k, v, bt[1:2].contiguous(), i32([[0], [0], [1], [16]]), H, scale, window,
-                    single_rows=True, max_context=17)
+    one = (q[1:2, :H * dh], k, v, bt[1:2].contiguous(), i32([[0], [0], [1], [16]]), H, scale, window)
+    ops().attention(one[0], out, *one[1:], single_rows=True, max_context=17)
     assert torch.allclose(out.float(), want[1:2], **TOL[torch.bfloat16])
+    if (H * dh) % 32 == 0:
+        packed = ops().packed_rows(1, H * dh, DEV)
+        ops().attention(one[0], packed, *one[1:], single_rows=True, max_context=17)
+        assert torch.equal(packed.rows(), out)
+        with pytest.raises(ops().KernelError, match="decode kernel only"):
+            ops().attention(one[0], packed, *one[1:], tiles_wide=one[4])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

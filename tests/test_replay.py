@@ -175,6 +175,37 @@ def test_long_context_with_heads_of_64(model_folders, dtype):
         U.assert_close(got[f"r{i}"], want[i], dtype, f"long context {dtype} request {i}")
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["C", "D"])
+@pytest.mark.parametrize("graphs", [False, True])
+def test_twelve_requests_decode_together(model_folders, name, graphs):
+    """Steps of 9 to 64 rows hand their bfloat16 rows from kernel to kernel in the packed layout
+    (LayerNorm, the decode attention and the first feed-forward product write it, the few-rows
+    product reads it).  C's feed-forward width is no multiple of 32, so its second product takes
+    ordinary rows; D packs all of them."""
+    from denno_beta_amd.config import EngineOptions
+    from denno_beta_amd.engine import ModelRunner, StepEntry
+    folder = model_folders(name, "bfloat16")
+    seqs = sequences(name, (40, 25, 70, 33, 90, 21, 58, 64, 30, 47, 36, 81), seed=40)
+    want = plain_logits(folder, seqs)
+    r = ModelRunner.from_folder(folder, EngineOptions(dtype="bfloat16", page_size=16, cache_tokens=12 * 96,
+                                                      max_live=12, use_graphs=graphs))
+    assert r.model.blocks[0].mixer.packed_input(12) and not r.model.blocks[0].mixer.packed_input(8)
+    assert r.model.blocks[0].ffn.down.packed_input(12) == (name == "D")
+    for i in range(12):
+        r.start_request(i)
+    tail = 20
+    got = r.step([StepEntry(i, s[:-tail], list(range(len(s) - tail))) for i, s in enumerate(seqs)]).cpu()
+    at = 0
+    for i, s in enumerate(seqs):
+        U.assert_close(got[at:at + len(s) - tail], want[i][:len(s) - tail], "bfloat16", f"prompt of request {i}")
+        at += len(s) - tail
+    for j in range(tail, 0, -1):
+        got = r.step([StepEntry(i, [s[len(s) - j]], [0]) for i, s in enumerate(seqs)]).cpu()
+        for i, s in enumerate(seqs):
+            U.assert_close(got[i:i + 1], want[i][len(s) - j:len(s) - j + 1], "bfloat16", f"request {i}, {j} from its end")
+
+
 def test_weights_stored_in_32_bit_stay_so_in_a_bfloat16_engine(backend, model_folders):
     """A folder stored in 32-bit, run with --dtype bfloat16: the matrices stay 32-bit and their
     products run in 32-bit on widened activations; the result is at least as close to the plain

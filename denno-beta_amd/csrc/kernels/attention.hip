@@ -396,10 +396,12 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
 
 // ---------------------------------------------------------------------------------------
 // decode: one row per request, request s being tile s and row s of the step (tile_seq[s] < 0:
-// padding; tile_pos0[s]: its position).  The context is cut into n_splits runs of `chunks` * 256 keys;
-// a workgroup walks its run 256 keys at a time (4 waves of 64 keys, each with a running
-// maximum, sum and weighted values, joined through LDS at the end) and, if there is more than
-// one split, a second kernel joins the splits' results in split order
+// padding; tile_pos0[s]: its position).  A workgroup has 4, 8 or 16 waves, 64 keys each at a time
+// (its chunk: 256, 512 or 1024 keys), chosen so that a short context is one chunk: every load of
+// a wave is then issued at once, behind one lookup of its pages.  The context is cut into
+// n_splits runs of `chunks` chunks; a workgroup walks its run chunk by chunk (each wave with a
+// running maximum, sum and weighted values, joined through LDS at the end) and, if there is
+// more than one split, a second kernel joins the splits' results in split order
 // (crates/denno-engine/kernels/kernels_elem.cu:577-603 has this two-kernel shape).
 // Scores: dh/8 lanes share a key, 16 bytes each, so one load instruction reads whole keys side
 // by side; all loads of 64 keys are issued before the first is used.  Values: lane = dim,
@@ -407,10 +409,8 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
 // exchanges inside the loop.
 // ---------------------------------------------------------------------------------------
 namespace decode {
-constexpr int CHUNK = 256;   // keys that a workgroup's 4 waves take at a time, 64 each
-
-template <int LPK>   // lanes per key = dh / 8
-__global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out,
+template <int LPK, int WAVES>   // lanes per key = dh / 8; waves per workgroup
+__global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out,
                                                        int ldo, const bf16_t* __restrict__ k_pool,
                                                        const bf16_t* __restrict__ v_pool,
                                                        const int32_t* __restrict__ block_tables, int max_blocks,
@@ -423,8 +423,9 @@ __global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__
   constexpr int KPI = 64 / LPK;          // keys per load instruction
   constexpr int DPL = (DH + 63) / 64;    // dims per lane in the second product
   constexpr int GROUP = LPK < 8 ? LPK : 8;   // load instructions issued together
-  __shared__ float wm[4], wl[4];
-  __shared__ float wacc[4][DH];
+  constexpr int CHUNK = WAVES * 64;          // keys that the workgroup's waves take at a time
+  __shared__ float wm[WAVES], wl[WAVES];
+  __shared__ float wacc[WAVES][DH];
   // In a step of single rows request s brings row s and is tile s: the block table and the query
   // are addressed by the workgroup's index, so their loads do not wait for the tile table's.
   const int split = blockIdx.x, h = blockIdx.y, tile = blockIdx.z;
@@ -540,11 +541,13 @@ __global__ __launch_bounds__(256) void partial_kernel(const bf16_t* __restrict__
   for (int i = 0; i < DPL; ++i)
     if (lane + 64 * i < DH) wacc[wave][lane + 64 * i] = acc[i];
   __syncthreads();
-  for (int d = threadIdx.x; d < DH; d += 256) {
-    float M = fmaxf(fmaxf(wm[0], wm[1]), fmaxf(wm[2], wm[3]));
+  for (int d = threadIdx.x; d < DH; d += WAVES * 64) {
+    float M = wm[0];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) M = fmaxf(M, wm[w]);
     float L = 0.f, A = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < WAVES; ++w) {
       if (wm[w] > NEG_INF) {
         float f = __expf(wm[w] - M);
         L += wl[w] * f;
@@ -589,24 +592,33 @@ __global__ void join_kernel(const float* __restrict__ part, bf16_t* __restrict__
 }  // namespace decode
 
 // part: 32-bit workspace of n_tiles * H * n_splits * (dh + 2) floats (unused when n_splits == 1);
-// the splits cover n_splits * chunks * 256 keys, which must reach the longest context.
+// waves: 4, 8 or 16 per workgroup (16 up to a head size of 64, 8 up to 128); the splits cover
+// n_splits * chunks * waves * 64 keys, which must reach the longest context.
 // ldo == 0: out is a packed matrix of H * dh columns (a multiple of 32)
 extern "C" int dn_attention_decode(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
                                    const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
                                    const int32_t* tile_row0, const int32_t* tile_pos0, int n_tiles, float* part,
-                                   int n_splits, int chunks, int H, int Hkv, int dh, int page_size, float scale,
-                                   int window, hipStream_t stream) {
+                                   int n_splits, int chunks, int waves, int H, int Hkv, int dh, int page_size,
+                                   float scale, int window, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (Hkv < 1 || H % Hkv != 0 || page_size % 16 != 0 || max_blocks < 1 || n_splits < 1 || chunks < 1 ||
       ldq % 8 != 0 || ldo < 0 || (ldo == 0 && (H * dh) % 32 != 0) || reinterpret_cast<uintptr_t>(q) % 16 != 0 || reinterpret_cast<uintptr_t>(k_pool) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(v_pool) % 16 != 0)
     return DN_ERR_SHAPE;
-  dim3 grid(n_splits, H, n_tiles), block(256);
-#define DN_DECODE(L)                                                                                              \
-  hipLaunchKernelGGL(decode::partial_kernel<L>, grid, block, 0, stream, static_cast<const bf16_t*>(q), ldq,       \
-                     static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),                          \
+  if (waves != 4 && !(waves == 8 && dh <= 128) && !(waves == 16 && dh <= 64)) return DN_ERR_SHAPE;
+  dim3 grid(n_splits, H, n_tiles), block(waves * 64);
+#define DN_DECODE_W(L, W)                                                                                          \
+  hipLaunchKernelGGL((decode::partial_kernel<L, W>), grid, block, 0, stream, static_cast<const bf16_t*>(q), ldq,   \
+                     static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),                           \
                      static_cast<const bf16_t*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0, tile_pos0, \
                      part, n_splits, chunks, H, Hkv, page_size, scale, window)
+#define DN_DECODE(L)                  \
+  if (waves == 16) {                  \
+    if constexpr (L <= 8) DN_DECODE_W(L, 16); \
+  } else if (waves == 8) {            \
+    if constexpr (L <= 16) DN_DECODE_W(L, 8);  \
+  } else                              \
+    DN_DECODE_W(L, 4)
   switch (dh) {
     case 16: DN_DECODE(2); break;
     case 32: DN_DECODE(4); break;
@@ -616,6 +628,7 @@ extern "C" int dn_attention_decode(const void* q, int ldq, void* out, int ldo, c
     default: return DN_ERR_SHAPE;
   }
 #undef DN_DECODE
+#undef DN_DECODE_W
   if (n_splits > 1)
     hipLaunchKernelGGL(decode::join_kernel, dim3(n_tiles, H), dim3(64), 0, stream, part, static_cast<bf16_t*>(out),
                        ldo, tile_seq, tile_row0, n_splits, H, dh);

@@ -53,7 +53,7 @@ def _declare(name, lib):
         "attention": {
             "dn_attention": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, I, P],
             "dn_attention_flash": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, P],
-            "dn_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, F, I, P],
+            "dn_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, I, F, I, P],
         },
         "sampling": {
             "dn_sample": [P, I, I, I, P, P, P, P],
@@ -330,7 +330,7 @@ def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
 
 FLASH_HEAD_DIMS = (16, 32, 48, 64, 96, 128)
 DECODE_HEAD_DIMS = (16, 32, 64, 128, 256)
-DECODE_SPLIT = 256
+DECODE_SPLIT = 256     # the decode kernel's smallest chunk; captured decode steps round contexts up to it
 
 
 def decode_attention_applies(dtype, page_size, head_dim, single_rows, max_context):
@@ -375,9 +375,15 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
     _need(decode or not out_packed, "attention: packed rows as out are written by the decode kernel only")
     if decode:
         n_tiles = tiles.shape[1]
+        # a workgroup's waves take 64 keys each at a time: as many waves as make the context one
+        # chunk (every load issued at once), within what the head size leaves registers for
+        # (where the batch alone gives two workgroups or more per CU the chip is busy anyway, and
+        # the smallest workgroups were measured fastest)
+        waves = 4 if max_context <= 256 or n_tiles * n_heads >= 512 else 8 if max_context <= 512 else 16
+        waves = min(waves, 16 if dh <= 64 else 8 if dh <= 128 else 4)
         # the context is split over workgroups only where the batch alone does not give about one
         # workgroup per CU: a second kernel has to join the splits
-        total_chunks = -(-max_context // DECODE_SPLIT)
+        total_chunks = -(-max_context // (waves * 64))
         n_splits = max(1, min(total_chunks, 256 // max(1, n_tiles * n_heads)))
         chunks = -(-total_chunks // n_splits)
         n_splits = -(-total_chunks // chunks)
@@ -388,7 +394,7 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
         _ok(lib.dn_attention_decode(
             q.data_ptr(), ldq, out.data_ptr(), ldo, k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(),
             block_tables.shape[1], base, base + 4 * n_tiles, base + 12 * n_tiles, n_tiles, part.data_ptr(), n_splits,
-            chunks, n_heads, Hkv, dh, ps, float(scale), int(window), _stream()), "attention (decode)")
+            chunks, waves, n_heads, Hkv, dh, ps, float(scale), int(window), _stream()), "attention (decode)")
         return out
     if fast and tiles_wide is not None and dh in FLASH_HEAD_DIMS:
         _dev(tiles_wide, "tiles_wide", _I32, 2)

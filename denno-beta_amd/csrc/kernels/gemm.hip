@@ -523,13 +523,13 @@ static int launch(const void* A, int lda, const void* W, const float* bias, void
   return 0;
 }
 
-template <int WM, int BK>
+template <int WM, int BK, int TM = 2>
 static int launch_bk(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr,
                      int M, int N, int K, int out_dtype, int epi, const KVScatter* kv, hipStream_t stream) {
-  if (kv) return launch<bf16_t, WM, 2, 2, BK, true>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, kv, stream);
+  if (kv) return launch<bf16_t, WM, TM, 2, BK, true>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, kv, stream);
   if (out_dtype == DN_BF16)
-    return launch<bf16_t, WM, 2, 2, BK, false>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, nullptr, stream);
-  return launch<float, WM, 2, 2, BK, false>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, nullptr, stream);
+    return launch<bf16_t, WM, TM, 2, BK, false>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, nullptr, stream);
+  return launch<float, WM, TM, 2, BK, false>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, epi, nullptr, stream);
 }
 
 static int run(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr, int M,
@@ -539,6 +539,10 @@ static int run(const void* A, int lda, const void* W, const float* bias, void* C
   // of 64 (half the barriers).  Both measured; see profiles/.
   const long tiles = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
   if (tiles >= 512) return launch_bk<4, 32>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream);
+  // Fewer tiles than CUs: 64 x 128 tiles (each wave 32 x 64) make twice as many workgroups
+  // (2048 x 1600: 54 -> 41 us with K = 1600, 122 -> 105 us with K = 6400).
+  if (tiles < 256 && M > 64)
+    return launch_bk<2, 64, 1>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream);
   return launch_bk<2, 64>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream);
 }
 }  // namespace tiled

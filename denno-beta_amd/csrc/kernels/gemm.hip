@@ -41,6 +41,27 @@ struct KVScatter {
 };
 
 
+// The same for four columns nn .. nn + 3 (nn a multiple of 4, so they are one head's): a key's
+// four dims are 8 bytes side by side.
+__device__ __forceinline__ void scatter_kv4(const KVScatter& kv, int m, int nn, const bf16_t* cv) {
+  if (nn < kv.q_width) return;
+  int c = nn - kv.q_width;
+  const bool is_value = c >= kv.kv_width;
+  if (is_value) c -= kv.kv_width;
+  const int slot = kv.slot_map[m];
+  if (slot < 0) return;
+  const int page = slot / kv.page_size, off = slot % kv.page_size;
+  const int hh = c / kv.dh, d = c % kv.dh;
+  const size_t base = (static_cast<size_t>(page) * kv.Hkv + hh) * kv.page_size * kv.dh;
+  if (is_value) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) kv.v_pool[base + static_cast<size_t>(d + e) * kv.page_size + off] = cv[e];
+  } else {
+    *reinterpret_cast<uint2*>(kv.k_pool + base + static_cast<size_t>(off) * kv.dh + d) =
+        *reinterpret_cast<const uint2*>(cv);
+  }
+}
+
 __device__ __forceinline__ void scatter_kv(const KVScatter& kv, int m, int nn, bf16_t cv) {
   if (nn < kv.q_width) return;
   int c = nn - kv.q_width;
@@ -369,6 +390,7 @@ static bool takes(const void* A, int lda, const void* W, int M, int K, int packe
 namespace tiled {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
 constexpr int XCDS = 8;
 
@@ -474,7 +496,52 @@ __global__ __launch_bounds__(WM * 128) __attribute__((amdgpu_waves_per_eu(2))) v
     }
     __syncthreads();     // the next set is written and this one has been read by every wave
   }
-  // acc[i][j][r]: row m0 + wm + 32 i + 8 (r / 4) + 4 g + r % 4, column n0 + wn + 32 j + lane % 32
+  // acc[i][j][r]: row m0 + wm + 32 i + 8 (r / 4) + 4 g + r % 4, column n0 + wn + 32 j + lane % 32:
+  // a lane holds one column, so stores straight from the accumulators would be 2 or 4 bytes at a
+  // stride of a row.  Each wave turns its 32 x 32 blocks round through a piece of LDS of its own
+  // (the slabs are done with: the loop ended at a barrier) and stores 16 bytes per lane along rows.
+  // Rows that do not allow that (a width or leading dimension that is no multiple of 4) take the
+  // element-wise path.
+  const bool vec = N % 4 == 0 && (resid ? ldr % 4 == 0 && reinterpret_cast<uintptr_t>(resid) % 16 == 0
+                                        : ldc % 4 == 0 && reinterpret_cast<uintptr_t>(C) % 16 == 0);
+  if (vec) {
+    constexpr int RS = 40;                               // floats per row of the piece: no bank shared by the two halves
+    float* piece = reinterpret_cast<float*>(lds) + wave * (32 * RS);
+    const int prow = lane / 8, pcol = (lane % 8) * 4;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int nb = n0 + wn + j * 32;
+      const float bv = (bias && nb + r32 < N) ? bias[nb + r32] : 0.f;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float v = acc[i][j][r] + bv;
+          piece[(8 * (r / 4) + 4 * g + (r % 4)) * RS + r32] = resid ? v : apply_epilogue(v, epi);
+        }
+        const int n = nb + pcol;
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const int lr = it * 8 + prow, m = m0 + wm + i * 32 + lr;
+          const floatx4 v = *reinterpret_cast<const floatx4*>(piece + lr * RS + pcol);
+          if (m >= M || n >= N) continue;
+          if (resid) {
+            floatx4* x = reinterpret_cast<floatx4*>(resid + static_cast<size_t>(m) * ldr + n);
+            *x = *x + v;
+          } else if constexpr (sizeof(TC) == 4) {
+            *reinterpret_cast<floatx4*>(C + static_cast<size_t>(m) * ldc + n) = v;
+          } else {
+            alignas(8) bf16_t cv[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) cv[e] = from_float<bf16_t>(v[e]);
+            *reinterpret_cast<uint2*>(C + static_cast<size_t>(m) * ldc + n) = *reinterpret_cast<const uint2*>(cv);
+            if constexpr (KV) scatter_kv4(kv, m, n, cv);
+          }
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int n = n0 + wn + j * 32 + r32;

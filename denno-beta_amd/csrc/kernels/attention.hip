@@ -189,8 +189,12 @@ __device__ __forceinline__ __bf16 to_bf16(float f) { return static_cast<__bf16>(
 namespace flash {
 constexpr int ROWS = 128;
 
+// Two waves per SIMD are asked for: with room for one wave only, the compiler keeps the MFMA
+// results in accumulation registers and copies all of them to and fro around the rescaling of
+// every tile (200 moves a tile).
 template <int DH16>
-__global__ __launch_bounds__(256) void kernel(const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void kernel(
+    const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo,
                                                const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
                                                const int32_t* __restrict__ block_tables, int max_blocks,
                                                const int32_t* __restrict__ tile_seq,
@@ -245,8 +249,11 @@ __global__ __launch_bounds__(256) void kernel(const bf16_t* __restrict__ q, int 
     const int key = kt_ + qcol;      // as A operand the lane's row is a key
     const int page = qcol < 16 ? pg[0] : pg[1];
     const bool ok = key <= hi_w && page >= 0;
+    // the key's place in its page: the tile's two runs of 16 start at offsets that are the same for
+    // every lane (a division on the scalar unit, not one per lane)
+    const int off = (qcol < 16 ? kt_ % page_size : (kt_ + 16) % page_size) + qcol % 16;
     // never a conditional load: a key outside reads the pool's first key and is dropped
-    const bf16_t* kr = k_pool + (ok ? ((static_cast<size_t>(page) * Hkv + hk) * page_size + key % page_size) * DH : 0) + g * 8;
+    const bf16_t* kr = k_pool + (ok ? ((static_cast<size_t>(page) * Hkv + hk) * page_size + off) * DH : 0) + g * 8;
 #pragma unroll
     for (int c = 0; c < DH16; ++c) kf[c] = *reinterpret_cast<const bf16x8*>(kr + c * 16);
     return ok;
@@ -326,11 +333,14 @@ __global__ __launch_bounds__(256) void kernel(const bf16_t* __restrict__ q, int 
     for (int a0 = 0; a0 < 2; ++a0)
 #pragma unroll
       for (int j = 0; j < 8; ++j) pb[a0][j] = to_bf16(p[8 * a0 + j]);
-    // alpha belongs to the lane's query, and so do all of the lane's accumulators
+    // alpha belongs to the lane's query, and so do all of the lane's accumulators; once the running
+    // maxima have settled it is 1 for the whole wave, tile after tile
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+      for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+    }
 #pragma unroll
     for (int a0 = 0; a0 < 2; ++a0) {
       if (pg[a0] < 0) continue;       // the same for every lane of the wave

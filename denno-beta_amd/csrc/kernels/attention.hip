@@ -176,53 +176,72 @@ __device__ __forceinline__ __bf16 to_bf16(float f) { return static_cast<__bf16>(
 
 // ---------------------------------------------------------------------------------------
 // flash: portions of prompts.  A workgroup takes up to 128 consecutive rows of one request
-// and one head; each of its 4 waves owns 32 rows and walks the keys in tiles of 32 with
-// v_mfma_f32_32x32x16_bf16, operands straight from the pages, one tile ahead of their use (the
-// waves of a workgroup read the same keys at nearly the same time, so they meet in cache).
+// and one head.  It has GROUPS x 4 waves: wave w owns the 32 rows 32 (w % 4), and the groups
+// share out the keys, tile of 32 by tile (group w / 4 takes tiles w / 4, w / 4 + GROUPS, ...):
+// what a wave does for one tile is a chain of dependent steps (scores, maximum, exponentials,
+// sum, values) of some thousand cycles whatever else runs, so a row's time is the number of
+// tiles its wave walks; two groups halve it, and join their running maxima, sums and weighted
+// values through LDS at the end, in group order.
+// A tile's keys and values come from the pages once per workgroup, 16 bytes per thread along
+// rows (two cache lines per 16 lanes), and lie in LDS for the four waves that need them, two
+// steps deep: the tiles of the step after the next are on their way to registers while this
+// step's are multiplied.
 //   S^T[key, q] = K . Q^T : lane (key = lane % 32, half g = lane / 32) gives 8 dims of a key.
 //   The result leaves each lane with 16 keys of ONE query (its column), so the running
 //   softmax is lane-local but for one exchange between the halves.
 //   O^T[d, q] += V^T . P^T : the lane's 16 probabilities are, eight by eight, exactly the
 //   B operand of two MFMAs whose k slots are the keys 16a + 4g + {0..3, 8..11}; the A
-//   operand reads those keys of dim d from the transposed value pages, 8 bytes at a time.
+//   operand reads those keys of dim d from the transposed values, 8 bytes at a time.
+// Two waves per SIMD at least are asked for: with room for one wave only, the compiler keeps the
+// MFMA results in accumulation registers and copies all of them to and fro around every rescaling.
 // ---------------------------------------------------------------------------------------
 namespace flash {
 constexpr int ROWS = 128;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
 
-// Two waves per SIMD are asked for: with room for one wave only, the compiler keeps the MFMA
-// results in accumulation registers and copies all of them to and fro around the rescaling of
-// every tile (200 moves a tile).
-template <int DH16>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void kernel(
-    const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo,
-                                               const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
-                                               const int32_t* __restrict__ block_tables, int max_blocks,
-                                               const int32_t* __restrict__ tile_seq,
-                                               const int32_t* __restrict__ tile_row0,
-                                               const int32_t* __restrict__ tile_nrows,
-                                               const int32_t* __restrict__ tile_pos0, int H, int Hkv, int page_size,
-                                               float scale, int window) {
+template <int DH16, int GROUPS>
+__global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2))) void kernel(
+    const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, const bf16_t* __restrict__ k_pool,
+    const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_row0,
+    const int32_t* __restrict__ tile_nrows, const int32_t* __restrict__ tile_pos0, int H, int Hkv, int page_size,
+    float scale, int window) {
   constexpr int DH = DH16 * 16;
   constexpr int DB = (DH + 31) / 32;
+  constexpr int CH = DH / 8;                 // 16-byte chunks in a key
+  constexpr int KROW = (CH + 1) * 8;         // a key's row in LDS, one chunk of padding: 16 rows, 16 bank groups
+  constexpr int VROW = 40;                   // a dim's row of 32 keys in LDS, 16 bytes of padding
+  constexpr int KCH = 32 * CH, VCH = DH * 4; // chunks of a tile of keys, of values
+  constexpr int KU = (KCH + 255) / 256, VU = (VCH + 255) / 256;
+  constexpr int KSZ = 32 * KROW, TSZ = KSZ + DH * VROW;     // elements of a tile's keys, of a whole tile
+  constexpr int STEP = 32 * GROUPS;          // keys per step
+  constexpr int JOIN = 2 + 16 * DB;          // floats a lane hands over at the end
+  constexpr int BYTES_TILES = 2 * GROUPS * TSZ * 2, BYTES_JOIN = GROUPS > 1 ? 4 * 64 * JOIN * 4 : 0;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[BYTES_TILES > BYTES_JOIN ? BYTES_TILES : BYTES_JOIN];
+  bf16_t* const tiles_lds = reinterpret_cast<bf16_t*>(smem);      // [2 steps][GROUPS][keys | values]
   const int tile = blockIdx.x, h = blockIdx.y;
   const int seq = tile_seq[tile];
-  if (seq < 0) return;
+  if (seq < 0) return;                       // the whole workgroup
   const int row0 = tile_row0[tile], nrows = tile_nrows[tile], pos0 = tile_pos0[tile];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-  const int wrow0 = wave * 32;
-  if (wrow0 >= nrows) return;   // no barrier follows: a wave without rows may leave
+  const int grp = wave / 4;                  // which tiles this wave multiplies
+  const int t = threadIdx.x % 256, ti = threadIdx.x / 256;   // this thread carries chunk t of the step's tile ti
+  const int wrow0 = (wave % 4) * 32;
+  const bool has_rows = wrow0 < nrows;       // a wave without rows still carries tiles into LDS
   const int qcol = lane % 32, g = lane / 32;
   const int hk = h / (H / Hkv);
   const int32_t* bt = block_tables + static_cast<size_t>(seq) * max_blocks;
   const bool row_ok = wrow0 + qcol < nrows;
-  const int my_row = row_ok ? wrow0 + qcol : nrows - 1;
+  const int my_row = min(wrow0 + qcol, nrows - 1);
   const int my_pos = pos0 + my_row;
   const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
-  const int lo_w = window > 0 ? max(0, pos0 + wrow0 - window + 1) : 0;
+  const int lo_w = window > 0 ? max(0, pos0 + wrow0 - window + 1) : 0;      // this wave's keys
   const int hi_w = pos0 + min(wrow0 + 31, nrows - 1);
+  const int lo_g = window > 0 ? max(0, pos0 - window + 1) : 0;              // the workgroup's
+  const int hi_g = pos0 + nrows - 1;
   const float NEG_INF = -INFINITY;
   const float scale2 = scale * 1.44269504088896340736f;    // log2(e)
-  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
 
   bf16x8 qf[DH16];
   {
@@ -237,128 +256,176 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
     for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
   float m = NEG_INF, l = 0.f;
 
-  // The keys of the next tile and the values of this one are asked for before this tile's
-  // scores are computed, and the page numbers one tile further ahead still: what a tile needs has
-  // been on its way for a whole tile's arithmetic when it is used.  A tile of 32 keys lies in two
-  // pages (or in one, if pages are longer): pg[0] for keys kt .. kt+15, pg[1] for kt+16 .. kt+31.
+  // A tile of 32 keys lies in two pages (or in one, if pages are longer): pg[0] for keys
+  // kt .. kt+15, pg[1] for kt+16 .. kt+31; -1 beyond the rows' last key.
   auto pages_of = [&](int kt_, int* pg) {
-    pg[0] = kt_ <= hi_w ? bt[kt_ / page_size] : -1;
-    pg[1] = kt_ + 16 <= hi_w ? bt[(kt_ + 16) / page_size] : -1;
+    pg[0] = kt_ <= hi_g ? bt[kt_ / page_size] : -1;
+    pg[1] = kt_ + 16 <= hi_g ? bt[(kt_ + 16) / page_size] : -1;
   };
-  auto load_keys = [&](int kt_, const int* pg, bf16x8* kf) -> bool {
-    const int key = kt_ + qcol;      // as A operand the lane's row is a key
-    const int page = qcol < 16 ? pg[0] : pg[1];
-    const bool ok = key <= hi_w && page >= 0;
-    // the key's place in its page: the tile's two runs of 16 start at offsets that are the same for
-    // every lane (a division on the scalar unit, not one per lane)
-    const int off = (qcol < 16 ? kt_ % page_size : (kt_ + 16) % page_size) + qcol % 16;
-    // never a conditional load: a key outside reads the pool's first key and is dropped
-    const bf16_t* kr = k_pool + (ok ? ((static_cast<size_t>(page) * Hkv + hk) * page_size + off) * DH : 0) + g * 8;
+  // Thread t's share of its tile: chunk t (+ 256 u) of the keys, counted along a key's dims and
+  // then from key to key, and of the values, counted along a dim's 16 keys of a page, then from
+  // dim to dim, then the second run of 16.  Never a conditional load: what has no page reads the
+  // pool's start and is stored as zeros.
+  u32x4 kreg[KU], vreg[VU];
+  auto fetch = [&](int kt_, const int* pg) {
+    const int off0 = kt_ % page_size, off1 = (kt_ + 16) % page_size;
 #pragma unroll
-    for (int c = 0; c < DH16; ++c) kf[c] = *reinterpret_cast<const bf16x8*>(kr + c * 16);
-    return ok;
-  };
-  int kt = (lo_w / 32) * 32;
-  int pg[2], pg_next[2];
-  pages_of(kt, pg);
-  bf16x8 kf[DH16];
-  bool k_ok = load_keys(kt, pg, kf);
-  pages_of(kt + 32, pg_next);
-  for (; kt <= hi_w; kt += 32) {
-    // this tile's values: as A operand the lane's row is a dim, its 8 k slots the keys
-    // 16 a0 + 4 g + {0..3, 8..11} of the tile
-    bf16x4 vlo[2][DB], vhi[2][DB];
-#pragma unroll
-    for (int a0 = 0; a0 < 2; ++a0) {
-      const int kb = kt + 16 * a0;
-      const bf16_t* vb = v_pool + (pg[a0] >= 0 ? (static_cast<size_t>(pg[a0]) * Hkv + hk) * DH * page_size + kb % page_size : 0) + 4 * g;
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const bf16_t* vr = vb + static_cast<size_t>(min(32 * db + qcol, DH - 1)) * page_size;
-        vlo[a0][db] = *reinterpret_cast<const bf16x4*>(vr);
-        vhi[a0][db] = *reinterpret_cast<const bf16x4*>(vr + 8);
-      }
+    for (int u = 0; u < KU; ++u) {
+      const int idx = min(t + 256 * u, KCH - 1), key = idx / CH, ch = idx % CH;
+      const int page = key < 16 ? pg[0] : pg[1];
+      const int off = (key < 16 ? off0 : off1) + key % 16;
+      kreg[u] = *reinterpret_cast<const u32x4*>(
+          k_pool + (page >= 0 ? ((static_cast<size_t>(page) * Hkv + hk) * page_size + off) * DH : 0) + ch * 8);
     }
-    bf16x8 kf_next[DH16];
-    const bool k_ok_next = load_keys(kt + 32, pg_next, kf_next);
-    int pg_far[2];
-    pages_of(kt + 64, pg_far);
+#pragma unroll
+    for (int u = 0; u < VU; ++u) {
+      const int idx = min(t + 256 * u, VCH - 1), a0 = idx / (DH * 2), d = (idx % (DH * 2)) / 2, half = idx % 2;
+      const int page = pg[a0];
+      vreg[u] = *reinterpret_cast<const u32x4*>(
+          v_pool + (page >= 0 ? ((static_cast<size_t>(page) * Hkv + hk) * DH + d) * page_size + (a0 ? off1 : off0) : 0) +
+          half * 8);
+    }
+  };
+  auto stash = [&](const int* pg, bf16_t* dst) {
+#pragma unroll
+    for (int u = 0; u < KU; ++u) {
+      const int idx = t + 256 * u, key = idx / CH, ch = idx % CH;
+      if (idx < KCH)
+        *reinterpret_cast<u32x4*>(dst + key * KROW + ch * 8) = (key < 16 ? pg[0] : pg[1]) >= 0 ? kreg[u] : zero4;
+    }
+#pragma unroll
+    for (int u = 0; u < VU; ++u) {
+      const int idx = t + 256 * u, a0 = idx / (DH * 2), d = (idx % (DH * 2)) / 2, half = idx % 2;
+      if (idx < VCH)
+        *reinterpret_cast<u32x4*>(dst + KSZ + d * VROW + a0 * 16 + half * 8) = pg[a0] >= 0 ? vreg[u] : zero4;
+    }
+  };
 
-    floatx16 s;
+  // Step kt first puts the tiles of step kt + STEP (asked for during the step before) from
+  // registers into the half of LDS that the step before read (every wave has left it: the
+  // barrier), then asks for the tiles of step kt + 2 STEP, then multiplies.
+  const int kt0 = (lo_g / STEP) * STEP;
+  const int mine = 32 * ti;                  // this thread carries the tile at kt + mine
+  int pg_now[2], pg_reg[2], pg_far[2];       // pages of the tile in registers and of the one to ask for next
+  pages_of(kt0 + mine, pg_now);
+  fetch(kt0 + mine, pg_now);
+  pages_of(kt0 + STEP + mine, pg_reg);
+  stash(pg_now, tiles_lds + ti * TSZ);
+  fetch(kt0 + STEP + mine, pg_reg);
+  pages_of(kt0 + 2 * STEP + mine, pg_far);
+  __syncthreads();
+  int buf = 0;
+  for (int kt = kt0; kt <= hi_g; kt += STEP, buf ^= 1) {
+    if (kt + STEP <= hi_g) stash(pg_reg, tiles_lds + ((buf ^ 1) * GROUPS + ti) * TSZ);
+    if (kt + 2 * STEP <= hi_g) fetch(kt + 2 * STEP + mine, pg_far);
+    pg_reg[0] = pg_far[0], pg_reg[1] = pg_far[1];
+    pages_of(kt + 3 * STEP + mine, pg_far);
+
+    const int kw = kt + 32 * grp;            // this wave's tile of the step
+    if (has_rows && kw <= hi_w && kw + 31 >= lo_w) {     // the same for the whole wave
+      const bf16_t* Kb = tiles_lds + (buf * GROUPS + grp) * TSZ;
+      const bf16_t* Vb = Kb + KSZ;
+      floatx16 s;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) s[i] = 0.f;
+      for (int i = 0; i < 16; ++i) s[i] = 0.f;
 #pragma unroll
-    for (int c = 0; c < DH16; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_ok ? kf[c] : zero8, qf[c], s, 0, 0, 0);
-    // s[i]: key kt + 8*(i/4) + 4*g + i%4, query = this lane's column.  Scores are kept times
-    // log2(e), so that each probability is one multiply-add and one v_exp_f32.  Only a tile that
-    // touches the causal edge (or the window's) of one of the wave's rows needs the mask; the
-    // others skip it, the same for the whole wave.
-    const bool edge = kt + 31 > pos0 + wrow0 || (window > 0 && kt < hi_w - window + 1);
-    float tmax = NEG_INF;
-    if (edge) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        int key = kt + 8 * (i / 4) + 4 * g + (i % 4);
-        bool ok = key >= my_lo && key <= my_pos;
-        s[i] = ok ? s[i] * scale2 : NEG_INF;
-        tmax = fmaxf(tmax, s[i]);
+      for (int c = 0; c < DH16; ++c) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Kb + qcol * KROW + (2 * c + g) * 8);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[c], s, 0, 0, 0);
       }
-    } else {
+      // s[i]: key kw + 8*(i/4) + 4*g + i%4, query = this lane's column.  Scores are kept times
+      // log2(e), so that each probability is one multiply-add and one v_exp_f32.  Only a tile that
+      // touches the causal edge (or the window's) of one of the wave's rows needs the mask; the
+      // others skip it, the same for the whole wave.
+      const bool edge = kw + 31 > pos0 + wrow0 || (window > 0 && kw < hi_w - window + 1);
+      float tmax = NEG_INF;
+      if (edge) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        s[i] *= scale2;
-        tmax = fmaxf(tmax, s[i]);
+        for (int i = 0; i < 16; ++i) {
+          int key = kw + 8 * (i / 4) + 4 * g + (i % 4);
+          bool ok = key >= my_lo && key <= my_pos;
+          s[i] = ok ? s[i] * scale2 : NEG_INF;
+          tmax = fmaxf(tmax, s[i]);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          s[i] *= scale2;
+          tmax = fmaxf(tmax, s[i]);
+        }
+      }
+      tmax = fmaxf(tmax, other_half(tmax));
+      float p[16];
+      float psum = 0.f, alpha = 1.f;
+      if (tmax > NEG_INF) {
+        float m_new = fmaxf(m, tmax);
+        alpha = __builtin_amdgcn_exp2f(m - m_new);      // m = -inf at first: 2^-inf = 0
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          p[i] = __builtin_amdgcn_exp2f(s[i] - m_new);  // a masked score is -inf: 0
+          psum += p[i];
+        }
+        m = m_new;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) p[i] = 0.f;
+      }
+      psum += other_half(psum);
+      l = l * alpha + psum;
+      bf16x8 pb[2];
+#pragma unroll
+      for (int a0 = 0; a0 < 2; ++a0)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pb[a0][j] = to_bf16(p[8 * a0 + j]);
+      // alpha belongs to the lane's query, and so do all of the lane's accumulators; once the running
+      // maxima have settled it is 1 for the whole wave, tile after tile
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+      }
+      // values: as A operand the lane's row is a dim, its 8 k slots the keys 16 a0 + 4 g + {0..3, 8..11}
+#pragma unroll
+      for (int a0 = 0; a0 < 2; ++a0) {
+        if (kw + 16 * a0 > hi_w) continue;       // the same for every lane of the wave: all its probabilities are 0
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const bf16_t* vr = Vb + min(32 * db + qcol, DH - 1) * VROW + 16 * a0 + 4 * g;
+          const bf16x4 vlo = *reinterpret_cast<const bf16x4*>(vr), vhi = *reinterpret_cast<const bf16x4*>(vr + 8);
+          bf16x8 vf = bf16x8{vlo[0], vlo[1], vlo[2], vlo[3], vhi[0], vhi[1], vhi[2], vhi[3]};
+          if (32 * db + qcol >= DH) vf = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[a0], o[db], 0, 0, 0);
+        }
       }
     }
-    tmax = fmaxf(tmax, other_half(tmax));
-    float p[16];
-    float psum = 0.f, alpha = 1.f;
-    if (tmax > NEG_INF) {
-      float m_new = fmaxf(m, tmax);
-      alpha = __builtin_amdgcn_exp2f(m - m_new);      // m = -inf at first: 2^-inf = 0
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        p[i] = __builtin_amdgcn_exp2f(s[i] - m_new);  // a masked score is -inf: 0
-        psum += p[i];
-      }
-      m = m_new;
-    } else {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) p[i] = 0.f;
-    }
-    psum += other_half(psum);
-    l = l * alpha + psum;
-    bf16x8 pb[2];
-#pragma unroll
-    for (int a0 = 0; a0 < 2; ++a0)
-#pragma unroll
-      for (int j = 0; j < 8; ++j) pb[a0][j] = to_bf16(p[8 * a0 + j]);
-    // alpha belongs to the lane's query, and so do all of the lane's accumulators; once the running
-    // maxima have settled it is 1 for the whole wave, tile after tile
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+    __syncthreads();      // the other half of LDS is written and this one has been read by every wave
+  }
+  if constexpr (GROUPS > 1) {
+    // the second group hands its maxima, sums and weighted values to the first, lane to lane (both
+    // hold the same queries in the same lanes); the tiles in LDS are done with
+    float* join = reinterpret_cast<float*>(smem) + ((wave % 4) * 64 + lane) * JOIN;
+    if (grp == 1) {
+      join[0] = m;
+      join[1] = l;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+        for (int i = 0; i < 16; ++i) join[2 + 16 * db + i] = o[db][i];
     }
+    __syncthreads();
+    if (grp == 1) return;
+    const float m1 = join[0], l1 = join[1];
+    const float m_new = fmaxf(m, m1);
+    const float f0 = m > NEG_INF ? __builtin_amdgcn_exp2f(m - m_new) : 0.f;
+    const float f1 = m1 > NEG_INF ? __builtin_amdgcn_exp2f(m1 - m_new) : 0.f;
+    l = l * f0 + l1 * f1;
 #pragma unroll
-    for (int a0 = 0; a0 < 2; ++a0) {
-      if (pg[a0] < 0) continue;       // the same for every lane of the wave
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        bf16x8 vf = bf16x8{vlo[a0][db][0], vlo[a0][db][1], vlo[a0][db][2], vlo[a0][db][3],
-                           vhi[a0][db][0], vhi[a0][db][1], vhi[a0][db][2], vhi[a0][db][3]};
-        if (32 * db + qcol >= DH) vf = zero8;
-        o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[a0], o[db], 0, 0, 0);
-      }
-    }
-#pragma unroll
-    for (int c = 0; c < DH16; ++c) kf[c] = kf_next[c];
-    k_ok = k_ok_next;
-    pg[0] = pg_next[0], pg[1] = pg_next[1];
-    pg_next[0] = pg_far[0], pg_next[1] = pg_far[1];
+      for (int i = 0; i < 16; ++i) o[db][i] = o[db][i] * f0 + join[2 + 16 * db + i] * f1;
   }
-  if (row_ok) {
+  if (has_rows && row_ok) {
     const float inv = 1.0f / l;
     bf16_t* orow = out + static_cast<size_t>(row0 + my_row) * ldo + h * DH;
 #pragma unroll
@@ -385,22 +452,34 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
   if (Hkv < 1 || H % Hkv != 0 || page_size % 16 != 0 || max_blocks < 1 || ldq % 8 != 0 || ldo % 4 != 0 ||
       reinterpret_cast<uintptr_t>(q) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 8 != 0)
     return DN_ERR_SHAPE;
-  dim3 grid(n_tiles, H), block(256);
-#define DN_FLASH(D)                                                                                               \
-  hipLaunchKernelGGL(flash::kernel<D>, grid, block, 0, stream, static_cast<const bf16_t*>(q), ldq,                \
+  // Two groups of waves where the workgroups are fewer than the CUs (a wave's chain of dependent
+  // steps per tile then bounds the time, and two groups halve the tiles a wave walks: 1 request,
+  // 128 rows after 896: 40 -> 29 us); with more workgroups the SIMDs are busy and the second
+  // group's share of carrying tiles only adds work (2 x 1024 rows: 52 -> 66 us).  Up to a head
+  // size of 64: beyond, the tiles of two groups do not fit 64 KB of LDS.
+  dim3 grid(n_tiles, H);
+  const bool two = static_cast<long>(n_tiles) * H <= 256;
+#define DN_FLASH_G(D, G)                                                                                          \
+  hipLaunchKernelGGL((flash::kernel<D, G>), grid, dim3(256 * G), 0, stream, static_cast<const bf16_t*>(q), ldq,   \
                      static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),                          \
                      static_cast<const bf16_t*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0, tile_nrows, \
                      tile_pos0, H, Hkv, page_size, scale, window)
+#define DN_FLASH(D, G) \
+  if (G == 2 && two)   \
+    DN_FLASH_G(D, G);  \
+  else                 \
+    DN_FLASH_G(D, 1)
   switch (dh) {
-    case 16: DN_FLASH(1); break;
-    case 32: DN_FLASH(2); break;
-    case 48: DN_FLASH(3); break;
-    case 64: DN_FLASH(4); break;
-    case 96: DN_FLASH(6); break;
-    case 128: DN_FLASH(8); break;
+    case 16: DN_FLASH(1, 2); break;
+    case 32: DN_FLASH(2, 2); break;
+    case 48: DN_FLASH(3, 2); break;
+    case 64: DN_FLASH(4, 2); break;
+    case 96: DN_FLASH(6, 1); break;
+    case 128: DN_FLASH(8, 1); break;
     default: return DN_ERR_SHAPE;
   }
 #undef DN_FLASH
+#undef DN_FLASH_G
   return dn_launch_status();
 }
 

@@ -257,6 +257,21 @@ def test_attention_mfma_kernel_for_portions(H, Hkv, dh, ps, window):
     assert torch.allclose(out.float(), want, **TOL[torch.bfloat16])
 
 
+@pytest.mark.parametrize("H,Hkv,dh,ps,window", [(8, 8, 64, 16, 0), (8, 2, 32, 32, 40)])
+def test_attention_mfma_kernel_with_many_workgroups(H, Hkv, dh, ps, window):
+    """More workgroups than CUs: the kernel then runs one group of waves per workgroup, not two."""
+    g = torch.Generator().manual_seed(3)
+    new_rows = [int(n) for n in torch.randint(1, 200, (36,), generator=g)]
+    seq_lens = [n + int(x) for n, x in zip(new_rows, torch.randint(0, 150, (36,), generator=g))]
+    q, k, v, bt, tiles, T = paged_case(seq_lens, new_rows, H, Hkv, dh, ps, torch.bfloat16, seed=H + dh)
+    assert paged_case.wide.shape[1] * H > 256
+    scale = 1 / math.sqrt(dh)
+    out = torch.zeros(T, H * dh, dtype=torch.bfloat16, device=DEV)
+    ops().attention(q[:, :H * dh], out, k, v, bt, tiles, H, scale, window, tiles_wide=paged_case.wide)
+    want = R.attention(q[:, :H * dh], torch.zeros(T, H * dh, device=DEV), k, v, bt, tiles, H, scale, window)
+    assert torch.allclose(out.float(), want, **TOL[torch.bfloat16])
+
+
 @pytest.mark.parametrize("H,Hkv,dh,ps,window", [(4, 4, 16, 16, 0), (25, 25, 64, 16, 0), (6, 2, 32, 32, 0),
                                                 (2, 1, 128, 64, 0), (3, 3, 256, 16, 0), (5, 5, 64, 16, 100),
                                                 (2, 2, 64, 32, 300)])

@@ -38,6 +38,7 @@ struct KVScatter {
   bf16_t* k_pool;
   bf16_t* v_pool;
   int q_width, kv_width, dh, page_size, Hkv;
+  int c_cols;     // columns of C that are stored: all of them, or q_width (nobody reads keys and values from C)
 };
 
 
@@ -301,7 +302,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
         resid[static_cast<size_t>(m) * ldr + nn] = epi_x[p][r] + v;
       } else {
         TC cv = from_float<TC>(apply_epilogue(v, epi));
-        C[(packed & PACKED_C) ? packed_index(m, nn, N / 32) : static_cast<size_t>(m) * ldc + nn] = cv;
+        if (!KV || nn < kv.c_cols)
+          C[(packed & PACKED_C) ? packed_index(m, nn, N / 32) : static_cast<size_t>(m) * ldc + nn] = cv;
         if constexpr (KV) scatter_kv(kv, m, nn, cv);
       }
     }
@@ -519,6 +521,41 @@ __global__ __launch_bounds__(WM * 128) __attribute__((amdgpu_waves_per_eu(2))) v
           const float v = acc[i][j][r] + bv;
           piece[(8 * (r / 4) + 4 * g + (r % 4)) * RS + r32] = resid ? v : apply_epilogue(v, epi);
         }
+        if constexpr (KV) {
+          // A block of value columns: a value's place in its page is [dim][offset], so four rows
+          // (tokens) whose slots follow one another from an offset that is a multiple of 4 are 8
+          // bytes side by side for one dim.  Lane = column, and the block is read down its columns.
+          if (nb >= kv.q_width + kv.kv_width && nb >= kv.c_cols) {
+            const int cc = nb + r32 - kv.q_width - kv.kv_width, hh = cc / kv.dh, d = cc % kv.dh;
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+              const int lr = it * 8 + g * 4, m = m0 + wm + i * 32 + lr;
+              alignas(8) bf16_t cv[4];
+              int slot[4];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                cv[e] = from_float<bf16_t>(piece[(lr + e) * RS + r32]);
+                slot[e] = m + e < M ? kv.slot_map[m + e] : -1;
+              }
+              if (nb + r32 >= N) continue;
+              const bool run = slot[0] >= 0 && slot[0] % 4 == 0 && slot[1] == slot[0] + 1 && slot[2] == slot[0] + 2 &&
+                               slot[3] == slot[0] + 3;
+              if (run) {
+                const int page = slot[0] / kv.page_size, off = slot[0] % kv.page_size;
+                *reinterpret_cast<uint2*>(kv.v_pool + ((static_cast<size_t>(page) * kv.Hkv + hh) * kv.dh + d) * kv.page_size +
+                                          off) = *reinterpret_cast<const uint2*>(cv);
+              } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                  if (slot[e] < 0) continue;
+                  const int page = slot[e] / kv.page_size, off = slot[e] % kv.page_size;
+                  kv.v_pool[((static_cast<size_t>(page) * kv.Hkv + hh) * kv.dh + d) * kv.page_size + off] = cv[e];
+                }
+              }
+            }
+            continue;
+          }
+        }
         const int n = nb + pcol;
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
@@ -534,7 +571,8 @@ __global__ __launch_bounds__(WM * 128) __attribute__((amdgpu_waves_per_eu(2))) v
             alignas(8) bf16_t cv[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) cv[e] = from_float<bf16_t>(v[e]);
-            *reinterpret_cast<uint2*>(C + static_cast<size_t>(m) * ldc + n) = *reinterpret_cast<const uint2*>(cv);
+            if (!KV || n < kv.c_cols)
+              *reinterpret_cast<uint2*>(C + static_cast<size_t>(m) * ldc + n) = *reinterpret_cast<const uint2*>(cv);
             if constexpr (KV) scatter_kv4(kv, m, n, cv);
           }
         }
@@ -559,7 +597,7 @@ __global__ __launch_bounds__(WM * 128) __attribute__((amdgpu_waves_per_eu(2))) v
           *x = *x + v;
         } else {
           const TC cv = from_float<TC>(apply_epilogue(v, epi));
-          C[static_cast<size_t>(m) * ldc + n] = cv;
+          if (!KV || n < kv.c_cols) C[static_cast<size_t>(m) * ldc + n] = cv;
           if constexpr (KV) scatter_kv(kv, m, n, cv);
         }
       }
@@ -659,18 +697,20 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
 
 // The fused projection q | k | v with packed W: C = A . W^T + bias as dn_gemm computes it, and the
 // key and value columns also go to their pages (see KVScatter), from the epilogue of the few-rows
-// or of the tiled kernel.  a_packed: A is packed (at most 64 rows).
+// or of the tiled kernel.  a_packed: A is packed (at most 64 rows).  c_cols: N, or q_width: C then
+// is [M, q_width] and gets the query columns only.
 extern "C" int dn_gemm_qkv(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, int M, int N,
                            int K, const int32_t* slot_map, void* k_pool, void* v_pool, int q_width, int Hkv, int dh,
-                           int page_size, int a_packed, hipStream_t stream) {
+                           int page_size, int a_packed, int c_cols, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   const int packed = PACKED_W | (a_packed ? PACKED_A : 0);
   if (K <= 0 || (lda < K && !a_packed)) return DN_ERR_SHAPE;
   const bool few = skinny::takes(A, lda, W, M, K, packed);
   if (!few && (a_packed || !tiled::takes(A, lda, W, K))) return DN_ERR_SHAPE;
-  if (q_width < 0 || q_width + 2 * Hkv * dh != N || page_size < 1) return DN_ERR_SHAPE;
+  if (q_width < 0 || q_width + 2 * Hkv * dh != N || page_size < 1 || dh % 4 != 0) return DN_ERR_SHAPE;
+  if ((c_cols != N && c_cols != q_width) || ldc < c_cols) return DN_ERR_SHAPE;
   KVScatter kv{slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_width, Hkv * dh, dh,
-               page_size, Hkv};
+               page_size, Hkv, c_cols};
   if (few) {
     skinny::Call c{A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, packed, &kv};
     skinny::run(c, stream);

@@ -48,7 +48,7 @@ def _declare(name, lib):
         "gemm": {
             "dn_gemm": [P, I, P, P, P, I, P, I, I, I, I, I, I, I, I, P],
             "dn_pack_matrix": [P, P, I, I, P],
-            "dn_gemm_qkv": [P, I, P, P, P, I, I, I, I, P, P, P, I, I, I, I, I, P],
+            "dn_gemm_qkv": [P, I, P, P, P, I, I, I, I, P, P, P, I, I, I, I, I, I, P],
         },
         "attention": {
             "dn_attention": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, I, P],
@@ -298,20 +298,23 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
 
 
 def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
-    """out = a @ w.T + bias, the fused projection q | k | v; the key columns (q_width ..) and the
-    value columns after them also go to the slots slot_map[t] of the pools, as kv_write does.
-    One kernel with a PackedMatrix and bfloat16 all through (the cache write is in the product's
-    epilogue), else two."""
+    """The fused projection q | k | v = a @ w.T + bias: the key columns (q_width ..) and the value
+    columns after them go to the slots slot_map[t] of the pools, as kv_write does.  out: [M, N], or
+    [M, q_width] for the queries alone (nothing reads keys and values from out).  Returns the
+    queries [M, q_width] (a view of out).  One kernel with a PackedMatrix and bfloat16 all through
+    (the cache write is in the product's epilogue), else two, and out must then be [M, N]."""
     n_pages, Hkv, ps, dh = k_pool.shape
     kvw = Hkv * dh
+    M, K = a.shape
+    N = w.shape[0]
+    _need(N == q_width + 2 * kvw, "linear_qkv: columns are not q | k | v")
+    _need(not isinstance(out, PackedMatrix) and out.dim() == 2 and out.shape[0] == M and out.shape[1] in (N, q_width),
+          f"linear_qkv: out must be [{M}, {N}] or [{M}, {q_width}]")
     if isinstance(w, PackedMatrix) and out.dtype == torch.bfloat16:
         _dev(out, "out", None, 2)
         _dev(slot_map, "slot_map", _I32, 1), _dev(k_pool, "k_pool", (torch.bfloat16,), 4)
         _dev(v_pool, "v_pool", (torch.bfloat16,), 4)
-        M, K = a.shape
         lda, N, packed = _operands(a, w, "linear_qkv")
-        _need(tuple(out.shape) == (M, N), "linear_qkv: shapes")
-        _need(N == q_width + 2 * kvw, "linear_qkv: columns are not q | k | v")
         _need(k_pool.is_contiguous() and v_pool.is_contiguous() and tuple(v_pool.shape) == (n_pages, Hkv, dh, ps),
               "linear_qkv: pools")
         _need(slot_map.is_contiguous() and slot_map.shape[0] == M, "linear_qkv: slot_map")
@@ -321,11 +324,12 @@ def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
         _ok(_lib("gemm").dn_gemm_qkv(a.data_ptr(), lda, w.data_ptr(), _ptr(bias), out.data_ptr(),
                                      _rows(out, "out"), M, N, K, slot_map.data_ptr(), k_pool.data_ptr(),
                                      v_pool.data_ptr(), q_width, Hkv, dh, ps, int(bool(packed & PACKED_A)),
-                                     _stream()), "linear_qkv")
-        return out
+                                     out.shape[1], _stream()), "linear_qkv")
+        return out[:, :q_width]
+    _need(out.shape[1] == N, "linear_qkv: without the fused kernel out must hold all columns")
     linear(a, w, bias, out=out)
     kv_write(out, q_width, q_width + kvw, slot_map, k_pool, v_pool)
-    return out
+    return out[:, :q_width]
 
 
 FLASH_HEAD_DIMS = (16, 32, 48, 64, 96, 128)

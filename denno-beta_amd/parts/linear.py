@@ -65,8 +65,10 @@ class Linear:
         return ops.linear(a, self.weight, self.bias, out=out, epilogue=epilogue)
 
     def project_qkv(self, a, out_dtype, slot_map, k_pool, v_pool, q_width):
-        """The fused projection whose key and value columns also go to the cache's pages."""
+        """The fused projection: the key and value columns go to the cache's pages, the queries
+        [M, q_width] come back (where one kernel does both, the other columns are stored nowhere else)."""
         if a.dtype != self.weight.dtype:
             a = ops.cast(a.contiguous(), torch.empty(a.shape, dtype=self.weight.dtype, device=a.device))
-        out = torch.empty((a.shape[0], self.out_features), dtype=out_dtype, device=a.device)
+        fused = isinstance(self.weight, ops.PackedMatrix) and out_dtype == torch.bfloat16
+        out = torch.empty((a.shape[0], q_width if fused else self.out_features), dtype=out_dtype, device=a.device)
         return ops.linear_qkv(a, self.weight, self.bias, out, slot_map, k_pool, v_pool, q_width)

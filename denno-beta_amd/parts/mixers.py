@@ -51,16 +51,16 @@ class CausalSelfAttention(Part):
         act = self.runtime.act_dtype
         g = ctx.groups[cache.group]
         if cache.writes:
-            qkv = self.qkv.project_qkv(h, act, g.slot_map, cache.k, cache.v, self.q_width)
+            q = self.qkv.project_qkv(h, act, g.slot_map, cache.k, cache.v, self.q_width)
         else:
-            qkv = self.qkv(h, out_dtype=act)
+            q = self.qkv(h, out_dtype=act)[:, :self.q_width]
         # a pure decode step's kernel hands its rows to the output projection packed
         if self.out.packed_input(h.shape[0]) and ops.decode_attention_applies(
                 act, cache.k.shape[2], self.head_dim, g.single_rows, g.max_context):
             o = ops.packed_rows(h.shape[0], self.q_width, h.device)
         else:
             o = torch.empty((h.shape[0], self.q_width), dtype=act, device=h.device)
-        ops.attention(qkv[:, :self.q_width], o, cache.k, cache.v, g.block_tables, g.tiles, self.n_heads,
+        ops.attention(q, o, cache.k, cache.v, g.block_tables, g.tiles, self.n_heads,
                       self.scale, self.window, tiles_wide=g.tiles_wide, single_rows=g.single_rows,
                       max_context=g.max_context)
         self.out(o, residual=accumulate_into)

@@ -141,4 +141,4 @@ def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
     linear(a, w, bias, out=out)
     kvw = k_pool.shape[1] * k_pool.shape[3]
     kv_write(out, q_width, q_width + kvw, slot_map, k_pool, v_pool)
-    return out
+    return out[:, :q_width]

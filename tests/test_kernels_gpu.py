@@ -113,14 +113,25 @@ def test_linear(in_dtype, M, N, K):
 
 
 @pytest.mark.parametrize("M", [1, 8, 20, 64, 70, 300])
-def test_linear_qkv_writes_the_cache(M):
+@pytest.mark.parametrize("slots_in", ["any order", "runs"])
+@pytest.mark.parametrize("queries_only", [False, True])
+def test_linear_qkv_writes_the_cache(M, slots_in, queries_only):
     """The fused projection with the cache write in its epilogue (of the few-rows kernel or of the
-    tiled one) against the product followed by the separate write."""
-    H, Hkv, dh, ps, n_pages, K = 6, 2, 32, 16, 20, 96
+    tiled one) against the product followed by the separate write.  Slots in any order, or as a
+    prompt's portion has them: runs of consecutive slots (the tiled kernel then stores a dim's
+    values of four tokens at once), starting anywhere.  The output holds all columns, or the
+    queries alone."""
+    H, Hkv, dh, ps, n_pages, K = 6, 2, 32, 16, 40, 96
     N = (H + 2 * Hkv) * dh
     a, w, bias = rnd(M, K, seed=1, dtype=torch.bfloat16), rnd(N, K, seed=2, dtype=torch.bfloat16, scale=0.2), rnd(N, seed=3)
     g = torch.Generator().manual_seed(M)
-    slots = torch.randperm(n_pages * ps, generator=g)[:M].to(torch.int32)
+    if slots_in == "runs":
+        starts, slots = [8, 10, 40, 101], []     # disjoint for 300 rows; the first and third run start 4-aligned
+        for i in range(M):
+            slots.append(starts[i * 4 // max(M, 1)] + i)       # four runs
+        slots = torch.tensor(slots, dtype=torch.int32)
+    else:
+        slots = torch.randperm(n_pages * ps, generator=g)[:M].to(torch.int32)
     if M > 2:
         slots[2] = -1
     slots = slots.to(DEV)
@@ -128,12 +139,13 @@ def test_linear_qkv_writes_the_cache(M):
              torch.zeros(n_pages, Hkv, dh, ps, dtype=torch.bfloat16, device=DEV)]
     want_pools = [torch.zeros_like(p) for p in pools]
     w = ops().pack_matrix(w)
-    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
-    ops().linear_qkv(a, w, bias, out, slots, pools[0], pools[1], H * dh)
-    want = torch.empty_like(out)
+    out = torch.full((M, H * dh if queries_only else N), 7.0, dtype=torch.bfloat16, device=DEV)
+    queries = ops().linear_qkv(a, w, bias, out, slots, pools[0], pools[1], H * dh)
+    want = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
     ops().linear(a, w, bias, out=want)
     R.kv_write(want, H * dh, (H + Hkv) * dh, slots, want_pools[0], want_pools[1])
-    assert torch.equal(out, want) and torch.equal(pools[0], want_pools[0]) and torch.equal(pools[1], want_pools[1])
+    assert torch.equal(queries, want[:, :H * dh]) and (queries_only or torch.equal(out, want))
+    assert torch.equal(pools[0], want_pools[0]) and torch.equal(pools[1], want_pools[1])
     assert pools[0].abs().sum() > 0 and pools[1].abs().sum() > 0
 
 

@@ -225,7 +225,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   bf16x8 b[U][NB];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    const int ks = wave + u * WAVES;
+    const int ks = 2 * (wave + (u / 2) * WAVES) + u % 2;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
       b[u][nb] = *reinterpret_cast<const bf16x8*>(ks < ksteps ? wblk[nb] + ks * 512 : W + lane * 8);
@@ -247,13 +247,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = floatx4{0.f, 0.f, 0.f, 0.f};
-  for (int ks0 = wave; ks0 < ksteps; ks0 += WAVES * U) {
+  // the steps go to the waves in pairs: wave w takes steps 2w, 2w + 1, 2 (w + WAVES), ... (the same
+  // shares as in gemm16_kernel, so that both sum in the same order)
+  for (int p0 = wave; 2 * p0 < ksteps; p0 += WAVES * (U / 2)) {
     bf16x8 a[U][MB];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int ks = ks0 + u * WAVES;
+      const int ks = 2 * (p0 + (u / 2) * WAVES) + u % 2;
       const bool ok = ks < ksteps && ks * 32 + g * 8 < K;
-      if (ks0 != wave) {
+      if (p0 != wave) {
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
           b[u][nb] = *reinterpret_cast<const bf16x8*>(ks < ksteps ? wblk[nb] + ks * 512 : W + lane * 8);
@@ -264,7 +266,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int ks = ks0 + u * WAVES;
+      const int ks = 2 * (p0 + (u / 2) * WAVES) + u % 2;
       const bool ok = ks < ksteps && ks * 32 + g * 8 < K;
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
@@ -310,6 +312,101 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   }
 }
 
+// Up to 16 rows of A in rows.  In the operands' layout 16 lanes are 16 rows, and a load of A from
+// memory touches as many cache lines (four times as many lookups as the packed W costs, and they
+// were what this product of 8 rows waited for).  Here a wave takes the steps of K in pairs
+// (wave w: steps 2w, 2w + 1, then 2 (w + WAVES), ...), so that a row's share of a pair is one cache
+// line of 128 bytes; it loads A eight lanes to a row, turns each pair round through a piece of LDS
+// of its own (no barrier: a wave's LDS operations keep their order) and reads the operands from
+// there.  16 columns per workgroup, sums joined through LDS in wave order, as in gemm_kernel.
+template <int WAVES, typename TC, bool KV>
+__global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __restrict__ A, int lda,
+                                                             const bf16_t* __restrict__ W,
+                                                             const float* __restrict__ bias, TC* __restrict__ C,
+                                                             int ldc, float* __restrict__ resid, int ldr, int M,
+                                                             int N, int K, int epi, KVScatter kv) {
+  typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+  constexpr int U = 4;                                     // pairs of steps in flight per wave
+  constexpr int ROW = 9 * 8;                               // elements per row of a wave's piece: 8 chunks and one of padding
+  __shared__ floatx4 red[WAVES][64];
+  __shared__ __attribute__((aligned(16))) bf16_t turn[WAVES][16 * ROW];
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int col = lane % 16, g = lane / 16;
+  const int n0 = blockIdx.x * 16;
+  const int ksteps = (K + 31) / 32, npairs = (ksteps + 1) / 2, nblocks = (N + 15) / 16;
+  const bf16_t* wblk = W + (static_cast<size_t>(min(static_cast<int>(blockIdx.x), nblocks - 1)) * ksteps * 64 + lane) * 8;
+  const bool two = M > 8;                                  // rows 8 .. 15 need a second load per pair
+  // what the epilogue will read is asked for first of all (wave 0 finishes the block)
+  float epi_bias = 0.f;
+  float epi_x[4] = {0.f, 0.f, 0.f, 0.f};
+  if (wave == 0) {
+    const int nn = min(n0 + col, N - 1);
+    if (bias) epi_bias = bias[nn];
+    if (resid) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) epi_x[r] = resid[static_cast<size_t>(min(g * 4 + r, M - 1)) * ldr + nn];
+    }
+  }
+  // never a conditional load; a step beyond K reads W's first block and meets zeros of A
+  const int lrow = lane / 8, lch = lane % 8;               // as loader: row and 16-byte chunk of the pair's 128 bytes
+  const bf16_t* a0 = A + static_cast<size_t>(min(lrow, M - 1)) * lda + lch * 8;
+  const bf16_t* a1 = A + static_cast<size_t>(min(lrow + 8, M - 1)) * lda + lch * 8;
+  bf16_t* mine = turn[wave];
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int p0 = wave; p0 < npairs; p0 += WAVES * U) {
+    bf16x8 b[U][2];
+    u32x4 al[U][2];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int p = p0 + u * WAVES, ks = 2 * p;
+      b[u][0] = *reinterpret_cast<const bf16x8*>(ks < ksteps ? wblk + ks * 512 : W + lane * 8);
+      b[u][1] = *reinterpret_cast<const bf16x8*>(ks + 1 < ksteps ? wblk + (ks + 1) * 512 : W + lane * 8);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int p = p0 + u * WAVES;
+      const bool ok = p * 64 + lch * 8 < K;
+      al[u][0] = *reinterpret_cast<const u32x4*>(ok ? a0 + p * 64 : a0);
+      al[u][1] = *reinterpret_cast<const u32x4*>(ok && two ? a1 + p * 64 : a0);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int p = p0 + u * WAVES;
+      const bool ok = p < npairs && p * 64 + lch * 8 < K;
+      *reinterpret_cast<u32x4*>(mine + lrow * ROW + lch * 8) = ok ? al[u][0] : zero4;
+      if (two) *reinterpret_cast<u32x4*>(mine + (lrow + 8) * ROW + lch * 8) = ok ? al[u][1] : zero4;
+      // as operand: lane (row col, chunk g) of each of the pair's two steps
+      const bf16x8 f0 = *reinterpret_cast<const bf16x8*>(mine + col * ROW + g * 8);
+      const bf16x8 f1 = *reinterpret_cast<const bf16x8*>(mine + col * ROW + (4 + g) * 8);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, b[u][0], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1, b[u][1], acc, 0, 0, 0);
+    }
+  }
+  red[wave][lane] = acc;
+  __syncthreads();
+  // acc[r] of lane (col, g) is row g*4 + r, column n0 + col
+  if (wave == 0) {
+    const int nn = n0 + col;
+    floatx4 sm = red[0][lane];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) sm += red[w][lane];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = g * 4 + r;
+      if (m >= M || nn >= N) continue;
+      const float v = sm[r] + epi_bias;
+      if (resid) {
+        resid[static_cast<size_t>(m) * ldr + nn] = epi_x[r] + v;
+      } else {
+        const TC cv = from_float<TC>(apply_epilogue(v, epi));
+        if (!KV || nn < kv.c_cols) C[static_cast<size_t>(m) * ldc + nn] = cv;
+        if constexpr (KV) scatter_kv(kv, m, nn, cv);
+      }
+    }
+  }
+}
+
 struct Call {
   const void* A; int lda; const void* W; const float* bias; void* C; int ldc; float* resid; int ldr;
   int M, N, K, out_dtype, epi, packed;
@@ -332,6 +429,21 @@ static void launch(const Call& c, hipStream_t stream) {
   return launch_one<MB, NB, WAVES, U, float, false>(c, stream);
 }
 
+template <int WAVES, typename TC, bool KV>
+static void launch16_one(const Call& c, hipStream_t stream) {
+  KVScatter kv = c.kv ? *c.kv : KVScatter{};
+  hipLaunchKernelGGL((gemm16_kernel<WAVES, TC, KV>), dim3((c.N + 15) / 16), dim3(WAVES * 64), 0, stream,
+                     static_cast<const bf16_t*>(c.A), c.lda, static_cast<const bf16_t*>(c.W), c.bias,
+                     static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N, c.K, c.epi, kv);
+}
+
+template <int WAVES>
+static void launch16(const Call& c, hipStream_t stream) {
+  if (c.kv) return launch16_one<WAVES, bf16_t, true>(c, stream);
+  if (c.out_dtype == DN_BF16) return launch16_one<WAVES, bf16_t, false>(c, stream);
+  return launch16_one<WAVES, float, false>(c, stream);
+}
+
 // With more than 16 rows every workgroup reads all of A (16 cache lines per load and 16 lanes,
 // as A lies in rows), so wider workgroups read less in total, as long as enough of them remain
 // to keep the memory system busy.  Measured at 64 rows: 2 column blocks where N >= 4096 (20 ->
@@ -339,6 +451,7 @@ static void launch(const Call& c, hipStream_t stream) {
 template <int WAVES>
 static void launch_mb(const Call& c, hipStream_t stream) {
   const int mb = (c.M + 15) / 16;
+  if (mb == 1 && !(c.packed & (PACKED_A | PACKED_C)) && c.M > 1) return launch16<WAVES>(c, stream);
   if (mb == 1) return launch<1, 1, WAVES, 8>(c, stream);
   if (c.N >= 32768) {
     switch (mb) {

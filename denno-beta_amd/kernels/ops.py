@@ -164,7 +164,7 @@ class PackedMatrix:
 
 
 PACKED_ROWS_MAX = 64     # the few-rows product's limit
-PACKED_ROWS_MIN = 9      # below, rows in the ordinary layout were measured as fast or faster (one row: 10 % faster)
+PACKED_ROWS_MIN = 17     # up to 16 rows the few-rows product turns ordinary rows round itself, as fast or faster
 
 
 def packed_rows(n_rows, width, device) -> PackedMatrix:

@@ -178,21 +178,22 @@ def test_long_context_with_heads_of_64(model_folders, dtype):
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", ["C", "D"])
 @pytest.mark.parametrize("graphs", [False, True])
-def test_twelve_requests_decode_together(model_folders, name, graphs):
-    """Steps of 9 to 64 rows hand their bfloat16 rows from kernel to kernel in the packed layout
+def test_twenty_requests_decode_together(model_folders, name, graphs):
+    """Steps of 17 to 64 rows hand their bfloat16 rows from kernel to kernel in the packed layout
     (LayerNorm, the decode attention and the first feed-forward product write it, the few-rows
     product reads it).  C's feed-forward width is no multiple of 32, so its second product takes
     ordinary rows; D packs all of them."""
     from denno_beta_amd.config import EngineOptions
     from denno_beta_amd.engine import ModelRunner, StepEntry
     folder = model_folders(name, "bfloat16")
-    seqs = sequences(name, (40, 25, 70, 33, 90, 21, 58, 64, 30, 47, 36, 81), seed=40)
+    seqs = sequences(name, (40, 25, 70, 33, 90, 21, 58, 64, 30, 47, 36, 81, 22, 55, 73, 38, 61, 27, 44, 66), seed=40)
+    n = len(seqs)
     want = plain_logits(folder, seqs)
-    r = ModelRunner.from_folder(folder, EngineOptions(dtype="bfloat16", page_size=16, cache_tokens=12 * 96,
-                                                      max_live=12, use_graphs=graphs))
-    assert r.model.blocks[0].mixer.packed_input(12) and not r.model.blocks[0].mixer.packed_input(8)
-    assert r.model.blocks[0].ffn.down.packed_input(12) == (name == "D")
-    for i in range(12):
+    r = ModelRunner.from_folder(folder, EngineOptions(dtype="bfloat16", page_size=16, cache_tokens=n * 96,
+                                                      max_live=n, use_graphs=graphs))
+    assert r.model.blocks[0].mixer.packed_input(n) and not r.model.blocks[0].mixer.packed_input(16)
+    assert r.model.blocks[0].ffn.down.packed_input(n) == (name == "D")
+    for i in range(n):
         r.start_request(i)
     tail = 20
     got = r.step([StepEntry(i, s[:-tail], list(range(len(s) - tail))) for i, s in enumerate(seqs)]).cpu()

@@ -548,6 +548,25 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
   for (int c = 0; c < chunks; ++c) {
     const int kbase = key0 + c * CHUNK + wave * 64;
     if (kbase > pos || kbase + 64 <= lo) continue;     // the same for the whole wave; no barrier in this loop
+    // values: lane = dim; 16 keys of one page at a time.  They are asked for first, before the keys
+    // (whose use would otherwise stand between them and memory): keys and values then make one trip
+    bf16x8 v0[4][DPL], v1[4][DPL];
+    bool live[4];
+#pragma unroll
+    for (int blk = 0; blk < 4; ++blk) {
+      const int kb = kbase + blk * 16;
+      live[blk] = kb <= pos && kb + 16 > lo;
+      const int kk = live[blk] ? kb : (pos / 16) * 16;
+      const int page = bt[kk / page_size];
+      live[blk] = live[blk] && page >= 0;
+      const bf16_t* vb = v_pool + (static_cast<size_t>(max(page, 0)) * Hkv + hk) * DH * page_size + kk % page_size;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        const int d = min(lane + 64 * i, DH - 1);
+        v0[blk][i] = *reinterpret_cast<const bf16x8*>(vb + static_cast<size_t>(d) * page_size);
+        v1[blk][i] = *reinterpret_cast<const bf16x8*>(vb + static_cast<size_t>(d) * page_size + 8);
+      }
+    }
     // scores: lane (key group grp, part sub of the key); after the sum over the key's lanes every
     // lane of group grp holds, in sc[it], the score of key kbase + it * KPI + grp
     float sc[LPK];
@@ -570,24 +589,6 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
         for (int i = 0; i < 8; ++i) dot = fmaf(qr[i], static_cast<float>(kv[u][i]), dot);
         dot = group_reduce<LPK>(dot, SumOp());
         sc[it0 + u] = (key >= lo && key <= pos) ? dot : NEG_INF;
-      }
-    }
-    // values: lane = dim; 16 keys of one page at a time, all loads of the 64 keys before their use
-    bf16x8 v0[4][DPL], v1[4][DPL];
-    bool live[4];
-#pragma unroll
-    for (int blk = 0; blk < 4; ++blk) {
-      const int kb = kbase + blk * 16;
-      live[blk] = kb <= pos && kb + 16 > lo;
-      const int kk = live[blk] ? kb : (pos / 16) * 16;
-      const int page = bt[kk / page_size];
-      live[blk] = live[blk] && page >= 0;
-      const bf16_t* vb = v_pool + (static_cast<size_t>(max(page, 0)) * Hkv + hk) * DH * page_size + kk % page_size;
-#pragma unroll
-      for (int i = 0; i < DPL; ++i) {
-        const int d = min(lane + 64 * i, DH - 1);
-        v0[blk][i] = *reinterpret_cast<const bf16x8*>(vb + static_cast<size_t>(d) * page_size);
-        v1[blk][i] = *reinterpret_cast<const bf16x8*>(vb + static_cast<size_t>(d) * page_size + 8);
       }
     }
     float m_c = NEG_INF;

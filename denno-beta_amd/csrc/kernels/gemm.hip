@@ -354,9 +354,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
   bf16_t* mine = turn[wave];
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
   floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int p0 = wave; p0 < npairs; p0 += WAVES * U) {
-    bf16x8 b[U][2];
-    u32x4 al[U][2];
+  // a round: U pairs of steps per wave, all its loads issued at once.  Measured and dropped: asking
+  // for the next round before this one is used, into a second set of registers (K = 6400: 10.3 ->
+  // 11.2 us), and sharing a block's 16 columns among 2 or 4 workgroups where blocks are few (1600
+  // columns, K = 6400: 10.3 -> 9.6 and 12.5 us; K = 1600: no gain)
+  auto ask = [&](int p0, bf16x8 (*b)[2], u32x4 (*al)[2]) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int p = p0 + u * WAVES, ks = 2 * p;
@@ -370,6 +372,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
       al[u][0] = *reinterpret_cast<const u32x4*>(ok ? a0 + p * 64 : a0);
       al[u][1] = *reinterpret_cast<const u32x4*>(ok && two ? a1 + p * 64 : a0);
     }
+  };
+  auto use = [&](int p0, const bf16x8 (*b)[2], const u32x4 (*al)[2]) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int p = p0 + u * WAVES;
@@ -382,6 +386,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, b[u][0], acc, 0, 0, 0);
       acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1, b[u][1], acc, 0, 0, 0);
     }
+  };
+  bf16x8 b0[U][2];
+  u32x4 al0[U][2];
+  for (int p0 = wave; p0 < npairs; p0 += WAVES * U) {
+    ask(p0, b0, al0);
+    use(p0, b0, al0);
   }
   red[wave][lane] = acc;
   __syncthreads();

@@ -45,9 +45,12 @@ class FixedState:
 
 @dataclass
 class Runtime:
-    """What parts need to know about the engine they are bound into."""
+    """What parts need to know about the engine they are bound into.  `position` is the model's
+    position encoding (set by the model before it binds its parts): a mixer asks it to turn its
+    queries and keys if it is of the kind that does (`rotates`)."""
     act_dtype: torch.dtype
     device: torch.device
+    position: Optional["Part"] = None
 
 
 class Part:

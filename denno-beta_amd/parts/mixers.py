@@ -50,7 +50,16 @@ class CausalSelfAttention(Part):
     def forward(self, h, ctx, cache, accumulate_into):
         act = self.runtime.act_dtype
         g = ctx.groups[cache.group]
-        if cache.writes:
+        position = self.runtime.position
+        if position is not None and getattr(position, "rotates", False):
+            # queries and keys are turned by their positions before the keys go to the cache: the
+            # product, the turn and the cache write are three steps here, not one kernel
+            qkv = self.qkv(h, out_dtype=act)
+            q = qkv[:, :self.q_width]
+            position.rotate(q, qkv[:, self.q_width:self.q_width + self.kv_width], ctx)
+            if cache.writes:
+                ops.kv_write(qkv, self.q_width, self.q_width + self.kv_width, g.slot_map, cache.k, cache.v)
+        elif cache.writes:
             q = self.qkv.project_qkv(h, act, g.slot_map, cache.k, cache.v, self.q_width)
         else:
             q = self.qkv(h, out_dtype=act)[:, :self.q_width]

@@ -135,6 +135,7 @@ class DecoderModel:
     # -- binding -------------------------------------------------------------------------
     def bind(self, tensors: Dict[str, torch.Tensor], runtime: Runtime):
         self.runtime = runtime
+        runtime.position = self.position          # mixers ask it to turn their queries and keys, if it does that
         for p in self.all_parts():
             p.bind(tensors, runtime)
         if self.head is not None:

@@ -1,8 +1,10 @@
 """Position encodings and the token table.
 
 A position encoding acts in one of two places: it gives a table that the embedding stage adds
-to the token rows (`table()`), or it turns queries and keys inside a mixer (`rotate`).  One
-that does not act in a place returns None there / leaves q and k as they are.
+to the token rows (`table()`), or it turns queries and keys inside a mixer (`rotates = True` and
+`rotate(q, k, ctx)`, which changes q [T, heads * dh] and k [T, kv heads * dh] in place, rows
+ctx.positions; a mixer that keeps keys then writes the turned keys to its cache).  One that does
+not act in a place returns None there / has `rotates = False`.
 """
 from __future__ import annotations
 
@@ -29,6 +31,7 @@ class TokenEmbedding(Part):
 class LearnedAbsolutePositions(Part):
     """x[i] += wpe[position_i]                    (crates/denno-engine/src/model/gpt2.rs:142-150)"""
     graph_safe = True
+    rotates = False
 
     def __init__(self, n_positions: int, width: int, name: str):
         self.n_positions, self.width, self.name = n_positions, width, name
@@ -50,6 +53,8 @@ class LearnedAbsolutePositions(Part):
 @POSITIONS.register("none")
 class NoPositions(Part):
     graph_safe = True
+    rotates = False
+
     def __init__(self):
         pass
 

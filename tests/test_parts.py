@@ -285,3 +285,156 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(backend):
         for i in range(len(seqs)):
             U.assert_close(got[f"r{i}"], want[i], "float32", f"toy model, {kind}, request {i}")
     r.cache.manager.check()
+
+
+# -- a toy position encoding that turns queries and keys, a toy feed-forward with routing --------
+def register_toy_rotation_and_experts():
+    from denno_beta_amd.parts import FEED_FORWARDS, POSITIONS, Part
+    from denno_beta_amd.weights import ParamSpec
+    if "toy_rotation" in POSITIONS:
+        return
+
+    @POSITIONS.register("toy_rotation")
+    class ToyRotation(Part):
+        """Pairs (2i, 2i + 1) of every head of q and k are turned by the angle position * base^(-2i/dh)."""
+        rotates = True
+
+        def __init__(self, head_dim, base):
+            self.head_dim, self.base = head_dim, base
+
+        def table(self):
+            return None
+
+        def rotate(self, q, k, ctx):
+            for t in (q, k):
+                turn_pairs(t, ctx.positions.to(torch.float32), self.head_dim, self.base)
+            return q, k
+
+    @FEED_FORWARDS.register("toy_experts")
+    class ToyExperts(Part):
+        """A router picks one expert per row (the first maximum of h R^T, in 32-bit); that expert's
+        two products with a tanh GELU between them are added into the residual stream."""
+
+        def __init__(self, width, inner, n_experts, prefix):
+            self.width, self.inner, self.n, self.prefix = width, inner, n_experts, prefix
+
+        def param_specs(self):
+            specs = [ParamSpec(self.prefix + "router", (self.n, self.width), "matrix", ("normal", 0.0, 0.5))]
+            for e in range(self.n):
+                specs += [ParamSpec(f"{self.prefix}e{e}.up", (self.inner, self.width), "matrix", ("normal", 0.0, 0.2)),
+                          ParamSpec(f"{self.prefix}e{e}.down", (self.width, self.inner), "matrix", ("normal", 0.0, 0.2))]
+            return specs
+
+        def bind(self, tensors, runtime):
+            super().bind(tensors, runtime)
+            self.router = tensors[self.prefix + "router"].float()
+            self.up = [tensors[f"{self.prefix}e{e}.up"].float() for e in range(self.n)]
+            self.down = [tensors[f"{self.prefix}e{e}.down"].float() for e in range(self.n)]
+
+        def forward(self, h, ctx, accumulate_into):
+            h = h.float()
+            choice = first_max(h @ self.router.t())
+            for e in range(self.n):
+                rows = (choice == e).nonzero().flatten()
+                if len(rows):
+                    accumulate_into[rows] += P.gelu_tanh(h[rows] @ self.up[e].t()) @ self.down[e].t()
+
+
+def first_max(scores):
+    """Index of each row's first maximum."""
+    best = scores.max(dim=-1, keepdim=True).values
+    return (scores == best).float().argmax(dim=-1)
+
+
+def turn_pairs(t, positions, head_dim, base):
+    """In place: in every head of t [T, heads * head_dim], the pair (2i, 2i + 1) turned by
+    positions[row] * base^(-2i / head_dim); angles, sines and the products in 32-bit."""
+    T, W = t.shape
+    x = t.float().reshape(T, W // head_dim, head_dim // 2, 2)
+    i = torch.arange(head_dim // 2, device=t.device, dtype=torch.float32)
+    angle = positions.to(t.device)[:, None, None] * base ** (-2.0 * i / head_dim)[None, None, :]
+    c, s = torch.cos(angle), torch.sin(angle)
+    a, b = x[..., 0], x[..., 1]
+    t.copy_(torch.stack([a * c - b * s, a * s + b * c], dim=-1).reshape(T, W).to(t.dtype))
+
+
+def rotation_model():
+    from denno_beta_amd.parts import DecoderSpec, LayerCall, LayerSpec
+    E = 32
+    layers = []
+    for i, (heads, kv_heads) in enumerate(((2, 2), (4, 2))):
+        p = f"L{i}."
+        dh = E // heads
+        layers.append(LayerSpec(
+            "pre_norm", ("layernorm", dict(width=E, eps=1e-5, weight_name=p + "n1.g", bias_name=None)),
+            ("causal_attention", dict(width=E, n_heads=heads, n_kv_heads=kv_heads, head_dim=16, scale=0.25,
+                                      qkv_weight=p + "qkv.w", qkv_bias=None, out_weight=p + "o.w", out_bias=None))
+            if heads == 2 else
+            ("causal_attention", dict(width=E, n_heads=heads, n_kv_heads=kv_heads, head_dim=16, scale=0.25,
+                                      qkv_weight=p + "qkv.w", qkv_bias=None, out_weight=p + "o.w", out_bias=None)),
+            ("layernorm", dict(width=E, eps=1e-5, weight_name=p + "n2.g", bias_name=None)),
+            ("toy_experts", dict(width=E, inner=48, n_experts=3, prefix=p + "ffn."))))
+        assert dh in (16, 8)
+    return DecoderSpec(vocab=50, width=E, max_positions=128, token_table="tok",
+                       position=("toy_rotation", dict(head_dim=16, base=50.0)), layers=layers,
+                       run_order=[LayerCall(i, i) for i in range(len(layers))],
+                       final_norm=("layernorm", dict(width=E, eps=1e-5, weight_name="nf.g", bias_name=None)))
+
+
+def rotation_plain(spec, st, seq, positions=None):
+    """The same model on one whole sequence with the plain functions; `positions` other than
+    0, 1, 2, ... shift every token."""
+    T = len(seq)
+    pos = torch.arange(T, dtype=torch.float32) if positions is None else positions
+    x = st["tok"][torch.tensor(seq)]
+    for i, ls in enumerate(spec.layers):
+        p = f"L{i}."
+        a = ls.mixer[1]
+        H, Hkv, dh = a["n_heads"], a["n_kv_heads"], a["head_dim"]
+        h = P.layer_norm(x, st[p + "n1.g"], 0.0, 1e-5)
+        qkv = h @ st[p + "qkv.w"].t()
+        q, k, v = qkv[:, :H * dh].clone(), qkv[:, H * dh:(H + Hkv) * dh].clone(), qkv[:, (H + Hkv) * dh:]
+        turn_pairs(q, pos, dh, 50.0)
+        turn_pairs(k, pos, dh, 50.0)
+        # query head hd reads key head hd // (H / Hkv): spread keys and values out to H heads
+        spread = lambda t: t.reshape(T, Hkv, 1, dh).expand(T, Hkv, H // Hkv, dh).reshape(T, H * dh)   # noqa: E731
+        x = x + P.causal_attention(q, spread(k), spread(v), H, a["scale"]) @ st[p + "o.w"].t()
+        h = P.layer_norm(x, st[p + "n2.g"], 0.0, 1e-5)
+        f = ls.ffn[1]
+        choice = first_max(h @ st[f["prefix"] + "router"].t())
+        out = torch.zeros_like(x)
+        for t in range(T):
+            e = int(choice[t])
+            out[t] = P.gelu_tanh(h[t] @ st[f"{f['prefix']}e{e}.up"].t()) @ st[f"{f['prefix']}e{e}.down"].t()
+        x = x + out
+    return P.layer_norm(x, st["nf.g"], 0.0, 1e-5) @ st["tok"].t()
+
+
+def test_toy_rotation_and_toy_experts_are_registered_built_and_stepped(backend):
+    """A position encoding that turns queries and keys before the keys go to the cache (with fewer
+    key heads than query heads in one layer) and a feed-forward that routes rows to experts, both
+    defined here; the framework's files do not change."""
+    from denno_beta_amd.engine import ModelRunner
+    register_toy_rotation_and_experts()
+    spec = rotation_model()
+    tensors = draw(spec, backend)
+    for name in tensors:              # sharp attention, so that a wrong turn of a query or key shows in the logits
+        if name.endswith("qkv.w"):
+            tensors[name] *= 25.0
+    r = ModelRunner(spec, tensors, options(backend, cache_tokens=192))
+    st = {k: v.float().cpu() for k, v in tensors.items()}
+    seqs = [seeded_tokens(i, n, 50) for i, n in enumerate((30, 11, 47, 25, 40))]
+    want = [rotation_plain(spec, st, s) for s in seqs]
+    for kind, steps in (("whole", U.whole_trace(seqs)), ("tail", U.tail_decode_trace(seqs, 8)),
+                        ("mixed", U.mixed_trace(seqs, seed=3))):
+        got = U.replay(r, steps)
+        for i in range(len(seqs)):
+            U.assert_close(got[f"r{i}"], want[i], "float32", f"rotation and experts, {kind}, request {i}")
+    r.cache.manager.check()
+    # the plain model is pinned by what a rotation must keep: only distances between positions
+    # count, so shifting every position by the same amount changes nothing; and the rotation does
+    # act (without it the logits differ)
+    shifted = rotation_plain(spec, st, seqs[0], positions=torch.arange(len(seqs[0]), dtype=torch.float32) + 7.0)
+    assert torch.allclose(shifted, want[0], atol=2e-4)
+    still = rotation_plain(spec, st, seqs[0], positions=torch.zeros(len(seqs[0])))
+    assert (still - want[0]).abs().max() > 0.05

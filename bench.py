@@ -64,7 +64,8 @@ def main():
     V, E, P = cfg["vocab_size"], cfg["n_embd"], cfg["n_positions"]
     if a.context + a.warmup + a.steps + 1 > P:
         a.steps = P - a.context - a.warmup - 1
-    opts = EngineOptions(dtype=a.dtype, page_size=16, cache_tokens=64 * P, max_live=64, max_batch_tokens=4096,
+    live = max(64, a.batch)
+    opts = EngineOptions(dtype=a.dtype, page_size=16, cache_tokens=live * P, max_live=live, max_batch_tokens=4096,
                          prefill_chunk=1024, use_graphs=not a.no_graphs, seed=0)
     runner = ModelRunner.from_random(cfg, seed=0, options=opts, stored=a.dtype)
     gen = torch.Generator().manual_seed(0)

@@ -427,7 +427,8 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
   }
   if (has_rows && row_ok) {
     const float inv = 1.0f / l;
-    bf16_t* orow = out + static_cast<size_t>(row0 + my_row) * ldo + h * DH;
+    // rows, or packed rows (ldo == 0): four dims from a multiple of 4 are 8 bytes side by side in both
+    const int orow_i = row0 + my_row;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -436,7 +437,9 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
         if (d0 < DH) {
           bf16x4 w = {to_bf16(o[db][4 * a] * inv), to_bf16(o[db][4 * a + 1] * inv), to_bf16(o[db][4 * a + 2] * inv),
                       to_bf16(o[db][4 * a + 3] * inv)};
-          *reinterpret_cast<bf16x4*>(orow + d0) = w;
+          bf16_t* dst = ldo > 0 ? out + static_cast<size_t>(orow_i) * ldo + h * DH + d0
+                                : out + packed_index(orow_i, h * DH + d0, H * DH / 32);
+          *reinterpret_cast<bf16x4*>(dst) = w;
         }
       }
   }
@@ -449,8 +452,10 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
                                   int n_tiles, int H, int Hkv, int dh, int page_size, float scale, int window,
                                   hipStream_t stream) {
   if (n_tiles <= 0) return 0;
-  if (Hkv < 1 || H % Hkv != 0 || page_size % 16 != 0 || max_blocks < 1 || ldq % 8 != 0 || ldo % 4 != 0 ||
-      reinterpret_cast<uintptr_t>(q) % 16 != 0 || reinterpret_cast<uintptr_t>(out) % 8 != 0)
+  // ldo == 0: out is a packed matrix of H * dh columns (a multiple of 32)
+  if (Hkv < 1 || H % Hkv != 0 || page_size % 16 != 0 || max_blocks < 1 || ldq % 8 != 0 || ldo % 4 != 0 || ldo < 0 ||
+      (ldo == 0 && (H * dh) % 32 != 0) || reinterpret_cast<uintptr_t>(q) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(out) % 8 != 0)
     return DN_ERR_SHAPE;
   // Two groups of waves where the workgroups are fewer than the CUs (a wave's chain of dependent
   // steps per tile then bounds the time, and two groups halve the tiles a wave walks: 1 request,

@@ -4,9 +4,9 @@
 //
 // Three kernels behind dn_gemm.  plain: 32-bit multiply-adds in a fixed order over K, whatever
 // M is, so a row's result does not depend on what else is in the batch; it is the whole 32-bit
-// path and takes bfloat16 operands too (converted exactly on load).  skinny: bfloat16, up to 64
-// rows, MFMA, bound by reading W once (decode).  tiled: bfloat16, many rows, MFMA through LDS
-// (prefill).
+// path and takes bfloat16 operands too (converted exactly on load).  skinny: bfloat16, up to 256
+// rows, MFMA, waves split K, bound by reading W once (decode, and steps of a few short prompt
+// portions).  tiled: bfloat16, many rows, MFMA through LDS (prefill).
 //
 // The two MFMA kernels take W packed (dn_pack_matrix): blocks of 16 rows x 32 columns, block
 // (n / 16, k / 32) at ((n / 16) * ceil(K / 32) + k / 32) * 512 elements, and inside a block the
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const TI* __restrict__ A, int
 
 
 // ---------------------------------------------------------------------------------------
-// Few rows (M <= 64), bfloat16: the decode step's products, bound by reading W once.
+// Few rows (M <= 256), bfloat16: the decode step's products, bound by reading W once.
 // A workgroup owns 16, 32 or 64 output columns; its waves split K in steps of 32 (wave w takes
 // steps w, w + WAVES, ...), each feeding v_mfma_f32_16x16x32_bf16 with one packed block of W per
 // 16 columns straight from memory (16 bytes per lane) and the matching 16 bytes of up to four
@@ -463,6 +463,17 @@ static void launch_mb(const Call& c, hipStream_t stream) {
   const int mb = (c.M + 15) / 16;
   if (mb == 1 && !(c.packed & (PACKED_A | PACKED_C)) && c.M > 1) return launch16<WAVES>(c, stream);
   if (mb == 1) return launch<1, 1, WAVES, 8>(c, stream);
+  if (mb > 4) {
+    // 65 to 256 rows: 16 columns per workgroup, the waves' sums for all row blocks through LDS.
+    // Measured against the tiled kernel (which has too few tiles to fill the chip here, and walks
+    // K = 6400 in a hundred steps whatever M is), the four products of a GPT-2 XL layer with
+    // packed rows: 56 against 158 us at 65 to 96 rows, 67 at 128, 87 at 192, 108 at 256; with
+    // rows in the ordinary layout 80, 127, 181 and 234 us.
+    if (mb <= 6) return launch<6, 1, WAVES, 2>(c, stream);
+    if (mb <= 8) return launch<8, 1, WAVES, 2>(c, stream);
+    if (mb <= 12) return launch<12, 1, WAVES, 2>(c, stream);
+    return launch<16, 1, WAVES, 2>(c, stream);
+  }
   if (c.N >= 32768) {
     switch (mb) {
       case 2: return launch<2, 4, WAVES, 4>(c, stream);
@@ -494,7 +505,7 @@ static void run(const Call& c, hipStream_t stream) {
 // A must allow 16-byte loads: in rows with K and lda multiples of 8 and the base aligned, or packed
 // (K a multiple of 32 then: nothing zeroes a packed block's columns beyond K); W is packed
 static bool takes(const void* A, int lda, const void* W, int M, int K, int packed) {
-  if (M > 64 || reinterpret_cast<uintptr_t>(A) % 16 != 0 || reinterpret_cast<uintptr_t>(W) % 16 != 0) return false;
+  if (M > 256 || reinterpret_cast<uintptr_t>(A) % 16 != 0 || reinterpret_cast<uintptr_t>(W) % 16 != 0) return false;
   return (packed & PACKED_A) ? K % 32 == 0 : (K % 8 == 0 && lda % 8 == 0);
 }
 }  // namespace skinny
@@ -777,7 +788,7 @@ static int run(const void* A, int lda, const void* W, const float* bias, void* C
 
 // packed: bit flags.  W in rows of K elements (the plain kernel, any dtype), or packed bfloat16
 // (PACKED_W 1: the MFMA kernels, which need A in bfloat16 and loadable 16 bytes at a time).  With
-// at most 64 rows A may be packed too (PACKED_A 2; lda is not read) and so may a bfloat16 C
+// at most 256 rows A may be packed too (PACKED_A 2; lda is not read) and so may a bfloat16 C
 // (PACKED_C 4; N a multiple of 32; ldc is not read).
 extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid,
                        int ldr, int M, int N, int K, int in_dtype, int out_dtype, int epilogue, int packed,
@@ -786,7 +797,7 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
   if (K <= 0 || K % 4 != 0 || (lda < K && !(packed & PACKED_A))) return DN_ERR_SHAPE;
   if (epilogue < EPI_NONE || epilogue > EPI_GELU_ERF) return DN_ERR_SHAPE;
   if (resid != nullptr && epilogue != EPI_NONE) return DN_ERR_SHAPE;
-  if ((packed & (PACKED_A | PACKED_C)) && (!(packed & PACKED_W) || M > 64)) return DN_ERR_SHAPE;
+  if ((packed & (PACKED_A | PACKED_C)) && (!(packed & PACKED_W) || M > 256)) return DN_ERR_SHAPE;
   if ((packed & PACKED_C) && (resid != nullptr || out_dtype != DN_BF16 || N % 32 != 0)) return DN_ERR_SHAPE;
   if (packed & PACKED_W) {
     if (in_dtype != DN_BF16) return DN_ERR_DTYPE;
@@ -820,7 +831,7 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
 
 // The fused projection q | k | v with packed W: C = A . W^T + bias as dn_gemm computes it, and the
 // key and value columns also go to their pages (see KVScatter), from the epilogue of the few-rows
-// or of the tiled kernel.  a_packed: A is packed (at most 64 rows).  c_cols: N, or q_width: C then
+// or of the tiled kernel.  a_packed: A is packed (at most 256 rows).  c_cols: N, or q_width: C then
 // is [M, q_width] and gets the query columns only.
 extern "C" int dn_gemm_qkv(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, int M, int N,
                            int K, const int32_t* slot_map, void* k_pool, void* v_pool, int q_width, int Hkv, int dh,

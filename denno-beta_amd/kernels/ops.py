@@ -135,7 +135,7 @@ class PackedMatrix:
     elements; inside it row n % 16, columns (k % 32) // 8 * 8 .. + 7 at (((k % 32) // 8) * 16 + n % 16) * 8.
     `linear` takes it for the MFMA kernels.  Every bfloat16 weight is held so (rows and columns
     beyond N and K are zeros), and so are the bfloat16 rows that one kernel hands to the next
-    while a step has at most 64 of them (`packed_rows`; K a multiple of 32, rows beyond N are
+    while a step has at most 256 of them (`packed_rows`; K a multiple of 32, rows beyond N are
     not written and never read into a result)."""
     __slots__ = ("data", "shape")
     dtype = torch.bfloat16
@@ -163,12 +163,12 @@ class PackedMatrix:
         return self.data.view(nb, ks, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(nb * 16, ks * 32)[:N, :K].contiguous()
 
 
-PACKED_ROWS_MAX = 64     # the few-rows product's limit
+PACKED_ROWS_MAX = 256    # the few-rows product's limit
 PACKED_ROWS_MIN = 17     # up to 16 rows the few-rows product turns ordinary rows round itself, as fast or faster
 
 
 def packed_rows(n_rows, width, device) -> PackedMatrix:
-    """An empty packed matrix for n_rows <= 64 rows of activations."""
+    """An empty packed matrix for n_rows <= 256 rows of activations."""
     _need(n_rows <= PACKED_ROWS_MAX and width % 32 == 0,
           f"packed rows: at most {PACKED_ROWS_MAX} rows of a width that is a multiple of 32, not {n_rows} x {width}")
     data = torch.empty(-(-n_rows // 16) * (width // 32) * 512, dtype=torch.bfloat16, device=device)
@@ -268,7 +268,7 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
     """out = epilogue(a @ w.T + bias), or residual += a @ w.T + bias (32-bit, in place).
     a: [M, K] rows contiguous; w: [N, K] held [out, in], in rows (the plain kernel: 32-bit, or a
     reference for bfloat16) or a PackedMatrix (the MFMA kernels); bias: 32-bit [N].  With a packed
-    w and at most 64 rows, a and a bfloat16 out may be packed rows."""
+    w and at most 256 rows, a and a bfloat16 out may be packed rows."""
     M, K = a.shape
     _need(K % 8 == 0, f"linear: the inner size {K} must be a multiple of 8")
     lda, N, packed = _operands(a, w, "linear")
@@ -338,9 +338,16 @@ DECODE_SPLIT = 256     # the decode kernel's smallest chunk; captured decode ste
 
 
 def decode_attention_applies(dtype, page_size, head_dim, single_rows, max_context):
-    """Whether `attention` takes the split kernel of pure decode steps (which can write packed rows)."""
+    """Whether `attention` takes the split kernel of pure decode steps."""
     return (dtype == torch.bfloat16 and page_size % 16 == 0 and bool(single_rows) and head_dim in DECODE_HEAD_DIMS
             and max_context > 0)
+
+
+def attention_writes_packed(dtype, page_size, head_dim, single_rows, max_context, tiles_wide):
+    """Whether `attention` with these arguments takes one of the two bfloat16 kernels, which can write
+    packed rows (the plain kernel cannot)."""
+    return decode_attention_applies(dtype, page_size, head_dim, single_rows, max_context) or (
+        dtype == torch.bfloat16 and page_size % 16 == 0 and tiles_wide is not None and head_dim in FLASH_HEAD_DIMS)
 
 
 def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, window=0, tiles_wide=None,
@@ -356,8 +363,8 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
     max_context: the longest context then.
 
     Three kernels: 32-bit takes the plain one; bfloat16 takes the MFMA kernel over tiles_wide, or,
-    for a pure decode step, the split kernel (out may then be packed rows); a head size that those
-    do not take falls to the plain one."""
+    for a pure decode step, the split kernel (with both, out may be packed rows); a head size that
+    those do not take falls to the plain one."""
     out_packed = isinstance(out, PackedMatrix)
     _dev(q, "q", _FLOATS, 2)
     if not out_packed:
@@ -376,7 +383,8 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
     lib = _lib("attention")
     fast = q.dtype == torch.bfloat16 and ps % 16 == 0 and ldq % 8 == 0 and q.data_ptr() % 16 == 0
     decode = fast and decode_attention_applies(q.dtype, ps, dh, single_rows, max_context)
-    _need(decode or not out_packed, "attention: packed rows as out are written by the decode kernel only")
+    _need(not out_packed or (fast and attention_writes_packed(q.dtype, ps, dh, single_rows, max_context, tiles_wide)),
+          "attention: packed rows as out are written by the bfloat16 kernels only")
     if decode:
         n_tiles = tiles.shape[1]
         # a workgroup's waves take 64 keys each at a time: as many waves as make the context one

@@ -63,9 +63,9 @@ class CausalSelfAttention(Part):
             q = self.qkv.project_qkv(h, act, g.slot_map, cache.k, cache.v, self.q_width)
         else:
             q = self.qkv(h, out_dtype=act)[:, :self.q_width]
-        # a pure decode step's kernel hands its rows to the output projection packed
-        if self.out.packed_input(h.shape[0]) and ops.decode_attention_applies(
-                act, cache.k.shape[2], self.head_dim, g.single_rows, g.max_context):
+        # the bfloat16 kernels hand their rows to the output projection packed, if it wants that
+        if self.out.packed_input(h.shape[0]) and ops.attention_writes_packed(
+                act, cache.k.shape[2], self.head_dim, g.single_rows, g.max_context, g.tiles_wide):
             o = ops.packed_rows(h.shape[0], self.q_width, h.device)
         else:
             o = torch.empty((h.shape[0], self.q_width), dtype=act, device=h.device)

@@ -149,7 +149,7 @@ def test_linear_qkv_writes_the_cache(M, slots_in, queries_only):
     assert pools[0].abs().sum() > 0 and pools[1].abs().sum() > 0
 
 
-@pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64, 65, 100, 130, 200, 256])
 @pytest.mark.parametrize("N,K", [(1600, 1600), (4800, 1600), (96, 6400), (33024, 64)])
 def test_linear_with_packed_rows(M, N, K):
     """The few-rows product reading packed rows and writing them gives, bit for bit, what it gives
@@ -181,14 +181,14 @@ def test_linear_with_packed_rows(M, N, K):
 def test_packed_rows_are_refused_where_no_kernel_takes_them():
     o = ops()
     w = o.pack_matrix(rnd(64, 64, dtype=torch.bfloat16))
-    with pytest.raises(o.KernelError, match="at most 64 rows"):
-        o.packed_rows(65, 64, DEV)
+    with pytest.raises(o.KernelError, match="at most 256 rows"):
+        o.packed_rows(257, 64, DEV)
     with pytest.raises(o.KernelError, match="multiple of 32"):
         o.packed_rows(4, 48, DEV)
     with pytest.raises(o.KernelError, match="need a packed matrix"):
         o.linear(o.packed_rows(4, 64, DEV), rnd(64, 64, dtype=torch.bfloat16), None, out=torch.empty(4, 64, dtype=torch.bfloat16, device=DEV))
     with pytest.raises(o.KernelError, match="packed rows as out"):
-        o.linear(rnd(70, 64, dtype=torch.bfloat16), w, None, out=o.PackedMatrix(torch.empty(5 * 2 * 512, dtype=torch.bfloat16, device=DEV), (70, 64)))
+        o.linear(rnd(270, 64, dtype=torch.bfloat16), w, None, out=o.PackedMatrix(torch.empty(17 * 2 * 512, dtype=torch.bfloat16, device=DEV), (270, 64)))
     with pytest.raises(o.KernelError, match="bfloat16 rows"):
         o.linear(rnd(4, 64), w, None, out=torch.empty(4, 64, device=DEV))
 
@@ -267,6 +267,15 @@ def test_attention_mfma_kernel_for_portions(H, Hkv, dh, ps, window):
     ops().attention(q[:, :H * dh], out, k, v, bt, tiles, H, scale, window, tiles_wide=paged_case.wide)
     want = R.attention(q[:, :H * dh], torch.zeros(T, H * dh, device=DEV), k, v, bt, tiles, H, scale, window)
     assert torch.allclose(out.float(), want, **TOL[torch.bfloat16])
+    if (H * dh) % 32 == 0:
+        # the first 200 rows as packed rows (the same requests, the long portion cut short)
+        new_rows[0] = 107
+        q2, k2, v2, bt2, tiles2, T2 = paged_case(seq_lens, new_rows, H, Hkv, dh, ps, torch.bfloat16, seed=H + dh)
+        rows = torch.zeros(T2, H * dh, dtype=torch.bfloat16, device=DEV)
+        ops().attention(q2[:, :H * dh], rows, k2, v2, bt2, tiles2, H, scale, window, tiles_wide=paged_case.wide)
+        packed = ops().packed_rows(T2, H * dh, DEV)
+        ops().attention(q2[:, :H * dh], packed, k2, v2, bt2, tiles2, H, scale, window, tiles_wide=paged_case.wide)
+        assert T2 == 200 and torch.equal(packed.rows(), rows)
 
 
 @pytest.mark.parametrize("H,Hkv,dh,ps,window", [(8, 8, 64, 16, 0), (8, 2, 32, 32, 40)])
@@ -315,8 +324,8 @@ def test_attention_split_kernel_for_decoding(H, Hkv, dh, ps, window):
         packed = ops().packed_rows(1, H * dh, DEV)
         ops().attention(one[0], packed, *one[1:], single_rows=True, max_context=17)
         assert torch.equal(packed.rows(), out)
-        with pytest.raises(ops().KernelError, match="decode kernel only"):
-            ops().attention(one[0], packed, *one[1:], tiles_wide=one[4])
+        with pytest.raises(ops().KernelError, match="bfloat16 kernels only"):
+            ops().attention(one[0], packed, *one[1:])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

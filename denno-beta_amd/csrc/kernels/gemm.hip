@@ -30,6 +30,18 @@ __device__ __forceinline__ float apply_epilogue(float v, int epi) {
   return v;
 }
 
+// The same for the MFMA kernels, whose results are rounded to bfloat16: the tanh form as
+// v / (1 + 2^(-2 log2(e) u)) with the hardware's exponential and reciprocal (a dozen instructions
+// where tanhf takes several dozen; after a product of 2048 x 6400 the difference was 10 us of 65).
+__device__ __forceinline__ float apply_epilogue_fast(float v, int epi) {
+  if (epi == EPI_GELU_TANH) {
+    const float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+    return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-2.8853900817779268f * u));
+  }
+  if (epi == EPI_GELU_ERF) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+  return v;
+}
+
 // Where a fused projection's key and value columns go besides C: columns q_width .. of row m are
 // the keys, then the values, of the token whose slot is slot_map[m] (page * page_size + offset,
 // < 0: none).  Pools as in the cache: keys [page, Hkv, page_size, dh], values [page, Hkv, dh, page_size].
@@ -303,7 +315,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
       if (resid) {
         resid[static_cast<size_t>(m) * ldr + nn] = epi_x[p][r] + v;
       } else {
-        TC cv = from_float<TC>(apply_epilogue(v, epi));
+        TC cv = from_float<TC>(apply_epilogue_fast(v, epi));
         if (!KV || nn < kv.c_cols)
           C[(packed & PACKED_C) ? packed_index(m, nn, N / 32) : static_cast<size_t>(m) * ldc + nn] = cv;
         if constexpr (KV) scatter_kv(kv, m, nn, cv);
@@ -409,7 +421,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
       if (resid) {
         resid[static_cast<size_t>(m) * ldr + nn] = epi_x[r] + v;
       } else {
-        const TC cv = from_float<TC>(apply_epilogue(v, epi));
+        const TC cv = from_float<TC>(apply_epilogue_fast(v, epi));
         if (!KV || nn < kv.c_cols) C[static_cast<size_t>(m) * ldc + nn] = cv;
         if constexpr (KV) scatter_kv(kv, m, nn, cv);
       }
@@ -653,7 +665,7 @@ __global__ __launch_bounds__(WM * 128) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const float v = acc[i][j][r] + bv;
-          piece[(8 * (r / 4) + 4 * g + (r % 4)) * RS + r32] = resid ? v : apply_epilogue(v, epi);
+          piece[(8 * (r / 4) + 4 * g + (r % 4)) * RS + r32] = resid ? v : apply_epilogue_fast(v, epi);
         }
         if constexpr (KV) {
           // A block of value columns: a value's place in its page is [dim][offset], so four rows
@@ -730,7 +742,7 @@ __global__ __launch_bounds__(WM * 128) __attribute__((amdgpu_waves_per_eu(2))) v
           float* x = resid + static_cast<size_t>(m) * ldr + n;
           *x = *x + v;
         } else {
-          const TC cv = from_float<TC>(apply_epilogue(v, epi));
+          const TC cv = from_float<TC>(apply_epilogue_fast(v, epi));
           if (!KV || n < kv.c_cols) C[static_cast<size_t>(m) * ldc + n] = cv;
           if constexpr (KV) scatter_kv(kv, m, n, cv);
         }
@@ -786,6 +798,242 @@ static int run(const void* A, int lda, const void* W, const float* bias, void* C
 }
 }  // namespace tiled
 
+// ---------------------------------------------------------------------------------------
+// Many rows, bfloat16, slabs carried from memory straight into LDS (global_load_lds_dwordx4: 16
+// bytes per lane, lane l's at the wave's LDS address + 16 l, no register and no LDS store between).
+// A slab of 32 along K is a list of 1 KB blocks in the packed layout, 16 rows x 32 columns each:
+// a block of W is 1 KB of memory as it lies; a block of A is made by the load itself (lane
+// l fetches the 16 bytes at row l % 16, column 8 (l / 16) of the block, which puts them where
+// v_mfma_f32_16x16x32_bf16 wants them).  A wave's operand read is then one ds_read_b128 per
+// block at 16 l: no swizzle, no bank shared.  STAGES slabs are in flight (vmcnt counts a wave's
+// own loads; one barrier per slab publishes them and frees the slab read before).
+//
+// The MFMA takes W as its first operand and A as its second: a lane then holds four consecutive
+// columns of one row of C, which it stores as 8 bytes (bfloat16) or adds as 16 (the 32-bit
+// residual) without a turn through LDS; for the fused QKV product they are one key's or one
+// value's four dims.
+//
+// What bounds these products here is the traffic from L2 into the CUs and the rounding of tiles to
+// 256 CUs, not the matrix cores: measured per tile and slab, time = 2.26e-7 us x BM x BN (matrix
+// cores at nine tenths of their peak) + 3.07e-5 us x (BM + BN) (loads), the two adding up rather
+// than overlapping, + 1.9e-4 us x BM x BN for the stores at the end.  So the tile is chosen per
+// product from a list, by that model: the largest that still fills the chip in whole rounds
+// (2048 x 4800 x 1600: 256 x 160 tiles are 240 workgroups, one round, 42 us where 256 x 128 tiles
+// took two rounds and 59 us; 2048 x 6400: 256 x 224, 53 against 66 us).
+// ---------------------------------------------------------------------------------------
+namespace direct {
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+constexpr int XCDS = 8, CUS = 256, LDS_PER_CU = 160 * 1024;
+
+// not a template: the host pass must not see the builtin inside one
+__device__ __forceinline__ void load_to_lds(const void* src, void* dst) {
+  __builtin_amdgcn_global_load_lds(src, dst, 16, 0, 0);
+}
+
+template <int N>
+__device__ __forceinline__ void wait_loads() {      // until at most N of this wave's loads are in flight
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// WM x WN waves, each TM x TN blocks of 16 x 16: the tile is 16 WM TM rows x 16 WN TN columns
+template <typename TC, int WM, int WN, int TM, int TN, int STAGES, bool KV>
+__global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __restrict__ A, int lda,
+                                                           const bf16_t* __restrict__ W, const float* __restrict__ bias,
+                                                           TC* __restrict__ C, int ldc, float* __restrict__ resid, int ldr,
+                                                           int M, int N, int K, int epi, int tiles_m, int tiles_n,
+                                                           KVScatter kv) {
+  constexpr int NW = WM * WN;
+  constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
+  constexpr int AB = BM / 16, WB = BN / 16;              // 1 KB blocks per slab
+  constexpr int SLAB = (AB + WB) * 64;                   // in u32x4
+  constexpr int HI = (AB + WB + NW - 1) / NW, REM = (AB + WB) % NW;   // waves below REM load HI blocks, the others HI - 1
+  static_assert((STAGES - 2) * HI < 64, "vmcnt has six bits");
+  extern __shared__ u32x4 lds[];
+  const int total = tiles_m * tiles_n;
+  int pid = blockIdx.x;
+  if (total % XCDS == 0) pid = (pid % XCDS) * (total / XCDS) + pid / XCDS;   // an XCD walks down a column of tiles
+  const int tm = pid % tiles_m, tn = pid / tiles_m;
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int lane = threadIdx.x % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+  const int wmb = (wave / WN) * TM, wnb = (wave % WN) * TN;     // in blocks
+  const int ksteps = K / 32, nblocks = (N + 15) / 16;
+
+  floatx4 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // where this lane's share of each of the wave's blocks starts; a row beyond M or a block of
+  // columns beyond N is replaced by the last inside (its results are not stored)
+  const bf16_t* src[HI];
+  int step[HI];
+#pragma unroll
+  for (int u = 0; u < HI; ++u) {
+    const int b = min(wave + u * NW, AB + WB - 1);
+    if (b < AB) {
+      src[u] = A + static_cast<size_t>(min(m0 + b * 16 + lane % 16, M - 1)) * lda + (lane / 16) * 8;
+      step[u] = 32;
+    } else {
+      src[u] = W + static_cast<size_t>(min(n0 / 16 + b - AB, nblocks - 1)) * ksteps * 512 + lane * 8;
+      step[u] = 512;
+    }
+  }
+  auto issue = [&](int kt) {
+    u32x4* slab = lds + (kt % STAGES) * SLAB;
+#pragma unroll
+    for (int u = 0; u < HI; ++u) {
+      const int b = wave + u * NW;
+      if (u < HI - 1 || REM == 0 || wave < REM) load_to_lds(src[u] + static_cast<size_t>(kt) * step[u], slab + b * 64);
+    }
+  };
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s)
+    if (s < ksteps) issue(s);
+  for (int kt = 0; kt < ksteps; ++kt) {
+    // slab kt of this wave has landed when only the loads of the STAGES - 2 slabs after it are out
+    if (kt + STAGES - 2 < ksteps) {
+      if (REM == 0 || wave < REM)
+        wait_loads<(STAGES - 2) * HI>();
+      else
+        wait_loads<(STAGES - 2) * (HI - 1)>();
+    } else {
+      wait_loads<0>();
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();      // every wave's share of slab kt is there, and slab kt - 1 has been read
+    if (kt + STAGES - 1 < ksteps) issue(kt + STAGES - 1);
+    const u32x4* slab = lds + (kt % STAGES) * SLAB;
+    bf16x8 af[TM], wf[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[i] = __builtin_bit_cast(bf16x8, slab[(wmb + i) * 64 + lane]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) wf[j] = __builtin_bit_cast(bf16x8, slab[(AB + wnb + j) * 64 + lane]);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], af[i], acc[i][j], 0, 0, 0);
+  }
+  // acc[i][j][r]: row m0 + 16 (wmb + i) + lane % 16, column n0 + 16 (wnb + j) + 4 (lane / 16) + r
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + (wnb + j) * 16 + (lane / 16) * 4;
+    if (n >= N) continue;
+    const floatx4 bv = bias ? *reinterpret_cast<const floatx4*>(bias + n) : floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int m = m0 + (wmb + i) * 16 + lane % 16;
+      if (m >= M) continue;
+      const floatx4 v = acc[i][j] + bv;
+      if (resid) {
+        floatx4* x = reinterpret_cast<floatx4*>(resid + static_cast<size_t>(m) * ldr + n);
+        *x = *x + v;
+      } else if constexpr (sizeof(TC) == 4) {
+        floatx4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = apply_epilogue_fast(v[r], epi);
+        *reinterpret_cast<floatx4*>(C + static_cast<size_t>(m) * ldc + n) = o;
+      } else {
+        alignas(8) bf16_t cv[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) cv[r] = from_float<bf16_t>(apply_epilogue_fast(v[r], epi));
+        if (!KV || n < kv.c_cols)
+          *reinterpret_cast<uint2*>(C + static_cast<size_t>(m) * ldc + n) = *reinterpret_cast<const uint2*>(cv);
+        if constexpr (KV) scatter_kv4(kv, m, n, cv);
+      }
+    }
+  }
+}
+
+// everything 16 bytes at a time: slabs of 32 along K, rows of A and C (or the residual) and the bias
+static bool takes(const void* A, int lda, const void* W, const float* bias, const void* C, int ldc, const float* resid,
+                  int ldr, int N, int K, int out_dtype) {
+  auto aligned = [](const void* p, int a) { return reinterpret_cast<uintptr_t>(p) % a == 0; };
+  if (K % 32 != 0 || lda % 8 != 0 || N % 4 != 0 || !aligned(A, 16) || !aligned(W, 16) || !aligned(bias, 16)) return false;
+  if (resid) return ldr % 4 == 0 && aligned(resid, 16);
+  return ldc % 4 == 0 && aligned(C, out_dtype == DN_F32 ? 16 : 8);
+}
+
+struct Args {
+  const void* A; int lda; const void* W; const float* bias; void* C; int ldc; float* resid; int ldr;
+  int M, N, K, out_dtype, epi; const KVScatter* kv;
+};
+
+template <typename TC, int WM, int WN, int TM, int TN, int STAGES, bool KV>
+static int launch(const Args& a, hipStream_t stream) {
+  constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
+  const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
+  constexpr size_t lds = static_cast<size_t>(STAGES) * (BM + BN) / 16 * 1024;
+  static bool raised = false;      // more than 64 KB of LDS has to be asked for once per kernel
+  if (lds > 65536 && !raised) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<TC, WM, WN, TM, TN, STAGES, KV>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (e != hipSuccess) return static_cast<int>(e);
+    raised = true;
+  }
+  hipLaunchKernelGGL((gemm_kernel<TC, WM, WN, TM, TN, STAGES, KV>), dim3(tiles_m * tiles_n), dim3(WM * WN * 64), lds,
+                     stream, static_cast<const bf16_t*>(a.A), a.lda, static_cast<const bf16_t*>(a.W), a.bias,
+                     static_cast<TC*>(a.C), a.ldc, a.resid, a.ldr, a.M, a.N, a.K, a.epi, tiles_m, tiles_n,
+                     a.kv ? *a.kv : KVScatter{});
+  return 0;
+}
+
+template <int WM, int WN, int TM, int TN, int STAGES>
+static int launch_as(const Args& a, hipStream_t stream) {
+  if (a.kv) return launch<bf16_t, WM, WN, TM, TN, STAGES, true>(a, stream);
+  if (a.out_dtype == DN_BF16 && !a.resid) return launch<bf16_t, WM, WN, TM, TN, STAGES, false>(a, stream);
+  return launch<float, WM, WN, TM, TN, STAGES, false>(a, stream);
+}
+
+// The tiles on offer: rows x columns, slabs in flight.  256 rows: 8 waves as 4 x 2, one workgroup
+// per CU; the two small ones leave room for two and three workgroups per CU.
+struct Shape { int bm, bn, stages; };
+constexpr Shape SHAPES[] = {{64, 128, 4}, {128, 128, 4}, {256, 128, 4}, {256, 160, 4}, {256, 192, 4},
+                            {256, 224, 4}, {256, 256, 4}, {256, 320, 3}};
+
+static double model_us(const Shape& s, int M, int N, int K) {
+  const double tiles = static_cast<double>((M + s.bm - 1) / s.bm) * ((N + s.bn - 1) / s.bn);
+  const size_t lds = static_cast<size_t>(s.stages) * (s.bm + s.bn) / 16 * 1024;
+  // two workgroups that share a CU hide some of each other's waits (measured: 1.5 to 1.8 times one's time for two rounds)
+  const double whole = static_cast<double>((static_cast<long>(tiles) + CUS - 1) / CUS);
+  const double rounds = 2 * lds <= LDS_PER_CU && whole > 1 ? 0.9 * whole : whole;
+  const double area = static_cast<double>(s.bm) * s.bn;
+  return rounds * (K * (2.26e-7 * area + 3.07e-5 * (s.bm + s.bn)) + 1.9e-4 * area);
+}
+
+static int pick(int M, int N, int K) {
+  int best = 0;
+  double best_us = 1e30;
+  for (int i = 0; i < static_cast<int>(sizeof(SHAPES) / sizeof(SHAPES[0])); ++i) {
+    const double us = model_us(SHAPES[i], M, N, K);
+    if (us < best_us) best_us = us, best = i;
+  }
+  return best;
+}
+
+static int run(const Args& a, hipStream_t stream) {
+  switch (pick(a.M, a.N, a.K)) {
+    case 0: return launch_as<2, 2, 2, 4, 4>(a, stream);
+    case 1: return launch_as<4, 2, 2, 4, 4>(a, stream);
+    case 2: return launch_as<4, 2, 4, 4, 4>(a, stream);
+    case 3: return launch_as<4, 2, 4, 5, 4>(a, stream);
+    case 4: return launch_as<4, 2, 4, 6, 4>(a, stream);
+    case 5: return launch_as<4, 2, 4, 7, 4>(a, stream);
+    case 6: return launch_as<4, 2, 4, 8, 4>(a, stream);
+    default: return launch_as<4, 2, 4, 10, 3>(a, stream);
+  }
+}
+}  // namespace direct
+
+// the tile that a product of these sizes gets from the kernel above: rows * 1000 + columns
+extern "C" int dn_gemm_tile(int M, int N, int K) {
+  const direct::Shape& s = direct::SHAPES[direct::pick(M, N, K)];
+  return s.bm * 1000 + s.bn;
+}
+
 // packed: bit flags.  W in rows of K elements (the plain kernel, any dtype), or packed bfloat16
 // (PACKED_W 1: the MFMA kernels, which need A in bfloat16 and loadable 16 bytes at a time).  With
 // at most 256 rows A may be packed too (PACKED_A 2; lda is not read) and so may a bfloat16 C
@@ -808,7 +1056,11 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
     }
     if (packed & (PACKED_A | PACKED_C)) return DN_ERR_SHAPE;
     if (!tiled::takes(A, lda, W, K)) return DN_ERR_SHAPE;
-    int rc = tiled::run(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr, stream);
+    int rc;
+    if (direct::takes(A, lda, W, bias, C, ldc, resid, ldr, N, K, out_dtype))
+      rc = direct::run(direct::Args{A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr}, stream);
+    else
+      rc = tiled::run(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr, stream);
     return rc != 0 ? rc : dn_launch_status();
   }
   dim3 grid((N + plain::BN - 1) / plain::BN, (M + plain::BM - 1) / plain::BM), block(256);
@@ -850,7 +1102,11 @@ extern "C" int dn_gemm_qkv(const void* A, int lda, const void* W, const float* b
     skinny::run(c, stream);
     return dn_launch_status();
   }
-  int rc = tiled::run(A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv, stream);
+  int rc;
+  if (direct::takes(A, lda, W, bias, C, ldc, nullptr, 0, N, K, DN_BF16))
+    rc = direct::run(direct::Args{A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv}, stream);
+  else
+    rc = tiled::run(A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv, stream);
   return rc != 0 ? rc : dn_launch_status();
 }
 

@@ -112,7 +112,39 @@ def test_linear(in_dtype, M, N, K):
         assert torch.allclose(out, exact("none"), **tol)
 
 
-@pytest.mark.parametrize("M", [1, 8, 20, 64, 70, 300])
+def test_linear_with_every_tile_of_the_many_rows_kernel():
+    """Beyond 256 rows the tile is chosen per product from a list: every tile on the list, on sizes
+    that are no multiple of it, with a short K (fewer slabs than the kernel keeps in flight) and a
+    longer one, for each kind of output."""
+    o = ops()
+    tile = o._lib("gemm").dn_gemm_tile
+    cases = {}
+    for K in (64, 416):             # per tile the smallest product that gets it
+        for M in range(260, 4200, 140):
+            for N in range(136, 10000, 232):
+                t = tile(M, N, K)
+                if t not in cases or M * N < cases[t][0] * cases[t][1]:
+                    cases[t] = (M, N, K)
+    assert len(cases) == 8, sorted(cases)
+    tol = dict(TOL[torch.bfloat16])
+    for M, N, K in cases.values():
+        a, w, bias = rnd(M, K, seed=1, dtype=torch.bfloat16), rnd(N, K, seed=2, dtype=torch.bfloat16, scale=0.2), rnd(N, seed=3)
+        wp = o.pack_matrix(w)
+        exact = (a.double() @ w.double().t() + bias.double()).float()
+        for out_dtype in (torch.float32, torch.bfloat16):
+            out = torch.empty(M, N, dtype=out_dtype, device=DEV)
+            o.linear(a, wp, bias, out=out)
+            assert torch.allclose(out.float(), exact, **tol), (M, N, K, out_dtype)
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        o.linear(a, wp, bias, out=out, epilogue="gelu_tanh")
+        assert torch.allclose(out.float(), torch.nn.functional.gelu(exact, approximate="tanh"), **tol), (M, N, K)
+        res = rnd(M, N, seed=4)
+        want = res + exact
+        o.linear(a, wp, bias, residual=res)
+        assert torch.allclose(res, want, **tol), (M, N, K)
+
+
+@pytest.mark.parametrize("M", [1, 8, 20, 64, 70, 300, 1000])
 @pytest.mark.parametrize("slots_in", ["any order", "runs"])
 @pytest.mark.parametrize("queries_only", [False, True])
 def test_linear_qkv_writes_the_cache(M, slots_in, queries_only):
@@ -121,12 +153,12 @@ def test_linear_qkv_writes_the_cache(M, slots_in, queries_only):
     prompt's portion has them: runs of consecutive slots (the tiled kernel then stores a dim's
     values of four tokens at once), starting anywhere.  The output holds all columns, or the
     queries alone."""
-    H, Hkv, dh, ps, n_pages, K = 6, 2, 32, 16, 40, 96
+    H, Hkv, dh, ps, n_pages, K = 6, 2, 32, 16, max(40, (M + 101) // 16 + 1), 96
     N = (H + 2 * Hkv) * dh
     a, w, bias = rnd(M, K, seed=1, dtype=torch.bfloat16), rnd(N, K, seed=2, dtype=torch.bfloat16, scale=0.2), rnd(N, seed=3)
     g = torch.Generator().manual_seed(M)
     if slots_in == "runs":
-        starts, slots = [8, 10, 40, 101], []     # disjoint for 300 rows; the first and third run start 4-aligned
+        starts, slots = [8, 10, 40, 101], []     # the first and third run start 4-aligned
         for i in range(M):
             slots.append(starts[i * 4 // max(M, 1)] + i)       # four runs
         slots = torch.tensor(slots, dtype=torch.int32)

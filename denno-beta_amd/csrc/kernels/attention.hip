@@ -219,7 +219,9 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
   constexpr int BYTES_TILES = 2 * GROUPS * TSZ * 2, BYTES_JOIN = GROUPS > 1 ? 4 * 64 * JOIN * 4 : 0;
   __shared__ __attribute__((aligned(16))) unsigned char smem[BYTES_TILES > BYTES_JOIN ? BYTES_TILES : BYTES_JOIN];
   bf16_t* const tiles_lds = reinterpret_cast<bf16_t*>(smem);      // [2 steps][GROUPS][keys | values]
-  const int tile = blockIdx.x, h = blockIdx.y;
+  // workgroups start in the order of the tile table, all heads of a tile together: the table lists
+  // the tiles with the longest contexts first, so the longest work is not what starts last
+  const int h = blockIdx.x, tile = blockIdx.y;
   const int seq = tile_seq[tile];
   if (seq < 0) return;                       // the whole workgroup
   const int row0 = tile_row0[tile], nrows = tile_nrows[tile], pos0 = tile_pos0[tile];
@@ -462,7 +464,8 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
   // 128 rows after 896: 40 -> 29 us); with more workgroups the SIMDs are busy and the second
   // group's share of carrying tiles only adds work (2 x 1024 rows: 52 -> 66 us).  Up to a head
   // size of 64: beyond, the tiles of two groups do not fit 64 KB of LDS.
-  dim3 grid(n_tiles, H);
+  if (n_tiles > 65535) return DN_ERR_SHAPE;      // the grid's second dimension
+  dim3 grid(H, n_tiles);
   const bool two = static_cast<long>(n_tiles) * H <= 256;
 #define DN_FLASH_G(D, G)                                                                                          \
   hipLaunchKernelGGL((flash::kernel<D, G>), grid, dim3(256 * G), 0, stream, static_cast<const bf16_t*>(q), ldq,   \

@@ -802,10 +802,12 @@ static int run(const void* A, int lda, const void* W, const float* bias, void* C
 // Many rows, bfloat16, slabs carried from memory straight into LDS (global_load_lds_dwordx4: 16
 // bytes per lane, lane l's at the wave's LDS address + 16 l, no register and no LDS store between).
 // A slab of 32 along K is a list of 1 KB blocks in the packed layout, 16 rows x 32 columns each:
-// a block of W is 1 KB of memory as it lies; a block of A is made by the load itself (lane
-// l fetches the 16 bytes at row l % 16, column 8 (l / 16) of the block, which puts them where
-// v_mfma_f32_16x16x32_bf16 wants them).  A wave's operand read is then one ds_read_b128 per
-// block at 16 l: no swizzle, no bank shared.  STAGES slabs are in flight (vmcnt counts a wave's
+// a block of W is 1 KB of memory as it lies and is read back at 16 l by lane l; a block of A is
+// made by the load itself, in an order of its own: the vector cache looks a load's lines up per 16
+// lanes, so 16 lanes take 64 bytes from each of four rows (four lines) and not 16 bytes from each of
+// sixteen (with a lane per row the lookups, 52 per load on average, kept the cache busy for three
+// quarters of the kernel's time), and the four 16-byte pieces of a row are exchanged by the row's
+// number so that the operand read (lane l wants row l % 16, piece l / 16) meets every bank once.  STAGES slabs are in flight (vmcnt counts a wave's
 // own loads; one barrier per slab publishes them and frees the slab read before).
 //
 // The MFMA takes W as its first operand and A as its second: a lane then holds four consecutive
@@ -860,6 +862,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
   const int wmb = (wave / WN) * TM, wnb = (wave % WN) * TN;     // in blocks
   const int ksteps = K / 32, nblocks = (N + 15) / 16;
+  // where the 16 bytes of row lane % 16, columns 8 (lane / 16) .. of a block of A lie in its 1 KB
+  // (see the loads below): any 8 and any 16 consecutive lanes read all banks once
+  const int aslot = 16 * (lane % 4) + 4 * ((lane % 16) / 4) + ((lane / 16) ^ (lane % 4));
 
   floatx4 acc[TM][TN];
 #pragma unroll
@@ -875,7 +880,10 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
   for (int u = 0; u < HI; ++u) {
     const int b = min(wave + u * NW, AB + WB - 1);
     if (b < AB) {
-      src[u] = A + static_cast<size_t>(min(m0 + b * 16 + lane % 16, M - 1)) * lda + (lane / 16) * 8;
+      // 16 lanes in a row take 64 bytes from each of four rows (g, g + 4, g + 8, g + 12 of the block):
+      // four cache lines, where a lane per row would touch sixteen
+      const int g = lane / 16, h = (lane % 16) / 4, piece = (lane % 4) ^ g;
+      src[u] = A + static_cast<size_t>(min(m0 + b * 16 + 4 * h + g, M - 1)) * lda + piece * 8;
       step[u] = 32;
     } else {
       src[u] = W + static_cast<size_t>(min(n0 / 16 + b - AB, nblocks - 1)) * ksteps * 512 + lane * 8;
@@ -909,7 +917,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
     const u32x4* slab = lds + (kt % STAGES) * SLAB;
     bf16x8 af[TM], wf[TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) af[i] = __builtin_bit_cast(bf16x8, slab[(wmb + i) * 64 + lane]);
+    for (int i = 0; i < TM; ++i) af[i] = __builtin_bit_cast(bf16x8, slab[(wmb + i) * 64 + aslot]);
 #pragma unroll
     for (int j = 0; j < TN; ++j) wf[j] = __builtin_bit_cast(bf16x8, slab[(AB + wnb + j) * 64 + lane]);
 #pragma unroll

@@ -89,6 +89,9 @@ def plan_rows(entries: Sequence[StepEntry], starts: Sequence[int], vocab: int, m
         for i in range(0, n, WIDE_TILE_ROWS):
             wide.append((s, row0 + i, min(WIDE_TILE_ROWS, n - i), start + i))
         row_start.append(row0 + n)
+    # a tile's work grows with the keys before its last row: the kernel starts workgroups in this
+    # order, the longest first (with the shortest last, the chip runs empty evenly)
+    wide.sort(key=lambda t: -(t[3] + t[2]))
     return tokens, positions, logit_rows, row_start, tiles, wide
 
 

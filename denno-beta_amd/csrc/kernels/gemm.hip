@@ -684,7 +684,7 @@ __global__ __launch_bounds__(WM * 128) __attribute__((amdgpu_waves_per_eu(2))) v
                 slot[e] = m + e < M ? kv.slot_map[m + e] : -1;
               }
               if (nb + r32 >= N) continue;
-              const bool run = slot[0] >= 0 && slot[0] % 4 == 0 && slot[1] == slot[0] + 1 && slot[2] == slot[0] + 2 &&
+              const bool run = kv.page_size % 4 == 0 && slot[0] >= 0 && slot[0] % 4 == 0 && slot[1] == slot[0] + 1 && slot[2] == slot[0] + 2 &&
                                slot[3] == slot[0] + 3;
               if (run) {
                 const int page = slot[0] / kv.page_size, off = slot[0] % kv.page_size;
@@ -834,6 +834,21 @@ __device__ __forceinline__ void load_to_lds(const void* src, void* dst) {
   __builtin_amdgcn_global_load_lds(src, dst, 16, 0, 0);
 }
 
+// element `which` (0..3, the lane's own choice) of the vector that lane E of this lane's quad holds
+template <int E>
+__device__ __forceinline__ float quad_pick(const floatx4& v, int which) {
+  const float b0 = dpp_move<0x55 * E>(v[0]), b1 = dpp_move<0x55 * E>(v[1]), b2 = dpp_move<0x55 * E>(v[2]),
+              b3 = dpp_move<0x55 * E>(v[3]);
+  return which == 0 ? b0 : which == 1 ? b1 : which == 2 ? b2 : b3;
+}
+
+// four values rounded to bfloat16, as the 8 bytes of one store (built in registers: an array that
+// is read back through a pointer of another type can end up in scratch memory)
+__device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
+  return uint2{static_cast<uint32_t>(from_float<bf16_t>(a).bits) | static_cast<uint32_t>(from_float<bf16_t>(b).bits) << 16,
+               static_cast<uint32_t>(from_float<bf16_t>(c).bits) | static_cast<uint32_t>(from_float<bf16_t>(d).bits) << 16};
+}
+
 template <int N>
 __device__ __forceinline__ void wait_loads() {      // until at most N of this wave's loads are in flight
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -926,12 +941,54 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
       for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], af[i], acc[i][j], 0, 0, 0);
   }
   // acc[i][j][r]: row m0 + 16 (wmb + i) + lane % 16, column n0 + 16 (wnb + j) + 4 (lane / 16) + r
-#pragma unroll
+  //
+  // Where the fused projection's keys and values go is worked out once per row, outside the loop over
+  // the column blocks (a slot's page and offset are divisions by numbers known only at run time; done
+  // per block and lane they cost more than the product's own epilogue).  Keys: the lane's row.  Values:
+  // in its page a value lies as [dim][offset], so four tokens whose slots follow one another from a
+  // multiple of 4 are 8 bytes side by side for one dim: the four lanes of a quad, which hold four
+  // tokens x four dims, exchange them (a 4 x 4 turn), and each stores four tokens of one dim.
+  int kpage[KV ? TM : 1], koff[KV ? TM : 1], vpage[KV ? TM : 1], voff[KV ? TM : 1];
+  if constexpr (KV) {
+#pragma clang loop unroll(full)
+    for (int i = 0; i < TM; ++i) {
+      const int m = m0 + (wmb + i) * 16 + lane % 16, mq = m - lane % 4;
+      const int slot = m < M ? kv.slot_map[m] : -1;
+      kpage[i] = slot >= 0 ? slot / kv.page_size : -1;
+      koff[i] = slot >= 0 ? slot % kv.page_size : 0;
+      int sq[4];
+#pragma clang loop unroll(full)
+      for (int e = 0; e < 4; ++e) sq[e] = mq + e < M ? kv.slot_map[mq + e] : -1;
+      const bool run = kv.page_size % 4 == 0 && sq[0] >= 0 && sq[0] % 4 == 0 && sq[1] == sq[0] + 1 && sq[2] == sq[0] + 2 &&
+                       sq[3] == sq[0] + 3;
+      vpage[i] = run ? sq[0] / kv.page_size : -1;
+      voff[i] = run ? sq[0] % kv.page_size : 0;
+    }
+  }
+  // every load of the epilogue before its first store: a wait for a load is a wait for the stores
+  // issued before it as well (one counter), and a load per column block made the blocks take turns
+  floatx4 bvs[TN];
+#pragma clang loop unroll(full)
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + (wnb + j) * 16 + (lane / 16) * 4;
+    bvs[j] = bias && n < N ? *reinterpret_cast<const floatx4*>(bias + n) : floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+#pragma clang loop unroll(full)
   for (int j = 0; j < TN; ++j) {
     const int n = n0 + (wnb + j) * 16 + (lane / 16) * 4;
     if (n >= N) continue;
-    const floatx4 bv = bias ? *reinterpret_cast<const floatx4*>(bias + n) : floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
+    const floatx4 bv = bvs[j];
+    // the block's place among the keys or the values: head hh, dims d .. d + 3 (a block of 16 columns is
+    // all queries, all keys or all values, and of one head: the widths are multiples of 16)
+    bool is_key = false, is_value = false;
+    int hh = 0, d = 0;
+    if constexpr (KV) {
+      is_key = n >= kv.q_width && n < kv.q_width + kv.kv_width;
+      is_value = n >= kv.q_width + kv.kv_width;
+      const int c = n - kv.q_width - (is_value ? kv.kv_width : 0);
+      hh = c / kv.dh, d = c % kv.dh;
+    }
+#pragma clang loop unroll(full)
     for (int i = 0; i < TM; ++i) {
       const int m = m0 + (wmb + i) * 16 + lane % 16;
       if (m >= M) continue;
@@ -941,16 +998,43 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
         *x = *x + v;
       } else if constexpr (sizeof(TC) == 4) {
         floatx4 o;
-#pragma unroll
+#pragma clang loop unroll(full)
         for (int r = 0; r < 4; ++r) o[r] = apply_epilogue_fast(v[r], epi);
         *reinterpret_cast<floatx4*>(C + static_cast<size_t>(m) * ldc + n) = o;
       } else {
-        alignas(8) bf16_t cv[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) cv[r] = from_float<bf16_t>(apply_epilogue_fast(v[r], epi));
-        if (!KV || n < kv.c_cols)
-          *reinterpret_cast<uint2*>(C + static_cast<size_t>(m) * ldc + n) = *reinterpret_cast<const uint2*>(cv);
-        if constexpr (KV) scatter_kv4(kv, m, n, cv);
+        const uint2 cv = pack4(apply_epilogue_fast(v[0], epi), apply_epilogue_fast(v[1], epi), apply_epilogue_fast(v[2], epi),
+                               apply_epilogue_fast(v[3], epi));
+        if (!KV || n < kv.c_cols) *reinterpret_cast<uint2*>(C + static_cast<size_t>(m) * ldc + n) = cv;
+        if constexpr (KV) {
+          if (is_key && kpage[i] >= 0)
+            *reinterpret_cast<uint2*>(kv.k_pool + ((static_cast<size_t>(kpage[i]) * kv.Hkv + hh) * kv.page_size + koff[i]) * kv.dh +
+                                      d) = cv;
+        }
+      }
+    }
+    if constexpr (KV) {
+      if (is_value) {
+        const int q = lane % 4;       // this lane's dim of the four after the turn
+#pragma clang loop unroll(full)
+        for (int i = 0; i < TM; ++i) {
+          const int mq = m0 + (wmb + i) * 16 + (lane % 16) / 4 * 4;      // the quad's first token
+          const floatx4 v = acc[i][j] + bv;
+          // token mq + e, dim d + q: lane e of the quad holds it in v[q]
+          const float t0 = quad_pick<0>(v, q), t1 = quad_pick<1>(v, q), t2 = quad_pick<2>(v, q), t3 = quad_pick<3>(v, q);
+          if (vpage[i] >= 0) {
+            *reinterpret_cast<uint2*>(kv.v_pool + ((static_cast<size_t>(vpage[i]) * kv.Hkv + hh) * kv.dh + d + q) * kv.page_size +
+                                      voff[i]) = pack4(t0, t1, t2, t3);
+          } else {
+#pragma clang loop unroll(full)
+            for (int e = 0; e < 4; ++e) {
+              const int slot = mq + e < M ? kv.slot_map[mq + e] : -1;
+              if (slot < 0) continue;
+              const int page = slot / kv.page_size, off = slot % kv.page_size;
+              kv.v_pool[((static_cast<size_t>(page) * kv.Hkv + hh) * kv.dh + d + q) * kv.page_size + off] =
+                  from_float<bf16_t>(e == 0 ? t0 : e == 1 ? t1 : e == 2 ? t2 : t3);
+            }
+          }
+        }
       }
     }
   }

@@ -181,7 +181,9 @@ __device__ __forceinline__ __bf16 to_bf16(float f) { return static_cast<__bf16>(
 // what a wave does for one tile is a chain of dependent steps (scores, maximum, exponentials,
 // sum, values) of some thousand cycles whatever else runs, so a row's time is the number of
 // tiles its wave walks; two groups halve it, and join their running maxima, sums and weighted
-// values through LDS at the end, in group order.
+// values through LDS at the end, in group order.  With one group a wave takes two tiles per step
+// (up to a head size of 96: the tiles of two steps must fit 64 KB of LDS), under one maximum, one
+// sum and one rescaling (2 x 1024 rows: 58 -> 50 us).
 // A tile's keys and values come from the pages once per workgroup, 16 bytes per thread along
 // rows (two cache lines per 16 lanes), and lie in LDS for the four waves that need them, two
 // steps deep: the tiles of the step after the next are on their way to registers while this
@@ -199,7 +201,7 @@ namespace flash {
 constexpr int ROWS = 128;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
 
-template <int DH16, int GROUPS>
+template <int DH16, int GROUPS, int TPS>     // head size / 16; groups of 4 waves; tiles a wave takes per step
 __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2))) void kernel(
     const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
@@ -214,11 +216,11 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
   constexpr int KCH = 32 * CH, VCH = DH * 4; // chunks of a tile of keys, of values
   constexpr int KU = (KCH + 255) / 256, VU = (VCH + 255) / 256;
   constexpr int KSZ = 32 * KROW, TSZ = KSZ + DH * VROW;     // elements of a tile's keys, of a whole tile
-  constexpr int STEP = 32 * GROUPS;          // keys per step
+  constexpr int STEP = 32 * GROUPS * TPS;    // keys per step
   constexpr int JOIN = 2 + 16 * DB;          // floats a lane hands over at the end
-  constexpr int BYTES_TILES = 2 * GROUPS * TSZ * 2, BYTES_JOIN = GROUPS > 1 ? 4 * 64 * JOIN * 4 : 0;
+  constexpr int BYTES_TILES = 2 * GROUPS * TPS * TSZ * 2, BYTES_JOIN = GROUPS > 1 ? 4 * 64 * JOIN * 4 : 0;
   __shared__ __attribute__((aligned(16))) unsigned char smem[BYTES_TILES > BYTES_JOIN ? BYTES_TILES : BYTES_JOIN];
-  bf16_t* const tiles_lds = reinterpret_cast<bf16_t*>(smem);      // [2 steps][GROUPS][keys | values]
+  bf16_t* const tiles_lds = reinterpret_cast<bf16_t*>(smem);      // [2 steps][GROUPS][TPS][keys | values]
   // workgroups start in the order of the tile table, all heads of a tile together: the table lists
   // the tiles with the longest contexts first, so the longest work is not what starts last
   const int h = blockIdx.x, tile = blockIdx.y;
@@ -227,7 +229,7 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
   const int row0 = tile_row0[tile], nrows = tile_nrows[tile], pos0 = tile_pos0[tile];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int grp = wave / 4;                  // which tiles this wave multiplies
-  const int t = threadIdx.x % 256, ti = threadIdx.x / 256;   // this thread carries chunk t of the step's tile ti
+  const int t = threadIdx.x % 256, ti = threadIdx.x / 256;   // this thread carries chunk t of the step's tiles ti TPS ..
   const int wrow0 = (wave % 4) * 32;
   const bool has_rows = wrow0 < nrows;       // a wave without rows still carries tiles into LDS
   const int qcol = lane % 32, g = lane / 32;
@@ -260,21 +262,21 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
 
   // A tile of 32 keys lies in two pages (or in one, if pages are longer): pg[0] for keys
   // kt .. kt+15, pg[1] for kt+16 .. kt+31; -1 beyond the rows' last key.
-  auto pages_of = [&](int kt_, int* pg) {
-    pg[0] = kt_ <= hi_g ? bt[kt_ / page_size] : -1;
-    pg[1] = kt_ + 16 <= hi_g ? bt[(kt_ + 16) / page_size] : -1;
+  struct Pages { int a, b; };
+  auto pages_of = [&](int kt_) {
+    return Pages{kt_ <= hi_g ? bt[kt_ / page_size] : -1, kt_ + 16 <= hi_g ? bt[(kt_ + 16) / page_size] : -1};
   };
   // Thread t's share of its tile: chunk t (+ 256 u) of the keys, counted along a key's dims and
   // then from key to key, and of the values, counted along a dim's 16 keys of a page, then from
   // dim to dim, then the second run of 16.  Never a conditional load: what has no page reads the
   // pool's start and is stored as zeros.
-  u32x4 kreg[KU], vreg[VU];
-  auto fetch = [&](int kt_, const int* pg) {
+  u32x4 kregs[TPS][KU], vregs[TPS][VU];
+  auto fetch = [&](int kt_, const Pages pg, u32x4* kreg, u32x4* vreg) {
     const int off0 = kt_ % page_size, off1 = (kt_ + 16) % page_size;
 #pragma unroll
     for (int u = 0; u < KU; ++u) {
       const int idx = min(t + 256 * u, KCH - 1), key = idx / CH, ch = idx % CH;
-      const int page = key < 16 ? pg[0] : pg[1];
+      const int page = key < 16 ? pg.a : pg.b;
       const int off = (key < 16 ? off0 : off1) + key % 16;
       kreg[u] = *reinterpret_cast<const u32x4*>(
           k_pool + (page >= 0 ? ((static_cast<size_t>(page) * Hkv + hk) * page_size + off) * DH : 0) + ch * 8);
@@ -282,24 +284,24 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
     for (int u = 0; u < VU; ++u) {
       const int idx = min(t + 256 * u, VCH - 1), a0 = idx / (DH * 2), d = (idx % (DH * 2)) / 2, half = idx % 2;
-      const int page = pg[a0];
+      const int page = a0 ? pg.b : pg.a;
       vreg[u] = *reinterpret_cast<const u32x4*>(
           v_pool + (page >= 0 ? ((static_cast<size_t>(page) * Hkv + hk) * DH + d) * page_size + (a0 ? off1 : off0) : 0) +
           half * 8);
     }
   };
-  auto stash = [&](const int* pg, bf16_t* dst) {
+  auto stash = [&](const Pages pg, bf16_t* dst, const u32x4* kreg, const u32x4* vreg) {
 #pragma unroll
     for (int u = 0; u < KU; ++u) {
       const int idx = t + 256 * u, key = idx / CH, ch = idx % CH;
       if (idx < KCH)
-        *reinterpret_cast<u32x4*>(dst + key * KROW + ch * 8) = (key < 16 ? pg[0] : pg[1]) >= 0 ? kreg[u] : zero4;
+        *reinterpret_cast<u32x4*>(dst + key * KROW + ch * 8) = (key < 16 ? pg.a : pg.b) >= 0 ? kreg[u] : zero4;
     }
 #pragma unroll
     for (int u = 0; u < VU; ++u) {
       const int idx = t + 256 * u, a0 = idx / (DH * 2), d = (idx % (DH * 2)) / 2, half = idx % 2;
       if (idx < VCH)
-        *reinterpret_cast<u32x4*>(dst + KSZ + d * VROW + a0 * 16 + half * 8) = pg[a0] >= 0 ? vreg[u] : zero4;
+        *reinterpret_cast<u32x4*>(dst + KSZ + d * VROW + a0 * 16 + half * 8) = (a0 ? pg.b : pg.a) >= 0 ? vreg[u] : zero4;
     }
   };
 
@@ -307,78 +309,113 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
   // registers into the half of LDS that the step before read (every wave has left it: the
   // barrier), then asks for the tiles of step kt + 2 STEP, then multiplies.
   const int kt0 = (lo_g / STEP) * STEP;
-  const int mine = 32 * ti;                  // this thread carries the tile at kt + mine
-  int pg_now[2], pg_reg[2], pg_far[2];       // pages of the tile in registers and of the one to ask for next
-  pages_of(kt0 + mine, pg_now);
-  fetch(kt0 + mine, pg_now);
-  pages_of(kt0 + STEP + mine, pg_reg);
-  stash(pg_now, tiles_lds + ti * TSZ);
-  fetch(kt0 + STEP + mine, pg_reg);
-  pages_of(kt0 + 2 * STEP + mine, pg_far);
+  const int mine = 32 * TPS * ti;            // this thread carries the tiles at kt + mine + 32 c
+  Pages pg_now[TPS], pg_reg[TPS], pg_far[TPS];    // pages of the tiles in registers and of those to ask for next
+#pragma clang loop unroll(full)
+  for (int c = 0; c < TPS; ++c) {
+    pg_now[c] = pages_of(kt0 + mine + 32 * c);
+    fetch(kt0 + mine + 32 * c, pg_now[c], kregs[c], vregs[c]);
+    pg_reg[c] = pages_of(kt0 + STEP + mine + 32 * c);
+  }
+#pragma clang loop unroll(full)
+  for (int c = 0; c < TPS; ++c) {
+    stash(pg_now[c], tiles_lds + (ti * TPS + c) * TSZ, kregs[c], vregs[c]);
+    fetch(kt0 + STEP + mine + 32 * c, pg_reg[c], kregs[c], vregs[c]);
+    pg_far[c] = pages_of(kt0 + 2 * STEP + mine + 32 * c);
+  }
   __syncthreads();
   int buf = 0;
   for (int kt = kt0; kt <= hi_g; kt += STEP, buf ^= 1) {
-    if (kt + STEP <= hi_g) stash(pg_reg, tiles_lds + ((buf ^ 1) * GROUPS + ti) * TSZ);
-    if (kt + 2 * STEP <= hi_g) fetch(kt + 2 * STEP + mine, pg_far);
-    pg_reg[0] = pg_far[0], pg_reg[1] = pg_far[1];
-    pages_of(kt + 3 * STEP + mine, pg_far);
+#pragma clang loop unroll(full)
+    for (int c = 0; c < TPS; ++c) {
+      if (kt + STEP <= hi_g) stash(pg_reg[c], tiles_lds + (((buf ^ 1) * GROUPS + ti) * TPS + c) * TSZ, kregs[c], vregs[c]);
+      if (kt + 2 * STEP <= hi_g) fetch(kt + 2 * STEP + mine + 32 * c, pg_far[c], kregs[c], vregs[c]);
+      pg_reg[c] = pg_far[c];
+      pg_far[c] = pages_of(kt + 3 * STEP + mine + 32 * c);
+    }
 
-    const int kw = kt + 32 * grp;            // this wave's tile of the step
-    if (has_rows && kw <= hi_w && kw + 31 >= lo_w) {     // the same for the whole wave
-      const bf16_t* Kb = tiles_lds + (buf * GROUPS + grp) * TSZ;
-      const bf16_t* Vb = Kb + KSZ;
-      floatx16 s;
+    // this wave's tiles of the step: kw0 + 32 c.  They share one maximum, one sum and one rescaling:
+    // the chain of dependent steps (scores, maximum, exponentials, sum, values) is as long for two
+    // tiles as for one, and it is that chain, not the work, which a wave's time is made of
+    const int kw0 = kt + 32 * TPS * grp;
+    bool act[TPS], any = false;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) s[i] = 0.f;
+    for (int c = 0; c < TPS; ++c) {
+      act[c] = has_rows && kw0 + 32 * c <= hi_w && kw0 + 32 * c + 31 >= lo_w;     // the same for the whole wave
+      any = any || act[c];
+    }
+    if (any) {
+      const bf16_t* Tb = tiles_lds + (buf * GROUPS + grp) * TPS * TSZ;
+      floatx16 s[TPS];
 #pragma unroll
-      for (int c = 0; c < DH16; ++c) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Kb + qcol * KROW + (2 * c + g) * 8);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[c], s, 0, 0, 0);
+      for (int c = 0; c < TPS; ++c) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[c][i] = 0.f;
+        if (!act[c]) continue;
+        const bf16_t* Kb = Tb + c * TSZ;
+#pragma unroll
+        for (int cc = 0; cc < DH16; ++cc) {
+          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Kb + qcol * KROW + (2 * cc + g) * 8);
+          s[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[cc], s[c], 0, 0, 0);
+        }
       }
-      // s[i]: key kw + 8*(i/4) + 4*g + i%4, query = this lane's column.  Scores are kept times
+      // s[c][i]: key kw + 8*(i/4) + 4*g + i%4, query = this lane's column.  Scores are kept times
       // log2(e), so that each probability is one multiply-add and one v_exp_f32.  Only a tile that
       // touches the causal edge (or the window's) of one of the wave's rows needs the mask; the
       // others skip it, the same for the whole wave.
-      const bool edge = kw + 31 > pos0 + wrow0 || (window > 0 && kw < hi_w - window + 1);
       float tmax = NEG_INF;
-      if (edge) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          int key = kw + 8 * (i / 4) + 4 * g + (i % 4);
-          bool ok = key >= my_lo && key <= my_pos;
-          s[i] = ok ? s[i] * scale2 : NEG_INF;
-          tmax = fmaxf(tmax, s[i]);
-        }
-      } else {
+      for (int c = 0; c < TPS; ++c) {
+        const int kw = kw0 + 32 * c;
+        const bool edge = kw + 31 > pos0 + wrow0 || (window > 0 && kw < hi_w - window + 1);
+        if (!act[c]) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          s[i] *= scale2;
-          tmax = fmaxf(tmax, s[i]);
+          for (int i = 0; i < 16; ++i) s[c][i] = NEG_INF;
+        } else if (edge) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            int key = kw + 8 * (i / 4) + 4 * g + (i % 4);
+            bool ok = key >= my_lo && key <= my_pos;
+            s[c][i] = ok ? s[c][i] * scale2 : NEG_INF;
+            tmax = fmaxf(tmax, s[c][i]);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            s[c][i] *= scale2;
+            tmax = fmaxf(tmax, s[c][i]);
+          }
         }
       }
       tmax = fmaxf(tmax, other_half(tmax));
-      float p[16];
+      float p[TPS][16];
       float psum = 0.f, alpha = 1.f;
       if (tmax > NEG_INF) {
         float m_new = fmaxf(m, tmax);
         alpha = __builtin_amdgcn_exp2f(m - m_new);      // m = -inf at first: 2^-inf = 0
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          p[i] = __builtin_amdgcn_exp2f(s[i] - m_new);  // a masked score is -inf: 0
-          psum += p[i];
-        }
+        for (int c = 0; c < TPS; ++c)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            p[c][i] = __builtin_amdgcn_exp2f(s[c][i] - m_new);  // a masked score is -inf: 0
+            psum += p[c][i];
+          }
         m = m_new;
       } else {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) p[i] = 0.f;
+        for (int c = 0; c < TPS; ++c)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) p[c][i] = 0.f;
       }
       psum += other_half(psum);
       l = l * alpha + psum;
-      bf16x8 pb[2];
+      bf16x8 pb[TPS][2];
 #pragma unroll
-      for (int a0 = 0; a0 < 2; ++a0)
+      for (int c = 0; c < TPS; ++c)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) pb[a0][j] = to_bf16(p[8 * a0 + j]);
+        for (int a0 = 0; a0 < 2; ++a0)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) pb[c][a0][j] = to_bf16(p[c][8 * a0 + j]);
       // alpha belongs to the lane's query, and so do all of the lane's accumulators; once the running
       // maxima have settled it is 1 for the whole wave, tile after tile
       if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
@@ -389,15 +426,20 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
       }
       // values: as A operand the lane's row is a dim, its 8 k slots the keys 16 a0 + 4 g + {0..3, 8..11}
 #pragma unroll
-      for (int a0 = 0; a0 < 2; ++a0) {
-        if (kw + 16 * a0 > hi_w) continue;       // the same for every lane of the wave: all its probabilities are 0
+      for (int c = 0; c < TPS; ++c) {
+        if (!act[c]) continue;
+        const bf16_t* Vb = Tb + c * TSZ + KSZ;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const bf16_t* vr = Vb + min(32 * db + qcol, DH - 1) * VROW + 16 * a0 + 4 * g;
-          const bf16x4 vlo = *reinterpret_cast<const bf16x4*>(vr), vhi = *reinterpret_cast<const bf16x4*>(vr + 8);
-          bf16x8 vf = bf16x8{vlo[0], vlo[1], vlo[2], vlo[3], vhi[0], vhi[1], vhi[2], vhi[3]};
-          if (32 * db + qcol >= DH) vf = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[a0], o[db], 0, 0, 0);
+        for (int a0 = 0; a0 < 2; ++a0) {
+          if (kw0 + 32 * c + 16 * a0 > hi_w) continue;       // the same for every lane of the wave: all its probabilities are 0
+#pragma unroll
+          for (int db = 0; db < DB; ++db) {
+            const bf16_t* vr = Vb + min(32 * db + qcol, DH - 1) * VROW + 16 * a0 + 4 * g;
+            const bf16x4 vlo = *reinterpret_cast<const bf16x4*>(vr), vhi = *reinterpret_cast<const bf16x4*>(vr + 8);
+            bf16x8 vf = bf16x8{vlo[0], vlo[1], vlo[2], vlo[3], vhi[0], vhi[1], vhi[2], vhi[3]};
+            if (32 * db + qcol >= DH) vf = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[c][a0], o[db], 0, 0, 0);
+          }
         }
       }
     }
@@ -467,16 +509,16 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
   if (n_tiles > 65535) return DN_ERR_SHAPE;      // the grid's second dimension
   dim3 grid(H, n_tiles);
   const bool two = static_cast<long>(n_tiles) * H <= 256;
-#define DN_FLASH_G(D, G)                                                                                          \
-  hipLaunchKernelGGL((flash::kernel<D, G>), grid, dim3(256 * G), 0, stream, static_cast<const bf16_t*>(q), ldq,   \
+#define DN_FLASH_G(D, G, T)                                                                                        \
+  hipLaunchKernelGGL((flash::kernel<D, G, T>), grid, dim3(256 * G), 0, stream, static_cast<const bf16_t*>(q), ldq, \
                      static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),                          \
                      static_cast<const bf16_t*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0, tile_nrows, \
                      tile_pos0, H, Hkv, page_size, scale, window)
-#define DN_FLASH(D, G) \
-  if (G == 2 && two)   \
-    DN_FLASH_G(D, G);  \
-  else                 \
-    DN_FLASH_G(D, 1)
+#define DN_FLASH(D, G)    \
+  if (G == 2 && two)      \
+    DN_FLASH_G(D, G, 1);  \
+  else                    \
+    DN_FLASH_G(D, 1, (D <= 6 ? 2 : 1))
   switch (dh) {
     case 16: DN_FLASH(1, 2); break;
     case 32: DN_FLASH(2, 2); break;

@@ -2,13 +2,15 @@
 // [out, in], K contiguous for both operands.  Epilogues: bias, GELU (tanh or erf form),
 // or accumulation into the 32-bit residual stream (x += A.W^T + bias).
 //
-// Three kernels behind dn_gemm.  plain: 32-bit multiply-adds in a fixed order over K, whatever
+// Four kernels behind dn_gemm.  plain: 32-bit multiply-adds in a fixed order over K, whatever
 // M is, so a row's result does not depend on what else is in the batch; it is the whole 32-bit
 // path and takes bfloat16 operands too (converted exactly on load).  skinny: bfloat16, up to 256
 // rows, MFMA, waves split K, bound by reading W once (decode, and steps of a few short prompt
-// portions).  tiled: bfloat16, many rows, MFMA through LDS (prefill).
+// portions).  direct: bfloat16, many rows, MFMA, slabs from memory straight into LDS, the tile
+// chosen per product (prefill).  tiled: the same sizes through registers into swizzled LDS; it takes
+// what direct refuses (K no multiple of 32, rows or a bias that do not allow 16-byte accesses).
 //
-// The two MFMA kernels take W packed (dn_pack_matrix): blocks of 16 rows x 32 columns, block
+// The MFMA kernels take W packed (dn_pack_matrix): blocks of 16 rows x 32 columns, block
 // (n / 16, k / 32) at ((n / 16) * ceil(K / 32) + k / 32) * 512 elements, and inside a block the
 // 8 elements k % 32 / 8 * 8 .. + 7 of row n % 16 at ((k % 32 / 8) * 16 + n % 16) * 8: the 16 bytes
 // that lane (n % 16) + 16 * (k % 32 / 8) feeds to v_mfma_f32_16x16x32_bf16.  A wave then reads 1 KB

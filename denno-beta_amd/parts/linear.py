@@ -47,7 +47,7 @@ class Linear:
         (ops.packed_rows): whoever makes them asks here.  From 17 to 256 rows: a wave of the few-rows
         product then reads 1 KB in one piece where rows of the ordinary layout cost it 16 cache
         lines per 16 lanes (up to 16 rows its kernel loads along rows and turns them round in LDS;
-        beyond 256 the tiled kernel reads rows)."""
+        beyond 256 the many-rows kernels read rows)."""
         return self.few_rows(n_rows) and n_rows >= ops.PACKED_ROWS_MIN and self.in_features % 32 == 0
 
     def __call__(self, a, out_dtype=None, epilogue="none", residual=None, packed_out=False):

@@ -77,12 +77,12 @@ __device__ __forceinline__ void scatter_kv4(const KVScatter& kv, int m, int nn, 
   }
 }
 
-__device__ __forceinline__ void scatter_kv(const KVScatter& kv, int m, int nn, bf16_t cv) {
+// slot: the row's entry of the slot map (a kernel that ends with this asks for it when it starts)
+__device__ __forceinline__ void scatter_kv_at(const KVScatter& kv, int slot, int nn, bf16_t cv) {
   if (nn < kv.q_width) return;
   int c = nn - kv.q_width;
   const bool is_value = c >= kv.kv_width;
   if (is_value) c -= kv.kv_width;
-  const int slot = kv.slot_map[m];
   if (slot < 0) return;
   const int page = slot / kv.page_size, off = slot % kv.page_size;
   const int hh = c / kv.dh, d = c % kv.dh;
@@ -91,6 +91,10 @@ __device__ __forceinline__ void scatter_kv(const KVScatter& kv, int m, int nn, b
     kv.v_pool[base + static_cast<size_t>(d) * kv.page_size + off] = cv;
   else
     kv.k_pool[base + static_cast<size_t>(off) * kv.dh + d] = cv;
+}
+
+__device__ __forceinline__ void scatter_kv(const KVScatter& kv, int m, int nn, bf16_t cv) {
+  scatter_kv_at(kv, kv.slot_map[m], nn, cv);
 }
 
 namespace plain {
@@ -213,16 +217,28 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   // what the epilogue will read (bias, the residual stream) is asked for first of all
   float epi_bias[PASSES];
   float epi_x[PASSES][4];
+  int epi_slot[KV ? PASSES : 1][4];
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     const int blk = wave + p * WAVES;
     epi_bias[p] = 0.f;
 #pragma unroll
     for (int r = 0; r < 4; ++r) epi_x[p][r] = 0.f;
+    if constexpr (KV) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) epi_slot[p][r] = -1;
+    }
     if (blk < BLOCKS) {
       const int mb = blk / NB, nb = blk % NB;
       const int nn = min(n0 + nb * 16 + col, N - 1);
       if (bias) epi_bias[p] = bias[nn];
+      if constexpr (KV) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = mb * 16 + g * 4 + r;
+          epi_slot[p][r] = m < M ? kv.slot_map[m] : -1;
+        }
+      }
       if (resid) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -320,7 +336,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
         TC cv = from_float<TC>(apply_epilogue_fast(v, epi));
         if (!KV || nn < kv.c_cols)
           C[(packed & PACKED_C) ? packed_index(m, nn, N / 32) : static_cast<size_t>(m) * ldc + nn] = cv;
-        if constexpr (KV) scatter_kv(kv, m, nn, cv);
+        if constexpr (KV) scatter_kv_at(kv, epi_slot[p][r], nn, cv);
       }
     }
   }
@@ -353,9 +369,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
   // what the epilogue will read is asked for first of all (wave 0 finishes the block)
   float epi_bias = 0.f;
   float epi_x[4] = {0.f, 0.f, 0.f, 0.f};
+  int epi_slot[4] = {-1, -1, -1, -1};
   if (wave == 0) {
     const int nn = min(n0 + col, N - 1);
     if (bias) epi_bias = bias[nn];
+    if constexpr (KV) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) epi_slot[r] = g * 4 + r < M ? kv.slot_map[g * 4 + r] : -1;
+    }
     if (resid) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) epi_x[r] = resid[static_cast<size_t>(min(g * 4 + r, M - 1)) * ldr + nn];
@@ -425,7 +446,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
       } else {
         const TC cv = from_float<TC>(apply_epilogue_fast(v, epi));
         if (!KV || nn < kv.c_cols) C[static_cast<size_t>(m) * ldc + nn] = cv;
-        if constexpr (KV) scatter_kv(kv, m, nn, cv);
+        if constexpr (KV) scatter_kv_at(kv, epi_slot[r], nn, cv);
       }
     }
   }

@@ -1104,10 +1104,12 @@ static int launch_as(const Args& a, hipStream_t stream) {
 }
 
 // The tiles on offer: rows x columns, slabs in flight.  256 rows: 8 waves as 4 x 2, one workgroup
-// per CU; the two small ones leave room for two and three workgroups per CU.
+// per CU; the small ones leave room for several workgroups per CU.  64 x 64 and 32 x 64 (4 waves) are
+// for products with few rows and a long K, whose larger tiles would leave most CUs idle (512 x 1600 x
+// 6400: 50 -> 39 us; 300 rows: 50 -> 37 us).
 struct Shape { int bm, bn, stages; };
 constexpr Shape SHAPES[] = {{64, 128, 4}, {128, 128, 4}, {256, 128, 4}, {256, 160, 4}, {256, 192, 4},
-                            {256, 224, 4}, {256, 256, 4}, {256, 320, 3}};
+                            {256, 224, 4}, {256, 256, 4}, {256, 320, 3}, {64, 64, 4}, {32, 64, 4}};
 
 static double model_us(const Shape& s, int M, int N, int K) {
   const double tiles = static_cast<double>((M + s.bm - 1) / s.bm) * ((N + s.bn - 1) / s.bn);
@@ -1138,7 +1140,9 @@ static int run(const Args& a, hipStream_t stream) {
     case 4: return launch_as<4, 2, 4, 6, 4>(a, stream);
     case 5: return launch_as<4, 2, 4, 7, 4>(a, stream);
     case 6: return launch_as<4, 2, 4, 8, 4>(a, stream);
-    default: return launch_as<4, 2, 4, 10, 3>(a, stream);
+    case 7: return launch_as<4, 2, 4, 10, 3>(a, stream);
+    case 8: return launch_as<2, 2, 2, 2, 4>(a, stream);
+    default: return launch_as<2, 2, 1, 2, 4>(a, stream);
   }
 }
 }  // namespace direct

@@ -125,7 +125,7 @@ def test_linear_with_every_tile_of_the_many_rows_kernel():
                 t = tile(M, N, K)
                 if t not in cases or M * N < cases[t][0] * cases[t][1]:
                     cases[t] = (M, N, K)
-    assert len(cases) == 8, sorted(cases)
+    assert len(cases) == 10, sorted(cases)
     tol = dict(TOL[torch.bfloat16])
     for M, N, K in cases.values():
         a, w, bias = rnd(M, K, seed=1, dtype=torch.bfloat16), rnd(N, K, seed=2, dtype=torch.bfloat16, scale=0.2), rnd(N, seed=3)

@@ -882,8 +882,8 @@ template <typename TC, int WM, int WN, int TM, int TN, int STAGES, bool KV>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __restrict__ A, int lda,
                                                            const bf16_t* __restrict__ W, const float* __restrict__ bias,
                                                            TC* __restrict__ C, int ldc, float* __restrict__ resid, int ldr,
-                                                           int M, int N, int K, int epi, int tiles_m, int tiles_n,
-                                                           KVScatter kv) {
+                                                           int M, int N, int K, int epi, int packed, int tiles_m,
+                                                           int tiles_n, KVScatter kv) {
   constexpr int NW = WM * WN;
   constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
   constexpr int AB = BM / 16, WB = BN / 16;              // 1 KB blocks per slab
@@ -902,7 +902,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
   const int ksteps = K / 32, nblocks = (N + 15) / 16;
   // where the 16 bytes of row lane % 16, columns 8 (lane / 16) .. of a block of A lie in its 1 KB
   // (see the loads below): any 8 and any 16 consecutive lanes read all banks once
-  const int aslot = 16 * (lane % 4) + 4 * ((lane % 16) / 4) + ((lane / 16) ^ (lane % 4));
+  // (a packed A is in the operand's order already: lane l reads at 16 l)
+  const int aslot = (packed & PACKED_A) ? lane : 16 * (lane % 4) + 4 * ((lane % 16) / 4) + ((lane / 16) ^ (lane % 4));
 
   floatx4 acc[TM][TN];
 #pragma unroll
@@ -921,8 +922,13 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
       // 16 lanes in a row take 64 bytes from each of four rows (g, g + 4, g + 8, g + 12 of the block):
       // four cache lines, where a lane per row would touch sixteen
       const int g = lane / 16, h = (lane % 16) / 4, piece = (lane % 4) ^ g;
-      src[u] = A + static_cast<size_t>(min(m0 + b * 16 + 4 * h + g, M - 1)) * lda + piece * 8;
-      step[u] = 32;
+      if (packed & PACKED_A) {      // a block of packed rows is 1 KB as it lies, like a block of W
+        src[u] = A + static_cast<size_t>(min(m0 / 16 + b, (M + 15) / 16 - 1)) * ksteps * 512 + lane * 8;
+        step[u] = 512;
+      } else {
+        src[u] = A + static_cast<size_t>(min(m0 + b * 16 + 4 * h + g, M - 1)) * lda + piece * 8;
+        step[u] = 32;
+      }
     } else {
       src[u] = W + static_cast<size_t>(min(n0 / 16 + b - AB, nblocks - 1)) * ksteps * 512 + lane * 8;
       step[u] = 512;
@@ -1027,7 +1033,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
       } else {
         const uint2 cv = pack4(apply_epilogue_fast(v[0], epi), apply_epilogue_fast(v[1], epi), apply_epilogue_fast(v[2], epi),
                                apply_epilogue_fast(v[3], epi));
-        if (!KV || n < kv.c_cols) *reinterpret_cast<uint2*>(C + static_cast<size_t>(m) * ldc + n) = cv;
+        // (in packed rows, four columns from a multiple of 4 are 8 bytes side by side too)
+        if (!KV || n < kv.c_cols)
+          *reinterpret_cast<uint2*>(C + ((packed & PACKED_C) ? packed_index(m, n, N / 32) : static_cast<size_t>(m) * ldc + n)) = cv;
         if constexpr (KV) {
           if (is_key && kpage[i] >= 0)
             *reinterpret_cast<uint2*>(kv.k_pool + ((static_cast<size_t>(kpage[i]) * kv.Hkv + hh) * kv.page_size + koff[i]) * kv.dh +
@@ -1065,16 +1073,18 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
 
 // everything 16 bytes at a time: slabs of 32 along K, rows of A and C (or the residual) and the bias
 static bool takes(const void* A, int lda, const void* W, const float* bias, const void* C, int ldc, const float* resid,
-                  int ldr, int N, int K, int out_dtype) {
+                  int ldr, int N, int K, int out_dtype, int packed) {
   auto aligned = [](const void* p, int a) { return reinterpret_cast<uintptr_t>(p) % a == 0; };
-  if (K % 32 != 0 || lda % 8 != 0 || N % 4 != 0 || !aligned(A, 16) || !aligned(W, 16) || !aligned(bias, 16)) return false;
+  if (K % 32 != 0 || N % 4 != 0 || !aligned(A, 16) || !aligned(W, 16) || !aligned(bias, 16)) return false;
+  if (!(packed & PACKED_A) && lda % 8 != 0) return false;
   if (resid) return ldr % 4 == 0 && aligned(resid, 16);
+  if (packed & PACKED_C) return N % 32 == 0 && out_dtype == DN_BF16 && aligned(C, 8);
   return ldc % 4 == 0 && aligned(C, out_dtype == DN_F32 ? 16 : 8);
 }
 
 struct Args {
   const void* A; int lda; const void* W; const float* bias; void* C; int ldc; float* resid; int ldr;
-  int M, N, K, out_dtype, epi; const KVScatter* kv;
+  int M, N, K, out_dtype, epi, packed; const KVScatter* kv;
 };
 
 template <typename TC, int WM, int WN, int TM, int TN, int STAGES, bool KV>
@@ -1091,7 +1101,7 @@ static int launch(const Args& a, hipStream_t stream) {
   }
   hipLaunchKernelGGL((gemm_kernel<TC, WM, WN, TM, TN, STAGES, KV>), dim3(tiles_m * tiles_n), dim3(WM * WN * 64), lds,
                      stream, static_cast<const bf16_t*>(a.A), a.lda, static_cast<const bf16_t*>(a.W), a.bias,
-                     static_cast<TC*>(a.C), a.ldc, a.resid, a.ldr, a.M, a.N, a.K, a.epi, tiles_m, tiles_n,
+                     static_cast<TC*>(a.C), a.ldc, a.resid, a.ldr, a.M, a.N, a.K, a.epi, a.packed, tiles_m, tiles_n,
                      a.kv ? *a.kv : KVScatter{});
   return 0;
 }
@@ -1131,6 +1141,17 @@ static int pick(int M, int N, int K) {
   return best;
 }
 
+// Up to 256 rows the few-rows kernel takes the product too (both read and write packed rows).
+// Measured on GPT-2 XL's four products, few rows against many: 1600 -> 4800 with the cache write 13.9
+// / 14.0 us at 128 rows, 20.4 / 14.5 at 160 and 192, 27.8 / 19.7 at 256; 1600 -> 6400 with GELU 13.1 /
+// 12.9, 19.3 / 17.6, 23.5 / 18.0; the two that end in 1,600 columns stay with the few-rows kernel at
+// every size (8.8 / 11.6 and 26.8 / 37.4 us at 192 rows): 64-row tiles of so few columns leave most
+// CUs idle.
+static bool beats_few_rows(int M, int N, int K) {
+  (void)K;
+  return M > 128 && N >= 4096;
+}
+
 static int run(const Args& a, hipStream_t stream) {
   switch (pick(a.M, a.N, a.K)) {
     case 0: return launch_as<2, 2, 2, 4, 4>(a, stream);
@@ -1168,18 +1189,20 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
   if ((packed & PACKED_C) && (resid != nullptr || out_dtype != DN_BF16 || N % 32 != 0)) return DN_ERR_SHAPE;
   if (packed & PACKED_W) {
     if (in_dtype != DN_BF16) return DN_ERR_DTYPE;
-    if (skinny::takes(A, lda, W, M, K, packed)) {
+    const bool few = skinny::takes(A, lda, W, M, K, packed);
+    const bool many = direct::takes(A, lda, W, bias, C, ldc, resid, ldr, N, K, out_dtype, packed);
+    if (many && (!few || direct::beats_few_rows(M, N, K))) {
+      int rc = direct::run(direct::Args{A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, packed, nullptr}, stream);
+      return rc != 0 ? rc : dn_launch_status();
+    }
+    if (few) {
       skinny::Call c{A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, packed, nullptr};
       skinny::run(c, stream);
       return dn_launch_status();
     }
     if (packed & (PACKED_A | PACKED_C)) return DN_ERR_SHAPE;
     if (!tiled::takes(A, lda, W, K)) return DN_ERR_SHAPE;
-    int rc;
-    if (direct::takes(A, lda, W, bias, C, ldc, resid, ldr, N, K, out_dtype))
-      rc = direct::run(direct::Args{A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr}, stream);
-    else
-      rc = tiled::run(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr, stream);
+    int rc = tiled::run(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, nullptr, stream);
     return rc != 0 ? rc : dn_launch_status();
   }
   dim3 grid((N + plain::BN - 1) / plain::BN, (M + plain::BM - 1) / plain::BM), block(256);
@@ -1211,21 +1234,22 @@ extern "C" int dn_gemm_qkv(const void* A, int lda, const void* W, const float* b
   const int packed = PACKED_W | (a_packed ? PACKED_A : 0);
   if (K <= 0 || (lda < K && !a_packed)) return DN_ERR_SHAPE;
   const bool few = skinny::takes(A, lda, W, M, K, packed);
-  if (!few && (a_packed || !tiled::takes(A, lda, W, K))) return DN_ERR_SHAPE;
+  const bool many = direct::takes(A, lda, W, bias, C, ldc, nullptr, 0, N, K, DN_BF16, packed);
+  if (!few && !many && (a_packed || !tiled::takes(A, lda, W, K))) return DN_ERR_SHAPE;
   if (q_width < 0 || q_width + 2 * Hkv * dh != N || page_size < 1 || dh % 4 != 0) return DN_ERR_SHAPE;
   if ((c_cols != N && c_cols != q_width) || ldc < c_cols) return DN_ERR_SHAPE;
   KVScatter kv{slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_width, Hkv * dh, dh,
                page_size, Hkv, c_cols};
+  if (many && (!few || direct::beats_few_rows(M, N, K))) {
+    int rc = direct::run(direct::Args{A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, packed, &kv}, stream);
+    return rc != 0 ? rc : dn_launch_status();
+  }
   if (few) {
     skinny::Call c{A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, packed, &kv};
     skinny::run(c, stream);
     return dn_launch_status();
   }
-  int rc;
-  if (direct::takes(A, lda, W, bias, C, ldc, nullptr, 0, N, K, DN_BF16))
-    rc = direct::run(direct::Args{A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv}, stream);
-  else
-    rc = tiled::run(A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv, stream);
+  int rc = tiled::run(A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, &kv, stream);
   return rc != 0 ? rc : dn_launch_status();
 }
 

@@ -23,7 +23,11 @@ TINY_C = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n
 # a fourth with the head size and context of the large models (4 heads of 64, 1024 positions)
 TINY_D = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n_embd=256, n_head=4,
               vocab_size=5003, n_positions=1024, layer_norm_epsilon=1e-5, activation_function="gelu_new")
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
+# a fifth, one wide layer: its products have the widths (more than 4,096 columns) at which steps of
+# 129 to 256 rows change kernels
+WIDE_E = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=1, n_embd=1408, n_head=22,
+              vocab_size=300, n_positions=64, layer_norm_epsilon=1e-5, activation_function="gelu_new")
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3), "E": (WIDE_E, 4)}
 
 
 def pytest_configure(config):

@@ -181,6 +181,38 @@ def test_linear_qkv_writes_the_cache(M, slots_in, queries_only):
     assert pools[0].abs().sum() > 0 and pools[1].abs().sum() > 0
 
 
+@pytest.mark.parametrize("M", [100, 129, 200, 256, 300])
+@pytest.mark.parametrize("rows_in", ["packed", "rows"])
+def test_linear_qkv_with_many_columns(M, rows_in):
+    """The fused projection where its columns are many (the many-rows kernel takes it from 129 rows on,
+    with packed rows too): heads of 48, a grouped cache, pages of 32, slots in runs that start anywhere."""
+    if rows_in == "packed" and M > 256:
+        pytest.skip("packed rows end at 256")
+    o = ops()
+    H, Hkv, dh, ps, K = 64, 16, 48, 32, 160
+    N = (H + 2 * Hkv) * dh
+    assert N >= 4096
+    n_pages = (M + 40) // ps + 2
+    a, w, bias = rnd(M, K, seed=1, dtype=torch.bfloat16), rnd(N, K, seed=2, dtype=torch.bfloat16, scale=0.2), rnd(N, seed=3)
+    slots = torch.tensor([(5 if i < M // 3 else 12 if i < 2 * M // 3 else 33) + i for i in range(M)], dtype=torch.int32)
+    slots[7] = -1
+    slots = slots.to(DEV)
+    pools = [torch.zeros(n_pages, Hkv, ps, dh, dtype=torch.bfloat16, device=DEV),
+             torch.zeros(n_pages, Hkv, dh, ps, dtype=torch.bfloat16, device=DEV)]
+    want_pools = [torch.zeros_like(p) for p in pools]
+    wp = o.pack_matrix(w)
+    out = torch.full((M, H * dh), 7.0, dtype=torch.bfloat16, device=DEV)
+    queries = o.linear_qkv(o.pack_matrix(a) if rows_in == "packed" else a, wp, bias, out, slots, pools[0], pools[1], H * dh)
+    want = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    o.linear(a, wp, bias, out=want)
+    R.kv_write(want, H * dh, (H + Hkv) * dh, slots, want_pools[0], want_pools[1])
+    assert torch.equal(queries, want[:, :H * dh])
+    assert torch.equal(pools[0], want_pools[0]) and torch.equal(pools[1], want_pools[1])
+    assert pools[0].abs().sum() > 0 and pools[1].abs().sum() > 0
+    exact = (a.double() @ w.double().t() + bias.double()).float()
+    assert torch.allclose(want.float(), exact, **TOL[torch.bfloat16])
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64, 65, 100, 130, 200, 256])
 @pytest.mark.parametrize("N,K", [(1600, 1600), (4800, 1600), (96, 6400), (33024, 64)])
 def test_linear_with_packed_rows(M, N, K):

@@ -207,6 +207,32 @@ def test_twenty_requests_decode_together(model_folders, name, graphs):
             U.assert_close(got[i:i + 1], want[i][len(s) - j:len(s) - j + 1], "bfloat16", f"request {i}, {j} from its end")
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("n", [150, 230])
+def test_many_requests_on_a_wide_layer(model_folders, n):
+    """Steps of 129 to 256 rows of a model whose products are wide: the rows stay packed from kernel to
+    kernel, the two products with many columns go to the many-rows kernel (the projection with its
+    cache write among them), the other two to the few-rows kernel.  The prompts run in one step of
+    three rows each (more than 256 rows: ordinary rows), then every request decodes."""
+    from denno_beta_amd.config import EngineOptions
+    from denno_beta_amd.engine import ModelRunner, StepEntry
+    folder = model_folders("E", "bfloat16")
+    seqs = sequences("E", [7] * n, seed=90)
+    want = plain_logits(folder, seqs)
+    r = ModelRunner.from_folder(folder, EngineOptions(dtype="bfloat16", page_size=16, cache_tokens=n * 16,
+                                                      max_live=n, use_graphs=False))
+    assert r.model.blocks[0].mixer.packed_input(n) and r.model.blocks[0].ffn.down.packed_input(n)
+    for i in range(n):
+        r.start_request(i)
+    got = r.step([StepEntry(i, s[:3], [0, 1, 2]) for i, s in enumerate(seqs)]).cpu()
+    for i in range(n):
+        U.assert_close(got[3 * i:3 * i + 3], want[i][:3], "bfloat16", f"prompt of request {i}")
+    for j in range(3, 7):
+        got = r.step([StepEntry(i, [s[j]], [0]) for i, s in enumerate(seqs)]).cpu()
+        for i in range(n):
+            U.assert_close(got[i:i + 1], want[i][j:j + 1], "bfloat16", f"request {i}, token {j}")
+
+
 def test_weights_stored_in_32_bit_stay_so_in_a_bfloat16_engine(backend, model_folders):
     """A folder stored in 32-bit, run with --dtype bfloat16: the matrices stay 32-bit and their
     products run in 32-bit on widened activations; the result is at least as close to the plain

@@ -269,7 +269,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   for (int mb = 0; mb < MB; ++mb) {
     int row = mb * 16 + col;
     a_ok[mb] = row < M;
-    arow[mb] = (packed & PACKED_A) ? A + (static_cast<size_t>(mb) * ksteps * 64 + lane) * 8
+    // (a block of rows beyond M, where MB is more than the rows need, reads the last one again: packed
+    // rows end with the block that holds row M - 1)
+    arow[mb] = (packed & PACKED_A) ? A + (static_cast<size_t>(min(mb, (M + 15) / 16 - 1)) * ksteps * 64 + lane) * 8
                                    : A + static_cast<size_t>(a_ok[mb] ? row : 0) * lda + g * 8;
   }
   floatx4 acc[MB][NB];

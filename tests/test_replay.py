@@ -75,6 +75,44 @@ def test_every_cutting_matches_the_plain_implementation(backend, model_folders, 
                 U.assert_close(b, a, dtype, f"{name} {dtype} {kind} vs whole, request {i}")
 
 
+def _cfg(L, E, H, I, V, P, eps=1e-5, act="gelu_new", inv=False):
+    return dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=L, n_embd=E, n_head=H, n_inner=I,
+                vocab_size=V, n_positions=P, layer_norm_epsilon=eps, activation_function=act,
+                scale_attn_by_inverse_layer_idx=inv)
+
+
+OTHER_SIZES = {
+    "one head of 80": _cfg(1, 80, 1, 320, 101, 160, 1e-3),                        # no MFMA attention kernel takes 80
+    "three heads of 112": _cfg(2, 336, 3, 1000, 777, 200, 1e-6, "gelu", True),    # nor 112; widths no multiple of 32
+    "three heads of 16": _cfg(4, 48, 3, 64, 50, 130),                             # a feed-forward narrower than 4 E
+    "two heads of 256": _cfg(1, 512, 2, 2048, 1000, 300),                         # the largest head size
+    "five heads of 48": _cfg(2, 240, 5, 960, 333, 260, 1e-5, "gelu", True),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(OTHER_SIZES))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_other_head_sizes_and_widths(tmp_path, name, dtype):
+    """Every head size in steps of 16 has a kernel (the MFMA kernels for some, the plain one for the
+    rest), and widths need be no multiple of 32: four cuttings of four requests each, one of them
+    to the last position but two."""
+    from denno_beta_amd.weights import write_model_folder
+    cfg = OTHER_SIZES[name]
+    folder = str(tmp_path)
+    write_model_folder(folder, cfg, 7, "float32")
+    P = cfg["n_positions"]
+    seqs = [seeded_tokens(20 + i, n, cfg["vocab_size"]) for i, n in enumerate((7, 70, P - 3, 40))]
+    want = plain_logits(folder, seqs)
+    for kind, steps in (("whole", U.whole_trace(seqs)), ("tail", U.tail_decode_trace(seqs, 32)),
+                        ("chunks", U.chunk_trace(seqs)), ("mixed", U.mixed_trace(seqs, seed=5))):
+        r = runner_for(folder, dtype, "cuda:0", cache_tokens=U.max_live_tokens(steps))
+        got = U.replay(r, steps)
+        r.cache.manager.check()
+        for i in range(len(seqs)):
+            U.assert_close(got[f"r{i}"], want[i], dtype, f"{name} {dtype} {kind} request {i}")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_and_first_tokens(backend, model_folders, dtype):
     """A sequence decoded token by token from its first token on, across many pages."""

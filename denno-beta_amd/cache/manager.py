@@ -55,6 +55,11 @@ def host_library():
             "dn_cache_pages_held": (I, [P, L, I]), "dn_cache_pages_needed": (I, [P, L, I, I, I]),
             "dn_cache_pages_peak": (I, [P, I, I, I]), "dn_cache_live": (I, [P]), "dn_cache_check": (I, [P]),
             "dn_cache_reuse_count": (L, [P, I]),
+            "dn_cache_lengths": (I, [P, c_void_p, I, c_void_p, IP]),
+            "dn_cache_reserve_step": (I, [P, c_void_p, c_void_p, I, c_void_p, IP]),
+            "dn_cache_commit_step": (I, [P, c_void_p, c_void_p, I, IP]),
+            "dn_cache_max_blocks": (I, [P, I, c_void_p, I]),
+            "dn_cache_step_tables": (I, [P, I, c_void_p, c_void_p, c_void_p, I, I, I, c_void_p, c_void_p, I, IP]),
             "dn_sched_create": (P, [P, I, I, I, I, I]), "dn_sched_destroy": (None, [P]),
             "dn_sched_add": (I, [P, L, I, I]),
             "dn_sched_schedule": (I, [P, c_void_p, c_void_p, c_void_p, c_void_p, I, c_void_p, IP, I]),
@@ -138,6 +143,50 @@ class CacheManager:
         out = np.empty(max(n, 1), dtype=np.int32)
         self._chk(self._lib.dn_cache_block_table(self._h, rid, group, out.ctypes.data, n), "block table")
         return out[:n]
+
+    # -- a whole step in one call each ----------------------------------------------------
+    # rids: int64 array; lengths and counts: int32 arrays (numpy, contiguous)
+    def _chk_step(self, rc, failed, rids, what):
+        if rc < 0:
+            raise (OutOfPages if rc == OUT_OF_PAGES else CacheError)(rc, f"{what} (request {int(rids[failed.value])})")
+
+    def lengths(self, rids: np.ndarray) -> np.ndarray:
+        out = np.empty(len(rids), dtype=np.int32)
+        failed = c_int(0)
+        self._chk_step(self._lib.dn_cache_lengths(self._h, rids.ctypes.data, len(rids), out.ctypes.data, failed),
+                       failed, rids, "length")
+        return out
+
+    def reserve_step(self, rids: np.ndarray, new_lens: np.ndarray) -> np.ndarray:
+        """Pages for every entry's tokens, entry after entry (entries before one that fails keep
+        theirs); -> the requests' slots."""
+        slots = np.empty(len(rids), dtype=np.int32)
+        failed = c_int(0)
+        self._chk_step(self._lib.dn_cache_reserve_step(self._h, rids.ctypes.data, new_lens.ctypes.data, len(rids),
+                                                       slots.ctypes.data, failed), failed, rids, "reserve")
+        return slots
+
+    def commit_step(self, rids: np.ndarray, new_lens: np.ndarray):
+        failed = c_int(0)
+        self._chk_step(self._lib.dn_cache_commit_step(self._h, rids.ctypes.data, new_lens.ctypes.data, len(rids),
+                                                      failed), failed, rids, "commit")
+
+    def max_blocks(self, group: int, rids: np.ndarray) -> int:
+        return self._chk(self._lib.dn_cache_max_blocks(self._h, group, rids.ctypes.data, len(rids)), "block tables")
+
+    def step_tables(self, group: int, rids, starts, counts, block_tables: np.ndarray, slot_map: np.ndarray):
+        """Fills block_tables [rows >= entries, max_blocks] and slot_map [>= tokens] (int32, contiguous,
+        written in place: views of a pinned buffer will do) for the step's entries; -1 wherever
+        there is nothing.  Returns the entry's index if one of its tokens has no page (given back,
+        or never reserved), else -1."""
+        failed = c_int(0)
+        rc = self._lib.dn_cache_step_tables(self._h, group, rids.ctypes.data, starts.ctypes.data, counts.ctypes.data,
+                                            len(rids), block_tables.shape[0], block_tables.shape[1],
+                                            block_tables.ctypes.data, slot_map.ctypes.data, slot_map.shape[0], failed)
+        if rc == BAD_ARGUMENT:
+            return failed.value
+        self._chk_step(rc, failed, rids, "step tables")
+        return -1
 
     def free_pages(self, group: int) -> int:
         return self._chk(self._lib.dn_cache_free_pages(self._h, group), "free pages")

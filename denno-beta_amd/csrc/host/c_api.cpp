@@ -45,6 +45,24 @@ int dn_cache_pages_needed(void* c, int64_t rid, int from_len, int new_len, int g
 int dn_cache_pages_peak(void* c, int g, int total_len, int chunk) {
   return static_cast<CacheManager*>(c)->pages_peak(g, total_len, chunk);
 }
+int dn_cache_lengths(void* c, const int64_t* rids, int n, int* out, int* failed) {
+  return static_cast<CacheManager*>(c)->lengths(rids, n, out, failed);
+}
+int dn_cache_reserve_step(void* c, const int64_t* rids, const int* new_lens, int n, int* slots_out, int* failed) {
+  return static_cast<CacheManager*>(c)->reserve_step(rids, new_lens, n, slots_out, failed);
+}
+int dn_cache_commit_step(void* c, const int64_t* rids, const int* new_lens, int n, int* failed) {
+  return static_cast<CacheManager*>(c)->commit_step(rids, new_lens, n, failed);
+}
+int dn_cache_max_blocks(void* c, int g, const int64_t* rids, int n) {
+  return static_cast<CacheManager*>(c)->max_blocks(g, rids, n);
+}
+int dn_cache_step_tables(void* c, int g, const int64_t* rids, const int* starts, const int* counts, int n,
+                         int bt_rows, int max_blocks, int32_t* block_tables, int32_t* slot_map, int sm_len,
+                         int* failed) {
+  return static_cast<CacheManager*>(c)->step_tables(g, rids, starts, counts, n, bt_rows, max_blocks, block_tables,
+                                                    slot_map, sm_len, failed);
+}
 int dn_cache_live(void* c) { return static_cast<CacheManager*>(c)->live(); }
 int dn_cache_check(void* c) { return static_cast<CacheManager*>(c)->check(); }
 int64_t dn_cache_reuse_count(void* c, int g) { return static_cast<CacheManager*>(c)->reuse_count(g); }

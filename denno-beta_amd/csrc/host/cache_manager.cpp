@@ -128,6 +128,78 @@ int CacheManager::commit(int64_t rid, int new_len) {
   return kOk;
 }
 
+int CacheManager::lengths(const int64_t* rids, int n, int* out, int* failed) const {
+  for (int i = 0; i < n; ++i) {
+    auto it = by_rid_.find(rids[i]);
+    if (it == by_rid_.end()) {
+      *failed = i;
+      return kUnknown;
+    }
+    out[i] = it->second.len;
+  }
+  return kOk;
+}
+
+int CacheManager::reserve_step(const int64_t* rids, const int* new_lens, int n, int* slots_out, int* failed) {
+  for (int i = 0; i < n; ++i) {
+    int rc = reserve(rids[i], new_lens[i]);
+    if (rc != kOk) {
+      *failed = i;
+      return rc;
+    }
+    slots_out[i] = by_rid_.find(rids[i])->second.slot;
+  }
+  return kOk;
+}
+
+int CacheManager::commit_step(const int64_t* rids, const int* new_lens, int n, int* failed) {
+  for (int i = 0; i < n; ++i) {
+    int rc = commit(rids[i], new_lens[i]);
+    if (rc != kOk) {
+      *failed = i;
+      return rc;
+    }
+  }
+  return kOk;
+}
+
+int CacheManager::max_blocks(int g, const int64_t* rids, int n) const {
+  if (g < 0 || g >= n_groups()) return kBadArgument;
+  int most = 0;
+  for (int i = 0; i < n; ++i) {
+    auto it = by_rid_.find(rids[i]);
+    if (it == by_rid_.end()) return kUnknown;
+    most = std::max(most, static_cast<int>(it->second.tables[g].size()));
+  }
+  return most;
+}
+
+int CacheManager::step_tables(int g, const int64_t* rids, const int* starts, const int* counts, int n, int bt_rows,
+                              int max_blocks, int32_t* block_tables, int32_t* slot_map, int sm_len,
+                              int* failed) const {
+  if (g < 0 || g >= n_groups() || groups_[g].kind != kPaged || n > bt_rows || max_blocks < 1) return kBadArgument;
+  const int ps = groups_[g].page_size;
+  std::fill(block_tables, block_tables + static_cast<size_t>(bt_rows) * max_blocks, -1);
+  std::fill(slot_map, slot_map + sm_len, -1);
+  int row = 0;
+  for (int i = 0; i < n; ++i) {
+    *failed = i;
+    auto it = by_rid_.find(rids[i]);
+    if (it == by_rid_.end()) return kUnknown;
+    const auto& t = it->second.tables[g];
+    if (static_cast<int>(t.size()) > max_blocks || starts[i] < 0 || counts[i] < 0 || row + counts[i] > sm_len)
+      return kBadArgument;
+    std::copy(t.begin(), t.end(), block_tables + static_cast<size_t>(i) * max_blocks);
+    for (int j = 0; j < counts[i]; ++j) {
+      const int pos = starts[i] + j, blk = pos / ps;
+      if (blk >= static_cast<int>(t.size()) || t[blk] < 0) return kBadArgument;     // no page, or given back
+      slot_map[row + j] = t[blk] * ps + pos % ps;
+    }
+    row += counts[i];
+  }
+  return kOk;
+}
+
 int CacheManager::length(int64_t rid) const {
   auto it = by_rid_.find(rid);
   return it == by_rid_.end() ? static_cast<int>(kUnknown) : it->second.len;

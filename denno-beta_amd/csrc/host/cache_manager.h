@@ -53,6 +53,22 @@ class CacheManager {
   int pages_needed(int64_t rid, int from_len, int new_len, int group) const;
   // most pages that a request of `total_len` tokens, fed in portions of at most `chunk`, holds at once
   int pages_peak(int group, int total_len, int chunk) const;
+
+  // The same for all requests of a step in one call each (a step of 64 single tokens is otherwise
+  // some hundred calls across the language boundary).  On a failure *failed is the entry's index.
+  int lengths(const int64_t* rids, int n, int* out, int* failed) const;
+  // pages for every entry's tokens, entry after entry; entries before a failing one keep theirs
+  int reserve_step(const int64_t* rids, const int* new_lens, int n, int* slots_out, int* failed);
+  int commit_step(const int64_t* rids, const int* new_lens, int n, int* failed);
+  int max_blocks(int group, const int64_t* rids, int n) const;      // the longest block table, or < 0
+  // The tables that the kernels read for one group: block_tables [bt_rows, max_blocks] (row i: entry
+  // i's; -1 where there is no page, and in rows n .. bt_rows - 1) and slot_map [sm_len] (token j of
+  // entry i at sum(counts[:i]) + j: page * page_size + offset of position starts[i] + j; -1 beyond
+  // the entries' tokens).  kBadArgument if a table or the map is too small or a token's page was
+  // given back.
+  int step_tables(int group, const int64_t* rids, const int* starts, const int* counts, int n, int bt_rows,
+                  int max_blocks, int32_t* block_tables, int32_t* slot_map, int sm_len, int* failed) const;
+
   int live() const { return static_cast<int>(by_rid_.size()); }
   int n_groups() const { return static_cast<int>(groups_.size()); }
   const GroupSpec& group(int g) const { return groups_[g]; }

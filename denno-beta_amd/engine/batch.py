@@ -97,69 +97,60 @@ def plan_rows(entries: Sequence[StepEntry], starts: Sequence[int], vocab: int, m
 
 def build_context(entries: Sequence[StepEntry], cache, vocab: int, max_positions: int, device) -> StepContext:
     """Reserves pages for the entries' tokens (raising cache.OutOfPages; pages taken for
-    earlier entries stay with their requests) and builds the step's tables."""
+    earlier entries stay with their requests) and builds the step's tables.  The cache manager is
+    asked once per table for the whole step, not once per request."""
     mgr = cache.manager
-    starts = [mgr.length(e.rid) for e in entries]
+    rids = np.asarray([e.rid for e in entries], dtype=np.int64)
+    counts = np.asarray([len(e.tokens) for e in entries], dtype=np.int32)
+    starts_a = mgr.lengths(rids)
+    starts = starts_a.tolist()
     tokens, positions, logit_rows, row_start, tiles, wide = plan_rows(entries, starts, vocab, max_positions)
-    for e, start in zip(entries, starts):
-        mgr.reserve(e.rid, start + len(e.tokens))
+    slots_a = mgr.reserve_step(rids, starts_a + counts)
     T, S, R = len(tokens), len(entries), len(logit_rows)
-    slots = [mgr.slot(e.rid) for e in entries]
+    slots = slots_a.tolist()
 
-    parts = [("tokens", np.asarray(tokens, dtype=np.int32)),
-             ("positions", np.asarray(positions, dtype=np.int32)),
-             ("logit_rows", np.asarray(logit_rows, dtype=np.int32)),
-             ("state_slots", np.asarray(slots, dtype=np.int32)),
-             ("row_start", np.asarray(row_start, dtype=np.int32)),
-             ("tiles", np.ascontiguousarray(np.asarray(tiles, dtype=np.int32).T).reshape(-1)),
-             ("wide", np.ascontiguousarray(np.asarray(wide, dtype=np.int32).T).reshape(-1))]
-    single = all(len(e.tokens) == 1 for e in entries)
-    max_context = max(start + len(e.tokens) for e, start in zip(entries, starts))
-    group_meta = []
-    for g, layout in enumerate(cache.layouts):
-        if layout.kind != 0:
-            group_meta.append(None)
-            continue
-        tables = [mgr.block_table(e.rid, g) for e in entries]
-        max_blocks = max(len(t) for t in tables)
-        bt = np.full((S, max_blocks), -1, dtype=np.int32)
-        slot_map = np.full(T, -1, dtype=np.int32)
-        for s, (e, start, tab) in enumerate(zip(entries, starts, tables)):
-            bt[s, :len(tab)] = tab
-            n = len(e.tokens)
-            pos = np.arange(start, start + n)
-            pages = tab[pos // layout.page_size]
-            if (pages < 0).any():
-                raise BatchError(f"request {e.rid}: a token's page was given back already")
-            slot_map[row_start[s]:row_start[s] + n] = pages * layout.page_size + pos % layout.page_size
-        parts.append((f"bt{g}", bt.reshape(-1)))
-        parts.append((f"sm{g}", slot_map))
-        group_meta.append((layout, max_blocks))
-
-    total = sum(a.size for _, a in parts)
-    on_gpu = torch.device(device).type == "cuda"
-    host = torch.empty(total, dtype=torch.int32, pin_memory=on_gpu)
-    hv = host.numpy()
+    paged = [(g, layout, mgr.max_blocks(g, rids)) for g, layout in enumerate(cache.layouts) if layout.kind == 0]
+    sizes = [("tokens", T), ("positions", T), ("logit_rows", R), ("state_slots", S), ("row_start", S + 1),
+             ("tiles", 4 * len(tiles)), ("wide", 4 * len(wide))]
+    for g, _, max_blocks in paged:
+        sizes += [(f"bt{g}", S * max_blocks), (f"sm{g}", T)]
     offs, o = {}, 0
-    for name, a in parts:
-        hv[o:o + a.size] = a
-        offs[name] = (o, a.size)
-        o += a.size
+    for name, n in sizes:
+        offs[name] = (o, n)
+        o += n
+    on_gpu = torch.device(device).type == "cuda"
+    host = torch.empty(o, dtype=torch.int32, pin_memory=on_gpu)
+    hv = host.numpy()
+
+    def put(name, values):
+        b, n = offs[name]
+        hv[b:b + n] = values
+    put("tokens", tokens), put("positions", positions), put("logit_rows", logit_rows)
+    put("state_slots", slots_a), put("row_start", row_start)
+    put("tiles", np.asarray(tiles, dtype=np.int32).T.reshape(-1))
+    put("wide", np.asarray(wide, dtype=np.int32).T.reshape(-1))
+    for g, layout, max_blocks in paged:
+        (b0, n0), (b1, n1) = offs[f"bt{g}"], offs[f"sm{g}"]
+        bad = mgr.step_tables(g, rids, starts_a, counts, hv[b0:b0 + n0].reshape(S, max_blocks), hv[b1:b1 + n1])
+        if bad >= 0:
+            raise BatchError(f"request {entries[bad].rid}: a token's page was given back already")
     dev = host.to(device, non_blocking=True) if on_gpu else host
 
     def view(name):
         b, n = offs[name]
         return dev[b:b + n]
+    single = bool((counts == 1).all())
+    max_context = int((starts_a + counts).max())
     tiles_dev = view("tiles").view(4, -1)
     wide_dev = view("wide").view(4, -1)
     groups = []
-    for g, meta in enumerate(group_meta):
-        if meta is None:
+    max_blocks_of = {g: mb for g, _, mb in paged}
+    for g, layout in enumerate(cache.layouts):
+        if layout.kind != 0:
             groups.append(GroupStep(0, 0, None, None, None))
             continue
-        layout, max_blocks = meta
         groups.append(GroupStep(layout.page_size, layout.window, view(f"sm{g}"),
-                                view(f"bt{g}").view(S, max_blocks), tiles_dev, wide_dev, single, max_context))
+                                view(f"bt{g}").view(S, max_blocks_of[g]), tiles_dev, wide_dev, single, max_context))
     return StepContext(
         T=T, S=S, R=R, tokens=view("tokens"), positions=view("positions"), logit_rows=view("logit_rows"),
         state_slots=view("state_slots"), row_start=view("row_start"), groups=groups,

@@ -68,7 +68,8 @@ class DecodeGraph:
                                logit_rows=v("logit_rows"), state_slots=v("state_slots"), row_start=v("row_start"),
                                groups=groups, host_row_start=list(range(B + 1)), host_first_pos=[0] * B,
                                host_slots=[-1] * B, rids=[-1] * B)
-        self._fill(self.host[0].numpy(), [], [], [])
+        none = np.empty(0, dtype=np.int32)
+        self._fill(self.host[0].numpy(), np.empty(0, dtype=np.int64), none, none, none)
         self.dev.copy_(self.host[0])
         # once outside the capture (libraries load, allocator warms up), then the capture
         side = torch.cuda.Stream(device=dev)
@@ -85,46 +86,42 @@ class DecodeGraph:
         b, n = self.off[name]
         return self.dev[b:b + n]
 
-    def _fill(self, hv, entries, starts, slots):
-        B, n = self.B, len(entries)
+    def _fill(self, hv, rids, tokens, starts, slots):
+        """The step's tables into a host buffer: rids int64 [n], tokens, starts, slots int32 [n]."""
+        B, n = self.B, len(rids)
         mgr = self.runner.cache.manager
 
         def put(name, vals, fill):
             b, ln = self.off[name]
             hv[b:b + ln] = fill
-            hv[b:b + len(vals)] = vals
-        put("tokens", [int(e.tokens[0]) for e in entries], 0)
+            hv[b:b + n] = vals
+        steps = np.arange(n + 1, dtype=np.int32)
+        put("tokens", tokens, 0)
         put("positions", starts, 0)
-        put("logit_rows", list(range(n)), 0)
+        put("logit_rows", steps[:n], 0)
         put("state_slots", slots, -1)
-        put("row_start", list(range(n + 1)), n)
+        b, ln = self.off["row_start"]
+        hv[b:b + ln] = n
+        hv[b:b + n + 1] = steps
         b, ln = self.off["tiles"]
         t = hv[b:b + ln].reshape(4, B)
         t[0, :], t[1, :], t[2, :], t[3, :] = -1, 0, 1, 0
-        t[0, :n], t[1, :n], t[3, :n] = np.arange(n), np.arange(n), starts
+        t[0, :n], t[1, :n], t[3, :n] = steps[:n], steps[:n], starts
+        ones = np.ones(n, dtype=np.int32)
         for g, l in enumerate(self.layouts):
             if l.kind != 0:
                 continue
-            b, ln = self.off[f"bt{g}"]
-            bt = hv[b:b + ln].reshape(B, self.max_blocks[g])
-            bt[:] = -1
-            b, ln = self.off[f"sm{g}"]
-            sm = hv[b:b + ln]
-            sm[:] = -1
-            for s, (e, start) in enumerate(zip(entries, starts)):
-                tab = mgr.block_table(e.rid, g)
-                bt[s, :len(tab)] = tab
-                page = tab[start // l.page_size]
-                if page < 0:
-                    raise BatchError(f"request {e.rid}: a token's page was given back already")
-                sm[s] = page * l.page_size + start % l.page_size
+            (b0, n0), (b1, n1) = self.off[f"bt{g}"], self.off[f"sm{g}"]
+            bad = mgr.step_tables(g, rids, starts, ones, hv[b0:b0 + n0].reshape(B, self.max_blocks[g]), hv[b1:b1 + n1])
+            if bad >= 0:
+                raise BatchError(f"request {int(rids[bad])}: a token's page was given back already")
 
-    def run(self, entries: Sequence[StepEntry], starts: List[int], slots: List[int]) -> torch.Tensor:
+    def run(self, rids, tokens, starts, slots) -> torch.Tensor:
         i = self.turn
         self.turn ^= 1
         if self.copied[i] is not None:
             self.copied[i].synchronize()      # the copy that last read this host buffer has ended
-        self._fill(self.host[i].numpy(), entries, starts, slots)
+        self._fill(self.host[i].numpy(), rids, tokens, starts, slots)
         self.dev.copy_(self.host[i], non_blocking=True)
         ev = torch.cuda.Event()
         ev.record()
@@ -147,36 +144,38 @@ class DecodeGraphs:
         """Runs a pure decode step; -> logits [R, vocab] at the wanted places (a copy)."""
         runner = self.runner
         mgr, spec = runner.cache.manager, runner.spec
-        starts = [mgr.length(e.rid) for e in entries]
-        seen = set()
-        for e, start in zip(entries, starts):
-            if e.rid in seen:
-                raise BatchError(f"request {e.rid} appears twice in one step")
-            seen.add(e.rid)
-            if start + 1 > spec.max_positions:
-                raise BatchError(f"request {e.rid}: {start} tokens in the cache + 1 exceed the model's "
-                                 f"{spec.max_positions} positions")
-            if not 0 <= int(e.tokens[0]) < spec.vocab:
-                raise BatchError(f"request {e.rid}: token id {e.tokens[0]} is outside the vocabulary of {spec.vocab}")
-            for w in e.want:
-                if w != 0:
-                    raise BatchError(f"request {e.rid}: wanted place {w} is not among its 1 tokens")
-        for e, start in zip(entries, starts):
-            mgr.reserve(e.rid, start + 1)
-        slots = [mgr.slot(e.rid) for e in entries]
         n = len(entries)
+        rids = np.asarray([e.rid for e in entries], dtype=np.int64)
+        tokens = np.asarray([e.tokens[0] for e in entries], dtype=np.int64)
+        starts = mgr.lengths(rids)
+        if len(set(rids.tolist())) != n:
+            raise BatchError("a request appears twice in one step")
+        if int(starts.max()) + 1 > spec.max_positions:
+            i = int(starts.argmax())
+            raise BatchError(f"request {entries[i].rid}: {int(starts[i])} tokens in the cache + 1 exceed the model's "
+                             f"{spec.max_positions} positions")
+        if int(tokens.min()) < 0 or int(tokens.max()) >= spec.vocab:
+            i = int(np.flatnonzero((tokens < 0) | (tokens >= spec.vocab))[0])
+            raise BatchError(f"request {entries[i].rid}: token id {entries[i].tokens[0]} is outside the vocabulary of {spec.vocab}")
+        rows = []
+        for i, e in enumerate(entries):
+            if len(e.want) > 0:
+                if len(e.want) != 1 or e.want[0] != 0:
+                    w = [w for w in e.want if w != 0]
+                    raise BatchError(f"request {e.rid}: wanted place {w[0] if w else 0} is not among its 1 tokens")
+                rows.append(i)
+        new_lens = starts + 1
+        slots = mgr.reserve_step(rids, new_lens)
         B = batch_bucket(n, runner.options.max_live)
-        ctx_bucket = min(-(-(max(starts) + 1) // DECODE_SPLIT) * DECODE_SPLIT, -(-spec.max_positions // 16) * 16)
+        ctx_bucket = min(-(-int(new_lens.max()) // DECODE_SPLIT) * DECODE_SPLIT, -(-spec.max_positions // 16) * 16)
         key = (B, ctx_bucket)
         g = self.graphs.get(key)
         if g is None:
             g = self.graphs[key] = DecodeGraph(runner, B, ctx_bucket)
-        logits = g.run(entries, starts, slots)
-        rows = [i for i, e in enumerate(entries) if len(e.want) > 0]
+        logits = g.run(rids, tokens.astype(np.int32), starts, slots)
         if len(rows) == n:
             out = logits[:n].clone()
         else:
             out = logits[torch.tensor(rows, dtype=torch.long, device=logits.device)] if rows else logits[:0].clone()
-        for e, start in zip(entries, starts):
-            mgr.commit(e.rid, start + 1)
+        mgr.commit_step(rids, new_lens)
         return out

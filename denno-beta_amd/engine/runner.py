@@ -8,6 +8,7 @@ from __future__ import annotations
 
 from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..cache import CacheStorage
@@ -85,8 +86,8 @@ class ModelRunner:
             return self.graphs.step(entries)
         ctx = build_context(entries, self.cache, self.spec.vocab, self.spec.max_positions, self.device)
         logits = self.model.forward(ctx, self.cache)
-        mgr = self.cache.manager
-        for e, start in zip(entries, ctx.host_first_pos):
-            mgr.commit(e.rid, start + len(e.tokens))
+        self.cache.manager.commit_step(
+            np.asarray(ctx.rids, dtype=np.int64),
+            np.asarray([start + len(e.tokens) for e, start in zip(entries, ctx.host_first_pos)], dtype=np.int32))
         self.steps_run += 1
         return logits

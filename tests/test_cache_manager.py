@@ -165,3 +165,91 @@ def test_random_orders_keep_every_page_accounted(seed):
         m.release(rid)
     assert m.free_pages(0) == 24 and m.free_pages(1) == 12
     m.check()
+
+
+def _arr(vals, dtype):
+    import numpy as np
+    return np.asarray(vals, dtype=dtype)
+
+
+def test_a_whole_step_in_one_call_each_agrees_with_the_calls_per_request():
+    """lengths, reserve_step, max_blocks, step_tables and commit_step against the same done request
+    by request, over random steps of portions and single tokens, with a window in one group."""
+    import numpy as np
+    rng = random.Random(5)
+    layouts = [GroupLayout(PAGED, 40, 16, 0), GroupLayout(STATE), GroupLayout(PAGED, 40, 8, 20)]
+    a, b = CacheManager(layouts, 6), CacheManager(layouts, 6)
+    live = []
+    for step in range(200):
+        if len(live) < 5 and rng.random() < 0.3:
+            rid = 100 + step
+            assert a.add(rid) == b.add(rid)
+            live.append(rid)
+        if live and rng.random() < 0.1:
+            rid = live.pop(rng.randrange(len(live)))
+            assert a.release(rid) and b.release(rid)
+        chosen = [r for r in live if rng.random() < 0.7]
+        rng.shuffle(chosen)
+        chosen = [r for r in chosen if a.length(r) < 100]
+        if not chosen:
+            continue
+        rids = _arr(chosen, np.int64)
+        counts = _arr([rng.choice([1, 1, 2, 5, 17]) for _ in chosen], np.int32)
+        starts = a.lengths(rids)
+        assert starts.tolist() == [b.length(r) for r in chosen]
+        slots = a.reserve_step(rids, starts + counts)
+        for r, s, c in zip(chosen, starts.tolist(), counts.tolist()):
+            b.reserve(r, s + c)
+        assert slots.tolist() == [b.slot(r) for r in chosen]
+        for g in (0, 2):
+            ps = layouts[g].page_size
+            tables = [b.block_table(r, g) for r in chosen]
+            mb = a.max_blocks(g, rids)
+            assert mb == max(len(t) for t in tables)
+            rows = len(chosen) + 2                       # as a graph's bucket has rows beyond the requests
+            bt = np.full((rows, mb), 99, dtype=np.int32)
+            sm = np.full(int(counts.sum()) + 3, 99, dtype=np.int32)
+            assert a.step_tables(g, rids, starts, counts, bt, sm) == -1
+            want_bt = np.full((rows, mb), -1, dtype=np.int32)
+            want_sm = []
+            for i, (t, s, c) in enumerate(zip(tables, starts.tolist(), counts.tolist())):
+                want_bt[i, :len(t)] = t
+                want_sm += [int(t[p // ps]) * ps + p % ps for p in range(s, s + c)]
+            assert (bt == want_bt).all()
+            assert sm.tolist() == want_sm + [-1, -1, -1]
+        a.commit_step(rids, starts + counts)
+        for r, s, c in zip(chosen, starts.tolist(), counts.tolist()):
+            b.commit(r, s + c)
+        a.check(), b.check()
+        assert [a.free_pages(g) for g in (0, 2)] == [b.free_pages(g) for g in (0, 2)]
+    for r in live:
+        a.release(r)
+    a.check()
+    assert a.free_pages(0) == 40 and a.free_pages(2) == 40
+
+
+def test_a_step_that_runs_out_of_pages_names_the_request_and_keeps_the_earlier_ones():
+    import numpy as np
+    m = mk(n_pages=3)
+    m.add(1), m.add(2), m.add(3)
+    rids = _arr([1, 2, 3], np.int64)
+    with pytest.raises(OutOfPages, match="request 2"):
+        m.reserve_step(rids, _arr([16, 48, 16], np.int32))      # 1 + 3 pages of 3
+    assert m.block_table(1, 0).tolist() == [0] and m.block_table(2, 0).tolist() == [] and m.free_pages(0) == 2
+    with pytest.raises(CacheError, match="request 9"):
+        m.lengths(_arr([1, 9], np.int64))
+    m.check()
+
+
+def test_step_tables_refuse_a_token_without_a_page():
+    import numpy as np
+    m = mk(n_pages=8, page=4, window=4)
+    m.add(1)
+    m.reserve(1, 12), m.commit(1, 12)        # the window has passed the first block
+    assert m.block_table(1, 0).tolist()[0] == -1
+    rids, one = _arr([1], np.int64), _arr([1], np.int32)
+    bt, sm = np.zeros((1, 3), dtype=np.int32), np.zeros(1, dtype=np.int32)
+    assert m.step_tables(0, rids, _arr([2], np.int32), one, bt, sm) == 0        # position 2: its page was given back
+    assert m.step_tables(0, rids, _arr([12], np.int32), one, bt, sm) == 0       # position 12: never reserved
+    assert m.step_tables(0, rids, _arr([11], np.int32), one, bt, sm) == -1 and sm[0] == bt[0, 2] * 4 + 3
+    assert m.step_tables(0, rids, _arr([11], np.int32), one, np.zeros((1, 2), dtype=np.int32), sm) == 0   # table too small

@@ -45,6 +45,8 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration (0: all)")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--norm-kernels", action="store_true",
+                    help="run every norm as a kernel of its own, also in steps of few rows (for comparisons)")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     ap.add_argument("--only", choices=["decode", "prefill", "serving"], default=None,
                     help="run one workload and print a short line (decode, prefill: for profiling; serving: "
@@ -58,6 +60,9 @@ def main():
     from denno_beta_amd.config import EngineOptions
     from denno_beta_amd.engine import Engine, ModelRunner, SamplingParams, StepEntry
 
+    if a.norm_kernels:
+        from denno_beta_amd.kernels import ops
+        ops.NORM_STREAM_ROWS_MAX = 0
     if a.only == "serving":
         return serving(a)
     cfg, full_layers = xl_config(a.layers)

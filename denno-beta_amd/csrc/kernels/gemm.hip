@@ -351,12 +351,41 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
 // line of 128 bytes; it loads A eight lanes to a row, turns each pair round through a piece of LDS
 // of its own (no barrier: a wave's LDS operations keep their order) and reads the operands from
 // there.  16 columns per workgroup, sums joined through LDS in wave order, as in gemm_kernel.
-template <int WAVES, typename TC, bool KV>
+//
+// The norm that stands between two such products runs inside them (NORM_OUT in the product before
+// it, NORM_IN in the one after), so that it is no kernel of its own: a LayerNorm of 8 rows is 4 us
+// of launch and latency for no work.  With y = (x - mean) / sqrt(var + eps) * gamma + beta
+// (crates/denno-engine/src/tensor.rs:1101-1112),
+//     y . W^T + b = ((x * gamma) . W^T - mean * c1) / sqrt(var + eps) + c2,
+//     c1[n] = sum_k gamma[k] W[n,k],  c2[n] = sum_k beta[k] W[n,k] + b[n]      (made once per weight),
+// so the product itself runs on rows that are not normalised, and the norm is two numbers per row in
+// the epilogue.  NORM_OUT: a product that adds into the residual stream also stores the updated rows
+// times gamma (the next norm's), rounded to bfloat16, and, for each row, the mean and the sum of
+// squared distances from it of its 16 columns.  NORM_IN: A is such a copy; each wave joins two rows'
+// N / 16 pairs (means are averaged; the squares add up with 16 times the squared distance of each
+// block's mean from the row's: exact, and as stable as two passes over the row) while the operands
+// travel, and wave 0 applies them at the end.  The rows are rounded to bfloat16 before the mean is
+// taken off, not after: right where a row's mean is not large beside its spread.
+struct NormIO {
+  const float* stats_in;     // NORM_IN: [M][blocks_in][2]
+  int blocks_in;             // K / 16
+  const float* c1;           // NORM_IN: [N]  (c2 comes as the bias)
+  float eps;
+  const float* gamma_out;    // NORM_OUT: [N] the next norm's weight
+  bf16_t* copy_out;          // NORM_OUT: [M, ldcopy] the updated rows times gamma_out in bfloat16
+  int ldcopy;
+  float* stats_out;          // NORM_OUT: [M][N / 16][2]
+};
+#define NORM_NONE 0
+#define NORM_IN 1
+#define NORM_OUT 2
+
+template <int WAVES, typename TC, bool KV, int NORM = NORM_NONE>
 __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __restrict__ A, int lda,
                                                              const bf16_t* __restrict__ W,
                                                              const float* __restrict__ bias, TC* __restrict__ C,
                                                              int ldc, float* __restrict__ resid, int ldr, int M,
-                                                             int N, int K, int epi, KVScatter kv) {
+                                                             int N, int K, int epi, KVScatter kv, NormIO nio) {
   typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
   constexpr int U = 4;                                     // pairs of steps in flight per wave
   constexpr int ROW = 9 * 8;                               // elements per row of a wave's piece: 8 chunks and one of padding
@@ -368,6 +397,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
   const int ksteps = (K + 31) / 32, npairs = (ksteps + 1) / 2, nblocks = (N + 15) / 16;
   const bf16_t* wblk = W + (static_cast<size_t>(min(static_cast<int>(blockIdx.x), nblocks - 1)) * ksteps * 64 + lane) * 8;
   const bool two = M > 8;                                  // rows 8 .. 15 need a second load per pair
+  // NORM_IN: the rows' pairs of statistics are asked for before the operands (loads come back in the
+  // order asked): wave w joins rows w, w + WAVES, ...; a lane holds up to SP pairs of a row
+  constexpr int SP = 4, SR = 16 / WAVES;
+  __shared__ float rowstat[16][2];
   // what the epilogue will read is asked for first of all (wave 0 finishes the block)
   float epi_bias = 0.f;
   float epi_x[4] = {0.f, 0.f, 0.f, 0.f};
@@ -384,6 +417,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
       for (int r = 0; r < 4; ++r) epi_x[r] = resid[static_cast<size_t>(min(g * 4 + r, M - 1)) * ldr + nn];
     }
   }
+  // (after the epilogue's loads and before the operands': they are back before the operands are)
+  float2 st[SR][SP];
+  float epi_c1 = 0.f, epi_gamma = 1.f;
+  if constexpr (NORM == NORM_IN) {
+#pragma unroll
+    for (int t = 0; t < SR; ++t) {
+      const int row = min(wave + t * WAVES, M - 1);
+#pragma unroll
+      for (int i = 0; i < SP; ++i)
+        st[t][i] = *reinterpret_cast<const float2*>(nio.stats_in + (static_cast<size_t>(row) * nio.blocks_in + min(lane + 64 * i, nio.blocks_in - 1)) * 2);
+    }
+    epi_c1 = nio.c1[min(n0 + col, N - 1)];
+  }
+  if constexpr (NORM == NORM_OUT) epi_gamma = nio.gamma_out[min(n0 + col, N - 1)];
   // never a conditional load; a step beyond K reads W's first block and meets zeros of A
   const int lrow = lane / 8, lch = lane % 8;               // as loader: row and 16-byte chunk of the pair's 128 bytes
   const bf16_t* a0 = A + static_cast<size_t>(min(lrow, M - 1)) * lda + lch * 8;
@@ -426,8 +473,37 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
   };
   bf16x8 b0[U][2];
   u32x4 al0[U][2];
+  // NORM_IN: the first round is asked for by every wave, with or without steps of its own (so that the
+  // wait for the statistics, which were asked for before, counts these loads exactly and depends on
+  // no branch), and the rows' statistics are joined while it travels
+  if (NORM == NORM_IN || wave < npairs) ask(wave, b0, al0);
+  if constexpr (NORM == NORM_IN) {
+    // the rows' means and 1 / sqrt(var + eps) for wave 0, which meets them behind the barrier further down
+    const float blocks = static_cast<float>(nio.blocks_in);
+#pragma unroll
+    for (int t = 0; t < SR; ++t) {
+      const int row = wave + t * WAVES;
+      float sm = 0.f;
+#pragma unroll
+      for (int i = 0; i < SP; ++i)
+        if (lane + 64 * i < nio.blocks_in) sm += st[t][i].x;
+      const float mean = wave_sum(sm) / blocks;
+      float sq = 0.f;
+#pragma unroll
+      for (int i = 0; i < SP; ++i)
+        if (lane + 64 * i < nio.blocks_in) {
+          const float d = st[t][i].x - mean;
+          sq += st[t][i].y + 16.f * d * d;
+        }
+      const float var = wave_sum(sq) / (16.f * blocks);
+      if (lane == 0) {
+        rowstat[row][0] = row < M ? mean : 0.f;
+        rowstat[row][1] = row < M ? 1.0f / sqrtf(var + nio.eps) : 0.f;
+      }
+    }
+  }
   for (int p0 = wave; p0 < npairs; p0 += WAVES * U) {
-    ask(p0, b0, al0);
+    if (p0 != wave) ask(p0, b0, al0);
     use(p0, b0, al0);
   }
   red[wave][lane] = acc;
@@ -442,13 +518,29 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
     for (int r = 0; r < 4; ++r) {
       const int m = g * 4 + r;
       if (m >= M || nn >= N) continue;
-      const float v = sm[r] + epi_bias;
+      float v = sm[r] + epi_bias;
+      if constexpr (NORM == NORM_IN) v = (sm[r] - rowstat[m][0] * epi_c1) * rowstat[m][1] + epi_bias;
       if (resid) {
         resid[static_cast<size_t>(m) * ldr + nn] = epi_x[r] + v;
+        if constexpr (NORM == NORM_OUT)
+          nio.copy_out[static_cast<size_t>(m) * nio.ldcopy + nn] = from_float<bf16_t>((epi_x[r] + v) * epi_gamma);
       } else {
         const TC cv = from_float<TC>(apply_epilogue_fast(v, epi));
         if (!KV || nn < kv.c_cols) C[static_cast<size_t>(m) * ldc + nn] = cv;
         if constexpr (KV) scatter_kv_at(kv, epi_slot[r], nn, cv);
+      }
+    }
+    if constexpr (NORM == NORM_OUT) {
+      // a row's 16 columns of this block lie in the 16 lanes of a row of lanes (N is a multiple of 16)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float x = epi_x[r] + (sm[r] + epi_bias);
+        const float mean = group_reduce<16>(x, SumOp()) * (1.0f / 16.0f);
+        const float d = x - mean;
+        const float sq = group_reduce<16>(d * d, SumOp());
+        const int m = g * 4 + r;
+        if (col == 0 && m < M)
+          *reinterpret_cast<float2*>(nio.stats_out + (static_cast<size_t>(m) * nblocks + blockIdx.x) * 2) = float2{mean, sq};
       }
     }
   }
@@ -481,7 +573,25 @@ static void launch16_one(const Call& c, hipStream_t stream) {
   KVScatter kv = c.kv ? *c.kv : KVScatter{};
   hipLaunchKernelGGL((gemm16_kernel<WAVES, TC, KV>), dim3((c.N + 15) / 16), dim3(WAVES * 64), 0, stream,
                      static_cast<const bf16_t*>(c.A), c.lda, static_cast<const bf16_t*>(c.W), c.bias,
-                     static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N, c.K, c.epi, kv);
+                     static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N, c.K, c.epi, kv, NormIO{});
+}
+
+// the same with the norm before the product (NORM_IN: bfloat16 out) or after it (NORM_OUT: into the residual stream)
+template <int WAVES>
+static void launch16_norm(const Call& c, const NormIO& nio, int norm, hipStream_t stream) {
+  KVScatter kv = c.kv ? *c.kv : KVScatter{};
+  const dim3 grid((c.N + 15) / 16), block(WAVES * 64);
+#define DN_L16(TC, KV, NORM)                                                                                        \
+  hipLaunchKernelGGL((gemm16_kernel<WAVES, TC, KV, NORM>), grid, block, 0, stream, static_cast<const bf16_t*>(c.A), \
+                     c.lda, static_cast<const bf16_t*>(c.W), c.bias, static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr,  \
+                     c.M, c.N, c.K, c.epi, kv, nio)
+  if (norm == NORM_OUT)
+    DN_L16(float, false, NORM_OUT);
+  else if (c.kv)
+    DN_L16(bf16_t, true, NORM_IN);
+  else
+    DN_L16(bf16_t, false, NORM_IN);
+#undef DN_L16
 }
 
 template <int WAVES>
@@ -1222,6 +1332,57 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
   else
     return DN_ERR_DTYPE;
 #undef DN_LAUNCH
+  return dn_launch_status();
+}
+
+// A product of at most 16 rows that adds into the residual stream and leaves what the norm after it
+// needs: resid [M, N] += A . W^T + bias; copy [M, ldcopy] = the updated rows times gamma [N] (that
+// norm's weight) in bfloat16; stats [M][N / 16][2] = mean and sum of squared distances from it of
+// each row's blocks of 16 columns.  A [M, K] bfloat16 in rows, W packed, N a multiple of 16.
+extern "C" int dn_gemm_norm_out(const void* A, int lda, const void* W, const float* bias, float* resid, int ldr, int M,
+                                int N, int K, const float* gamma, void* copy, int ldcopy, float* stats,
+                                hipStream_t stream) {
+  if (M < 1 || M > 16 || N < 16 || N % 16 != 0 || K < 8 || lda < K || ldr < N || ldcopy < N || !resid || !copy || !stats ||
+      !gamma)
+    return DN_ERR_SHAPE;
+  if (!skinny::takes(A, lda, W, M, K, PACKED_W)) return DN_ERR_SHAPE;
+  skinny::Call c{A, lda, W, bias, nullptr, 0, resid, ldr, M, N, K, DN_F32, EPI_NONE, PACKED_W, nullptr};
+  skinny::NormIO nio{nullptr, 0, nullptr, 0.f, gamma, static_cast<bf16_t*>(copy), ldcopy, stats};
+  if (K >= 1024)
+    skinny::launch16_norm<8>(c, nio, NORM_OUT, stream);
+  else
+    skinny::launch16_norm<4>(c, nio, NORM_OUT, stream);
+  return dn_launch_status();
+}
+
+// The product after such a norm: C [M, N] bfloat16 = act(LayerNorm(x) . W^T + b), where A is the
+// copy of x times gamma [M, K] and stats [M][K / 16][2] what dn_gemm_norm_out left (K a multiple of
+// 16, at most 4,096), c1[n] = sum_k gamma[k] W[n,k] and c2[n] = sum_k beta[k] W[n,k] + b[n].  With
+// slot_map, the key and value columns go to their pages as in dn_gemm_qkv.
+extern "C" int dn_gemm_norm_in(const void* A, int lda, const float* stats, const float* c1, const float* c2,
+                               float eps, const void* W, void* C, int ldc, int M, int N, int K,
+                               int epilogue, const int32_t* slot_map, void* k_pool, void* v_pool, int q_width,
+                               int Hkv, int dh, int page_size, int c_cols, hipStream_t stream) {
+  if (M < 1 || M > 16 || N < 1 || K < 16 || K % 16 != 0 || K > 4096 || lda < K || !stats || !c1 || !c2 || !C)
+    return DN_ERR_SHAPE;
+  if (epilogue < EPI_NONE || epilogue > EPI_GELU_ERF) return DN_ERR_SHAPE;
+  if (!skinny::takes(A, lda, W, M, K, PACKED_W) || reinterpret_cast<uintptr_t>(stats) % 8 != 0) return DN_ERR_SHAPE;
+  KVScatter kv{};
+  if (slot_map) {
+    if (q_width < 0 || q_width + 2 * Hkv * dh != N || page_size < 1 || !k_pool || !v_pool || epilogue != EPI_NONE)
+      return DN_ERR_SHAPE;
+    if ((c_cols != N && c_cols != q_width) || ldc < c_cols) return DN_ERR_SHAPE;
+    kv = KVScatter{slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_width, Hkv * dh, dh,
+                   page_size, Hkv, c_cols};
+  } else if (ldc < N) {
+    return DN_ERR_SHAPE;
+  }
+  skinny::Call c{A, lda, W, c2, C, ldc, nullptr, 0, M, N, K, DN_BF16, epilogue, PACKED_W, slot_map ? &kv : nullptr};
+  skinny::NormIO nio{stats, K / 16, c1, eps, nullptr, nullptr, 0, nullptr};
+  if (K >= 1024)
+    skinny::launch16_norm<8>(c, nio, NORM_IN, stream);
+  else
+    skinny::launch16_norm<4>(c, nio, NORM_IN, stream);
   return dn_launch_status();
 }
 

@@ -48,6 +48,8 @@ def _declare(name, lib):
         "gemm": {
             "dn_gemm": [P, I, P, P, P, I, P, I, I, I, I, I, I, I, I, P],
             "dn_pack_matrix": [P, P, I, I, P],
+            "dn_gemm_norm_out": [P, I, P, P, P, I, I, I, I, P, P, I, P, P],
+            "dn_gemm_norm_in": [P, I, P, P, P, F, P, P, I, I, I, I, I, P, P, P, I, I, I, I, I, P],
             "dn_gemm_qkv": [P, I, P, P, P, I, I, I, I, P, P, P, I, I, I, I, I, I, P],
         },
         "attention": {
@@ -476,3 +478,94 @@ def penalties(logits, ctx, ctx_start, repetition, frequency, presence, ngram):
                                       repetition.data_ptr(), frequency.data_ptr(), presence.data_ptr(),
                                       ngram.data_ptr(), _stream()), "penalties")
     return logits
+
+
+# ---------------------------------------------------------------------------------------
+# A norm that runs inside the products before and after it (steps of at most 16 rows)
+# ---------------------------------------------------------------------------------------
+NORM_STREAM_ROWS_MAX = 16     # 0 switches it off: norms then run as kernels of their own
+NORM_STREAM_WIDTH_MAX = 4096
+
+
+def norm_stream_takes(n_rows, width, w):
+    """Whether linear_norm_out can leave, and linear_norm_in can use, the statistics of n_rows rows
+    of `width` columns with the packed weight w."""
+    return (isinstance(w, PackedMatrix) and 1 <= n_rows <= NORM_STREAM_ROWS_MAX and width % 16 == 0
+            and 16 <= width <= NORM_STREAM_WIDTH_MAX)
+
+
+def norm_stream_buffers(n_rows, width, device):
+    """(copy, stats): the residual stream's rows times the next norm's weight, in bfloat16
+    [n_rows, width], and, per row and block of 16 columns, the mean and the sum of squared distances
+    from it [n_rows, width / 16, 2]."""
+    return (torch.empty((n_rows, width), dtype=torch.bfloat16, device=device),
+            torch.empty((n_rows, width // 16, 2), dtype=torch.float32, device=device))
+
+
+def norm_folded(w_rows, bias, gamma, beta):
+    """(c1, c2) for linear_norm_in: with y = (x - mean) / sqrt(var + eps) * gamma + beta,
+    y @ w.T + bias = ((x * gamma) @ w.T - mean * c1) / sqrt(var + eps) + c2, where
+    c1 = w @ gamma and c2 = w @ beta + bias, in 32-bit from the weight as the kernel holds it.
+    w_rows: [N, K] (any float dtype); made once per pair of norm and weight."""
+    w = w_rows.float()
+    c1 = w @ gamma.float()
+    c2 = torch.zeros_like(c1) if beta is None else w @ beta.float()
+    if bias is not None:
+        c2 = c2 + bias.float()
+    return c1.contiguous(), c2.contiguous()
+
+
+def linear_norm_out(a, w, bias, residual, gamma, copy, stats):
+    """residual += a @ w.T + bias (32-bit, in place), and what a LayerNorm of the updated rows with
+    weight gamma needs: copy = the rows times gamma in bfloat16, stats = each row's means and
+    squared distances by blocks of 16 columns.  a: bfloat16 [M, K] in rows, M <= 16; w: PackedMatrix
+    [N, K], N a multiple of 16."""
+    _dev(a, "a", (torch.bfloat16,), 2), _dev(residual, "residual", (torch.float32,), 2)
+    M, K = a.shape
+    N = w.shape[0]
+    _need(norm_stream_takes(M, N, w) and w.shape[1] == K and K % 8 == 0, "linear_norm_out: sizes it does not take")
+    _need(tuple(residual.shape) == (M, N) and tuple(copy.shape) == (M, N) and copy.dtype == torch.bfloat16
+          and tuple(stats.shape) == (M, N // 16, 2) and stats.dtype == torch.float32 and stats.is_contiguous(),
+          "linear_norm_out: residual, copy or stats")
+    for v, name in ((bias, "bias"), (gamma, "gamma")):
+        if v is not None:
+            _dev(v, name, (torch.float32,), 1)
+            _need(v.is_contiguous() and v.shape[0] == N, f"linear_norm_out: {name}")
+    _need(gamma is not None, "linear_norm_out: gamma")
+    _ok(_lib("gemm").dn_gemm_norm_out(a.data_ptr(), _rows(a, "a"), w.data_ptr(), _ptr(bias), residual.data_ptr(),
+                                      _rows(residual, "residual"), M, N, K, gamma.data_ptr(), copy.data_ptr(),
+                                      _rows(copy, "copy"), stats.data_ptr(), _stream()), "linear_norm_out")
+    return residual
+
+
+def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None):
+    """out = epilogue(LayerNorm(x) @ w.T + bias) where copy and stats are what linear_norm_out left
+    of x (with this norm's gamma) and c1, c2 = norm_folded(w, bias, gamma, beta).  out: bfloat16
+    [M, N]; kv = (slot_map, k_pool, v_pool, q_width): a fused projection whose key and value columns
+    go to the cache (out may then hold the queries alone); returns out, or the queries."""
+    _dev(copy, "copy", (torch.bfloat16,), 2), _dev(out, "out", (torch.bfloat16,), 2)
+    M, K = copy.shape
+    N = w.shape[0]
+    _need(norm_stream_takes(M, K, w) and w.shape[1] == K, "linear_norm_in: sizes it does not take")
+    _need(tuple(stats.shape) == (M, K // 16, 2) and stats.dtype == torch.float32 and stats.is_contiguous(),
+          "linear_norm_in: stats")
+    for v, name in ((c1, "c1"), (c2, "c2")):
+        _dev(v, name, (torch.float32,), 1)
+        _need(v.is_contiguous() and v.shape[0] == N, f"linear_norm_in: {name}")
+    if kv is None:
+        _need(tuple(out.shape) == (M, N), "linear_norm_in: out shape")
+        args = (0, 0, 0, 0, 0, 0, 0, 0)
+    else:
+        slot_map, k_pool, v_pool, q_width = kv
+        n_pages, Hkv, ps, dh = k_pool.shape
+        _need(N == q_width + 2 * Hkv * dh and out.shape[0] == M and out.shape[1] in (N, q_width),
+              "linear_norm_in: columns are not q | k | v, or out's shape")
+        _dev(slot_map, "slot_map", _I32, 1), _dev(k_pool, "k_pool", (torch.bfloat16,), 4)
+        _dev(v_pool, "v_pool", (torch.bfloat16,), 4)
+        _need(k_pool.is_contiguous() and v_pool.is_contiguous() and tuple(v_pool.shape) == (n_pages, Hkv, dh, ps)
+              and slot_map.is_contiguous() and slot_map.shape[0] == M and dh % 4 == 0, "linear_norm_in: pools or slot map")
+        args = (slot_map.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), q_width, Hkv, dh, ps, out.shape[1])
+    _ok(_lib("gemm").dn_gemm_norm_in(copy.data_ptr(), _rows(copy, "copy"), stats.data_ptr(), c1.data_ptr(),
+                                     c2.data_ptr(), float(eps), w.data_ptr(), out.data_ptr(), _rows(out, "out"),
+                                     M, N, K, EPILOGUES[epilogue], *args, _stream()), "linear_norm_in")
+    return out if kv is None else out[:, :kv[3]]

@@ -51,6 +51,11 @@ class Runtime:
     act_dtype: torch.dtype
     device: torch.device
     position: Optional["Part"] = None
+    # what the last part that added into the residual stream left for the norm after it (StreamStats),
+    # or None; the model clears it where the stream changes in any other way
+    stream_stats: Optional["StreamStats"] = None
+    # the norm that will read the stream first after the block that runs now (set by the model), or None
+    next_norm: Optional["Part"] = None
 
 
 class Part:
@@ -73,9 +78,48 @@ class Part:
         The default, a tensor [rows, width], is always right."""
         return False
 
+    def prepare_lazy_norm(self, norm) -> None:
+        """Called once, after binding, with the norm that stands before this part in its block: a part
+        that can run that norm inside its own first kernel makes ready for it here."""
+
+    def takes_lazy_norm(self, n_rows: int, norm) -> bool:
+        """A mixer or feed-forward whose first kernel can run `norm` itself for a step of n_rows rows,
+        given what the part before left (StreamStats), says so here; the block then hands it a
+        LazyNorm in place of the normed rows.  The default, normed rows, is always right."""
+        return False
+
+    def writes_norm_stats(self, n_rows: int) -> bool:
+        """A mixer or feed-forward whose last kernel, as it adds into the residual stream, can leave
+        the statistics for the norm after it; its forward then takes `stats=` (a StreamStats)."""
+        return False
+
     # helpers ---------------------------------------------------------------
     def _take(self, tensors, name):
         return tensors[name]
+
+
+class StreamStats:
+    """What one norm of the residual stream's rows needs, left by the kernel that last added into
+    the stream: the rows times that norm's weight, rounded to bfloat16, and per row and block of 16
+    columns the mean and the sum of squared distances from it (kernels.ops.linear_norm_out /
+    linear_norm_in).  `norm` is the norm it was made for: nobody else may use it."""
+
+    def __init__(self, copy, stats, norm):
+        self.copy, self.stats, self.norm = copy, stats, norm
+        self.written = False
+
+
+class LazyNorm:
+    """Rows that are not normed yet: a norm, the residual stream it is to read and the statistics
+    that were left for it.  Whoever receives it runs the norm inside its own kernel or asks for
+    the rows (`rows()`)."""
+
+    def __init__(self, norm, x, dtype, stream: StreamStats):
+        self.norm, self.x, self.dtype, self.stream = norm, x, dtype, stream
+        self.shape, self.device = x.shape, x.device
+
+    def rows(self, packed=False):
+        return self.norm.forward(self.x, self.dtype, packed=packed)
 
 
 class Registry(dict):

@@ -35,8 +35,17 @@ class DenseMLP(Part):
     def packed_input(self, n_rows):
         return self.up.packed_input(n_rows)
 
-    def forward(self, h, ctx, accumulate_into):
+    def prepare_lazy_norm(self, norm):
+        self.up.fold_norm(norm)
+
+    def takes_lazy_norm(self, n_rows, norm):
+        return self.up.takes_lazy_norm(n_rows, norm)
+
+    def writes_norm_stats(self, n_rows):
+        return self.down.writes_norm_stats(n_rows)
+
+    def forward(self, h, ctx, accumulate_into, stats=None):
         n = h.shape[0]
         f = self.up(h, out_dtype=self.runtime.act_dtype, epilogue=ACTIVATION_EPILOGUES[self.activation],
                     packed_out=self.up.few_rows(n) and self.down.packed_input(n))
-        self.down(f, residual=accumulate_into)
+        self.down(f, residual=accumulate_into, stats=stats)

@@ -11,6 +11,7 @@ import torch
 
 from ..kernels import ops
 from ..weights.spec import ParamSpec
+from .base import LazyNorm
 
 
 class Linear:
@@ -22,6 +23,7 @@ class Linear:
         self.init_std = init_std
         self.weight = None
         self.bias = None
+        self._folded = {}      # id(norm) -> (c1, c2, eps): see fold_norm
 
     def param_specs(self):
         shape = (self.in_features, self.out_features) if self.stored_in_out else (self.out_features, self.in_features)
@@ -50,14 +52,50 @@ class Linear:
         beyond 256 the many-rows kernels read rows)."""
         return self.few_rows(n_rows) and n_rows >= ops.PACKED_ROWS_MIN and self.in_features % 32 == 0
 
-    def __call__(self, a, out_dtype=None, epilogue="none", residual=None, packed_out=False):
+    def fold_norm(self, norm):
+        """Makes ready to run `norm` (the norm that stands before this product) inside the product's
+        own kernel: ops.norm_folded, once."""
+        f = getattr(norm, "fused_params", None)
+        if f is None or not ops.norm_stream_takes(1, self.in_features, self.weight):
+            return
+        kind, gamma, beta, eps = f()
+        if kind == "layernorm":
+            self._folded[id(norm)] = (*ops.norm_folded(self.weight.rows(), self.bias, gamma, beta), eps)
+
+    def takes_lazy_norm(self, n_rows: int, norm) -> bool:
+        """Whether a call with n_rows rows can run `norm` in its own kernel (fold_norm has been called)."""
+        return id(norm) in self._folded and ops.norm_stream_takes(n_rows, self.in_features, self.weight)
+
+    def writes_norm_stats(self, n_rows: int) -> bool:
+        """Whether a call with n_rows rows that adds into the residual stream can leave what the norm after it needs."""
+        return ops.norm_stream_takes(n_rows, self.out_features, self.weight) and self.in_features % 8 == 0
+
+    def _fusable(self, a, out_dtype):
+        """(c1, c2, eps) if `a` is a LazyNorm that this call can run in its own kernel."""
+        if ((out_dtype or a.dtype) == torch.bfloat16 and a.stream is not None and a.stream.written
+                and a.stream.norm is a.norm and self.takes_lazy_norm(a.shape[0], a.norm)):
+            return self._folded[id(a.norm)]
+        return None
+
+    def __call__(self, a, out_dtype=None, epilogue="none", residual=None, packed_out=False, stats=None):
         """epilogue(a @ W^T + b) as a new [M, out] tensor of out_dtype (as packed rows if
         packed_out, for a Linear whose packed_input said so), or added into `residual` (32-bit) in
         place.  An input in another precision than the weight is converted to the weight's (exact
         from bfloat16 to 32-bit)."""
+        if isinstance(a, LazyNorm):
+            f = self._fusable(a, out_dtype) if residual is None and not packed_out else None
+            if f is not None:
+                out = torch.empty((a.shape[0], self.out_features), dtype=torch.bfloat16, device=a.device)
+                return ops.linear_norm_in(a.stream.copy, a.stream.stats, f[0], f[1], f[2], self.weight, out, epilogue=epilogue)
+            a = a.rows(packed=self.packed_input(a.shape[0]))
         if a.dtype != self.weight.dtype:
             a = ops.cast(a.contiguous(), torch.empty(a.shape, dtype=self.weight.dtype, device=a.device))
         if residual is not None:
+            if (stats is not None and isinstance(a, torch.Tensor) and a.dtype == torch.bfloat16
+                    and self.writes_norm_stats(a.shape[0])):
+                stats.written = True
+                return ops.linear_norm_out(a, self.weight, self.bias, residual, stats.norm.fused_params()[1],
+                                           stats.copy, stats.stats)
             return ops.linear(a, self.weight, self.bias, residual=residual)
         if packed_out:
             out = ops.packed_rows(a.shape[0], self.out_features, a.device)
@@ -68,6 +106,13 @@ class Linear:
     def project_qkv(self, a, out_dtype, slot_map, k_pool, v_pool, q_width):
         """The fused projection: the key and value columns go to the cache's pages, the queries
         [M, q_width] come back (where one kernel does both, the other columns are stored nowhere else)."""
+        if isinstance(a, LazyNorm):
+            f = self._fusable(a, out_dtype)
+            if f is not None:
+                out = torch.empty((a.shape[0], q_width), dtype=torch.bfloat16, device=a.device)
+                return ops.linear_norm_in(a.stream.copy, a.stream.stats, f[0], f[1], f[2], self.weight, out,
+                                          kv=(slot_map, k_pool, v_pool, q_width))
+            a = a.rows(packed=self.packed_input(a.shape[0]))
         if a.dtype != self.weight.dtype:
             a = ops.cast(a.contiguous(), torch.empty(a.shape, dtype=self.weight.dtype, device=a.device))
         fused = isinstance(self.weight, ops.PackedMatrix) and out_dtype == torch.bfloat16

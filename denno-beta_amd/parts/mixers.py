@@ -47,7 +47,16 @@ class CausalSelfAttention(Part):
     def packed_input(self, n_rows):
         return self.qkv.packed_input(n_rows)
 
-    def forward(self, h, ctx, cache, accumulate_into):
+    def prepare_lazy_norm(self, norm):
+        self.qkv.fold_norm(norm)
+
+    def takes_lazy_norm(self, n_rows, norm):
+        return self.qkv.takes_lazy_norm(n_rows, norm)
+
+    def writes_norm_stats(self, n_rows):
+        return self.out.writes_norm_stats(n_rows)
+
+    def forward(self, h, ctx, cache, accumulate_into, stats=None):
         act = self.runtime.act_dtype
         g = ctx.groups[cache.group]
         position = self.runtime.position
@@ -72,4 +81,4 @@ class CausalSelfAttention(Part):
         ops.attention(q, o, cache.k, cache.v, g.block_tables, g.tiles, self.n_heads,
                       self.scale, self.window, tiles_wide=g.tiles_wide, single_rows=g.single_rows,
                       max_context=g.max_context)
-        self.out(o, residual=accumulate_into)
+        self.out(o, residual=accumulate_into, stats=stats)

@@ -143,6 +143,10 @@ class DecoderModel:
         else:
             self.head = Linear(self.spec.width, self.spec.vocab, self.spec.token_table, None)
             self.head.bind(tensors)
+        for b in self.blocks:
+            after = getattr(b, "after_bind", None)     # an arrangement may make its parts ready for each other
+            if after is not None:
+                after()
         return self
 
     def weight_bytes(self, tensors=None):
@@ -171,8 +175,13 @@ class DecoderModel:
         rt = self.runtime
         x = torch.empty((ctx.T, self.spec.width), dtype=torch.float32, device=rt.device)
         ops.embed(ctx.tokens, ctx.positions, self.embedding.weight, self.position.table(), x)
-        for call in self.spec.run_order:
+        rt.stream_stats = None      # nobody has left anything for a norm of these rows yet
+        order = self.spec.run_order
+        for i, call in enumerate(order):
+            nxt = self.blocks[order[i + 1].layer] if i + 1 < len(order) else None
+            rt.next_norm = nxt.first_norm() if nxt is not None and hasattr(nxt, "first_norm") else None
             self.blocks[call.layer].forward(x, ctx, cache.view(call.cache, call.writes_cache), rt)
+        rt.stream_stats = rt.next_norm = None
         if ctx.R == 0:
             return torch.empty((0, self.spec.vocab), dtype=torch.float32, device=rt.device)
         h = self.final_norm.forward(x, rt.act_dtype, rows=ctx.logit_rows, packed=self.head.packed_input(ctx.R))

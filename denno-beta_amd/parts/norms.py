@@ -29,6 +29,10 @@ class LayerNorm(Part):
         self.weight = tensors[self.weight_name]
         self.bias = tensors[self.bias_name] if self.bias_name else None
 
+    def fused_params(self):
+        """What a kernel that runs this norm itself needs (parts.base.LazyNorm)."""
+        return ("layernorm", self.weight, self.bias, self.eps)
+
     def forward(self, x, out_dtype, rows=None, packed=False):
         n = x.shape[0] if rows is None else rows.shape[0]
         if packed:

@@ -68,6 +68,44 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
     return out
 
 
+def norm_folded(w_rows, bias, gamma, beta):
+    w = w_rows.float()
+    c1 = w @ gamma.float()
+    c2 = torch.zeros_like(c1) if beta is None else w @ beta.float()
+    return c1, (c2 if bias is None else c2 + bias.float())
+
+
+def linear_norm_out(a, w, bias, residual, gamma, copy, stats):
+    linear(a, w, bias, residual=residual)
+    copy.copy_(residual * gamma)
+    blocks = residual.view(residual.shape[0], -1, 16)
+    mean = blocks.mean(dim=-1)
+    stats[:, :, 0] = mean
+    stats[:, :, 1] = ((blocks - mean[:, :, None]) ** 2).sum(dim=-1)
+    return residual
+
+
+def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None):
+    """The kernel's own formula: the product of the rows that are not normalised, then the row's mean
+    and 1 / sqrt(var + eps), joined from the blocks' pairs, on the sums."""
+    mean = stats[:, :, 0].mean(dim=1, keepdim=True)
+    var = (stats[:, :, 1] + 16.0 * (stats[:, :, 0] - mean) ** 2).sum(dim=1, keepdim=True) / copy.shape[1]
+    y = (copy.float() @ w.float().t() - mean * c1) / torch.sqrt(var + eps) + c2
+    if epilogue == "gelu_tanh":
+        y = torch.nn.functional.gelu(y, approximate="tanh")
+    elif epilogue == "gelu_erf":
+        y = torch.nn.functional.gelu(y)
+    if kv is None:
+        out.copy_(y)
+        return out
+    slot_map, k_pool, v_pool, q_width = kv
+    hkv, dh = k_pool.shape[1], k_pool.shape[3]
+    full = y.to(out.dtype)
+    kv_write(full, q_width, q_width + hkv * dh, slot_map, k_pool, v_pool)
+    out.copy_(full[:, :out.shape[1]])
+    return out[:, :q_width]
+
+
 def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, window=0, tiles_wide=None,
               single_rows=False, max_context=0):
     n_pages, hkv, ps, dh = k_pool.shape

@@ -181,6 +181,96 @@ def test_linear_qkv_writes_the_cache(M, slots_in, queries_only):
     assert pools[0].abs().sum() > 0 and pools[1].abs().sum() > 0
 
 
+@pytest.mark.parametrize("M,E,I,epilogue", [(1, 64, 256, "gelu_tanh"), (8, 1600, 6400, "gelu_tanh"), (5, 96, 320, "gelu_erf"),
+                                            (16, 1600, 4800, "none"), (13, 2560, 1024, "none"), (3, 4096, 4112, "gelu_tanh"),
+                                            (9, 16, 16, "none"), (2, 336, 1000, "none")])
+def test_a_norm_inside_the_products_on_both_sides_of_it(M, E, I, epilogue):
+    """x += a W1^T + b1 leaves the rows times gamma in bfloat16 and their statistics by blocks of 16
+    columns; the next product runs on those rows and applies the norm to its sums: against the plain
+    references of both, against the three kernels one after the other (product into the stream,
+    LayerNorm, product), and a row alone."""
+    a = rnd(M, I, seed=1, dtype=torch.bfloat16)
+    x0 = rnd(M, E, seed=2, scale=3.0) + 1.5                   # rows whose mean is half their spread
+    w1, b1 = rnd(E, I, seed=3, dtype=torch.bfloat16, scale=0.05), rnd(E, seed=4)
+    w2, b2 = rnd(I, E, seed=5, dtype=torch.bfloat16, scale=0.1), rnd(I, seed=6)
+    gamma, beta = 1 + rnd(E, seed=7, scale=0.1), rnd(E, seed=8, scale=0.1)
+    p1, p2 = ops().pack_matrix(w1), ops().pack_matrix(w2)
+    assert ops().norm_stream_takes(M, E, p1)
+    for b in (beta, None):
+        x = x0.clone()
+        copy, stats = ops().norm_stream_buffers(M, E, DEV)
+        copy.fill_(7.0), stats.fill_(7.0)
+        ops().linear_norm_out(a, p1, b1, x, gamma, copy, stats)
+        x_ref, copy_ref, stats_ref = x0.clone(), torch.empty_like(copy), torch.empty_like(stats)
+        R.linear_norm_out(a, w1, b1, x_ref, gamma, copy_ref, stats_ref)
+        x_two = ops().linear(a, p1, b1, residual=x0.clone())
+        assert torch.equal(x, x_two)                                # the same sums as the kernel that leaves nothing
+        assert torch.allclose(x, x_ref, atol=2e-2, rtol=2e-2)
+        assert torch.equal(copy, (x * gamma).to(torch.bfloat16))
+        assert torch.allclose(stats[:, :, 0], stats_ref[:, :, 0], atol=1e-3, rtol=1e-3)
+        assert torch.allclose(stats[:, :, 1], stats_ref[:, :, 1], atol=1e-2, rtol=1e-2)
+        c1, c2 = ops().norm_folded(p2.rows(), b2, gamma, b)
+        c1r, c2r = R.norm_folded(w2, b2, gamma, b)
+        assert torch.allclose(c1, c1r, atol=1e-4, rtol=1e-4) and torch.allclose(c2, c2r, atol=1e-4, rtol=1e-4)
+        out = torch.full((M, I), 7.0, dtype=torch.bfloat16, device=DEV)
+        ops().linear_norm_in(copy, stats, c1, c2, 1e-5, p2, out, epilogue=epilogue)
+        plain = R.linear_norm_in(copy, stats, c1, c2, 1e-5, w2, torch.empty_like(out), epilogue=epilogue)
+        assert torch.allclose(out.float(), plain.float(), atol=3e-2, rtol=2e-2), (M, E, I)
+        # against the norm as a kernel of its own on the 32-bit rows: here the rows are rounded to
+        # bfloat16 before the mean is taken off, there after; the two differ by roundings only
+        h = ops().layernorm(x, gamma, b, 1e-5, torch.empty(M, E, dtype=torch.bfloat16, device=DEV))
+        three = ops().linear(h, p2, b2, out=torch.empty_like(out), epilogue=epilogue)
+        assert (out.float() - three.float()).norm() <= 1e-2 * three.float().norm(), (M, E, I)
+    alone = torch.empty(1, I, dtype=torch.bfloat16, device=DEV)
+    ops().linear_norm_in(copy[M - 1:M].contiguous(), stats[M - 1:M].contiguous(), c1, c2, 1e-5, p2, alone, epilogue=epilogue)
+    assert torch.equal(alone[0], out[M - 1])
+
+
+def test_a_norm_inside_a_fused_projection_writes_the_cache():
+    H, Hkv, dh, ps, n_pages, E, M = 6, 2, 48, 16, 12, 160, 7
+    N = (H + 2 * Hkv) * dh
+    x = rnd(M, E, seed=1, scale=2.0) + 0.7
+    gamma, beta = 1 + rnd(E, seed=2, scale=0.1), rnd(E, seed=3, scale=0.1)
+    copy = (x * gamma).to(torch.bfloat16)
+    stats = torch.empty(M, E // 16, 2, device=DEV)
+    blocks = x.view(M, -1, 16)
+    stats[:, :, 0] = blocks.mean(-1)
+    stats[:, :, 1] = ((blocks - blocks.mean(-1, keepdim=True)) ** 2).sum(-1)
+    w, bias = rnd(N, E, seed=4, dtype=torch.bfloat16, scale=0.2), rnd(N, seed=5)
+    wp = ops().pack_matrix(w)
+    c1, c2 = ops().norm_folded(wp.rows(), bias, gamma, beta)
+    slots = torch.randperm(n_pages * ps, generator=torch.Generator().manual_seed(M))[:M].to(torch.int32)
+    slots[2] = -1
+    slots = slots.to(DEV)
+    for queries_only in (False, True):
+        pools = [torch.zeros(n_pages, Hkv, ps, dh, dtype=torch.bfloat16, device=DEV),
+                 torch.zeros(n_pages, Hkv, dh, ps, dtype=torch.bfloat16, device=DEV)]
+        want_pools = [torch.zeros_like(p) for p in pools]
+        out = torch.full((M, H * dh if queries_only else N), 7.0, dtype=torch.bfloat16, device=DEV)
+        queries = ops().linear_norm_in(copy, stats, c1, c2, 1e-5, wp, out, kv=(slots, pools[0], pools[1], H * dh))
+        want = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        ops().linear_norm_in(copy, stats, c1, c2, 1e-5, wp, want)
+        R.kv_write(want, H * dh, (H + Hkv) * dh, slots, want_pools[0], want_pools[1])
+        assert torch.equal(queries, want[:, :H * dh]) and (queries_only or torch.equal(out, want))
+        assert torch.equal(pools[0], want_pools[0]) and torch.equal(pools[1], want_pools[1])
+        assert pools[0].abs().sum() > 0 and pools[1].abs().sum() > 0
+    h = ops().layernorm(x, gamma, beta, 1e-5, torch.empty(M, E, dtype=torch.bfloat16, device=DEV))
+    two = ops().linear(h, wp, bias, out=torch.empty(M, N, dtype=torch.bfloat16, device=DEV))
+    assert (want.float() - two.float()).norm() <= 1e-2 * two.float().norm()
+
+
+def test_the_norm_inside_products_refuses_what_it_cannot_take():
+    wp = ops().pack_matrix(rnd(32, 64, seed=2, dtype=torch.bfloat16))
+    assert not ops().norm_stream_takes(17, 64, wp) and not ops().norm_stream_takes(4, 40, wp)
+    assert not ops().norm_stream_takes(4, 8192, wp) and not ops().norm_stream_takes(4, 64, rnd(32, 64, dtype=torch.bfloat16))
+    copy, stats = ops().norm_stream_buffers(17, 64, DEV)
+    c = rnd(32, seed=3)
+    with pytest.raises(ops().KernelError):
+        ops().linear_norm_in(copy, stats, c, c, 1e-5, wp, torch.empty(17, 32, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(ops().KernelError):
+        ops().linear_norm_out(rnd(17, 64, dtype=torch.bfloat16), wp, None, rnd(17, 32), c, *ops().norm_stream_buffers(17, 32, DEV))
+
+
 @pytest.mark.parametrize("M", [100, 129, 200, 256, 300])
 @pytest.mark.parametrize("rows_in", ["packed", "rows"])
 def test_linear_qkv_with_many_columns(M, rows_in):

@@ -438,3 +438,49 @@ def test_toy_rotation_and_toy_experts_are_registered_built_and_stepped(backend):
     assert torch.allclose(shifted, want[0], atol=2e-4)
     still = rotation_plain(spec, st, seqs[0], positions=torch.zeros(len(seqs[0])))
     assert (still - want[0]).abs().max() > 0.05
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,rows", [("A", 1), ("B", 7), ("D", 16)])
+def test_norms_that_run_inside_the_products_beside_them(model_folders, name, rows):
+    """In a step of at most 16 rows the block's norms are no kernels of their own: the product
+    before a norm leaves what it needs, the product after it applies it.  The same steps with every
+    norm as a kernel: logits agree to bfloat16 rounding, the cache holds the same keys but for
+    roundings, and the products with a norm inside did run (two a layer, less the first layer's
+    first, whose rows come from the embedding)."""
+    from denno_beta_amd.engine import ModelRunner, StepEntry
+    from denno_beta_amd.kernels import ops
+    cfg = TINY[name][0]
+    folder = model_folders(name, "bfloat16")
+    seq = seeded_tokens(5, 40 + rows, cfg["vocab_size"])
+    calls = {"in": 0, "out": 0}
+    real_in, real_out = ops.linear_norm_in, ops.linear_norm_out
+
+    def count_in(*a, **k):
+        calls["in"] += 1
+        return real_in(*a, **k)
+
+    def count_out(*a, **k):
+        calls["out"] += 1
+        return real_out(*a, **k)
+    got = {}
+    limit = ops.NORM_STREAM_ROWS_MAX
+    try:
+        ops.linear_norm_in, ops.linear_norm_out = count_in, count_out
+        for inside in (True, False):
+            ops.NORM_STREAM_ROWS_MAX = limit if inside else 0
+            r = ModelRunner.from_folder(folder, options("cuda:0", "bfloat16", use_graphs=False))
+            r.start_request(0)
+            r.step([StepEntry(0, seq[:40], [])])                          # 40 rows: norms as kernels either way
+            before = dict(calls)
+            got[inside] = r.step([StepEntry(0, seq[40:], list(range(rows)))]).float().cpu()
+            if inside:
+                assert calls["in"] - before["in"] == 2 * cfg["n_layer"] - 1
+                assert calls["out"] - before["out"] == 2 * cfg["n_layer"] - 1
+            else:
+                assert calls == before
+    finally:
+        ops.linear_norm_in, ops.linear_norm_out, ops.NORM_STREAM_ROWS_MAX = real_in, real_out, limit
+    U.assert_close(got[True], got[False], "bfloat16", f"{name}: norms inside the products against norms as kernels")
+    want = P.PlainGPT2.from_folder(folder).logits(seq)[40:]
+    U.assert_close(got[True], want, "bfloat16", f"{name}: norms inside the products against the plain implementation")

@@ -191,13 +191,42 @@ namespace skinny {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
+// The norm that stands between two such products of few rows runs inside them (NORM_OUT in the product before
+// it, NORM_IN in the one after), so that it is no kernel of its own: a LayerNorm of 8 rows is 4 us
+// of launch and latency for no work.  With y = (x - mean) / sqrt(var + eps) * gamma + beta
+// (crates/denno-engine/src/tensor.rs:1101-1112),
+//     y . W^T + b = ((x * gamma) . W^T - mean * c1) / sqrt(var + eps) + c2,
+//     c1[n] = sum_k gamma[k] W[n,k],  c2[n] = sum_k beta[k] W[n,k] + b[n]      (made once per weight),
+// so the product itself runs on rows that are not normalised, and the norm is two numbers per row in
+// the epilogue.  NORM_OUT: a product that adds into the residual stream also stores the updated rows
+// times gamma (the next norm's), rounded to bfloat16, and, for each row, the mean and the sum of
+// squared distances from it of its 16 columns.  NORM_IN: A is such a copy; each wave joins two rows'
+// N / 16 pairs (means are averaged; the squares add up with 16 times the squared distance of each
+// block's mean from the row's: exact, and as stable as two passes over the row) while the operands
+// travel, and wave 0 applies them at the end.  The rows are rounded to bfloat16 before the mean is
+// taken off, not after: right where a row's mean is not large beside its spread.
+struct NormIO {
+  const float* stats_in;     // NORM_IN: [M][blocks_in][2]
+  int blocks_in;             // K / 16
+  const float* c1;           // NORM_IN: [N]  (c2 comes as the bias)
+  float eps;
+  const float* gamma_out;    // NORM_OUT: [N] the next norm's weight
+  bf16_t* copy_out;          // NORM_OUT: [M, ldcopy] the updated rows times gamma_out in bfloat16
+  int ldcopy;
+  float* stats_out;          // NORM_OUT: [M][N / 16][2]
+};
+#define NORM_NONE 0
+#define NORM_IN 1
+#define NORM_OUT 2
+
+
 // MB row blocks and NB column blocks of 16 per workgroup; U steps of K in flight per wave.
-template <int MB, int NB, int WAVES, int U, typename TC, bool KV>
+template <int MB, int NB, int WAVES, int U, typename TC, bool KV, int NORM = NORM_NONE>
 __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restrict__ A, int lda,
                                                            const bf16_t* __restrict__ W,
                                                            const float* __restrict__ bias, TC* __restrict__ C,
                                                            int ldc, float* __restrict__ resid, int ldr, int M, int N,
-                                                           int K, int epi, int packed, KVScatter kv) {
+                                                           int K, int epi, int packed, KVScatter kv, NormIO nio) {
   constexpr int BLOCKS = MB * NB;                          // 16 x 16 blocks of C in this workgroup
   constexpr int PASSES = (BLOCKS + WAVES - 1) / WAVES;     // wave w finishes blocks w, w + WAVES, ...
   __shared__ floatx4 red[WAVES][BLOCKS][64];
@@ -218,10 +247,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   float epi_bias[PASSES];
   float epi_x[PASSES][4];
   int epi_slot[KV ? PASSES : 1][4];
+  float epi_norm[NORM != NORM_NONE ? PASSES : 1];          // NORM_IN: c1 of the lane's column; NORM_OUT: the next norm's gamma
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     const int blk = wave + p * WAVES;
     epi_bias[p] = 0.f;
+    if constexpr (NORM != NORM_NONE) {
+      const int nn = min(n0 + (blk < BLOCKS ? blk % NB : 0) * 16 + col, N - 1);
+      epi_norm[p] = NORM == NORM_IN ? nio.c1[nn] : nio.gamma_out[nn];
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) epi_x[p][r] = 0.f;
     if constexpr (KV) {
@@ -246,6 +280,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
           epi_x[p][r] = resid[static_cast<size_t>(m) * ldr + nn];
         }
       }
+    }
+  }
+  // NORM_IN: wave w joins the statistics of rows w, w + WAVES, ...: their pairs are asked for now, before
+  // the operands (up to SP * 64 blocks of 16 columns a row)
+  constexpr int SP = 2, SR = MB * 16 / WAVES;
+  __shared__ float rowstat[NORM == NORM_IN ? MB * 16 : 1][2];
+  float2 st[NORM == NORM_IN ? SR : 1][SP];
+  if constexpr (NORM == NORM_IN) {
+#pragma unroll
+    for (int t = 0; t < SR; ++t) {
+      const int row = min(wave + t * WAVES, M - 1);
+#pragma unroll
+      for (int i = 0; i < SP; ++i)
+        st[t][i] = *reinterpret_cast<const float2*>(nio.stats_in + (static_cast<size_t>(row) * nio.blocks_in + min(lane + 64 * i, nio.blocks_in - 1)) * 2);
     }
   }
   // Loads are never conditional and nothing uses a loaded value before all loads of a round are
@@ -274,6 +322,33 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
     arow[mb] = (packed & PACKED_A) ? A + (static_cast<size_t>(min(mb, (M + 15) / 16 - 1)) * ksteps * 64 + lane) * 8
                                    : A + static_cast<size_t>(a_ok[mb] ? row : 0) * lda + g * 8;
   }
+  // NORM_IN: the rows' means and 1 / sqrt(var + eps), joined while the first round of operands travels (a
+  // wave does it in its first turn of the loop below, which every wave has: K >= 1024); the finishing
+  // waves meet them behind the barrier further down
+  auto join_stats = [&]() {
+    const float blocks = static_cast<float>(nio.blocks_in);
+#pragma unroll
+    for (int t = 0; t < SR; ++t) {
+      const int row = wave + t * WAVES;
+      float sm = 0.f;
+#pragma unroll
+      for (int i = 0; i < SP; ++i)
+        if (lane + 64 * i < nio.blocks_in) sm += st[t][i].x;
+      const float mean = wave_sum(sm) / blocks;
+      float sq = 0.f;
+#pragma unroll
+      for (int i = 0; i < SP; ++i)
+        if (lane + 64 * i < nio.blocks_in) {
+          const float d = st[t][i].x - mean;
+          sq += st[t][i].y + 16.f * d * d;
+        }
+      const float var = wave_sum(sq) / (16.f * blocks);
+      if (lane == 0) {
+        rowstat[row][0] = row < M ? mean : 0.f;
+        rowstat[row][1] = row < M ? 1.0f / sqrtf(var + nio.eps) : 0.f;
+      }
+    }
+  };
   floatx4 acc[MB][NB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
@@ -295,6 +370,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
         a[u][mb] = *reinterpret_cast<const bf16x8*>(ok ? arow[mb] + ks * astep : arow[mb]);
+    }
+    if constexpr (NORM == NORM_IN) {
+      if (p0 == wave) join_stats();
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -327,13 +405,30 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
     floatx4 s = red[0][blk][lane];
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) s += red[w][blk][lane];
+    if constexpr (NORM == NORM_OUT) {
+      // a row's 16 columns of this block lie in the 16 lanes of a row of lanes (N is a multiple of 16)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float x = epi_x[p][r] + (s[r] + epi_bias[p]);
+        const float mean = group_reduce<16>(x, SumOp()) * (1.0f / 16.0f);
+        const float d = x - mean;
+        const float sq = group_reduce<16>(d * d, SumOp());
+        const int m = mb * 16 + g * 4 + r;
+        if (col == 0 && m < M)
+          *reinterpret_cast<float2*>(nio.stats_out + (static_cast<size_t>(m) * nblocks + blockIdx.x * NB + nb) * 2) = float2{mean, sq};
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       int m = mb * 16 + g * 4 + r;
       if (m >= M || nn >= N) continue;
       float v = s[r] + epi_bias[p];
+      if constexpr (NORM == NORM_IN) v = (s[r] - rowstat[m][0] * epi_norm[p]) * rowstat[m][1] + epi_bias[p];
       if (resid) {
         resid[static_cast<size_t>(m) * ldr + nn] = epi_x[p][r] + v;
+        if constexpr (NORM == NORM_OUT)
+          nio.copy_out[nio.ldcopy > 0 ? static_cast<size_t>(m) * nio.ldcopy + nn : packed_index(m, nn, N / 32)] =
+              from_float<bf16_t>((epi_x[p][r] + v) * epi_norm[p]);
       } else {
         TC cv = from_float<TC>(apply_epilogue_fast(v, epi));
         if (!KV || nn < kv.c_cols)
@@ -351,35 +446,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
 // line of 128 bytes; it loads A eight lanes to a row, turns each pair round through a piece of LDS
 // of its own (no barrier: a wave's LDS operations keep their order) and reads the operands from
 // there.  16 columns per workgroup, sums joined through LDS in wave order, as in gemm_kernel.
-//
-// The norm that stands between two such products runs inside them (NORM_OUT in the product before
-// it, NORM_IN in the one after), so that it is no kernel of its own: a LayerNorm of 8 rows is 4 us
-// of launch and latency for no work.  With y = (x - mean) / sqrt(var + eps) * gamma + beta
-// (crates/denno-engine/src/tensor.rs:1101-1112),
-//     y . W^T + b = ((x * gamma) . W^T - mean * c1) / sqrt(var + eps) + c2,
-//     c1[n] = sum_k gamma[k] W[n,k],  c2[n] = sum_k beta[k] W[n,k] + b[n]      (made once per weight),
-// so the product itself runs on rows that are not normalised, and the norm is two numbers per row in
-// the epilogue.  NORM_OUT: a product that adds into the residual stream also stores the updated rows
-// times gamma (the next norm's), rounded to bfloat16, and, for each row, the mean and the sum of
-// squared distances from it of its 16 columns.  NORM_IN: A is such a copy; each wave joins two rows'
-// N / 16 pairs (means are averaged; the squares add up with 16 times the squared distance of each
-// block's mean from the row's: exact, and as stable as two passes over the row) while the operands
-// travel, and wave 0 applies them at the end.  The rows are rounded to bfloat16 before the mean is
-// taken off, not after: right where a row's mean is not large beside its spread.
-struct NormIO {
-  const float* stats_in;     // NORM_IN: [M][blocks_in][2]
-  int blocks_in;             // K / 16
-  const float* c1;           // NORM_IN: [N]  (c2 comes as the bias)
-  float eps;
-  const float* gamma_out;    // NORM_OUT: [N] the next norm's weight
-  bf16_t* copy_out;          // NORM_OUT: [M, ldcopy] the updated rows times gamma_out in bfloat16
-  int ldcopy;
-  float* stats_out;          // NORM_OUT: [M][N / 16][2]
-};
-#define NORM_NONE 0
-#define NORM_IN 1
-#define NORM_OUT 2
-
 template <int WAVES, typename TC, bool KV, int NORM = NORM_NONE>
 __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __restrict__ A, int lda,
                                                              const bf16_t* __restrict__ W,
@@ -558,7 +624,43 @@ static void launch_one(const Call& c, hipStream_t stream) {
   KVScatter kv = c.kv ? *c.kv : KVScatter{};
   hipLaunchKernelGGL((gemm_kernel<MB, NB, WAVES, U, TC, KV>), grid, block, 0, stream,
                      static_cast<const bf16_t*>(c.A), c.lda, static_cast<const bf16_t*>(c.W), c.bias,
-                     static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N, c.K, c.epi, c.packed, kv);
+                     static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N, c.K, c.epi, c.packed, kv, NormIO{});
+}
+
+// the same with the norm before the product (NORM_IN: bfloat16 out) or after it (NORM_OUT: into the
+// residual stream), for 17 to 64 rows
+template <int MB, int NB, int WAVES, int U>
+static void launch_norm(const Call& c, const NormIO& nio, int norm, hipStream_t stream) {
+  dim3 grid((c.N + 16 * NB - 1) / (16 * NB)), block(WAVES * 64);
+  KVScatter kv = c.kv ? *c.kv : KVScatter{};
+#define DN_LN(TC, KV, NORM)                                                                                        \
+  hipLaunchKernelGGL((gemm_kernel<MB, NB, WAVES, U, TC, KV, NORM>), grid, block, 0, stream,                       \
+                     static_cast<const bf16_t*>(c.A), c.lda, static_cast<const bf16_t*>(c.W), c.bias,             \
+                     static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N, c.K, c.epi, c.packed, kv, nio)
+  if (norm == NORM_OUT)
+    DN_LN(float, false, NORM_OUT);
+  else if (c.kv)
+    DN_LN(bf16_t, true, NORM_IN);
+  else
+    DN_LN(bf16_t, false, NORM_IN);
+#undef DN_LN
+}
+
+// 17 to 64 rows with a norm inside: the shapes that launch_mb picks for these rows (8 waves: K >= 1024)
+static void launch_mb_norm(const Call& c, const NormIO& nio, int norm, hipStream_t stream) {
+  const int mb = (c.M + 15) / 16;
+  if (c.N >= 4096) {
+    switch (mb) {
+      case 2: return launch_norm<2, 2, 8, 4>(c, nio, norm, stream);
+      case 3: return launch_norm<3, 2, 8, 4>(c, nio, norm, stream);
+      default: return launch_norm<4, 2, 8, 4>(c, nio, norm, stream);
+    }
+  }
+  switch (mb) {
+    case 2: return launch_norm<2, 1, 8, 8>(c, nio, norm, stream);
+    case 3: return launch_norm<3, 1, 8, 8>(c, nio, norm, stream);
+    default: return launch_norm<4, 1, 8, 8>(c, nio, norm, stream);
+  }
 }
 
 template <int MB, int NB, int WAVES, int U>
@@ -1335,20 +1437,25 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
   return dn_launch_status();
 }
 
-// A product of at most 16 rows that adds into the residual stream and leaves what the norm after it
-// needs: resid [M, N] += A . W^T + bias; copy [M, ldcopy] = the updated rows times gamma [N] (that
-// norm's weight) in bfloat16; stats [M][N / 16][2] = mean and sum of squared distances from it of
-// each row's blocks of 16 columns.  A [M, K] bfloat16 in rows, W packed, N a multiple of 16.
+// A product of few rows that adds into the residual stream and leaves what the norm after it needs:
+// resid [M, N] += A . W^T + bias; copy = the updated rows times gamma [N] (that norm's weight) in
+// bfloat16, in rows of ldcopy elements or (ldcopy == 0, N a multiple of 32) as packed rows; stats
+// [M][N / 16][2] = mean and sum of squared distances from it of each row's blocks of 16 columns.
+// A [M, K] bfloat16 in rows or (lda == 0) packed, W packed, N a multiple of 16.  Up to 16 rows (A in
+// rows), or 17 to 64 rows with K >= 1024.
 extern "C" int dn_gemm_norm_out(const void* A, int lda, const void* W, const float* bias, float* resid, int ldr, int M,
                                 int N, int K, const float* gamma, void* copy, int ldcopy, float* stats,
                                 hipStream_t stream) {
-  if (M < 1 || M > 16 || N < 16 || N % 16 != 0 || K < 8 || lda < K || ldr < N || ldcopy < N || !resid || !copy || !stats ||
-      !gamma)
-    return DN_ERR_SHAPE;
-  if (!skinny::takes(A, lda, W, M, K, PACKED_W)) return DN_ERR_SHAPE;
-  skinny::Call c{A, lda, W, bias, nullptr, 0, resid, ldr, M, N, K, DN_F32, EPI_NONE, PACKED_W, nullptr};
+  if (M < 1 || M > 64 || N < 16 || N % 16 != 0 || K < 8 || ldr < N || !resid || !copy || !stats || !gamma) return DN_ERR_SHAPE;
+  if ((lda != 0 && lda < K) || (ldcopy != 0 && ldcopy < N) || (ldcopy == 0 && N % 32 != 0)) return DN_ERR_SHAPE;
+  if (M <= 16 ? lda == 0 : K < 1024) return DN_ERR_SHAPE;
+  const int packed = PACKED_W | (lda == 0 ? PACKED_A : 0);
+  if (!skinny::takes(A, lda, W, M, K, packed)) return DN_ERR_SHAPE;
+  skinny::Call c{A, lda, W, bias, nullptr, 0, resid, ldr, M, N, K, DN_F32, EPI_NONE, packed, nullptr};
   skinny::NormIO nio{nullptr, 0, nullptr, 0.f, gamma, static_cast<bf16_t*>(copy), ldcopy, stats};
-  if (K >= 1024)
+  if (M > 16)
+    skinny::launch_mb_norm(c, nio, NORM_OUT, stream);
+  else if (K >= 1024)
     skinny::launch16_norm<8>(c, nio, NORM_OUT, stream);
   else
     skinny::launch16_norm<4>(c, nio, NORM_OUT, stream);
@@ -1356,17 +1463,21 @@ extern "C" int dn_gemm_norm_out(const void* A, int lda, const void* W, const flo
 }
 
 // The product after such a norm: C [M, N] bfloat16 = act(LayerNorm(x) . W^T + b), where A is the
-// copy of x times gamma [M, K] and stats [M][K / 16][2] what dn_gemm_norm_out left (K a multiple of
-// 16, at most 4,096), c1[n] = sum_k gamma[k] W[n,k] and c2[n] = sum_k beta[k] W[n,k] + b[n].  With
-// slot_map, the key and value columns go to their pages as in dn_gemm_qkv.
+// copy of x times gamma [M, K] (in rows, or lda == 0: packed rows) and stats [M][K / 16][2] what
+// dn_gemm_norm_out left, c1[n] = sum_k gamma[k] W[n,k] and c2[n] = sum_k beta[k] W[n,k] + b[n].
+// Up to 16 rows (A in rows, K a multiple of 16 up to 4,096), or 17 to 64 rows (K from 1,024 to 2,048).
+// With slot_map, the key and value columns go to their pages as in dn_gemm_qkv; without, ldc == 0 asks
+// for C in packed rows (17 rows and more, N a multiple of 32).
 extern "C" int dn_gemm_norm_in(const void* A, int lda, const float* stats, const float* c1, const float* c2,
                                float eps, const void* W, void* C, int ldc, int M, int N, int K,
                                int epilogue, const int32_t* slot_map, void* k_pool, void* v_pool, int q_width,
                                int Hkv, int dh, int page_size, int c_cols, hipStream_t stream) {
-  if (M < 1 || M > 16 || N < 1 || K < 16 || K % 16 != 0 || K > 4096 || lda < K || !stats || !c1 || !c2 || !C)
+  if (M < 1 || M > 64 || N < 1 || K < 16 || K % 16 != 0 || K > 4096 || (lda != 0 && lda < K) || !stats || !c1 || !c2 || !C)
     return DN_ERR_SHAPE;
+  if (M <= 16 ? lda == 0 : (K < 1024 || K > 2048)) return DN_ERR_SHAPE;
   if (epilogue < EPI_NONE || epilogue > EPI_GELU_ERF) return DN_ERR_SHAPE;
-  if (!skinny::takes(A, lda, W, M, K, PACKED_W) || reinterpret_cast<uintptr_t>(stats) % 8 != 0) return DN_ERR_SHAPE;
+  const int packed = PACKED_W | (lda == 0 ? PACKED_A : 0);
+  if (!skinny::takes(A, lda, W, M, K, packed) || reinterpret_cast<uintptr_t>(stats) % 8 != 0) return DN_ERR_SHAPE;
   KVScatter kv{};
   if (slot_map) {
     if (q_width < 0 || q_width + 2 * Hkv * dh != N || page_size < 1 || !k_pool || !v_pool || epilogue != EPI_NONE)
@@ -1374,12 +1485,15 @@ extern "C" int dn_gemm_norm_in(const void* A, int lda, const float* stats, const
     if ((c_cols != N && c_cols != q_width) || ldc < c_cols) return DN_ERR_SHAPE;
     kv = KVScatter{slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_width, Hkv * dh, dh,
                    page_size, Hkv, c_cols};
-  } else if (ldc < N) {
+  } else if (ldc == 0 ? (M <= 16 || N % 32 != 0) : ldc < N) {      // ldc == 0: C in packed rows (17 rows and more)
     return DN_ERR_SHAPE;
   }
-  skinny::Call c{A, lda, W, c2, C, ldc, nullptr, 0, M, N, K, DN_BF16, epilogue, PACKED_W, slot_map ? &kv : nullptr};
+  skinny::Call c{A, lda, W, c2, C, ldc, nullptr, 0, M, N, K, DN_BF16, epilogue, packed | (ldc == 0 ? PACKED_C : 0),
+                 slot_map ? &kv : nullptr};
   skinny::NormIO nio{stats, K / 16, c1, eps, nullptr, nullptr, 0, nullptr};
-  if (K >= 1024)
+  if (M > 16)
+    skinny::launch_mb_norm(c, nio, NORM_IN, stream);
+  else if (K >= 1024)
     skinny::launch16_norm<8>(c, nio, NORM_IN, stream);
   else
     skinny::launch16_norm<4>(c, nio, NORM_IN, stream);

@@ -483,23 +483,30 @@ def penalties(logits, ctx, ctx_start, repetition, frequency, presence, ngram):
 # ---------------------------------------------------------------------------------------
 # A norm that runs inside the products before and after it (steps of at most 16 rows)
 # ---------------------------------------------------------------------------------------
-NORM_STREAM_ROWS_MAX = 16     # 0 switches it off: norms then run as kernels of their own
+NORM_STREAM_ROWS_MAX = 64     # 0 switches it off: norms then run as kernels of their own
 NORM_STREAM_WIDTH_MAX = 4096
 
 
 def norm_stream_takes(n_rows, width, w):
-    """Whether linear_norm_out can leave, and linear_norm_in can use, the statistics of n_rows rows
-    of `width` columns with the packed weight w."""
-    return (isinstance(w, PackedMatrix) and 1 <= n_rows <= NORM_STREAM_ROWS_MAX and width % 16 == 0
-            and 16 <= width <= NORM_STREAM_WIDTH_MAX)
+    """Whether linear_norm_out can leave, and linear_norm_in can use, what a norm of n_rows rows of
+    `width` columns needs, with the packed weight w [out, in] of the product in question.  Up to 16
+    rows: widths that are multiples of 16, up to 4,096.  17 to 64 rows (the rows then travel
+    packed): widths that are multiples of 32 from 1,024 to 2,048, and products of at least 1,024 inner
+    columns."""
+    if not isinstance(w, PackedMatrix) or not 1 <= n_rows <= NORM_STREAM_ROWS_MAX:
+        return False
+    if n_rows <= 16:
+        return width % 16 == 0 and 16 <= width <= NORM_STREAM_WIDTH_MAX
+    return n_rows <= 64 and width % 32 == 0 and 1024 <= width <= 2048 and w.shape[1] >= 1024
 
 
 def norm_stream_buffers(n_rows, width, device):
-    """(copy, stats): the residual stream's rows times the next norm's weight, in bfloat16
-    [n_rows, width], and, per row and block of 16 columns, the mean and the sum of squared distances
-    from it [n_rows, width / 16, 2]."""
-    return (torch.empty((n_rows, width), dtype=torch.bfloat16, device=device),
-            torch.empty((n_rows, width // 16, 2), dtype=torch.float32, device=device))
+    """(copy, stats): the residual stream's rows times the next norm's weight, in bfloat16 ([n_rows,
+    width], from 17 rows on as packed rows), and, per row and block of 16 columns, the mean and
+    the sum of squared distances from it [n_rows, width / 16, 2]."""
+    copy = (packed_rows(n_rows, width, device) if n_rows >= PACKED_ROWS_MIN else
+            torch.empty((n_rows, width), dtype=torch.bfloat16, device=device))
+    return copy, torch.empty((n_rows, width // 16, 2), dtype=torch.float32, device=device)
 
 
 def norm_folded(w_rows, bias, gamma, beta):
@@ -515,26 +522,37 @@ def norm_folded(w_rows, bias, gamma, beta):
     return c1.contiguous(), c2.contiguous()
 
 
+def _rows_or_packed(t, name, M, width):
+    """The leading dimension of a bfloat16 [M, width] tensor in rows, or 0 for packed rows."""
+    if isinstance(t, PackedMatrix):
+        _need(tuple(t.shape) == (M, width) and width % 32 == 0, f"{name}: packed rows of another shape")
+        return 0
+    _dev(t, name, (torch.bfloat16,), 2)
+    _need(tuple(t.shape) == (M, width), f"{name}: shape")
+    return _rows(t, name)
+
+
 def linear_norm_out(a, w, bias, residual, gamma, copy, stats):
     """residual += a @ w.T + bias (32-bit, in place), and what a LayerNorm of the updated rows with
-    weight gamma needs: copy = the rows times gamma in bfloat16, stats = each row's means and
-    squared distances by blocks of 16 columns.  a: bfloat16 [M, K] in rows, M <= 16; w: PackedMatrix
-    [N, K], N a multiple of 16."""
-    _dev(a, "a", (torch.bfloat16,), 2), _dev(residual, "residual", (torch.float32,), 2)
+    weight gamma needs: copy = the rows times gamma in bfloat16 (a tensor, or packed rows), stats =
+    each row's means and squared distances by blocks of 16 columns.  a: bfloat16 [M, K] in rows or
+    packed rows; w: PackedMatrix [N, K], N a multiple of 16."""
+    _dev(residual, "residual", (torch.float32,), 2)
     M, K = a.shape
     N = w.shape[0]
     _need(norm_stream_takes(M, N, w) and w.shape[1] == K and K % 8 == 0, "linear_norm_out: sizes it does not take")
-    _need(tuple(residual.shape) == (M, N) and tuple(copy.shape) == (M, N) and copy.dtype == torch.bfloat16
-          and tuple(stats.shape) == (M, N // 16, 2) and stats.dtype == torch.float32 and stats.is_contiguous(),
-          "linear_norm_out: residual, copy or stats")
+    lda, ldcopy = _rows_or_packed(a, "a", M, K), _rows_or_packed(copy, "copy", M, N)
+    _need(M > 16 or lda > 0, "linear_norm_out: up to 16 rows come in rows")
+    _need(tuple(residual.shape) == (M, N) and tuple(stats.shape) == (M, N // 16, 2) and stats.dtype == torch.float32
+          and stats.is_contiguous(), "linear_norm_out: residual or stats")
     for v, name in ((bias, "bias"), (gamma, "gamma")):
         if v is not None:
             _dev(v, name, (torch.float32,), 1)
             _need(v.is_contiguous() and v.shape[0] == N, f"linear_norm_out: {name}")
     _need(gamma is not None, "linear_norm_out: gamma")
-    _ok(_lib("gemm").dn_gemm_norm_out(a.data_ptr(), _rows(a, "a"), w.data_ptr(), _ptr(bias), residual.data_ptr(),
+    _ok(_lib("gemm").dn_gemm_norm_out(a.data_ptr(), lda, w.data_ptr(), _ptr(bias), residual.data_ptr(),
                                       _rows(residual, "residual"), M, N, K, gamma.data_ptr(), copy.data_ptr(),
-                                      _rows(copy, "copy"), stats.data_ptr(), _stream()), "linear_norm_out")
+                                      ldcopy, stats.data_ptr(), _stream()), "linear_norm_out")
     return residual
 
 
@@ -543,10 +561,17 @@ def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None):
     of x (with this norm's gamma) and c1, c2 = norm_folded(w, bias, gamma, beta).  out: bfloat16
     [M, N]; kv = (slot_map, k_pool, v_pool, q_width): a fused projection whose key and value columns
     go to the cache (out may then hold the queries alone); returns out, or the queries."""
-    _dev(copy, "copy", (torch.bfloat16,), 2), _dev(out, "out", (torch.bfloat16,), 2)
     M, K = copy.shape
     N = w.shape[0]
     _need(norm_stream_takes(M, K, w) and w.shape[1] == K, "linear_norm_in: sizes it does not take")
+    if isinstance(out, PackedMatrix):
+        _need(kv is None and M > 16 and N % 32 == 0, "linear_norm_in: packed rows as out need 17 rows or more, N a multiple of 32, no cache write")
+        ldc = 0
+    else:
+        _dev(out, "out", (torch.bfloat16,), 2)
+        ldc = _rows(out, "out")
+    lda = _rows_or_packed(copy, "copy", M, K)
+    _need(M > 16 or lda > 0, "linear_norm_in: up to 16 rows come in rows")
     _need(tuple(stats.shape) == (M, K // 16, 2) and stats.dtype == torch.float32 and stats.is_contiguous(),
           "linear_norm_in: stats")
     for v, name in ((c1, "c1"), (c2, "c2")):
@@ -565,7 +590,7 @@ def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None):
         _need(k_pool.is_contiguous() and v_pool.is_contiguous() and tuple(v_pool.shape) == (n_pages, Hkv, dh, ps)
               and slot_map.is_contiguous() and slot_map.shape[0] == M and dh % 4 == 0, "linear_norm_in: pools or slot map")
         args = (slot_map.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), q_width, Hkv, dh, ps, out.shape[1])
-    _ok(_lib("gemm").dn_gemm_norm_in(copy.data_ptr(), _rows(copy, "copy"), stats.data_ptr(), c1.data_ptr(),
-                                     c2.data_ptr(), float(eps), w.data_ptr(), out.data_ptr(), _rows(out, "out"),
+    _ok(_lib("gemm").dn_gemm_norm_in(copy.data_ptr(), lda, stats.data_ptr(), c1.data_ptr(),
+                                     c2.data_ptr(), float(eps), w.data_ptr(), out.data_ptr(), ldc,
                                      M, N, K, EPILOGUES[epilogue], *args, _stream()), "linear_norm_in")
     return out if kv is None else out[:, :kv[3]]

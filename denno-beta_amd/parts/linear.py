@@ -56,7 +56,8 @@ class Linear:
         """Makes ready to run `norm` (the norm that stands before this product) inside the product's
         own kernel: ops.norm_folded, once."""
         f = getattr(norm, "fused_params", None)
-        if f is None or not ops.norm_stream_takes(1, self.in_features, self.weight):
+        if f is None or not (ops.norm_stream_takes(1, self.in_features, self.weight)
+                             or ops.norm_stream_takes(17, self.in_features, self.weight)):
             return
         kind, gamma, beta, eps = f()
         if kind == "layernorm":
@@ -83,16 +84,16 @@ class Linear:
         place.  An input in another precision than the weight is converted to the weight's (exact
         from bfloat16 to 32-bit)."""
         if isinstance(a, LazyNorm):
-            f = self._fusable(a, out_dtype) if residual is None and not packed_out else None
+            f = self._fusable(a, out_dtype) if residual is None and not (packed_out and a.shape[0] <= 16) else None
             if f is not None:
-                out = torch.empty((a.shape[0], self.out_features), dtype=torch.bfloat16, device=a.device)
+                out = (ops.packed_rows(a.shape[0], self.out_features, a.device) if packed_out else
+                       torch.empty((a.shape[0], self.out_features), dtype=torch.bfloat16, device=a.device))
                 return ops.linear_norm_in(a.stream.copy, a.stream.stats, f[0], f[1], f[2], self.weight, out, epilogue=epilogue)
             a = a.rows(packed=self.packed_input(a.shape[0]))
         if a.dtype != self.weight.dtype:
             a = ops.cast(a.contiguous(), torch.empty(a.shape, dtype=self.weight.dtype, device=a.device))
         if residual is not None:
-            if (stats is not None and isinstance(a, torch.Tensor) and a.dtype == torch.bfloat16
-                    and self.writes_norm_stats(a.shape[0])):
+            if stats is not None and a.dtype == torch.bfloat16 and self.writes_norm_stats(a.shape[0]):
                 stats.written = True
                 return ops.linear_norm_out(a, self.weight, self.bias, residual, stats.norm.fused_params()[1],
                                            stats.copy, stats.stats)

@@ -27,7 +27,11 @@ TINY_D = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n
 # 129 to 256 rows change kernels
 WIDE_E = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=1, n_embd=1408, n_head=22,
               vocab_size=300, n_positions=64, layer_norm_epsilon=1e-5, activation_function="gelu_new")
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3), "E": (WIDE_E, 4)}
+# a sixth, two layers of 1,024 columns: the least width at which steps of 17 to 64 rows run their norms
+# inside the products beside them, across the blocks' border too
+WIDE_F = dict(architectures=["GPT2LMHeadModel"], model_type="gpt2", n_layer=2, n_embd=1024, n_head=16,
+              vocab_size=300, n_positions=64, layer_norm_epsilon=1e-5, activation_function="gelu")
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3), "E": (WIDE_E, 4), "F": (WIDE_F, 5)}
 
 
 def pytest_configure(config):

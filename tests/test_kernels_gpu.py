@@ -226,6 +226,50 @@ def test_a_norm_inside_the_products_on_both_sides_of_it(M, E, I, epilogue):
     assert torch.equal(alone[0], out[M - 1])
 
 
+@pytest.mark.parametrize("M,E,I,epilogue", [(17, 1600, 6400, "gelu_tanh"), (40, 1408, 5632, "none"), (64, 1600, 4800, "gelu_tanh"),
+                                            (33, 1024, 1040, "none"), (50, 2048, 4096, "gelu_erf")])
+@pytest.mark.parametrize("layout", ["packed", "rows"])
+def test_a_norm_inside_products_of_17_to_64_rows(M, E, I, epilogue, layout):
+    """The same with the rows travelling packed, as they do from 17 rows on, or in rows: the product
+    into the stream reads packed rows and leaves a packed copy, the product after it reads that and
+    writes packed rows."""
+    pk = layout == "packed"
+    a = rnd(M, I, seed=1, dtype=torch.bfloat16)
+    x0 = rnd(M, E, seed=2, scale=3.0) + 1.5
+    w1, b1 = rnd(E, I, seed=3, dtype=torch.bfloat16, scale=0.05), rnd(E, seed=4)
+    w2, b2 = rnd(I, E, seed=5, dtype=torch.bfloat16, scale=0.1), rnd(I, seed=6)
+    gamma, beta = 1 + rnd(E, seed=7, scale=0.1), rnd(E, seed=8, scale=0.1)
+    p1, p2 = ops().pack_matrix(w1), ops().pack_matrix(w2)
+    assert ops().norm_stream_takes(M, E, p1) and ops().norm_stream_takes(M, E, p2)
+    x = x0.clone()
+    copy, stats = ops().norm_stream_buffers(M, E, DEV)
+    assert isinstance(copy, ops().PackedMatrix)
+    if not pk:
+        copy = torch.empty(M, E, dtype=torch.bfloat16, device=DEV)
+    ops().linear_norm_out(ops().pack_matrix(a) if pk and I % 32 == 0 else a, p1, b1, x, gamma, copy, stats)
+    x_two = ops().linear(a, p1, b1, residual=x0.clone())
+    assert torch.allclose(x, x_two, atol=1e-4, rtol=1e-5)          # the same product from rows and from packed rows
+    copy_rows = copy.rows() if pk else copy
+    assert torch.equal(copy_rows, (x * gamma).to(torch.bfloat16))
+    stats_ref = torch.empty_like(stats)
+    R.linear_norm_out(a, w1, b1, x0.clone(), gamma, torch.empty(M, E, dtype=torch.bfloat16, device=DEV), stats_ref)
+    assert torch.allclose(stats[:, :, 0], stats_ref[:, :, 0], atol=1e-3, rtol=1e-3)
+    assert torch.allclose(stats[:, :, 1], stats_ref[:, :, 1], atol=1e-2, rtol=1e-2)
+    c1, c2 = ops().norm_folded(p2.rows(), b2, gamma, beta)
+    out = ops().packed_rows(M, I, DEV) if pk and I % 32 == 0 else torch.full((M, I), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops().linear_norm_in(copy, stats, c1, c2, 1e-5, p2, out, epilogue=epilogue)
+    out_rows = out.rows() if isinstance(out, ops().PackedMatrix) else out
+    plain = R.linear_norm_in(copy_rows, stats, c1, c2, 1e-5, w2, torch.empty(M, I, dtype=torch.bfloat16, device=DEV), epilogue=epilogue)
+    assert torch.allclose(out_rows.float(), plain.float(), atol=3e-2, rtol=2e-2), (M, E, I)
+    h = ops().layernorm(x, gamma, beta, 1e-5, torch.empty(M, E, dtype=torch.bfloat16, device=DEV))
+    three = ops().linear(h, p2, b2, out=torch.empty(M, I, dtype=torch.bfloat16, device=DEV), epilogue=epilogue)
+    assert (out_rows.float() - three.float()).norm() <= 1e-2 * three.float().norm(), (M, E, I)
+    # the same rows among 16 give the same as among M (another kernel: to rounding)
+    few_copy, few_stats = copy_rows[:16].contiguous(), stats[:16].contiguous()
+    few = ops().linear_norm_in(few_copy, few_stats, c1, c2, 1e-5, p2, torch.empty(16, I, dtype=torch.bfloat16, device=DEV), epilogue=epilogue)
+    assert torch.allclose(few.float(), out_rows[:16].float(), atol=3e-2, rtol=2e-2)
+
+
 def test_a_norm_inside_a_fused_projection_writes_the_cache():
     H, Hkv, dh, ps, n_pages, E, M = 6, 2, 48, 16, 12, 160, 7
     N = (H + 2 * Hkv) * dh
@@ -261,7 +305,7 @@ def test_a_norm_inside_a_fused_projection_writes_the_cache():
 
 def test_the_norm_inside_products_refuses_what_it_cannot_take():
     wp = ops().pack_matrix(rnd(32, 64, seed=2, dtype=torch.bfloat16))
-    assert not ops().norm_stream_takes(17, 64, wp) and not ops().norm_stream_takes(4, 40, wp)
+    assert not ops().norm_stream_takes(17, 64, wp) and not ops().norm_stream_takes(4, 40, wp) and not ops().norm_stream_takes(65, 1600, wp)
     assert not ops().norm_stream_takes(4, 8192, wp) and not ops().norm_stream_takes(4, 64, rnd(32, 64, dtype=torch.bfloat16))
     copy, stats = ops().norm_stream_buffers(17, 64, DEV)
     c = rnd(32, seed=3)

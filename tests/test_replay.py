@@ -246,6 +246,46 @@ def test_twenty_requests_decode_together(model_folders, name, graphs):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("name,n", [("E", 20), ("E", 64), ("F", 17), ("F", 40), ("F", 64)])
+def test_up_to_64_requests_on_wide_layers(model_folders, name, n):
+    """Steps of 17 to 64 rows of models whose layers are 1,024 columns wide or more: the norms between
+    the products run inside them (counted: two a layer, less the first layer's first), the rows travel
+    packed.  Every request decodes from its second token on; at the end some requests have ended."""
+    from denno_beta_amd.config import EngineOptions
+    from denno_beta_amd.engine import ModelRunner, StepEntry
+    from denno_beta_amd.kernels import ops
+    folder = model_folders(name, "bfloat16")
+    layers = TINY[name][0]["n_layer"]
+    seqs = sequences(name, [7] * n, seed=70)
+    want = plain_logits(folder, seqs)
+    calls = []
+    real = ops.linear_norm_in
+    ops.linear_norm_in = lambda *a, **k: (calls.append(a[0].shape[0]), real(*a, **k))[1]
+    try:
+        r = ModelRunner.from_folder(folder, EngineOptions(dtype="bfloat16", page_size=16, cache_tokens=n * 16,
+                                                          max_live=n, use_graphs=False))
+        for i in range(n):
+            r.start_request(i)
+        for i in range(0, n, 8):       # the first tokens, eight requests to a step
+            got = r.step([StepEntry(k, seqs[k][:1], [0]) for k in range(i, min(i + 8, n))]).cpu()
+            for k in range(i, min(i + 8, n)):
+                U.assert_close(got[k - i:k - i + 1], want[k][:1], "bfloat16", f"first token of request {k}")
+        alive = list(range(n))
+        for j in range(1, 7):
+            calls.clear()
+            got = r.step([StepEntry(i, [seqs[i][j]], [0]) for i in alive]).cpu()
+            assert calls == [len(alive)] * (2 * layers - 1), calls
+            for row, i in enumerate(alive):
+                U.assert_close(got[row:row + 1], want[i][j:j + 1], "bfloat16", f"request {i}, token {j}")
+            if j == 3:                 # a third of them ends: fewer rows, another kernel shape
+                for i in alive[::3]:
+                    r.end_request(i)
+                alive = [i for i in alive if i % 3 != 0]
+    finally:
+        ops.linear_norm_in = real
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("n", [150, 230])
 def test_many_requests_on_a_wide_layer(model_folders, n):
     """Steps of 129 to 256 rows of a model whose products are wide: the rows stay packed from kernel to

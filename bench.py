@@ -60,9 +60,6 @@ def main():
     from denno_beta_amd.config import EngineOptions
     from denno_beta_amd.engine import Engine, ModelRunner, SamplingParams, StepEntry
 
-    if a.norm_kernels:
-        from denno_beta_amd.kernels import ops
-        ops.NORM_STREAM_ROWS_MAX = 0
     if a.only == "serving":
         return serving(a)
     cfg, full_layers = xl_config(a.layers)
@@ -71,7 +68,7 @@ def main():
         a.steps = P - a.context - a.warmup - 1
     live = max(64, a.batch)
     opts = EngineOptions(dtype=a.dtype, page_size=16, cache_tokens=live * P, max_live=live, max_batch_tokens=4096,
-                         prefill_chunk=1024, use_graphs=not a.no_graphs, seed=0)
+                         prefill_chunk=1024, use_graphs=not a.no_graphs, seed=0, norms_inside_products=not a.norm_kernels)
     runner = ModelRunner.from_random(cfg, seed=0, options=opts, stored=a.dtype)
     gen = torch.Generator().manual_seed(0)
     prompt = lambda n: torch.randint(0, V, (n,), generator=gen).tolist()   # noqa: E731
@@ -155,7 +152,7 @@ def serving(a):
     cfg = dict(architectures=["GPT2LMHeadModel"], n_layer=36, n_embd=1280, n_head=20, n_inner=5120, vocab_size=50257,
                n_positions=1024, layer_norm_epsilon=1e-5, activation_function="gelu_new")
     opts = EngineOptions(dtype=a.dtype, page_size=16, cache_tokens=64 * 1024, max_live=64, max_batch_tokens=2048,
-                         prefill_chunk=512, use_graphs=not a.no_graphs, seed=0)
+                         prefill_chunk=512, use_graphs=not a.no_graphs, seed=0, norms_inside_products=not a.norm_kernels)
     eng = Engine.from_random(cfg, 0, opts, stored=a.dtype)
     gen = torch.Generator().manual_seed(1)
     lengths = torch.randint(16, 769, (64,), generator=gen).tolist()

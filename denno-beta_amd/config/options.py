@@ -25,6 +25,7 @@ class EngineOptions:
     device: str = "cuda:0"
     use_graphs: bool = True            # replay pure-decode steps from captured HIP graphs
     seed: Optional[int] = None         # default seed of requests that bring none
+    norms_inside_products: bool = True  # steps of few rows: a norm between two products runs inside them (parts/blocks.py)
 
     def validate(self):
         if self.dtype not in DTYPES:

@@ -25,7 +25,8 @@ class ModelRunner:
         options.validate()
         self.spec, self.options, self.config = spec, options, config
         self.device = torch.device(options.device)
-        self.runtime = Runtime(act_dtype=_ACT[options.dtype], device=self.device)
+        self.runtime = Runtime(act_dtype=_ACT[options.dtype], device=self.device,
+                               norms_inside_products=options.norms_inside_products)
         self.model = spec.instantiate().bind(tensors, self.runtime)
         cache_tokens = options.cache_tokens or options.max_live * spec.max_positions
         self.cache = CacheStorage(self.model.cache_specs, kv_dtype=self.runtime.act_dtype,

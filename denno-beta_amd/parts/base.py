@@ -51,6 +51,7 @@ class Runtime:
     act_dtype: torch.dtype
     device: torch.device
     position: Optional["Part"] = None
+    norms_inside_products: bool = True     # EngineOptions.norms_inside_products
     # what the last part that added into the residual stream left for the norm after it (StreamStats),
     # or None; the model clears it where the stream changes in any other way
     stream_stats: Optional["StreamStats"] = None

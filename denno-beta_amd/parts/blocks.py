@@ -27,7 +27,7 @@ class PreNormBlock:
         # A norm is a kernel of its own, or, where the parts on both sides of it can (steps of few
         # rows), it runs inside them: the part before leaves what the norm needs as it adds into the
         # stream, the part after applies it in its own kernel (parts.base.StreamStats, LazyNorm).
-        n = x.shape[0]
+        n = x.shape[0] if runtime.norms_inside_products else 1 << 30      # (so many rows nobody takes)
         before = runtime.stream_stats
         if before is not None and not (before.written and before.norm is self.norm1
                                        and self.mixer.takes_lazy_norm(n, self.norm1)):

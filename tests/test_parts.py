@@ -464,14 +464,12 @@ def test_norms_that_run_inside_the_products_beside_them(model_folders, name, row
         calls["out"] += 1
         return real_out(*a, **k)
     got = {}
-    limit = ops.NORM_STREAM_ROWS_MAX
     try:
         ops.linear_norm_in, ops.linear_norm_out = count_in, count_out
         for inside in (True, False):
-            ops.NORM_STREAM_ROWS_MAX = limit if inside else 0
-            r = ModelRunner.from_folder(folder, options("cuda:0", "bfloat16", use_graphs=False))
+            r = ModelRunner.from_folder(folder, options("cuda:0", "bfloat16", use_graphs=False, norms_inside_products=inside))
             r.start_request(0)
-            r.step([StepEntry(0, seq[:40], [])])                          # 40 rows: norms as kernels either way
+            r.step([StepEntry(0, seq[:40], [])])
             before = dict(calls)
             got[inside] = r.step([StepEntry(0, seq[40:], list(range(rows)))]).float().cpu()
             if inside:
@@ -480,7 +478,7 @@ def test_norms_that_run_inside_the_products_beside_them(model_folders, name, row
             else:
                 assert calls == before
     finally:
-        ops.linear_norm_in, ops.linear_norm_out, ops.NORM_STREAM_ROWS_MAX = real_in, real_out, limit
+        ops.linear_norm_in, ops.linear_norm_out = real_in, real_out
     U.assert_close(got[True], got[False], "bfloat16", f"{name}: norms inside the products against norms as kernels")
     want = P.PlainGPT2.from_folder(folder).logits(seq)[40:]
     U.assert_close(got[True], want, "bfloat16", f"{name}: norms inside the products against the plain implementation")

@@ -18,6 +18,7 @@ from .rng import uniform
 class Sampler:
     def __init__(self, device):
         self.device = device
+        self._zeros = {}      # rows -> [2, rows] of zeros on the device: temperatures and uniforms of all-greedy steps
 
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
                counters: Sequence[int], contexts: Sequence[Sequence[int]]) -> List[int]:
@@ -42,11 +43,17 @@ class Sampler:
                 f32([p.frequency_penalty or 0.0 for p in params]),
                 f32([p.presence_penalty or 0.0 for p in params]),
                 torch.tensor([p.no_repeat_ngram_size or 0 for p in params], dtype=torch.int32, device=dev))
-        temps = [0.0 if p.greedy else p.effective_temperature for p in params]
-        us = [0.0 if p.greedy else uniform(s, n) for p, s, n in zip(params, seeds, counters)]
         out = torch.empty(R, dtype=torch.int32, device=dev)
-        t_dev = torch.tensor(temps, dtype=torch.float32, device=dev)
-        u_dev = torch.tensor(us, dtype=torch.float32, device=dev)
+        if all(p.greedy for p in params):
+            # nothing to bring to the device: a step of greedy rows costs no copy
+            tu = self._zeros.get(R)
+            if tu is None:
+                tu = self._zeros[R] = torch.zeros((2, R), dtype=torch.float32, device=dev)
+        else:
+            temps = [0.0 if p.greedy else p.effective_temperature for p in params]
+            us = [0.0 if p.greedy else uniform(s, n) for p, s, n in zip(params, seeds, counters)]
+            tu = torch.tensor([temps, us], dtype=torch.float32, device=dev)      # one copy for both
+        t_dev, u_dev = tu[0], tu[1]
         restricted = [r for r, p in enumerate(params)
                       if not p.greedy and (p.top_k is not None or p.top_p is not None)]
         ops.sample(logits, t_dev, u_dev, out)

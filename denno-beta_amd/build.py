@@ -34,7 +34,7 @@ LIBRARIES = {
              ["host/cache_manager.h", "host/scheduler.h"]),
     "elementwise": ("hip", ["kernels/elementwise.hip"], ["kernels/common.h"]),
     "gemm": ("hip", ["kernels/gemm.hip"], ["kernels/common.h"]),
-    "attention": ("hip", ["kernels/attention.hip"], ["kernels/common.h"]),
+    "attention": ("hip", ["kernels/attention.hip"], ["kernels/common.h", "kernels/attention.h"]),
     "sampling": ("hip", ["kernels/sampling.hip"], ["kernels/common.h"]),
 }
 

@@ -11,8 +11,11 @@
 // The key pool is [n_pages, Hkv, page_size, dh], the value pool [n_pages, Hkv, dh, page_size];
 // query head h reads key head h / (H / Hkv).
 #include "common.h"
+#include "attention.h"
 
 #include <math.h>
+
+#include <mutex>
 
 namespace plain {
 constexpr int BQ = 16;
@@ -773,4 +776,59 @@ extern "C" int dn_attention_decode(const void* q, int ldq, void* out, int ldo, c
     hipLaunchKernelGGL(decode::join_kernel, dim3(n_tiles, H), dim3(64), 0, stream, part, static_cast<bf16_t*>(out),
                        ldo, tile_seq, tile_row0, n_splits, H, dh);
   return dn_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// The split decode kernels with the library's own memory for the split results: for callers that
+// cannot allocate (attention.h).  `scratch` below is a host-side stand-in in host code, not a device
+// address; the address on each GPU comes from hipGetSymbolAddress, once per GPU, and is what the
+// kernels get.
+// ---------------------------------------------------------------------------------------
+static __device__ __align__(256) float scratch[DN_DECODE_STATIC_SCRATCH_FLOATS];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_lock;
+float* scratch_on_device[MAX_DEVICES];   // zero-initialised: not looked up yet
+
+// the address of `scratch` on the current GPU; 0 and *err set if it cannot be had
+float* scratch_here(int* err) {
+  int dev = -1;
+  hipError_t rc = hipGetDevice(&dev);
+  if (rc != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    *err = rc != hipSuccess ? static_cast<int>(rc) : DN_ERR_SHAPE;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(scratch_lock);
+  if (scratch_on_device[dev] == nullptr) {
+    void* p = nullptr;
+    rc = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (rc != hipSuccess || p == nullptr) {
+      *err = rc != hipSuccess ? static_cast<int>(rc) : DN_ERR_SCRATCH;
+      return nullptr;
+    }
+    scratch_on_device[dev] = static_cast<float*>(p);
+  }
+  return scratch_on_device[dev];
+}
+}  // namespace
+
+extern "C" int dn_attention_decode_static(const void* q, int ldq, void* out, int ldo, const void* k_pool,
+                                          const void* v_pool, const int32_t* block_tables, int max_blocks,
+                                          const int32_t* tile_seq, const int32_t* tile_row0,
+                                          const int32_t* tile_pos0, int n_tiles, int n_splits, int chunks, int waves,
+                                          int H, int Hkv, int dh, int page_size, float scale, int window,
+                                          hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (n_splits < 1 || H < 1 || dh < 1) return DN_ERR_SHAPE;
+  float* part = nullptr;
+  if (n_splits > 1) {
+    const long long need = static_cast<long long>(n_tiles) * H * n_splits * (dh + 2);
+    if (need > DN_DECODE_STATIC_SCRATCH_FLOATS) return DN_ERR_SCRATCH;
+    int err = 0;
+    part = scratch_here(&err);
+    if (part == nullptr) return err;
+  }
+  return dn_attention_decode(q, ldq, out, ldo, k_pool, v_pool, block_tables, max_blocks, tile_seq, tile_row0, tile_pos0,
+                             n_tiles, part, n_splits, chunks, waves, H, Hkv, dh, page_size, scale, window, stream);
 }

@@ -30,6 +30,15 @@ class OutOfPages(CacheError):
 
 
 @dataclass(frozen=True)
+class SlotState:
+    """A live request's record of fixed size (csrc/host/cache_manager.h): zero when its slot is given out."""
+    num_computed: int     # tokens in the cache = the next token's position
+    last_token: int       # the token sampled last, -1 before the first
+    rng_seed: int
+    rng_drawn: int        # numbers drawn from the request's generator so far
+
+
+@dataclass(frozen=True)
 class GroupLayout:
     kind: int            # PAGED or STATE
     n_pages: int = 0
@@ -50,6 +59,9 @@ def host_library():
             "dn_cache_create": (P, [I, IP, IP, IP, IP, I]), "dn_cache_destroy": (None, [P]),
             "dn_cache_add": (I, [P, L]), "dn_cache_release": (I, [P, L]), "dn_cache_reserve": (I, [P, L, I]),
             "dn_cache_commit": (I, [P, L, I]), "dn_cache_length": (I, [P, L]), "dn_cache_slot": (I, [P, L]),
+            "dn_cache_state": (I, [P, L, c_void_p]), "dn_cache_set_rng": (I, [P, L, ctypes.c_uint64, ctypes.c_uint64]),
+            "dn_cache_note_sampled": (I, [P, L, I]),
+            "dn_cache_rng_states": (I, [P, c_void_p, I, c_void_p, c_void_p, IP]),
             "dn_cache_generation": (L, [P, I]), "dn_cache_block_table": (I, [P, L, I, c_void_p, I]),
             "dn_cache_blocks": (I, [P, L, I]), "dn_cache_free_pages": (I, [P, I]),
             "dn_cache_pages_held": (I, [P, L, I]), "dn_cache_pages_needed": (I, [P, L, I, I, I]),
@@ -134,6 +146,30 @@ class CacheManager:
 
     def slot(self, rid: int) -> int:
         return self._chk(self._lib.dn_cache_slot(self._h, rid), f"slot of request {rid}")
+
+    # -- the request's slot record: position, generator, last token --------------------------
+    def state(self, rid: int) -> "SlotState":
+        out = np.empty(6, dtype=np.int64)
+        self._chk(self._lib.dn_cache_state(self._h, rid, out.ctypes.data), f"state of request {rid}")
+        v = out.tolist()
+        return SlotState(v[0], v[1], v[2] | (v[3] << 32), v[4] | (v[5] << 32))
+
+    def set_rng(self, rid: int, seed: int, drawn: int = 0):
+        """The request's generator: its seed and how many numbers it has given (a request that comes
+        back after preemption brings its count)."""
+        self._chk(self._lib.dn_cache_set_rng(self._h, rid, seed & (2 ** 64 - 1), drawn), f"generator of request {rid}")
+
+    def note_sampled(self, rid: int, token: int):
+        """One number was drawn from the request's generator and gave `token`."""
+        self._chk(self._lib.dn_cache_note_sampled(self._h, rid, token), f"sampled token of request {rid}")
+
+    def rng_states(self, rids: np.ndarray):
+        """-> (seeds, numbers drawn so far) of the requests, uint64 arrays."""
+        seeds, drawn = np.empty(len(rids), dtype=np.uint64), np.empty(len(rids), dtype=np.uint64)
+        failed = c_int(0)
+        self._chk_step(self._lib.dn_cache_rng_states(self._h, rids.ctypes.data, len(rids), seeds.ctypes.data,
+                                                     drawn.ctypes.data, failed), failed, rids, "generator")
+        return seeds, drawn
 
     def generation(self, slot: int) -> int:
         return self._lib.dn_cache_generation(self._h, slot)

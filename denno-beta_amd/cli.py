@@ -6,13 +6,20 @@
     denno info <model>
     denno random-model <folder> --config FILE --seed N [--dtype float32|bfloat16]
 
+    denno generate <model> --prompt-file FILE [--max-live N] [--page-size N] [--cache-tokens N]
+          [--prefill-chunk N] [--max-batch-tokens N] [--kv-policy preempt|reserve] ...
+
 `<model>` is a folder with config.json and model.safetensors (the reference resolves a hub id
 in its download cache, main.rs:555-565; there is no network here).  Option names and defaults
 are the reference's: max-tokens 128, temperature unset = 1.0 and 0 = greedy, seed unset =
 entropy.  `--quant` names the precision: the reference's fp32 (default there) and this
 engine's bf16; its int8 and q4 modes are not built.  Beyond the reference: `--prompt-ids`
 for token ids where the folder has no tokenizer.json, `--top-k`, `--top-p` (the reference's
-request parameters, crates/denno-engine/src/engine.rs:42-43), `--ignore-eos`.
+request parameters, crates/denno-engine/src/engine.rs:42-43), `--ignore-eos`; `--prompt-file` with
+one prompt a line (token ids separated by commas or blanks), which all go through the scheduler
+together, one line of output each in the file's order; and the engine's own options (`--max-live`,
+`--page-size`, `--cache-tokens`, `--prefill-chunk`, `--max-batch-tokens`, `--kv-policy`,
+`--no-graphs`), which the reference sets through DENNO_* environment variables.
 """
 from __future__ import annotations
 
@@ -44,12 +51,13 @@ def load_tokenizer(model_dir):
 
 
 def parser():
-    ap = argparse.ArgumentParser(prog="denno", description="GPT-2 inference engine for MI355X")
+    ap = argparse.ArgumentParser(prog="denno", description="inference engine for one MI355X")
     sub = ap.add_subparsers(dest="command", required=True)
     g = sub.add_parser("generate", help="one generation")
     g.add_argument("model", help="model folder")
     g.add_argument("--prompt", help="prompt text (needs tokenizer.json in the folder)")
     g.add_argument("--prompt-ids", help="prompt as comma-separated token ids")
+    g.add_argument("--prompt-file", help="several prompts, one a line, as token ids separated by commas or blanks")
     g.add_argument("--system", default=None)
     g.add_argument("--max-tokens", type=int, default=128)
     g.add_argument("--temperature", type=float, default=None, help="unset: 1.0; 0: greedy")
@@ -65,6 +73,16 @@ def parser():
     g.add_argument("--ignore-eos", action="store_true")
     g.add_argument("--cast-weights", action="store_true",
                    help="bf16: round matrices stored in 32-bit to bfloat16 at load")
+    g.add_argument("--max-live", type=int, default=None,
+                   help="most requests that hold cache at a time (default: 1, or up to 64 with --prompt-file)")
+    g.add_argument("--page-size", type=int, default=16, help="tokens in a page of the cache")
+    g.add_argument("--cache-tokens", type=int, default=None,
+                   help="size of the cache in tokens (default: max-live times the model's positions)")
+    g.add_argument("--prefill-chunk", type=int, default=512, help="longest portion of one prompt in one step")
+    g.add_argument("--max-batch-tokens", type=int, default=2048, help="token budget of one step")
+    g.add_argument("--kv-policy", default="preempt", choices=["preempt", "reserve"],
+                   help="when pages run out: preempt the youngest request, or admit only what can be reserved")
+    g.add_argument("--no-graphs", action="store_true", help="run decode steps kernel by kernel")
     i = sub.add_parser("info", help="what a model folder holds")
     i.add_argument("model")
     r = sub.add_parser("random-model", help="write a model folder with random weights")
@@ -82,7 +100,12 @@ def cmd_generate(a):
     if quant is None:
         raise SystemExit(f"--quant {a.quant}: this engine has fp32 and bf16; quantized weights are not built")
     tok = load_tokenizer(a.model)
-    if a.prompt_ids is not None:
+    if a.prompt_file is not None:
+        with open(a.prompt_file) as f:
+            prompts = [[int(x) for x in line.replace(",", " ").split()] for line in f if line.strip()]
+        if not prompts:
+            raise SystemExit(f"{a.prompt_file} holds no prompt")
+    elif a.prompt_ids is not None:
         ids = [int(x) for x in a.prompt_ids.replace(" ", "").split(",") if x]
     elif a.prompt is not None:
         if tok is None:
@@ -91,23 +114,29 @@ def cmd_generate(a):
         text = a.prompt if a.raw else fallback_template(a.system, a.prompt)
         ids = tok.encode(text).ids
     else:
-        raise SystemExit("one of --prompt and --prompt-ids is needed")
+        raise SystemExit("one of --prompt, --prompt-ids and --prompt-file is needed")
+    if a.prompt_file is None:
+        prompts = [ids]
     params = SamplingParams(
         max_tokens=a.max_tokens, temperature=a.temperature, top_k=a.top_k, top_p=a.top_p, seed=a.seed,
         repetition_penalty=a.repetition_penalty, frequency_penalty=a.frequency_penalty,
         presence_penalty=a.presence_penalty, no_repeat_ngram_size=a.no_repeat_ngram_size,
         ignore_eos=a.ignore_eos)
-    eng = Engine.from_folder(a.model, EngineOptions(dtype=quant, max_live=1, seed=a.seed), a.cast_weights)
-    out = eng.generate([ids], params)[0]
-    if a.raw or tok is None:
-        # the raw path stops at the end-of-sequence token without keeping it (main.rs:708-710)
-        eos = set(eng.spec.eos_token_ids)
-        if out and out[-1] in eos and not a.ignore_eos:
-            out = out[:-1]
-    if tok is not None and a.prompt is not None:
-        print(tok.decode(out))
-    else:
-        print(",".join(str(t) for t in out))
+    max_live = a.max_live if a.max_live is not None else min(len(prompts), 64)
+    eng = Engine.from_folder(a.model, EngineOptions(
+        dtype=quant, max_live=max_live, seed=a.seed, page_size=a.page_size, cache_tokens=a.cache_tokens,
+        prefill_chunk=a.prefill_chunk, max_batch_tokens=a.max_batch_tokens, kv_policy=a.kv_policy,
+        use_graphs=not a.no_graphs), a.cast_weights)
+    for out in eng.generate(prompts, params):
+        if a.raw or tok is None:
+            # the raw path stops at the end-of-sequence token without keeping it (main.rs:708-710)
+            eos = set(eng.spec.eos_token_ids)
+            if out and out[-1] in eos and not a.ignore_eos:
+                out = out[:-1]
+        if tok is not None and a.prompt is not None:
+            print(tok.decode(out))
+        else:
+            print(",".join(str(t) for t in out))
     return 0
 
 

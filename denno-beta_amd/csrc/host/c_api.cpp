@@ -32,6 +32,27 @@ int dn_cache_reserve(void* c, int64_t rid, int n) { return static_cast<CacheMana
 int dn_cache_commit(void* c, int64_t rid, int n) { return static_cast<CacheManager*>(c)->commit(rid, n); }
 int dn_cache_length(void* c, int64_t rid) { return static_cast<CacheManager*>(c)->length(rid); }
 int dn_cache_slot(void* c, int64_t rid) { return static_cast<CacheManager*>(c)->slot(rid); }
+// out: num_computed, last_token, then the seed and the count of numbers drawn as two 32-bit halves each (low first)
+int dn_cache_state(void* c, int64_t rid, int64_t* out) {
+  const denno::SlotState* s = static_cast<CacheManager*>(c)->state(rid);
+  if (!s) return denno::kUnknown;
+  out[0] = s->num_computed;
+  out[1] = s->last_token;
+  out[2] = static_cast<int64_t>(s->rng_seed & 0xffffffffu);
+  out[3] = static_cast<int64_t>(s->rng_seed >> 32);
+  out[4] = static_cast<int64_t>(s->rng_drawn & 0xffffffffu);
+  out[5] = static_cast<int64_t>(s->rng_drawn >> 32);
+  return denno::kOk;
+}
+int dn_cache_set_rng(void* c, int64_t rid, uint64_t seed, uint64_t drawn) {
+  return static_cast<CacheManager*>(c)->set_rng(rid, seed, drawn);
+}
+int dn_cache_note_sampled(void* c, int64_t rid, int token) {
+  return static_cast<CacheManager*>(c)->note_sampled(rid, token);
+}
+int dn_cache_rng_states(void* c, const int64_t* rids, int n, uint64_t* seeds, uint64_t* drawn, int* failed) {
+  return static_cast<CacheManager*>(c)->rng_states(rids, n, seeds, drawn, failed);
+}
 int64_t dn_cache_generation(void* c, int slot) { return static_cast<CacheManager*>(c)->generation(slot); }
 int dn_cache_block_table(void* c, int64_t rid, int g, int32_t* out, int cap) {
   return static_cast<CacheManager*>(c)->block_table(rid, g, out, cap);

@@ -6,7 +6,8 @@ namespace denno {
 
 CacheManager::CacheManager(const std::vector<GroupSpec>& groups, int max_requests)
     : groups_(groups), free_(groups.size()), used_before_(groups.size()), reuse_(groups.size(), 0),
-      slot_rid_(max_requests, -1), slot_gen_(max_requests, 0) {
+      slot_rid_(max_requests, -1), slot_gen_(max_requests, 0),
+      slot_state_(max_requests, SlotState{0, -1, 0, 0}) {
   for (size_t g = 0; g < groups_.size(); ++g) {
     if (groups_[g].kind != kPaged) continue;
     // a stack whose top is page 0, so a fresh pool hands pages out in ascending order
@@ -23,7 +24,7 @@ int CacheManager::add(int64_t rid) {
   Request r;
   r.slot = free_slots_.back();
   free_slots_.pop_back();
-  r.len = 0;
+  slot_state_[r.slot] = SlotState{0, -1, 0, 0};
   r.tables.resize(groups_.size());
   r.first_live.assign(groups_.size(), 0);
   slot_rid_[r.slot] = rid;
@@ -82,7 +83,7 @@ int CacheManager::reserve(int64_t rid, int new_len) {
   auto it = by_rid_.find(rid);
   if (it == by_rid_.end()) return kUnknown;
   Request& r = it->second;
-  if (new_len < r.len) return kBadArgument;
+  if (new_len < slot_state_[r.slot].num_computed) return kBadArgument;
   std::vector<int> need(groups_.size(), 0);
   for (size_t g = 0; g < groups_.size(); ++g) {
     if (groups_[g].kind != kPaged) continue;
@@ -106,13 +107,13 @@ int CacheManager::commit(int64_t rid, int new_len) {
   auto it = by_rid_.find(rid);
   if (it == by_rid_.end()) return kUnknown;
   Request& r = it->second;
-  if (new_len < r.len) return kBadArgument;
+  if (new_len < slot_state_[r.slot].num_computed) return kBadArgument;
   for (size_t g = 0; g < groups_.size(); ++g) {
     if (groups_[g].kind != kPaged) continue;
     int blocks = static_cast<int>(r.tables[g].size());
     if (new_len > blocks * groups_[g].page_size) return kBadArgument;   // commit without reserve
   }
-  r.len = new_len;
+  slot_state_[r.slot].num_computed = new_len;
   for (size_t g = 0; g < groups_.size(); ++g) {
     if (groups_[g].kind != kPaged) continue;
     int first = std::min(first_needed_block(static_cast<int>(g), new_len),
@@ -135,7 +136,7 @@ int CacheManager::lengths(const int64_t* rids, int n, int* out, int* failed) con
       *failed = i;
       return kUnknown;
     }
-    out[i] = it->second.len;
+    out[i] = slot_state_[it->second.slot].num_computed;
   }
   return kOk;
 }
@@ -202,12 +203,46 @@ int CacheManager::step_tables(int g, const int64_t* rids, const int* starts, con
 
 int CacheManager::length(int64_t rid) const {
   auto it = by_rid_.find(rid);
-  return it == by_rid_.end() ? static_cast<int>(kUnknown) : it->second.len;
+  return it == by_rid_.end() ? static_cast<int>(kUnknown) : slot_state_[it->second.slot].num_computed;
 }
 
 int CacheManager::slot(int64_t rid) const {
   auto it = by_rid_.find(rid);
   return it == by_rid_.end() ? static_cast<int>(kUnknown) : it->second.slot;
+}
+
+const SlotState* CacheManager::state(int64_t rid) const {
+  auto it = by_rid_.find(rid);
+  return it == by_rid_.end() ? nullptr : &slot_state_[it->second.slot];
+}
+
+int CacheManager::set_rng(int64_t rid, uint64_t seed, uint64_t drawn) {
+  auto it = by_rid_.find(rid);
+  if (it == by_rid_.end()) return kUnknown;
+  slot_state_[it->second.slot].rng_seed = seed;
+  slot_state_[it->second.slot].rng_drawn = drawn;
+  return kOk;
+}
+
+int CacheManager::note_sampled(int64_t rid, int32_t token) {
+  auto it = by_rid_.find(rid);
+  if (it == by_rid_.end()) return kUnknown;
+  slot_state_[it->second.slot].rng_drawn += 1;
+  slot_state_[it->second.slot].last_token = token;
+  return kOk;
+}
+
+int CacheManager::rng_states(const int64_t* rids, int n, uint64_t* seeds, uint64_t* drawn, int* failed) const {
+  for (int i = 0; i < n; ++i) {
+    auto it = by_rid_.find(rids[i]);
+    if (it == by_rid_.end()) {
+      *failed = i;
+      return kUnknown;
+    }
+    seeds[i] = slot_state_[it->second.slot].rng_seed;
+    drawn[i] = slot_state_[it->second.slot].rng_drawn;
+  }
+  return kOk;
 }
 
 int64_t CacheManager::generation(int slot) const {

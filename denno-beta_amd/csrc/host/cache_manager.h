@@ -34,6 +34,17 @@ struct GroupSpec {
   int window;      // 0: every key is kept; W > 0: a query at position p reads keys in (p - W, p]
 };
 
+// What a live request keeps beside its pages, in its slot: a record of fixed size, zero when the slot
+// is given out.  The reference keeps the position in its cache object and the sampler's generator in
+// the session (crates/denno-engine/src/kv_cache.rs:21, 133-135; engine.rs:251).  The generator here is
+// counter-based: its whole state is the seed and the count of numbers drawn.
+struct SlotState {
+  int32_t num_computed;   // tokens in the cache = the next token's position
+  int32_t last_token;     // the token sampled last, -1 before the first
+  uint64_t rng_seed;
+  uint64_t rng_drawn;     // numbers drawn from the generator so far
+};
+
 class CacheManager {
  public:
   CacheManager(const std::vector<GroupSpec>& groups, int max_requests);
@@ -44,6 +55,13 @@ class CacheManager {
   int commit(int64_t rid, int new_len);       // len = new_len; pages that a window has passed go back
   int length(int64_t rid) const;              // tokens committed, or kUnknown
   int slot(int64_t rid) const;
+  // the request's slot record; 0 if the id is not live.  set_rng: at admission (a request that was
+  // preempted brings the count it had); note_sampled: one more number drawn, `token` sampled with it
+  const SlotState* state(int64_t rid) const;
+  int set_rng(int64_t rid, uint64_t seed, uint64_t drawn);
+  int note_sampled(int64_t rid, int32_t token);
+  // seeds and counts of a step's requests in one call; on a failure *failed is the entry's index
+  int rng_states(const int64_t* rids, int n, uint64_t* seeds, uint64_t* drawn, int* failed) const;
   int64_t generation(int slot) const;         // bumped each time the slot is given out
   int block_table(int64_t rid, int group, int32_t* out, int cap) const;   // -> blocks; -1 marks a page given back
   int free_pages(int group) const;
@@ -78,8 +96,7 @@ class CacheManager {
 
  private:
   struct Request {
-    int slot;
-    int len;                                   // tokens committed
+    int slot;                                  // index of its SlotState (the position lives there)
     std::vector<std::vector<int32_t>> tables;  // [group][block] -> page, -1 once given back
     std::vector<int> first_live;               // [group] first block that is still held
   };
@@ -91,6 +108,7 @@ class CacheManager {
   std::vector<int64_t> reuse_;
   std::vector<int64_t> slot_rid_;              // [slot] rid, or -1
   std::vector<int64_t> slot_gen_;
+  std::vector<SlotState> slot_state_;          // [slot]
   std::vector<int> free_slots_;
   std::unordered_map<int64_t, Request> by_rid_;
 };

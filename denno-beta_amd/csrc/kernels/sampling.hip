@@ -185,9 +185,9 @@ __global__ __launch_bounds__(THREADS) void penalties_kernel(float* __restrict__ 
 // top-k / top-p (sampler.rs:372-435, 487-514): the m largest of z = logit/T (ties: the lower
 // index first) in descending order, e_i = exp(z_i - z_0); with top-p the list is cut where
 // the running sum of e_i / sum(e) reaches p; then the walk with u * sum(kept e) in that order.
-// m = min(k, 2048, V); with top-p alone m = min(2048, V), the reference's subset (where the
-// reference falls back to a full sort because the 2048 largest do not reach p, the tail
-// beyond them is dropped here).
+// m = min(k, 2048, V); with top-p alone m = min(2048, V), the reference's subset, and as there
+// (sampler.rs:387-435) a row whose cut does not fall before the last of the 2048 is not
+// decided here: its place in `undecided` is set and sample_full_kernel below takes it.
 // ---------------------------------------------------------------------------------------
 constexpr int CAND = 2048;
 
@@ -207,7 +207,8 @@ __global__ __launch_bounds__(THREADS) void sample_top_kernel(const float* __rest
                                                               const float* __restrict__ uniform,
                                                               const int32_t* __restrict__ top_k,
                                                               const float* __restrict__ top_p,
-                                                              int32_t* __restrict__ out) {
+                                                              int32_t* __restrict__ out,
+                                                              int32_t* __restrict__ undecided) {
   __shared__ uint32_t cand_key[CAND];
   __shared__ int32_t cand_idx[CAND];
   __shared__ float cand_e[CAND];
@@ -337,6 +338,9 @@ __global__ __launch_bounds__(THREADS) void sample_top_kernel(const float* __rest
         }
       }
     }
+    // top-p alone over a vocabulary larger than the subset: a cut that is not reached before the
+    // subset's last member needs the tail (sampler.rs:425-433)
+    undecided[blockIdx.x] = (k <= 0 && V > CAND && keep == m) ? 1 : 0;
     float total = 0.f;
     for (int i = 0; i < keep; ++i) total += cand_e[i];
     float u = uniform[r] * total;
@@ -350,6 +354,125 @@ __global__ __launch_bounds__(THREADS) void sample_top_kernel(const float* __rest
     }
     out[r] = pick;
   }
+}
+
+// ---------------------------------------------------------------------------------------
+// top-p over the whole vocabulary (sampler.rs:466-476, 487-514): every z = logit/T in descending
+// order (ties: the lower index first), e_i = exp(z_i - z_0), the list cut where the running sum of
+// e_i / sum(e) reaches p, then the walk with u * sum(kept e).  One workgroup per listed row sorts
+// the row in `work` (per row: n_pad keys, n_pad indices, n_pad numerators; n_pad the power of
+// two from V up).  Sums run in the list's order by segments: a thread adds its own stretch, one
+// thread adds the stretches' sums, so the result does not depend on timing.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(THREADS) void sample_full_kernel(const float* __restrict__ logits, int ld, int V,
+                                                               int n_pad, const int32_t* __restrict__ rows,
+                                                               const float* __restrict__ temperature,
+                                                               const float* __restrict__ uniform,
+                                                               const float* __restrict__ top_p,
+                                                               uint32_t* __restrict__ work,
+                                                               int32_t* __restrict__ out) {
+  __shared__ float seg_sum[THREADS];
+  __shared__ float seg_base[THREADS];
+  __shared__ float total_s;
+  __shared__ int first_s;
+  const int t = threadIdx.x;
+  const int r = rows[blockIdx.x];
+  const float* row = logits + static_cast<size_t>(r) * ld;
+  const float T = temperature[r];
+  uint32_t* key = work + static_cast<size_t>(blockIdx.x) * 3 * n_pad;
+  int32_t* idx = reinterpret_cast<int32_t*>(key + n_pad);
+  float* e = reinterpret_cast<float*>(key + 2 * static_cast<size_t>(n_pad));
+  for (int i = t; i < n_pad; i += THREADS) {
+    key[i] = i < V ? order_key(row[i] / T) : 0u;
+    idx[i] = i < V ? i : 0x7fffffff;
+  }
+  __syncthreads();
+  for (int size = 2; size <= n_pad; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      for (int i = t; i < n_pad / 2; i += THREADS) {
+        int a = 2 * i - (i & (stride - 1));
+        int b = a + stride;
+        bool descending = (a & size) == 0;
+        uint32_t ka = key[a], kb = key[b];
+        int ia = idx[a], ib = idx[b];
+        bool a_first = ka > kb || (ka == kb && ia < ib);
+        if (a_first != descending) {
+          key[a] = kb;
+          key[b] = ka;
+          idx[a] = ib;
+          idx[b] = ia;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  // a value that is NaN has key 0 like the padding but a real index, which sorts before the padding's:
+  // the first V places hold the row
+  const float z0 = key_value(key[0]);
+  const int seg = (V + THREADS - 1) / THREADS;
+  const int lo = min(V, t * seg), hi = min(V, lo + seg);
+  float s = 0.f;
+  for (int i = lo; i < hi; ++i) {
+    float v = key[i] != 0u ? expf(key_value(key[i]) - z0) : 0.f;     // key 0: NaN, which nothing can pick
+    e[i] = v;
+    s += v;
+  }
+  seg_sum[t] = s;
+  if (t == 0) first_s = V;
+  __syncthreads();
+  if (t == 0) {
+    float run = 0.f;
+    for (int k = 0; k < THREADS; ++k) {
+      seg_base[k] = run;
+      run += seg_sum[k];
+    }
+    total_s = run;
+  }
+  __syncthreads();
+  const float p = top_p[blockIdx.x];
+  int keep = V;
+  if (p < 1.0f) {
+    const float total = total_s;
+    float cum = seg_base[t] / total;
+    // (the reference adds e_i / total term by term; here a stretch starts from its base / total)
+    for (int i = lo; i < hi; ++i) {
+      cum += e[i] / total;
+      if (cum >= p) {
+        atomicMin(&first_s, i);
+        break;
+      }
+    }
+    __syncthreads();
+    keep = min(V, first_s + 1);
+    __syncthreads();
+  }
+  // the kept list's sum, then the walk
+  s = 0.f;
+  for (int i = lo; i < min(hi, keep); ++i) s += e[i];
+  seg_sum[t] = s;
+  if (t == 0) first_s = keep;
+  __syncthreads();
+  if (t == 0) {
+    float run = 0.f;
+    for (int k = 0; k < THREADS; ++k) {
+      seg_base[k] = run;
+      run += seg_sum[k];
+    }
+    total_s = run;
+  }
+  __syncthreads();
+  {
+    float u = uniform[r] * total_s - seg_base[t];
+    for (int i = lo; i < min(hi, keep); ++i) {
+      u -= e[i];
+      if (u <= 0.f) {
+        atomicMin(&first_s, i);
+        break;
+      }
+    }
+  }
+  __syncthreads();
+  if (t == 0) out[r] = idx[min(first_s, keep - 1)];
 }
 }  // namespace sampling
 
@@ -374,10 +497,21 @@ extern "C" int dn_penalties(float* logits, int ld, int R, int V, const int32_t* 
 
 extern "C" int dn_sample_top(const float* logits, int ld, int n_rows, int V, const int32_t* rows,
                              const float* temperature, const float* uniform, const int32_t* top_k,
-                             const float* top_p, int32_t* out, hipStream_t stream) {
+                             const float* top_p, int32_t* out, int32_t* undecided, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (V < 1 || ld < V) return DN_ERR_SHAPE;
   hipLaunchKernelGGL(sampling::sample_top_kernel, dim3(n_rows), dim3(sampling::THREADS), 0, stream, logits, ld, V,
-                     rows, temperature, uniform, top_k, top_p, out);
+                     rows, temperature, uniform, top_k, top_p, out, undecided);
+  return dn_launch_status();
+}
+
+// work: 3 * n_pad 32-bit words per listed row, n_pad the power of two from V up
+extern "C" int dn_sample_full(const float* logits, int ld, int n_rows, int V, int n_pad, const int32_t* rows,
+                              const float* temperature, const float* uniform, const float* top_p, void* work,
+                              int32_t* out, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (V < 1 || ld < V || n_pad < V || n_pad < 2 || (n_pad & (n_pad - 1)) != 0) return DN_ERR_SHAPE;
+  hipLaunchKernelGGL(sampling::sample_full_kernel, dim3(n_rows), dim3(sampling::THREADS), 0, stream, logits, ld, V,
+                     n_pad, rows, temperature, uniform, top_p, static_cast<uint32_t*>(work), out);
   return dn_launch_status();
 }

@@ -12,6 +12,7 @@ import time
 from dataclasses import dataclass, field
 from typing import Dict, Iterable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..config import EngineOptions
@@ -121,11 +122,15 @@ class Engine:
                                    "(a request larger than the cache should have been refused)")
             return []
         entries, sampled = [], []
+        manager = self.runner.cache.manager
         for p in plan:
             req = self.requests[p.rid]
             if p.start == 0:
-                # admitted (or admitted again after preemption): fixed-size states start at zero
-                self.runner.cache.reset_states(self.runner.cache.manager.slot(p.rid))
+                # admitted (or admitted again after preemption): fixed-size states start at zero, and the
+                # request's slot record gets its generator (seed, numbers drawn so far: a request that
+                # comes back after preemption goes on where it was, so its samples do not change)
+                self.runner.cache.reset_states(manager.slot(p.rid))
+                manager.set_rng(p.rid, req.seed, len(req.generated))
             wants = p.samples and len(req.generated) < req.max_new
             entries.append(StepEntry(p.rid, req.tokens[p.start:p.start + p.count], [p.count - 1] if wants else []))
             if wants:
@@ -137,9 +142,12 @@ class Engine:
             logits = self.runner.step(entries)
             for p in plan:
                 self.scheduler.step_done(p.rid, p.count)
-            tokens = self.sampler.sample(
-                logits, [r.params for r in sampled], [r.seed for r in sampled],
-                [len(r.generated) for r in sampled], [r.tokens for r in sampled])
+            # each request's generator lives in its slot record: the seed and the count of numbers drawn
+            seeds, drawn = manager.rng_states(np.asarray([r.rid for r in sampled], dtype=np.int64))
+            tokens = self.sampler.sample(logits, [r.params for r in sampled], seeds.tolist(), drawn.tolist(),
+                                         [r.tokens for r in sampled])
+            for r, tok in zip(sampled, tokens):
+                manager.note_sampled(r.rid, int(tok))
         except Exception:
             # the step's requests are dropped, their pages go back, the engine stays usable
             # (crates/denno-server/src/scheduler.rs:362-370, 457-469)

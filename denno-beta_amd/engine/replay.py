@@ -23,15 +23,22 @@ class TraceReplayer:
 
     def run_step(self, record: dict) -> Optional[torch.Tensor]:
         """-> logits [wanted, vocab] on the device, or None if the step wants none."""
-        entries = []
-        for e in record.get("entries", []):
-            name = str(e["id"])
-            if name not in self._rid:
-                self._rid[name] = self._next
-                self._next += 1
-                self.runner.start_request(self._rid[name])
-            entries.append(StepEntry(self._rid[name], e["tokens"], e.get("want", [])))
-        logits = self.runner.step(entries)
+        entries, started = [], []
+        try:
+            for e in record.get("entries", []):
+                name = str(e["id"])
+                if name not in self._rid:
+                    self.runner.start_request(self._next)
+                    self._rid[name] = self._next
+                    self._next += 1
+                    started.append(name)
+                entries.append(StepEntry(self._rid[name], e["tokens"], e.get("want", [])))
+            logits = self.runner.step(entries)
+        except Exception:
+            # a step that cannot run leaves nothing of the requests it would have started
+            for name in started:
+                self.runner.end_request(self._rid.pop(name))
+            raise
         for name in record.get("end", []):
             rid = self._rid.pop(str(name), None)
             if rid is not None:

@@ -24,7 +24,25 @@ class KernelError(RuntimeError):
     pass
 
 
+_fail_after = None      # fail_after_launches
+launches = 0            # kernel launches asked for through this module since import
+
+
+def fail_after_launches(n):
+    """Failure injection: the next n launches go through, the one after them raises KernelError on
+    the host before anything is launched (so every kernel that did start ends normally); then
+    launches go through again.  None: off.  The reference's tests wrap the model in one that fails
+    after it has written the cache (crates/denno-engine/src/engine.rs:3354-3385)."""
+    global _fail_after
+    _fail_after = None if n is None else launches + int(n)
+
+
 def _lib(name):
+    global launches, _fail_after
+    if _fail_after is not None and launches >= _fail_after:
+        _fail_after = None
+        raise KernelError(f"injected failure: launch number {launches + 1} was refused")
+    launches += 1
     lib = _libs.get(name)
     if lib is None:
         if not torch.cuda.is_available():
@@ -60,7 +78,8 @@ def _declare(name, lib):
         "sampling": {
             "dn_sample": [P, I, I, I, P, P, P, P],
             "dn_penalties": [P, I, I, I, P, P, P, P, P, P, P],
-            "dn_sample_top": [P, I, I, I, P, P, P, P, P, P, P],
+            "dn_sample_top": [P, I, I, I, P, P, P, P, P, P, P, P],
+            "dn_sample_full": [P, I, I, I, I, P, P, P, P, P, P, P],
         },
     }[name]
     for fn, args in sigs.items():
@@ -442,22 +461,46 @@ def sample(logits, temperature, uniform, out):
     return out
 
 
-def sample_top(logits, rows, temperature, uniform, top_k, top_p, out):
+def sample_top(logits, rows, temperature, uniform, top_k, top_p, out, undecided):
     """For the rows listed in `rows` (each with temperature > 0): top_k[j] largest candidates
     (0: no limit but the 2048 that the kernel keeps), cut at cumulative probability top_p[j]
     (1: no cut), then the walk with uniform[row].  temperature, uniform and out are indexed by
-    row, top_k and top_p by the place in `rows`."""
+    row, top_k, top_p and undecided by the place in `rows`.  undecided[j] = 1: top-p alone did not
+    find its cut before the last of the 2048 candidates; the row needs `sample_full`."""
     _dev(logits, "logits", (torch.float32,), 2), _dev(rows, "rows", _I32, 1)
     _dev(temperature, "temperature", (torch.float32,), 1), _dev(uniform, "uniform", (torch.float32,), 1)
     _dev(top_k, "top_k", _I32, 1), _dev(top_p, "top_p", (torch.float32,), 1), _dev(out, "out", _I32, 1)
+    _dev(undecided, "undecided", _I32, 1)
     R, V = logits.shape
     ld = _rows(logits, "logits")
     n = rows.shape[0]
-    _need(top_k.shape[0] == n and top_p.shape[0] == n, "sample_top: one top_k and top_p per listed row")
+    _need(top_k.shape[0] == n and top_p.shape[0] == n and undecided.shape[0] == n,
+          "sample_top: one top_k, top_p and undecided per listed row")
     _need(temperature.shape[0] == R and uniform.shape[0] == R and out.shape[0] == R, "sample_top: rows")
     _ok(_lib("sampling").dn_sample_top(logits.data_ptr(), ld, n, V, rows.data_ptr(), temperature.data_ptr(),
                                        uniform.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), out.data_ptr(),
-                                       _stream()), "sample_top")
+                                       undecided.data_ptr(), _stream()), "sample_top")
+    return out
+
+
+def sample_full(logits, rows, temperature, uniform, top_p, out):
+    """top-p over the whole sorted vocabulary for the rows listed in `rows` (each with temperature
+    > 0), then the walk with uniform[row]: what `sample_top` leaves undecided."""
+    _dev(logits, "logits", (torch.float32,), 2), _dev(rows, "rows", _I32, 1)
+    _dev(temperature, "temperature", (torch.float32,), 1), _dev(uniform, "uniform", (torch.float32,), 1)
+    _dev(top_p, "top_p", (torch.float32,), 1), _dev(out, "out", _I32, 1)
+    R, V = logits.shape
+    ld = _rows(logits, "logits")
+    n = rows.shape[0]
+    _need(top_p.shape[0] == n, "sample_full: one top_p per listed row")
+    _need(temperature.shape[0] == R and uniform.shape[0] == R and out.shape[0] == R, "sample_full: rows")
+    n_pad = 2
+    while n_pad < V:
+        n_pad *= 2
+    work = torch.empty(n * 3 * n_pad, dtype=torch.int32, device=logits.device)
+    _ok(_lib("sampling").dn_sample_full(logits.data_ptr(), ld, n, V, n_pad, rows.data_ptr(), temperature.data_ptr(),
+                                        uniform.data_ptr(), top_p.data_ptr(), work.data_ptr(), out.data_ptr(),
+                                        _stream()), "sample_full")
     return out
 
 

@@ -54,13 +54,26 @@ class Sampler:
             us = [0.0 if p.greedy else uniform(s, n) for p, s, n in zip(params, seeds, counters)]
             tu = torch.tensor([temps, us], dtype=torch.float32, device=dev)      # one copy for both
         t_dev, u_dev = tu[0], tu[1]
+        # top_p = 1 without top_k restricts nothing: such a row takes the plain walk over the whole
+        # vocabulary (the reference sorts it first, crates/denno-engine/src/sampler.rs:387-435, which
+        # gives the same distribution)
         restricted = [r for r, p in enumerate(params)
-                      if not p.greedy and (p.top_k is not None or p.top_p is not None)]
+                      if not p.greedy and (p.top_k is not None or (p.top_p is not None and p.top_p < 1.0))]
         ops.sample(logits, t_dev, u_dev, out)
-        if restricted:
-            rows = torch.tensor(restricted, dtype=torch.int32, device=dev)
-            ks = torch.tensor([params[r].top_k or 0 for r in restricted], dtype=torch.int32, device=dev)
-            ps = torch.tensor([params[r].top_p if params[r].top_p is not None else 1.0 for r in restricted],
-                              dtype=torch.float32, device=dev)
-            ops.sample_top(logits, rows, t_dev, u_dev, ks, ps, out)
-        return out.tolist()
+        if not restricted:
+            return out.tolist()
+        n = len(restricted)
+        top_p = [params[r].top_p if params[r].top_p is not None else 1.0 for r in restricted]
+        ints = torch.tensor([restricted, [params[r].top_k or 0 for r in restricted]], dtype=torch.int32, device=dev)
+        ps = torch.tensor(top_p, dtype=torch.float32, device=dev)
+        both = torch.empty(R + n, dtype=torch.int32, device=dev)       # tokens, then which listed rows are undecided
+        both[:R].copy_(out)
+        ops.sample_top(logits, ints[0], t_dev, u_dev, ints[1], ps, both[:R], both[R:])
+        host = both.tolist()
+        tokens, undecided = host[:R], [j for j in range(n) if host[R + j]]
+        if undecided:
+            # top-p alone whose cut lies beyond the 2,048 largest: the whole vocabulary, sorted
+            rows = torch.tensor([restricted[j] for j in undecided], dtype=torch.int32, device=dev)
+            ps = torch.tensor([top_p[j] for j in undecided], dtype=torch.float32, device=dev)
+            tokens = ops.sample_full(logits, rows, t_dev, u_dev, ps, both[:R]).tolist()
+        return tokens

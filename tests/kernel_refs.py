@@ -165,13 +165,26 @@ def penalties(logits, ctx, ctx_start, repetition, frequency, presence, ngram):
     return logits
 
 
-def sample_top(logits, rows, temperature, uniform, top_k, top_p, out):
+def sample_top(logits, rows, temperature, uniform, top_k, top_p, out, undecided):
     from plain import sampler_plain as sp
     for j, r in enumerate(rows.tolist()):
-        k = int(top_k[j]) or 2048
+        k, p = int(top_k[j]), float(top_p[j])
+        if k > 0:
+            out[r] = sp.top_k_top_p(logits[r].tolist(), float(temperature[r]), min(k, 2048),
+                                    None if p >= 1.0 else p, float(uniform[r]))
+            undecided[j] = 0
+        else:
+            tok, whole = sp.top_p_alone(logits[r].tolist(), float(temperature[r]), p, float(uniform[r]))
+            out[r], undecided[j] = tok, int(whole)
+    return out
+
+
+def sample_full(logits, rows, temperature, uniform, top_p, out):
+    from plain import sampler_plain as sp
+    for j, r in enumerate(rows.tolist()):
         p = float(top_p[j])
-        out[r] = sp.top_k_top_p(logits[r].tolist(), float(temperature[r]), min(k, 2048),
-                                None if p >= 1.0 else p, float(uniform[r]))
+        out[r] = sp.top_k_top_p(logits[r].tolist(), float(temperature[r]), None, None if p >= 1.0 else p,
+                                float(uniform[r]))
     return out
 
 

@@ -72,6 +72,40 @@ def top_k_top_p(logits, t, top_k, top_p, u):
     return z[len(probs) - 1][1]
 
 
+TOP_P_SUBSET = 2048      # sampler.rs:23
+
+
+def top_p_alone(logits, t, top_p, u):
+    """top-p without top-k (sampler.rs:387-435): over a vocabulary larger than 2,048 the cut is
+    looked for among the 2,048 largest, with probabilities relative to their sum; if it falls
+    before the last of them the token is drawn from that head of the list, else everything is
+    done over again on the whole sorted vocabulary (sample_legacy_full, :466-476).
+    -> (token, whether the whole vocabulary was needed)."""
+    n = len(logits)
+    if n > TOP_P_SUBSET:
+        z = [(f32(x) / f32(t), i) for i, x in enumerate(logits)]
+        z.sort(key=lambda a: (-a[0], a[1]))
+        sub = z[:TOP_P_SUBSET]
+        mx = sub[0][0]
+        probs = [math.exp(a[0] - mx) for a in sub]
+        total = sum(probs)
+        cum, cutoff = 0.0, TOP_P_SUBSET
+        for i, p in enumerate(probs):
+            cum += p / total
+            if cum >= top_p:
+                cutoff = i + 1
+                break
+        if cutoff < TOP_P_SUBSET:
+            pr = probs[:cutoff]
+            r = u * sum(pr)
+            for i, p in enumerate(pr):
+                r -= p
+                if r <= 0.0:
+                    return sub[i][1], False
+            return sub[cutoff - 1][1], False
+    return top_k_top_p(logits, t, None, top_p, u), n > TOP_P_SUBSET
+
+
 def repetition_penalty(logits, context, penalty):
     """Each distinct context token once: l > 0 -> l / p, else l * p (sampler.rs:42-58)."""
     out = list(logits)

@@ -3,6 +3,8 @@ Unit vectors after the reference's cache tests (crates/denno-engine/src/kv_cache
 turned from rows of one buffer into pages of a pool."""
 import random
 
+import numpy as np
+
 import pytest
 
 from denno_beta_amd.cache import PAGED, STATE, CacheError, CacheManager, GroupLayout, OutOfPages
@@ -81,6 +83,24 @@ def test_slots_and_generations():
     g = m.generation(a)
     m.release(10)
     assert m.add(12) == a and m.generation(a) == g + 1      # the slot is used again, under a new generation
+
+
+def test_a_slot_record_starts_at_zero_for_the_next_request():
+    m = mk(max_requests=1)
+    slot = m.add(10)
+    m.reserve(10, 20), m.commit(10, 20)
+    m.set_rng(10, 2 ** 63 + 5, 3)
+    m.note_sampled(10, 77)
+    st = m.state(10)
+    assert (st.num_computed, st.last_token, st.rng_seed, st.rng_drawn) == (20, 77, 2 ** 63 + 5, 4)
+    seeds, drawn = m.rng_states(np.asarray([10], dtype=np.int64))
+    assert seeds.tolist() == [2 ** 63 + 5] and drawn.tolist() == [4]
+    m.release(10)
+    with pytest.raises(CacheError, match="no live request"):
+        m.state(10)
+    assert m.add(11) == slot
+    st = m.state(11)
+    assert (st.num_computed, st.last_token, st.rng_seed, st.rng_drawn) == (0, -1, 0, 0)
 
 
 def test_freed_pages_are_used_again():

@@ -162,6 +162,100 @@ def test_a_failed_step_gives_everything_back(backend, model_folders):
     assert e.generate([prompt], sp)[0] == clean
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_step_that_fails_between_its_kernels(model_folders, dtype):
+    """A step that fails after some of its kernels have run (crates/denno-engine/src/engine.rs:3354-3438:
+    the reference's failing model errors after it has written the cache): keys and values of some
+    layers stand in pages that go back to the pool.  Whatever the kernel it fails at (the first of layer
+    0, one in the middle, the head's), every page and slot comes back, the other requests' error is
+    reported, and the next requests, which get those pages, give a clean engine's tokens bit for bit."""
+    from denno_beta_amd.engine import SamplingParams
+    from denno_beta_amd.kernels import ops
+    folder = model_folders("B", dtype)
+    prompts = [seeded_tokens(50 + i, n, 1000) for i, n in enumerate((40, 9, 75))]
+    sp = SamplingParams(max_tokens=6, temperature=0.0)
+    mk = lambda: engine_for(folder, dtype, "cuda:0", cache_tokens=256, use_graphs=False)   # noqa: E731
+    clean = mk().generate(prompts, sp)
+    e = mk()
+    for p in prompts:
+        e.add_request(p, sp)
+    e.step()
+    before = ops.launches
+    e.step()
+    per_step = ops.launches - before              # launches of the step that will fail, the sampling kernel last
+    assert per_step > 3 * 4
+    for n in (0, 3, per_step // 2, per_step - 3, per_step - 1):
+        e = mk()
+        rids = [e.add_request(p, sp) for p in prompts]
+        e.step()                                   # the prompts are in the cache, a token each is sampled
+        ops.fail_after_launches(n)
+        with pytest.raises(ops.KernelError, match="injected"):
+            e.step()
+        assert ops._fail_after is None
+        assert all(e.finish_reason(r) == "error" for r in rids) and not e.has_unfinished()
+        m = e.runner.cache.manager
+        assert m.live() == 0 and m.free_pages(0) == 16
+        m.check()
+        assert e.generate(prompts, sp) == clean, f"after a failure at launch {n}"
+        assert m.reuse_count(0) > 0
+    ops.fail_after_launches(None)
+
+
+def test_the_slot_record_holds_position_and_generator(backend, model_folders):
+    """A live request's slot record (position, generator, last token) follows what the engine does, is
+    zero for the next request that gets the slot, and carries a preempted request's generator on."""
+    from denno_beta_amd.engine import SamplingParams
+    from denno_beta_amd.sampling import uniform
+    e = engine_for(model_folders("A", "float32"), "float32", backend, cache_tokens=256, max_live=1)
+    m = e.runner.cache.manager
+    prompt = seeded_tokens(3, 11, 512)
+    rid = e.add_request(prompt, SamplingParams(max_tokens=3, temperature=0.7, seed=99))
+    e.step()
+    st = m.state(rid)
+    tok = e.requests[rid].generated[0]
+    assert (st.num_computed, st.last_token, st.rng_seed, st.rng_drawn) == (11, tok, 99, 1)
+    e.step()
+    st = m.state(rid)
+    assert (st.num_computed, st.last_token, st.rng_drawn) == (12, e.requests[rid].generated[1], 2)
+    while e.has_unfinished():
+        e.step()
+    other = e.add_request(prompt[:4], SamplingParams(max_tokens=2, temperature=0.0, seed=5))
+    e.step()
+    st = m.state(other)
+    assert m.slot(other) == 0 and (st.num_computed, st.rng_seed, st.rng_drawn) == (4, 5, 1)
+    assert uniform(99, 0) != uniform(99, 1)
+
+
+@pytest.mark.gpu
+def test_serving_at_large_layer_sizes_gives_each_request_its_solo_tokens(tmp_path):
+    """Two layers of GPT-2 Large's sizes, 24 requests with prompts of 16 to 300 tokens admitted into a
+    running batch, portions of 64, 200 tokens a step, so few pages that requests are put back: in 32-bit
+    every request's tokens are those of its run alone, as interleaved sessions equal solo ones in the
+    reference (crates/denno-engine/src/engine.rs:2449-2542)."""
+    import torch
+    from denno_beta_amd.config import EngineOptions
+    from denno_beta_amd.engine import Engine, SamplingParams
+    from denno_beta_amd.weights import write_model_folder
+    cfg = dict(architectures=["GPT2LMHeadModel"], n_layer=2, n_embd=1280, n_head=20, n_inner=5120, vocab_size=50257,
+               n_positions=1024, layer_norm_epsilon=1e-5, activation_function="gelu_new")
+    folder = write_model_folder(str(tmp_path), cfg, 3, "float32")
+    g = torch.Generator().manual_seed(4)
+    lengths = torch.randint(16, 301, (24,), generator=g).tolist()
+    prompts = [torch.randint(0, 50257, (n,), generator=g).tolist() for n in lengths]
+    sp = SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True)
+    mk = lambda **kw: Engine.from_folder(folder, EngineOptions(dtype="float32", page_size=16, **kw))   # noqa: E731
+    solo = mk(max_live=1, cache_tokens=1024)
+    want = [solo.generate([p], sp)[0] for p in prompts]
+    e = mk(max_live=8, cache_tokens=800, prefill_chunk=64, max_batch_tokens=200)
+    got = e.generate(prompts, sp)
+    assert got == want
+    assert sum(1 for r in e.records if r.decode_rows and r.prefill_rows) > 10, "few steps mixed prompts and decoding"
+    assert sum(r.preempted for r in e.records) > 0, "the pool was too large: nobody was put back"
+    e.runner.cache.manager.check()
+    assert e.runner.cache.manager.live() == 0
+
+
 def test_command_line(backend, model_folders):
     """`denno generate` with the reference's option names; greedy, against the plain implementation."""
     if backend == "cpu":
@@ -174,6 +268,29 @@ def test_command_line(backend, model_folders):
                           "--raw"], capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stderr
     assert [int(t) for t in out.stdout.strip().split(",")] == want
+
+
+def test_command_line_with_several_prompts(backend, model_folders, tmp_path):
+    """`denno generate --prompt-file`: five prompts through the scheduler at once, with three live
+    requests, portions of 8 tokens, 20 tokens a step and so few pages that requests wait or are put
+    back: every line equals the prompt's run alone."""
+    if backend == "cpu":
+        pytest.skip("the command line runs the HIP kernels")
+    folder = model_folders("A", "float32")
+    prompts = [seeded_tokens(30 + i, n, 512) for i, n in enumerate((9, 40, 17, 3, 60))]
+    plain = PlainGPT2.from_folder(folder)
+    want = [plain.greedy(p, 6) for p in prompts]
+    path = tmp_path / "prompts.txt"
+    path.write_text("".join((", " if i % 2 else " ").join(map(str, p)) + "\n" for i, p in enumerate(prompts)))
+    for policy in ("preempt", "reserve"):
+        out = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "denno"), "generate", folder, "--prompt-file",
+                              str(path), "--max-tokens", "6", "--temperature", "0", "--quant", "fp32", "--raw",
+                              "--max-live", "3", "--page-size", "16", "--cache-tokens", "128", "--prefill-chunk", "8",
+                              "--max-batch-tokens", "20", "--kv-policy", policy], capture_output=True, text=True,
+                             timeout=300)
+        assert out.returncode == 0, out.stderr
+        got = [[int(t) for t in line.split(",")] for line in out.stdout.strip().splitlines()]
+        assert got == want, policy
 
 
 def test_command_line_with_text(backend, model_folders, tmp_path):

@@ -557,6 +557,44 @@ def test_attention_window_edges():
         assert abs(out[pos, 0].item() - (lo + pos) / 2) < 1e-3, pos
 
 
+@pytest.mark.parametrize("H,dh,window,n", [(2, 64, 37, 700), (2, 64, 100, 700), (1, 128, 100, 1000), (3, 32, 300, 520)])
+def test_attention_window_edges_in_every_kernel(H, dh, window, n):
+    """All scores equal and values that name their position (dim p % dh is 1 at position p): the output is,
+    per dim, the share of the window's positions with that remainder, so one key too many or too few at
+    either edge of the window changes a dim by 1 / window, which is far above what bfloat16 rounds.
+    The 32-bit kernel, the bfloat16 kernel for portions and the bfloat16 kernel for single rows (with the
+    context split over workgroups where the head size makes chunks of 512 keys, so that a split lies
+    wholly before the window)."""
+    ps = 16
+    for dtype in (torch.float32, torch.bfloat16):
+        q, k, v, bt, tiles, T = paged_case([n], [n], H, H, dh, ps, dtype, seed=window)
+        k.zero_(), v.zero_()
+        pos = torch.arange(n, device=DEV)
+        pages, offs = bt[0, pos // ps].long(), pos % ps
+        for h in range(H):
+            v[pages, h, pos % dh, offs] = 1.0
+        # want[p, d]: how many positions of [lo, p] have remainder d, over the window's length
+        onehot = torch.zeros(n, dh, device=DEV)
+        onehot[pos, pos % dh] = 1.0
+        cum = torch.cat([torch.zeros(1, dh, device=DEV), onehot.cumsum(0)])
+        lo = (pos - window + 1).clamp(min=0)
+        want = ((cum[pos + 1] - cum[lo]) / (pos - lo + 1).unsqueeze(1)).repeat(1, H)
+        kinds = [dict()] if dtype == torch.float32 else [dict(tiles_wide=paged_case.wide)]
+        for kw in kinds:
+            out = torch.zeros(T, H * dh, dtype=dtype, device=DEV)
+            ops().attention(q[:, :H * dh], out, k, v, bt, tiles, H, 1.0, window, **kw)
+            worst = (out.float() - want).abs().max(dim=1).values
+            assert worst.max().item() < 0.2 / window, (dtype, int(worst.argmax()), worst.max().item())
+        if dtype == torch.bfloat16:
+            for p in sorted({0, 1, window - 2, window - 1, window, window + 1, 255, 256, 257, 511, 512, 513, n - 1}):
+                if p >= n:
+                    continue
+                out = torch.zeros(1, H * dh, dtype=dtype, device=DEV)
+                ops().attention(q[p:p + 1, :H * dh], out, k, v, bt, i32([[0], [0], [1], [p]]), H, 1.0, window,
+                                single_rows=True, max_context=min(-(-(p + 1) // 256) * 256, bt.shape[1] * ps))
+                assert (out[0].float() - want[p]).abs().max().item() < 0.2 / window, ("single row", p)
+
+
 def test_attention_rows_do_not_depend_on_the_batch():
     H, dh, ps = 4, 32, 16
     q, k, v, bt, tiles, T = paged_case([200, 90], [50, 90], H, H, dh, ps, torch.float32, seed=2)
@@ -612,9 +650,12 @@ def test_sample_top_and_penalties():
     for trial in range(5):
         u = torch.tensor([uniform(trial, i) for i in range(8)], device=DEV)
         out = torch.full((8,), -1, dtype=torch.int32, device=DEV)
-        ops().sample_top(logits, rows, temp, u, ks, ps, out)
-        want = R.sample_top(logits.cpu(), rows.cpu(), temp.cpu(), u.cpu(), ks.cpu(), ps.cpu(), torch.full((8,), -1, dtype=torch.int32))
+        undecided = torch.full((5,), -1, dtype=torch.int32, device=DEV)
+        ops().sample_top(logits, rows, temp, u, ks, ps, out, undecided)
+        want = R.sample_top(logits.cpu(), rows.cpu(), temp.cpu(), u.cpu(), ks.cpu(), ps.cpu(),
+                            torch.full((8,), -1, dtype=torch.int32), torch.zeros(5, dtype=torch.int32))
         assert out.tolist() == want.tolist(), trial
+        assert undecided.tolist() == [0] * 5          # a vocabulary within the 2,048 candidates is always decided
     assert out[2].item() == 10
     ctx = i32([3, 4, 3, 9, 4, 3] + [7, 8, 7, 8, 7])
     start = i32([0, 6, 6, 11])
@@ -624,3 +665,39 @@ def test_sample_top_and_penalties():
     ops().penalties(l, ctx, start, torch.tensor([1.5, 1.0, 1.0], device=DEV), torch.tensor([0.3, 0.0, 0.0], device=DEV),
                     torch.tensor([0.2, 0.0, 0.5], device=DEV), i32([0, 0, 2]))
     assert torch.allclose(l.cpu(), want, atol=1e-6) and l[2, 8].item() == float("-inf")
+
+
+def test_top_p_beyond_the_2048_largest_takes_the_whole_vocabulary():
+    """Flat logits over a vocabulary of 50,257 with top-p 0.9999: among the 2,048 largest the cut falls on
+    the last, so the subset kernel must leave the row undecided and the kernel over the whole sorted
+    vocabulary decide it, as the reference falls back to its full path (sampler.rs:387-435).  Tokens
+    outside the 2,048 largest are drawn, and each draw is the plain sampler's."""
+    from denno_beta_amd.sampling import Sampler, SamplingParams, uniform
+    V, n = 50257, 24
+    g = torch.Generator().manual_seed(8)
+    row = torch.randn(V, generator=g) * 0.05
+    row[777] = 0.5                                      # one clear head of the list
+    logits = row.repeat(n, 1).to(DEV).contiguous()
+    rows = i32(list(range(n)))
+    ps = torch.full((n,), 0.9999, device=DEV)
+    ps[n - 1] = 1e-6                                    # so small a p that the head alone is kept: decided in the subset
+    temp = torch.full((n,), 1.0, device=DEV)
+    u = torch.tensor([uniform(3, i) for i in range(n)], device=DEV)
+    out = torch.full((n,), -1, dtype=torch.int32, device=DEV)
+    undecided = torch.full((n,), -1, dtype=torch.int32, device=DEV)
+    ops().sample_top(logits, rows, temp, u, i32([0] * n), ps, out, undecided)
+    assert undecided.tolist() == [1] * (n - 1) + [0] and out[n - 1].item() == 777
+    ops().sample_full(logits, rows[:n - 1].contiguous(), temp, u, ps[:n - 1].contiguous(), out)
+    top = set(row.topk(2048).indices.tolist())
+    got = out.tolist()
+    assert sum(1 for t in got[:n - 1] if t not in top) > n // 2, "draws never left the 2,048 largest"
+    for i in range(0, n - 1, 4):
+        tok, whole = SP.top_p_alone(row.tolist(), 1.0, 0.9999, float(u[i]))
+        assert whole and tok == got[i], i
+    # the sampler does both steps, and with top_p = 1 takes the plain walk
+    sp = SamplingParams(temperature=1.0, top_p=0.9999, seed=3)
+    toks = Sampler(torch.device(DEV)).sample(logits[:4].clone(), [sp] * 4, [3] * 4, [0, 1, 2, 3], [[]] * 4)
+    assert toks == got[:4]
+    one = SamplingParams(temperature=1.0, top_p=1.0, seed=3)
+    toks = Sampler(torch.device(DEV)).sample(logits[:4].clone(), [one] * 4, [3] * 4, [0, 1, 2, 3], [[]] * 4)
+    assert toks == [SP.temperature_walk(row.tolist(), 1.0, uniform(3, i)) for i in range(4)]

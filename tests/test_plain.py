@@ -217,6 +217,27 @@ def test_top_k_and_top_p():
     assert {S.top_k_top_p(logits, 1.0, None, 0.1, u / 10) for u in range(10)} == {1}
 
 
+def test_top_p_alone_falls_back_to_the_whole_vocabulary():
+    """sampler.rs:387-435: over more than 2,048 tokens the cut is looked for among the 2,048 largest, with
+    probabilities relative to their sum: a row is decided there unless the cut falls on the last of them
+    (a flat row with p near 1), which needs the whole vocabulary, and then tokens beyond the 2,048 largest
+    are drawn.  Up to 2,048 tokens there is the whole vocabulary only."""
+    n = 3000
+    peaked = [0.0] * n
+    peaked[5], peaked[9] = 12.0, 11.0
+    tok, whole = S.top_p_alone(peaked, 1.0, 0.9, 0.99)
+    assert not whole and tok == 9 and S.top_p_alone(peaked, 1.0, 0.5, 0.99) == (5, False)
+    flat = [0.001 * ((i * 7919) % n) / n for i in range(n)]
+    order = sorted(range(n), key=lambda i: (-flat[i], i))
+    draws = [S.top_p_alone(flat, 1.0, 0.9, u / 50) for u in range(50)]
+    assert not any(whole for _, whole in draws)             # 0.9 of the 2,048 largest's mass lies among them
+    assert all(order.index(tok) < 0.9 * 2048 + 2 for tok, _ in draws)
+    draws = [S.top_p_alone(flat, 1.0, 0.9999, u / 50) for u in range(50)]
+    assert all(whole for _, whole in draws)
+    assert any(order.index(tok) >= 2048 for tok, _ in draws)
+    assert S.top_p_alone([1.0, 3.0, 2.0], 1.0, 0.1, 0.5) == (1, False)
+
+
 def test_penalties():
     l = [2.0, -2.0, 1.0, 0.5]
     assert S.repetition_penalty(l, [0, 1, 0], 2.0) == [1.0, -4.0, 1.0, 0.5]      # each distinct token once

@@ -160,6 +160,29 @@ def test_step_refuses_what_it_cannot_run(backend, model_folders):
     assert r.cache.manager.length(0) == 3
 
 
+def test_a_refused_step_leaves_nothing_of_the_requests_it_started(backend, model_folders):
+    """A replayed step that cannot run (a token outside the vocabulary, a request named twice, no pages
+    left) gives back the slots of the requests that it started; requests that were live before stay."""
+    from denno_beta_amd.cache import OutOfPages
+    from denno_beta_amd.engine import BatchError
+    from denno_beta_amd.engine.replay import TraceReplayer
+    r = runner_for(model_folders("A", "float32"), "float32", backend, cache_tokens=64, max_live=2)
+    rp = TraceReplayer(r)
+    rp.run_step({"step": 0, "entries": [{"id": "old", "tokens": [1, 2, 3], "want": []}], "end": []})
+    for bad, error in (([{"id": "new", "tokens": [5, 512], "want": []}], BatchError),
+                       ([{"id": "new", "tokens": [5], "want": []}, {"id": "new", "tokens": [6], "want": []}], BatchError),
+                       ([{"id": "new", "tokens": [1] * 60, "want": []}], OutOfPages)):
+        with pytest.raises(error):
+            rp.run_step({"step": 1, "entries": bad, "end": []})
+        assert rp.live() == ["old"] and r.cache.manager.live() == 1
+        r.cache.manager.check()
+    # the slot that the refused requests took and gave back serves the next one
+    out = rp.run_step({"step": 2, "entries": [{"id": "new", "tokens": [7, 8], "want": [1]},
+                                              {"id": "old", "tokens": [4], "want": [0]}], "end": ["new", "old"]})
+    assert out.shape == (2, 512) and rp.live() == [] and r.cache.manager.live() == 0
+    r.cache.manager.check()
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decode_graphs_replay_what_eager_steps_compute(model_folders, dtype):

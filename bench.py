@@ -4,27 +4,38 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one decode step of the engine (scheduler, step function, sampling): batch 8 from a
-512-token context by default.  One JSON line: decoded tokens a second, the prefill of 2,048
-tokens (two prompts of 1,024 in one step), the decode step's share of the HBM roofline, and
-decoding at batch 1 and 64.  Peaks are the published ones of MI355X.
+512-token context by default.  Every figure is the median of three blocks of K steps (of three runs for
+the prefill).  One JSON line: decoded tokens a second, the prefill of 2,048 tokens (two prompts of 1,024
+in one step), the decode step's share of the HBM roofline, decoding at batch 1 and 64 (`points`: tokens a
+second; `point_details`: milliseconds, bytes and share of the roofline of each), and the 32-bit engine's
+decode steps and prefill (`fp32`).  Peaks are the published ones of MI355X.
+
+    python bench.py --only decode|prefill [--kernel-times]   one workload; with --kernel-times kernel by
+                                                             kernel, each launch between two HIP events
+    python bench.py --only serving [--dtype float32]         BASELINE.json's configs[3] through the scheduler
+    python bench.py --only replay [--sequences 8]            BASELINE.json's configs[4] against the plain
+                                                             implementation, in four ways of cutting
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
-sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+SHORT = {"bfloat16": "bf16", "float32": "fp32"}
 
 
-def xl_config(n_layer):
-    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "BASELINE.json")) as f:
-        text = json.load(f)["configs"][2]
-    # the sizes that BASELINE.json's configs[2] names in words
+def baseline_config(index, n_layer=0):
+    """The sizes that BASELINE.json's configs[index] names in words -> (config.json keys, its layers)."""
     import re
+    with open(os.path.join(ROOT, "BASELINE.json")) as f:
+        text = json.load(f)["configs"][index]
     num = lambda key: int(re.search(key + r"=(\d+)", text).group(1))   # noqa: E731
     cfg = dict(architectures=["GPT2LMHeadModel"], n_layer=num("n_layer"), n_embd=num("n_embd"), n_head=num("n_head"),
                n_inner=num("n_inner"), vocab_size=num("vocab_size"), n_positions=num("n_positions"),
@@ -33,6 +44,102 @@ def xl_config(n_layer):
     if n_layer:
         cfg["n_layer"] = n_layer
     return cfg, full
+
+
+class Workloads:
+    """The decode and prefill measurements on one runner."""
+
+    def __init__(self, a, dtype):
+        import torch
+        from denno_beta_amd.config import EngineOptions
+        from denno_beta_amd.engine import ModelRunner
+        self.torch, self.a, self.dtype = torch, a, dtype
+        self.cfg, self.full_layers = baseline_config(2, a.layers)
+        P = self.cfg["n_positions"]
+        live = max(64, a.batch)
+        self.opts = EngineOptions(dtype=dtype, page_size=16, cache_tokens=live * P, max_live=live, max_batch_tokens=4096,
+                                  prefill_chunk=1024, use_graphs=not (a.no_graphs or a.kernel_times), seed=0,
+                                  norms_inside_products=not a.norm_kernels)
+        self.runner = ModelRunner.from_random(self.cfg, seed=0, options=self.opts, stored=dtype)
+        self.gen = torch.Generator().manual_seed(0)
+
+    def prompt(self, n):
+        return self.torch.randint(0, self.cfg["vocab_size"], (n,), generator=self.gen).tolist()
+
+    def decode(self, batch, steps, warmup, blocks=3):
+        """-> {ms, tok_s, bytes, frac, mean_context}: the median block of `steps` steps."""
+        from denno_beta_amd.engine import Engine, SamplingParams
+        a, P, sync = self.a, self.cfg["n_positions"], self.torch.cuda.synchronize
+        steps = max(1, min(steps, (P - a.context - warmup - 2) // blocks))
+        eng = Engine(self.runner, self.opts)
+        sp = SamplingParams(max_tokens=P, temperature=0.0, ignore_eos=True)
+        rids = [eng.add_request(self.prompt(a.context), sp) for _ in range(batch)]
+        while any(eng.scheduler.computed(r) < a.context for r in rids):
+            eng.step()
+        for _ in range(warmup):
+            eng.step()
+        times = []
+        for _ in range(blocks):
+            sync()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                eng.step()
+            sync()
+            times.append((time.perf_counter() - t0) / steps)
+        assert all(len(eng.requests[r].generated) >= blocks * steps for r in rids)
+        for r in rids:
+            eng.abort(r)
+        order = sorted(range(blocks), key=lambda i: times[i])
+        mid = order[blocks // 2]
+        mean_ctx = a.context + 1 + warmup + mid * steps + (steps - 1) / 2.0
+        nbytes = self.runner.model.weight_bytes() + batch * mean_ctx * self.runner.cache.bytes_per_token()
+        t = times[mid]
+        return {"ms": t * 1e3, "tok_s": batch / t, "bytes": nbytes, "frac": nbytes / t / 1e9 / HBM_PEAK_GBS,
+                "mean_context": mean_ctx, "steps": steps}
+
+    def prefill(self, reps=3):
+        """-> {value, tokens, ms, frac}: two prompts of 1,024 tokens in one step, the median of `reps`."""
+        from denno_beta_amd.engine import StepEntry
+        runner, sync = self.runner, self.torch.cuda.synchronize
+        times = []
+        for i in range(reps + 1):
+            seqs = [self.prompt(1024), self.prompt(1024)]
+            for j in range(2):
+                runner.start_request(1000 + j)
+            sync()
+            t0 = time.perf_counter()
+            runner.step([StepEntry(1000 + j, seqs[j], [1023]) for j in range(2)])
+            sync()
+            times.append(time.perf_counter() - t0)
+            for j in range(2):
+                runner.end_request(1000 + j)
+        t = statistics.median(times[1:])
+        cfg = self.cfg
+        V, E = cfg["vocab_size"], cfg["n_embd"]
+        mat = sum(w.numel() for w in _layer_matrices(runner))
+        flops = 2.0 * 2048 * mat + 2.0 * 2 * V * E + cfg["n_layer"] * 2 * (4.0 * E * 1024 * 1025 / 2)
+        return {"value": 2048 / t, "tokens": 2048, "ms": t * 1e3, "frac": flops / t / MFMA_PEAK[SHORT[self.dtype]]}
+
+
+def _layer_matrices(runner):
+    from denno_beta_amd.parts import Linear
+    seen = []
+    for b in runner.model.blocks:
+        for p in b.parts():
+            for v in vars(p).values():
+                if isinstance(v, Linear):
+                    seen.append(v.weight)
+    return seen
+
+
+def kernel_table(what):
+    """Prints the per-kernel shares that ops.time_launches measured."""
+    from denno_beta_amd.kernels import ops
+    times = ops.launch_times()
+    total = sum(ms for _, ms in times.values())
+    print(f"{what}: {total:.3f} ms in {sum(n for n, _ in times.values())} launches (each between two events)")
+    for name, (n, ms) in sorted(times.items(), key=lambda kv: -kv[1][1]):
+        print(f"  {ms / total * 100:5.1f} %  {ms / n * 1e3:8.1f} us x {n:5d}  {name}")
 
 
 def main():
@@ -47,116 +154,95 @@ def main():
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--norm-kernels", action="store_true",
                     help="run every norm as a kernel of its own, also in steps of few rows (for comparisons)")
-    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
-    ap.add_argument("--only", choices=["decode", "prefill", "serving"], default=None,
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64, the prefill and the 32-bit engine")
+    ap.add_argument("--kernel-times", action="store_true",
+                    help="with --only decode or prefill: every launch between two HIP events (no graphs), and a "
+                         "table of each kernel's share")
+    ap.add_argument("--sequences", type=int, default=8, help="--only replay: how many of the eight sequences")
+    ap.add_argument("--only", choices=["decode", "prefill", "serving", "replay"], default=None,
                     help="run one workload and print a short line (decode, prefill: for profiling; serving: "
-                         "BASELINE.json's configs[3], GPT-2 Large shape, 64 requests through the scheduler)")
+                         "BASELINE.json's configs[3], GPT-2 Large shape, 64 requests through the scheduler; replay: "
+                         "configs[4], GPT-2 Medium shape, against the plain implementation)")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
         sys.exit(2)
-
-    import torch
-    from denno_beta_amd.config import EngineOptions
-    from denno_beta_amd.engine import Engine, ModelRunner, SamplingParams, StepEntry
-
     if a.only == "serving":
         return serving(a)
-    cfg, full_layers = xl_config(a.layers)
-    V, E, P = cfg["vocab_size"], cfg["n_embd"], cfg["n_positions"]
-    if a.context + a.warmup + a.steps + 1 > P:
-        a.steps = P - a.context - a.warmup - 1
-    live = max(64, a.batch)
-    opts = EngineOptions(dtype=a.dtype, page_size=16, cache_tokens=live * P, max_live=live, max_batch_tokens=4096,
-                         prefill_chunk=1024, use_graphs=not a.no_graphs, seed=0, norms_inside_products=not a.norm_kernels)
-    runner = ModelRunner.from_random(cfg, seed=0, options=opts, stored=a.dtype)
-    gen = torch.Generator().manual_seed(0)
-    prompt = lambda n: torch.randint(0, V, (n,), generator=gen).tolist()   # noqa: E731
-    sync = torch.cuda.synchronize
+    if a.only == "replay":
+        return replay(a)
 
-    def decode_point(batch, steps, warmup):
-        eng = Engine(runner, opts)
-        sp = SamplingParams(max_tokens=P, temperature=0.0, ignore_eos=True)
-        rids = [eng.add_request(prompt(a.context), sp) for _ in range(batch)]
-        while any(eng.scheduler.computed(r) < a.context for r in rids):
-            eng.step()
-        for _ in range(warmup):
-            eng.step()
-        sync()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            eng.step()
-        sync()
-        dt = time.perf_counter() - t0
-        assert all(len(eng.requests[r].generated) >= steps for r in rids)
-        mean_ctx = a.context + 1 + warmup + (steps - 1) / 2.0
-        for r in rids:
-            eng.abort(r)
-        return dt / steps, mean_ctx
-
-    def prefill_point(reps=3):
-        times = []
-        for i in range(reps + 1):
-            seqs = [prompt(1024), prompt(1024)]
-            for j in range(2):
-                runner.start_request(1000 + j)
-            sync()
-            t0 = time.perf_counter()
-            runner.step([StepEntry(1000 + j, seqs[j], [1023]) for j in range(2)])
-            sync()
-            times.append(time.perf_counter() - t0)
-            for j in range(2):
-                runner.end_request(1000 + j)
-        return sorted(times[1:])[len(times[1:]) // 2]
-
-    if a.only == "prefill":
-        t = prefill_point()
-        print(json.dumps({"prefill_ms": t * 1e3, "tokens": 2048}))
+    w = Workloads(a, a.dtype)
+    if a.only in ("prefill", "decode"):
+        from denno_beta_amd.kernels import ops
+        if a.only == "prefill":
+            w.prefill(1)
+            if a.kernel_times:
+                ops.time_launches(True)
+            r = w.prefill(1 if a.kernel_times else 3)
+            print(json.dumps({"prefill_ms": r["ms"], "tokens": 2048, "frac": r["frac"]}))
+        else:
+            if a.kernel_times:
+                w.decode(a.batch, 2, 2, blocks=1)
+                ops.time_launches(True)
+            r = w.decode(a.batch, a.steps, a.warmup, blocks=1 if a.kernel_times else 3)
+            print(json.dumps({"decode_ms_per_step": r["ms"], "batch": a.batch, "mean_context": r["mean_context"],
+                              "frac": r["frac"]}))
+        if a.kernel_times:
+            kernel_table(f"{a.only}, {a.dtype}")
         return
-    step_s, mean_ctx = decode_point(a.batch, a.steps, a.warmup)
-    if a.only == "decode":
-        print(json.dumps({"decode_ms_per_step": step_s * 1e3, "batch": a.batch, "mean_context": mean_ctx}))
-        return
-    weight_bytes = runner.model.weight_bytes()
-    kv_bytes = a.batch * mean_ctx * runner.cache.bytes_per_token()
-    achieved = (weight_bytes + kv_bytes) / step_s / 1e9
-    short = "bf16" if a.dtype == "bfloat16" else "fp32"
+
+    main_point = w.decode(a.batch, a.steps, a.warmup)
+    cfg, short = w.cfg, SHORT[a.dtype]
     out = {
-        "metric": "GPT-2 XL decode tokens/s (batch 8, context 512)", "value": a.batch / step_s, "unit": "tokens/s",
-        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": step_s * 1e3, "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": short, "data": "synthetic",
-        "config": {"model": "gpt2-xl-shape", "n_layer": cfg["n_layer"], "n_layer_full": full_layers, "n_embd": E,
-                   "n_head": cfg["n_head"], "n_inner": cfg["n_inner"], "vocab_size": V, "n_positions": P,
-                   "global_batch": a.batch, "seq_len": a.context, "page_size": opts.page_size,
-                   "weights": "random N(0,0.02)", "graphs": opts.use_graphs, "parallelism": "single-gpu"},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS},
+        "metric": "GPT-2 XL decode tokens/s (batch 8, context 512)", "value": main_point["tok_s"], "unit": "tokens/s",
+        "n_gpus": 1, "steps": main_point["steps"], "warmup": a.warmup, "ms_per_step": main_point["ms"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": short, "data": "synthetic",
+        "config": {"model": "gpt2-xl-shape", "n_layer": cfg["n_layer"], "n_layer_full": w.full_layers,
+                   "n_embd": cfg["n_embd"], "n_head": cfg["n_head"], "n_inner": cfg["n_inner"],
+                   "vocab_size": cfg["vocab_size"], "n_positions": cfg["n_positions"], "global_batch": a.batch,
+                   "seq_len": a.context, "page_size": w.opts.page_size, "weights": "random N(0,0.02)",
+                   "graphs": w.opts.use_graphs, "timing": "median of 3 blocks", "parallelism": "single-gpu"},
+        "roofline": {"bound": "hbm", "achieved": main_point["bytes"] / main_point["ms"] / 1e6, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": main_point["frac"]},
     }
     if not a.no_points:
-        t = prefill_point()
-        mat = sum(w.numel() for w in _layer_matrices(runner))
-        flops = 2.0 * 2048 * mat + 2.0 * 2 * V * E + cfg["n_layer"] * 2 * (4.0 * E * 1024 * 1025 / 2)
-        out["prefill"] = {"value": 2048 / t, "tokens": 2048, "ms": t * 1e3, "frac": flops / t / MFMA_PEAK[short]}
-        b1, _ = decode_point(1, min(a.steps, 100), a.warmup)
-        b64, _ = decode_point(64, min(a.steps, 50), a.warmup)
-        out["points"] = {"decode_b1": 1 / b1, "decode_b64": 64 / b64}
+        out["prefill"] = w.prefill()
+        b1 = w.decode(1, min(a.steps, 100), a.warmup)
+        b64 = w.decode(64, min(a.steps, 50), a.warmup)
+        out["points"] = {"decode_b1": b1["tok_s"], "decode_b64": b64["tok_s"]}
+        keep = lambda r: {k: r[k] for k in ("ms", "tok_s", "bytes", "frac")}   # noqa: E731
+        out["point_details"] = {"decode_b1": keep(b1), f"decode_b{a.batch}": keep(main_point), "decode_b64": keep(b64)}
+        if a.dtype == "bfloat16":
+            # the true 32-bit engine at the same sizes: every product in the plain kernels
+            del w
+            import torch
+            torch.cuda.empty_cache()
+            f = Workloads(a, "float32")
+            f1, f8 = f.decode(1, min(a.steps, 10), 2), f.decode(8, min(a.steps, 10), 2)
+            out["fp32"] = {"decode_b1": keep(f1), "decode_b8": keep(f8), "prefill": f.prefill()}
     print(json.dumps(out))
+
+
+def large_config():
+    return baseline_config(3)[0]
 
 
 def serving(a):
     """GPT-2 Large shape, random weights: 64 requests with prompt lengths uniform in [16, 768], 256
-    generated tokens each, greedy, continuous batching with prompt portions of 512."""
+    generated tokens each, greedy, continuous batching with prompt portions of 512.  After the timed
+    run four of the requests run again, each alone: their tokens must be the same (32-bit: exactly; in
+    bfloat16 a step's kernels depend on its rows, so the share of equal tokens is reported)."""
     import torch
     from denno_beta_amd.config import EngineOptions
     from denno_beta_amd.engine import Engine, SamplingParams
-    cfg = dict(architectures=["GPT2LMHeadModel"], n_layer=36, n_embd=1280, n_head=20, n_inner=5120, vocab_size=50257,
-               n_positions=1024, layer_norm_epsilon=1e-5, activation_function="gelu_new")
+    cfg = large_config()
     opts = EngineOptions(dtype=a.dtype, page_size=16, cache_tokens=64 * 1024, max_live=64, max_batch_tokens=2048,
                          prefill_chunk=512, use_graphs=not a.no_graphs, seed=0, norms_inside_products=not a.norm_kernels)
     eng = Engine.from_random(cfg, 0, opts, stored=a.dtype)
     gen = torch.Generator().manual_seed(1)
     lengths = torch.randint(16, 769, (64,), generator=gen).tolist()
-    prompts = [torch.randint(0, 50257, (n,), generator=gen).tolist() for n in lengths]
+    prompts = [torch.randint(0, cfg["vocab_size"], (n,), generator=gen).tolist() for n in lengths]
     sp = SamplingParams(max_tokens=256, temperature=0.0, ignore_eos=True)
     eng.generate(prompts[:2], SamplingParams(max_tokens=4, temperature=0.0, ignore_eos=True))   # warm-up
     eng.records.clear()
@@ -167,24 +253,96 @@ def serving(a):
     dt = time.perf_counter() - t0
     assert all(len(o) == 256 for o in out)
     steps = len(eng.records)
+    records = list(eng.records)
+    same = []
+    for i in (0, 21, 42, 63):
+        alone = eng.generate([prompts[i]], sp)[0]
+        first_other = next((j for j in range(256) if alone[j] != out[i][j]), 256)
+        same.append(first_other)
+    if a.dtype == "float32" and min(same) < 256:
+        raise SystemExit(f"serving: a request's tokens differ from its run alone (equal tokens before the first "
+                         f"difference, of 256: {same})")
     print(json.dumps({
         "workload": "GPT-2 Large shape, 64 requests, prompts U[16,768], 256 new tokens, prefill portions of 512",
         "seconds": dt, "generated_tokens": 64 * 256, "generated_tokens_per_s": 64 * 256 / dt,
         "prompt_tokens": sum(lengths), "all_tokens_per_s": (64 * 256 + sum(lengths)) / dt, "steps": steps,
-        "mean_rows_per_step": sum(r.rows for r in eng.records) / steps,
-        "mixed_steps": sum(1 for r in eng.records if r.decode_rows and r.prefill_rows),
-        "preemptions": sum(r.preempted for r in eng.records), "dtype": a.dtype}))
+        "mean_rows_per_step": sum(r.rows for r in records) / steps,
+        "mixed_steps": sum(1 for r in records if r.decode_rows and r.prefill_rows),
+        "preemptions": sum(r.preempted for r in records), "dtype": a.dtype,
+        "tokens_equal_to_the_run_alone_before_the_first_difference": same}))
 
 
-def _layer_matrices(runner):
-    from denno_beta_amd.parts import Linear
-    seen = []
-    for b in runner.model.blocks:
-        for p in b.parts():
-            for v in vars(p).values():
-                if isinstance(v, Linear):
-                    seen.append(v.weight)
-    return seen
+def replay(a):
+    """BASELINE.json's configs[4]: GPT-2 Medium shape, random weights stored in 32-bit, seeded sequences of
+    1,024 tokens replayed whole, token by token, in portions of 128 and mixed (four live requests, pages
+    used again), every logit compared with the plain implementation's; and the cuttings with each other."""
+    import torch
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import replay_util as U
+    from plain.gpt2_plain import PlainGPT2
+    from denno_beta_amd.config import EngineOptions
+    from denno_beta_amd.engine import ModelRunner
+    from denno_beta_amd.engine.replay import TraceReplayer
+    from denno_beta_amd.weights import write_model_folder
+    import tempfile
+    cfg, _ = baseline_config(4, a.layers)
+    V, n = cfg["vocab_size"], cfg["n_positions"]
+    seqs = [torch.randint(0, V, (n,), generator=torch.Generator().manual_seed(100 + i)).tolist()
+            for i in range(a.sequences)]
+    token_by_token = []
+    for base in range(0, len(seqs), 4):          # four requests live at a time, a token of each per step
+        group = list(range(base, min(base + 4, len(seqs))))
+        for t in range(n):
+            token_by_token.append({"step": len(token_by_token), "end": [f"r{i}" for i in group] if t == n - 1 else [],
+                                   "entries": [{"id": f"r{i}", "tokens": seqs[i][t:t + 1], "want": [0]} for i in group]})
+    traces = {"whole": U.whole_trace(seqs), "token by token": token_by_token,
+              "portions of 128": U.chunk_trace(seqs, sizes=(128,)),
+              "mixed": U.mixed_trace(seqs, seed=3, sizes=(1, 1, 1, 2, 5, 17, 40, 128))}
+    result = {"workload": f"GPT-2 Medium shape, {cfg['n_layer']} layers, {len(seqs)} sequences of {n} tokens"}
+    with tempfile.TemporaryDirectory() as folder:
+        print("replay: writing the model and running the plain implementation ...", file=sys.stderr, flush=True)
+        write_model_folder(folder, cfg, 4, "float32")
+        plain = PlainGPT2.from_folder(folder)
+        want = []
+        for i, s in enumerate(seqs):
+            want.append(plain.logits(s, by_head=True).cuda())
+            print(f"replay: plain logits of sequence {i}", file=sys.stderr, flush=True)
+        for dtype in ("float32", "bfloat16"):
+            whole = None
+            for kind, steps in traces.items():
+                tokens = U.max_live_tokens(steps)
+                runner = ModelRunner.from_folder(folder, EngineOptions(dtype=dtype, page_size=16, cache_tokens=tokens,
+                                                                       max_live=4), cast_matrices=True)
+                rp = TraceReplayer(runner)
+                got = [torch.empty_like(wt) for wt in want]
+                pos = {}
+                for st in steps:
+                    out = rp.run_step(st)
+                    k = 0
+                    for e in st["entries"]:
+                        i, base = int(e["id"][1:]), pos.get(e["id"], 0)
+                        m = len(e["want"])
+                        got[i][torch.tensor([base + x for x in e["want"]], device="cuda")] = out[k:k + m]
+                        k += m
+                        pos[e["id"]] = base + len(e["tokens"])
+                runner.cache.manager.check()
+                worst = max((g - wt).abs().max().item() for g, wt in zip(got, want))
+                agree = sum((g.argmax(1) == wt.argmax(1)).sum().item() for g, wt in zip(got, want)) / (len(seqs) * n)
+                entry = {"worst_difference_from_plain": worst, "greedy_token_agreement": agree,
+                         "steps": len(steps), "pages_used_again": runner.cache.manager.reuse_count(0)}
+                if whole is None:
+                    whole = got
+                else:
+                    entry["equal_to_whole_bit_for_bit"] = all(torch.equal(g, wg) for g, wg in zip(got, whole))
+                    entry["worst_difference_from_whole"] = max((g - wg).abs().max().item() for g, wg in zip(got, whole))
+                result[f"{dtype}, {kind}"] = entry
+                print(f"replay: {dtype}, {kind}: {entry}", file=sys.stderr, flush=True)
+                del runner, rp
+                if kind != "whole":
+                    del got
+            del whole
+    result["largest_logit"] = max(wt.abs().max().item() for wt in want)
+    print(json.dumps(result))
 
 
 if __name__ == "__main__":

@@ -186,7 +186,7 @@ __device__ __forceinline__ __bf16 to_bf16(float f) { return static_cast<__bf16>(
 // tiles its wave walks; two groups halve it, and join their running maxima, sums and weighted
 // values through LDS at the end, in group order.  With one group a wave takes two tiles per step
 // (up to a head size of 96: the tiles of two steps must fit 64 KB of LDS), under one maximum, one
-// sum and one rescaling (2 x 1024 rows: 58 -> 50 us).
+// sum and one rescaling.
 // A tile's keys and values come from the pages once per workgroup, 16 bytes per thread along
 // rows (two cache lines per 16 lanes), and lie in LDS for the four waves that need them, two
 // steps deep: the tiles of the step after the next are on their way to registers while this
@@ -505,9 +505,8 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
       reinterpret_cast<uintptr_t>(out) % 8 != 0)
     return DN_ERR_SHAPE;
   // Two groups of waves where the workgroups are fewer than the CUs (a wave's chain of dependent
-  // steps per tile then bounds the time, and two groups halve the tiles a wave walks: 1 request,
-  // 128 rows after 896: 40 -> 29 us); with more workgroups the SIMDs are busy and the second
-  // group's share of carrying tiles only adds work (2 x 1024 rows: 52 -> 66 us).  Up to a head
+  // steps per tile then bounds the time, and two groups halve the tiles a wave walks); with more
+  // workgroups the SIMDs are busy and the second group's share of carrying tiles only adds work.  Up to a head
   // size of 64: beyond, the tiles of two groups do not fit 64 KB of LDS.
   if (n_tiles > 65535) return DN_ERR_SHAPE;      // the grid's second dimension
   dim3 grid(H, n_tiles);

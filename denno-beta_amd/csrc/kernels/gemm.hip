@@ -15,8 +15,8 @@
 // 8 elements k % 32 / 8 * 8 .. + 7 of row n % 16 at ((k % 32 / 8) * 16 + n % 16) * 8: the 16 bytes
 // that lane (n % 16) + 16 * (k % 32 / 8) feeds to v_mfma_f32_16x16x32_bf16.  A wave then reads 1 KB
 // in one piece per block; from rows of K elements the same load touches 16 cache lines per
-// group of 16 lanes, and the rate of those lookups, not of bytes, bounded the kernel (measured:
-// 8.3 -> 6.7 us for 8 x 1600 . 1600 x 4800).  Rows and columns beyond N and K are zeros.
+// group of 16 lanes, and the rate of those lookups, not of bytes, bounds the kernel.  Rows and
+// columns beyond N and K are zeros.
 #include "common.h"
 
 #define EPI_NONE 0
@@ -34,7 +34,7 @@ __device__ __forceinline__ float apply_epilogue(float v, int epi) {
 
 // The same for the MFMA kernels, whose results are rounded to bfloat16: the tanh form as
 // v / (1 + 2^(-2 log2(e) u)) with the hardware's exponential and reciprocal (a dozen instructions
-// where tanhf takes several dozen; after a product of 2048 x 6400 the difference was 10 us of 65).
+// where tanhf takes several dozen, which shows in the epilogue of a product with many columns).
 __device__ __forceinline__ float apply_epilogue_fast(float v, int epi) {
   if (epi == EPI_GELU_TANH) {
     const float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
@@ -192,8 +192,8 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 // The norm that stands between two such products of few rows runs inside them (NORM_OUT in the product before
-// it, NORM_IN in the one after), so that it is no kernel of its own: a LayerNorm of 8 rows is 4 us
-// of launch and latency for no work.  With y = (x - mean) / sqrt(var + eps) * gamma + beta
+// it, NORM_IN in the one after), so that it is no kernel of its own: a LayerNorm of a few rows is
+// all launch and latency and no work.  With y = (x - mean) / sqrt(var + eps) * gamma + beta
 // (crates/denno-engine/src/tensor.rs:1101-1112),
 //     y . W^T + b = ((x * gamma) . W^T - mean * c1) / sqrt(var + eps) + c2,
 //     c1[n] = sum_k gamma[k] W[n,k],  c2[n] = sum_k beta[k] W[n,k] + b[n]      (made once per weight),
@@ -504,10 +504,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
   bf16_t* mine = turn[wave];
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
   floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-  // a round: U pairs of steps per wave, all its loads issued at once.  Measured and dropped: asking
-  // for the next round before this one is used, into a second set of registers (K = 6400: 10.3 ->
-  // 11.2 us), and sharing a block's 16 columns among 2 or 4 workgroups where blocks are few (1600
-  // columns, K = 6400: 10.3 -> 9.6 and 12.5 us; K = 1600: no gain)
+  // a round: U pairs of steps per wave, all its loads issued at once (asking for the next round
+  // before this one is used, into a second set of registers, was slower)
   auto ask = [&](int p0, bf16x8 (*b)[2], u32x4 (*al)[2]) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -705,19 +703,17 @@ static void launch16(const Call& c, hipStream_t stream) {
 
 // With more than 16 rows every workgroup reads all of A (16 cache lines per load and 16 lanes,
 // as A lies in rows), so wider workgroups read less in total, as long as enough of them remain
-// to keep the memory system busy.  Measured at 64 rows: 2 column blocks where N >= 4096 (20 ->
-// 13 us for K = 1600), 4 for a vocabulary, 1 for N = 1600.
+// to keep the memory system busy: 2 column blocks per workgroup from 4,096 columns on, 4 from
+// 32,768 on, else 1.
 template <int WAVES>
 static void launch_mb(const Call& c, hipStream_t stream) {
   const int mb = (c.M + 15) / 16;
   if (mb == 1 && !(c.packed & (PACKED_A | PACKED_C)) && c.M > 1) return launch16<WAVES>(c, stream);
   if (mb == 1) return launch<1, 1, WAVES, 8>(c, stream);
   if (mb > 4) {
-    // 65 to 256 rows: 16 columns per workgroup, the waves' sums for all row blocks through LDS.
-    // Measured against the tiled kernel (which has too few tiles to fill the chip here, and walks
-    // K = 6400 in a hundred steps whatever M is), the four products of a GPT-2 XL layer with
-    // packed rows: 56 against 158 us at 65 to 96 rows, 67 at 128, 87 at 192, 108 at 256; with
-    // rows in the ordinary layout 80, 127, 181 and 234 us.
+    // 65 to 256 rows: 16 columns per workgroup, the waves' sums for all row blocks through LDS
+    // (the tiled kernel has too few tiles to fill the chip at so few rows, and walks a long K in
+    // as many steps whatever M is)
     if (mb <= 6) return launch<6, 1, WAVES, 2>(c, stream);
     if (mb <= 8) return launch<8, 1, WAVES, 2>(c, stream);
     if (mb <= 12) return launch<12, 1, WAVES, 2>(c, stream);
@@ -1024,11 +1020,10 @@ static int run(const void* A, int lda, const void* W, const float* bias, void* C
                int N, int K, int out_dtype, int epi, const KVScatter* kv, hipStream_t stream) {
   // Where 128 x 128 tiles would be many (two or more per CU), a workgroup of 8 waves takes 256 x 128
   // with slabs of 32 along K: each slab of W serves twice the rows.  Else 4 waves, 128 x 128, slabs
-  // of 64 (half the barriers).  Both measured; see profiles/.
+  // of 64 (half the barriers).
   const long tiles = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
   if (tiles >= 512) return launch_bk<4, 32>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream);
-  // Fewer tiles than CUs: 64 x 128 tiles (each wave 32 x 64) make twice as many workgroups
-  // (2048 x 1600: 54 -> 41 us with K = 1600, 122 -> 105 us with K = 6400).
+  // Fewer tiles than CUs: 64 x 128 tiles (each wave 32 x 64) make twice as many workgroups.
   if (tiles < 256 && M > 64)
     return launch_bk<2, 64, 1>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream);
   return launch_bk<2, 64>(A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epi, kv, stream);
@@ -1057,8 +1052,7 @@ static int run(const void* A, int lda, const void* W, const float* bias, void* C
 // cores at nine tenths of their peak) + 3.07e-5 us x (BM + BN) (loads), the two adding up rather
 // than overlapping, + 1.9e-4 us x BM x BN for the stores at the end.  So the tile is chosen per
 // product from a list, by that model: the largest that still fills the chip in whole rounds
-// (2048 x 4800 x 1600: 256 x 160 tiles are 240 workgroups, one round, 42 us where 256 x 128 tiles
-// took two rounds and 59 us; 2048 x 6400: 256 x 224, 53 against 66 us).
+// (a tile count just above a multiple of 256 costs a whole further round).
 // ---------------------------------------------------------------------------------------
 namespace direct {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
@@ -1356,11 +1350,8 @@ static int pick(int M, int N, int K) {
 }
 
 // Up to 256 rows the few-rows kernel takes the product too (both read and write packed rows).
-// Measured on GPT-2 XL's four products, few rows against many: 1600 -> 4800 with the cache write 13.9
-// / 14.0 us at 128 rows, 20.4 / 14.5 at 160 and 192, 27.8 / 19.7 at 256; 1600 -> 6400 with GELU 13.1 /
-// 12.9, 19.3 / 17.6, 23.5 / 18.0; the two that end in 1,600 columns stay with the few-rows kernel at
-// every size (8.8 / 11.6 and 26.8 / 37.4 us at 192 rows): 64-row tiles of so few columns leave most
-// CUs idle.
+// This one is the faster from 129 rows on where the product has 4,096 columns or more; with fewer
+// columns its 64-row tiles leave most CUs idle and the few-rows kernel stays ahead at every size.
 static bool beats_few_rows(int M, int N, int K) {
   (void)K;
   return M > 128 && N >= 4096;

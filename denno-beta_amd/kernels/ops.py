@@ -37,12 +37,39 @@ def fail_after_launches(n):
     _fail_after = None if n is None else launches + int(n)
 
 
+_timed = None           # time_launches: [(what, start event, end event)]
+_started = None
+
+
+def time_launches(on=True):
+    """Per-kernel timers behind one switch: while on, every launch made through this module stands between
+    two HIP events (steps must then run kernel by kernel, not from captured graphs).  `launch_times()`
+    gives what they measured.  The reference has its profiler behind DENNO_PROF in the same way
+    (crates/denno-engine/src/prof.rs)."""
+    global _timed, _started
+    _timed, _started = ([] if on else None), None
+
+
+def launch_times():
+    """-> {what: (launches, milliseconds in all)} of the launches since time_launches(True); waits for
+    the device."""
+    torch.cuda.synchronize()
+    out = {}
+    for what, a, b in _timed or []:
+        n, ms = out.get(what, (0, 0.0))
+        out[what] = (n + 1, ms + a.elapsed_time(b))
+    return out
+
+
 def _lib(name):
-    global launches, _fail_after
+    global launches, _fail_after, _started
     if _fail_after is not None and launches >= _fail_after:
         _fail_after = None
         raise KernelError(f"injected failure: launch number {launches + 1} was refused")
     launches += 1
+    if _timed is not None:
+        _started = torch.cuda.Event(enable_timing=True)
+        _started.record()
     lib = _libs.get(name)
     if lib is None:
         if not torch.cuda.is_available():
@@ -93,6 +120,12 @@ def _stream():
 
 
 def _ok(rc, what):
+    global _started
+    if _timed is not None and _started is not None:
+        end = torch.cuda.Event(enable_timing=True)
+        end.record()
+        _timed.append((what, _started, end))
+        _started = None
     if rc != 0:
         if rc == -1:
             raise KernelError(f"{what}: unsupported dtype combination")
@@ -303,7 +336,8 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
         _need(tuple(residual.shape) == (M, N) and epi == 0 and out is None, "linear: residual")
         ldr = _rows(residual, "residual")
         _ok(_lib("gemm").dn_gemm(a.data_ptr(), lda, wp, _ptr(bias), 0, 0, residual.data_ptr(), ldr,
-                                 M, N, K, _CODE[a.dtype], F32, 0, packed, _stream()), "linear")
+                                 M, N, K, _CODE[a.dtype], F32, 0, packed, _stream()),
+            "linear" if _timed is None else f"linear {K} -> {N}, added into the stream")
         return residual
     if isinstance(out, PackedMatrix):
         _need((packed & PACKED_W) and M <= PACKED_ROWS_MAX and N % 32 == 0 and out.device == a.device,
@@ -314,7 +348,8 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
         ldc = _rows(out, "out")
     _need(tuple(out.shape) == (M, N), "linear: out shape")
     _ok(_lib("gemm").dn_gemm(a.data_ptr(), lda, wp, _ptr(bias), out.data_ptr(), ldc, 0, 0, M, N, K,
-                             _CODE[a.dtype], _CODE[out.dtype], epi, packed, _stream()), "linear")
+                             _CODE[a.dtype], _CODE[out.dtype], epi, packed, _stream()),
+        "linear" if _timed is None else f"linear {K} -> {N}" + (f", {epilogue}" if epi else ""))
     return out
 
 
@@ -345,7 +380,8 @@ def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
         _ok(_lib("gemm").dn_gemm_qkv(a.data_ptr(), lda, w.data_ptr(), _ptr(bias), out.data_ptr(),
                                      _rows(out, "out"), M, N, K, slot_map.data_ptr(), k_pool.data_ptr(),
                                      v_pool.data_ptr(), q_width, Hkv, dh, ps, int(bool(packed & PACKED_A)),
-                                     out.shape[1], _stream()), "linear_qkv")
+                                     out.shape[1], _stream()),
+            "linear_qkv" if _timed is None else f"linear {K} -> {N}, cache write")
         return out[:, :q_width]
     _need(out.shape[1] == N, "linear_qkv: without the fused kernel out must hold all columns")
     linear(a, w, bias, out=out)
@@ -595,7 +631,8 @@ def linear_norm_out(a, w, bias, residual, gamma, copy, stats):
     _need(gamma is not None, "linear_norm_out: gamma")
     _ok(_lib("gemm").dn_gemm_norm_out(a.data_ptr(), lda, w.data_ptr(), _ptr(bias), residual.data_ptr(),
                                       _rows(residual, "residual"), M, N, K, gamma.data_ptr(), copy.data_ptr(),
-                                      ldcopy, stats.data_ptr(), _stream()), "linear_norm_out")
+                                      ldcopy, stats.data_ptr(), _stream()),
+        "linear_norm_out" if _timed is None else f"linear {K} -> {N}, added into the stream, leaves the next norm's statistics")
     return residual
 
 
@@ -635,5 +672,7 @@ def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None):
         args = (slot_map.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), q_width, Hkv, dh, ps, out.shape[1])
     _ok(_lib("gemm").dn_gemm_norm_in(copy.data_ptr(), lda, stats.data_ptr(), c1.data_ptr(),
                                      c2.data_ptr(), float(eps), w.data_ptr(), out.data_ptr(), ldc,
-                                     M, N, K, EPILOGUES[epilogue], *args, _stream()), "linear_norm_in")
+                                     M, N, K, EPILOGUES[epilogue], *args, _stream()),
+        "linear_norm_in" if _timed is None else
+        f"norm + linear {K} -> {N}" + (", cache write" if kv is not None else "") + (f", {epilogue}" if epilogue != "none" else ""))
     return out if kv is None else out[:, :kv[3]]

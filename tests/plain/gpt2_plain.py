@@ -89,6 +89,21 @@ def causal_attention(q, k, v, n_head, scale, first_position=0, window=None):
     return out
 
 
+def causal_attention_by_head(q, k, v, n_head, scale):
+    """The same result as causal_attention for a whole sequence from position 0, one head at a time
+    as matrices: scores of all pairs, -inf above the diagonal, softmax_rows, times the values.  For
+    sequences too long for the loop above; tests/test_plain.py holds the two against each other."""
+    n, e = q.shape
+    dh = e // n_head
+    out = torch.zeros_like(q)
+    above = torch.ones(n, n, dtype=torch.bool).triu(1)
+    for hd in range(n_head):
+        c = slice(hd * dh, (hd + 1) * dh)
+        s = (q[:, c] @ k[:, c].t()) * scale
+        out[:, c] = softmax_rows(s.masked_fill(above, float("-inf"))) @ v[:, c]
+    return out
+
+
 def attention_scale(head_dim, layer_idx, scale_attn_weights=True, scale_attn_by_inverse_layer_idx=False):
     """1/sqrt(dh) as the reference (model/gpt2.rs:174); config options of the
     architecture switch it off or divide further by (layer_idx + 1)."""
@@ -100,13 +115,13 @@ def attention_scale(head_dim, layer_idx, scale_attn_weights=True, scale_attn_by_
     return s
 
 
-def attention_block(h, p, n_head, scale):
+def attention_block(h, p, n_head, scale, attention=causal_attention):
     """qkv = h W + b, columns q | k | v; attention; output projection
     (model/gpt2.rs:155-208)."""
     e = h.shape[-1]
     qkv = linear_in_out(h, p["attn.c_attn.weight"], p["attn.c_attn.bias"])
     q, k, v = qkv[:, :e], qkv[:, e:2 * e], qkv[:, 2 * e:]
-    a = causal_attention(q, k, v, n_head, scale)
+    a = attention(q, k, v, n_head, scale)
     return linear_in_out(a, p["attn.c_proj.weight"], p["attn.c_proj.bias"])
 
 
@@ -116,9 +131,9 @@ def mlp_block(h, p, act):
     return linear_in_out(f, p["mlp.c_proj.weight"], p["mlp.c_proj.bias"])
 
 
-def block(x, p, n_head, scale, eps, act):
+def block(x, p, n_head, scale, eps, act, attention=causal_attention):
     """x += attn(LN1(x)); x += mlp(LN2(x))                      (model/gpt2.rs:152-220)"""
-    x = x + attention_block(layer_norm(x, p["ln_1.weight"], p["ln_1.bias"], eps), p, n_head, scale)
+    x = x + attention_block(layer_norm(x, p["ln_1.weight"], p["ln_1.bias"], eps), p, n_head, scale, attention)
     x = x + mlp_block(layer_norm(x, p["ln_2.weight"], p["ln_2.bias"], eps), p, act)
     return x
 
@@ -165,15 +180,17 @@ class PlainGPT2:
         pre = f"h.{i}."
         return {k[len(pre):]: v for k, v in self.t.items() if k.startswith(pre)}
 
-    def logits(self, tokens) -> torch.Tensor:
-        """[len(tokens), vocab] logits of one whole sequence starting at position 0."""
+    def logits(self, tokens, by_head=False) -> torch.Tensor:
+        """[len(tokens), vocab] logits of one whole sequence starting at position 0.
+        by_head: attention one head at a time as matrices (long sequences of deep models)."""
         tok = torch.as_tensor(tokens, dtype=torch.long)
         pos = torch.arange(len(tok))
         x = embed(tok, pos, self.t["wte.weight"], self.t["wpe.weight"])
         dh = self.n_embd // self.n_head
         for i in range(self.n_layer):
             scale = attention_scale(dh, i, self.scale_w, self.scale_inv)
-            x = block(x, self.layer_params(i), self.n_head, scale, self.eps, self.act)
+            x = block(x, self.layer_params(i), self.n_head, scale, self.eps, self.act,
+                      causal_attention_by_head if by_head else causal_attention)
         return head(x, self.t["ln_f.weight"], self.t["ln_f.bias"], self.eps, self.t["wte.weight"])
 
     def greedy(self, prompt, n_new):

@@ -92,6 +92,17 @@ def test_attention_is_the_library_routine(n_head, dh):
     assert torch.allclose(got, want.transpose(0, 1).reshape(n, e), atol=1e-5)
 
 
+def test_attention_by_head_is_the_loop(model_folders):
+    """The matrix form that long sequences use gives what the loop over queries gives."""
+    n, n_head, dh = 70, 3, 32
+    q, k, v = rnd(n, n_head * dh, seed=4), rnd(n, n_head * dh, seed=5), rnd(n, n_head * dh, seed=6)
+    assert torch.allclose(P.causal_attention_by_head(q, k, v, n_head, 0.4), P.causal_attention(q, k, v, n_head, 0.4),
+                          atol=2e-6)
+    plain = P.PlainGPT2.from_folder(model_folders("B", "float32"))
+    seq = seeded_tokens(1, 90, 1000)
+    assert torch.allclose(plain.logits(seq, by_head=True), plain.logits(seq), atol=2e-6)
+
+
 def test_attention_first_position_returns_value():
     q, k, v = rnd(1, 32, seed=1), rnd(1, 32, seed=2), rnd(1, 32, seed=3)
     assert torch.equal(P.causal_attention(q, k, v, 2, 1.0), v)

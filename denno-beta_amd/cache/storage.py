@@ -24,7 +24,8 @@ _TORCH = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.i
 class CacheStorage:
     def __init__(self, cache_specs: Sequence, *, kv_dtype: torch.dtype, page_size: int, cache_tokens: int,
                  max_live: int, device, allocate: bool = True):
-        """cache_specs[i]: the need of cache i (PagedKV, FixedState or None)."""
+        """cache_specs[i]: the need of cache i (PagedKV, FixedState or None).  kv_dtype: what pages hold
+        whose PagedKV names no dtype of its own."""
         self.page_size, self.max_live, self.device, self.kv_dtype = page_size, max_live, device, kv_dtype
         self.group_specs: List = []
         self.members: List[List[int]] = []
@@ -56,11 +57,12 @@ class CacheStorage:
             if isinstance(cs, PagedKV):
                 shape = (n, n_pages, cs.n_kv_heads, page_size, cs.head_dim)
                 vshape = (n, n_pages, cs.n_kv_heads, cs.head_dim, page_size)   # a page's values transposed
+                dt = _TORCH[cs.dtype] if cs.dtype is not None else kv_dtype
                 if allocate:
                     # zeros, not empty: a page's unwritten tail is read (masked) by attention,
                     # and must hold numbers, not whatever bits the allocator left
-                    self.k.append(torch.zeros(shape, dtype=kv_dtype, device=device))
-                    self.v.append(torch.zeros(vshape, dtype=kv_dtype, device=device))
+                    self.k.append(torch.zeros(shape, dtype=dt, device=device))
+                    self.v.append(torch.zeros(vshape, dtype=dt, device=device))
                 else:
                     self.k.append(None), self.v.append(None)
                 self.state.append(None)
@@ -101,5 +103,6 @@ class CacheStorage:
         total = 0
         for g, cs in enumerate(self.group_specs):
             if isinstance(cs, PagedKV):
-                total += len(self.members[g]) * 2 * cs.n_kv_heads * cs.head_dim * torch.empty((), dtype=self.kv_dtype).element_size()
+                dt = _TORCH[cs.dtype] if cs.dtype is not None else self.kv_dtype
+                total += len(self.members[g]) * 2 * cs.n_kv_heads * cs.head_dim * torch.empty((), dtype=dt).element_size()
         return total

@@ -1,8 +1,7 @@
 from .base import ConfigError, read_config_json
-from .gpt2 import GPT2Config
 from .options import EngineOptions
 from .registry import (Architecture, known_architectures, load_config, register_architecture,
                        resolve_architecture)
 
-__all__ = ["ConfigError", "read_config_json", "GPT2Config", "EngineOptions", "Architecture",
+__all__ = ["ConfigError", "read_config_json", "EngineOptions", "Architecture",
            "known_architectures", "load_config", "register_architecture", "resolve_architecture"]

@@ -4,13 +4,13 @@
 #include "common.h"
 
 // ---------------------------------------------------------------------------------------
-// x[t,:] = wte[token_t,:] + wpe[pos_t,:]      (crates/denno-engine/src/model/gpt2.rs:142-150)
-// wpe may be null (an architecture whose positions enter elsewhere).
+// x[t,:] = wte[token_t,:] * token_scale + wpe[pos_t,:]   (crates/denno-engine/src/model/gpt2.rs:142-150,
+// where the scale is 1).  wpe may be null (an architecture whose positions enter elsewhere).
 // ---------------------------------------------------------------------------------------
 template <typename TW>
 __global__ void embed_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ positions,
                              const TW* __restrict__ wte, const TW* __restrict__ wpe, float* __restrict__ x,
-                             int T, int E, int vocab, int n_pos) {
+                             int T, int E, int vocab, int n_pos, float token_scale) {
   int t = blockIdx.x;
   if (t >= T) return;
   int tok = tokens[t];
@@ -20,6 +20,7 @@ __global__ void embed_kernel(const int32_t* __restrict__ tokens, const int32_t* 
     float v = __uint_as_float(0x7fc00000u);   // an id outside the table: NaN, never a neighbour's row
     if (ok) {
       v = to_float(wte[static_cast<size_t>(tok) * E + e]);
+      if (token_scale != 1.0f) v *= token_scale;
       if (wpe != nullptr) v += to_float(wpe[static_cast<size_t>(pos) * E + e]);
     }
     x[static_cast<size_t>(t) * E + e] = v;
@@ -27,15 +28,18 @@ __global__ void embed_kernel(const int32_t* __restrict__ tokens, const int32_t* 
 }
 
 extern "C" int dn_embed(const int32_t* tokens, const int32_t* positions, const void* wte, const void* wpe,
-                        float* x, int T, int E, int vocab, int n_pos, int table_dtype, hipStream_t stream) {
+                        float* x, int T, int E, int vocab, int n_pos, int table_dtype, float token_scale,
+                        hipStream_t stream) {
   if (T <= 0) return 0;
   dim3 grid(T), block(256);
   if (table_dtype == DN_F32)
     hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, tokens, positions,
-                       static_cast<const float*>(wte), static_cast<const float*>(wpe), x, T, E, vocab, n_pos);
+                       static_cast<const float*>(wte), static_cast<const float*>(wpe), x, T, E, vocab, n_pos,
+                       token_scale);
   else if (table_dtype == DN_BF16)
     hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, tokens, positions,
-                       static_cast<const bf16_t*>(wte), static_cast<const bf16_t*>(wpe), x, T, E, vocab, n_pos);
+                       static_cast<const bf16_t*>(wte), static_cast<const bf16_t*>(wpe), x, T, E, vocab, n_pos,
+                       token_scale);
   else
     return DN_ERR_DTYPE;
   return dn_launch_status();
@@ -227,5 +231,25 @@ extern "C" int dn_cast(const void* in, void* out, long long n, int in_dtype, int
                        static_cast<bf16_t*>(out), static_cast<size_t>(n));
   else
     return DN_ERR_DTYPE;
+  return dn_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// What a head may do to its logits, in place: l = l * scale, then, if cap > 0, l = cap * tanh(l / cap).
+// ---------------------------------------------------------------------------------------
+__global__ void logits_post_kernel(float* __restrict__ logits, int ld, int V, float scale, float cap) {
+  float* row = logits + static_cast<size_t>(blockIdx.y) * ld;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < V; i += gridDim.x * blockDim.x) {
+    float l = row[i] * scale;
+    if (cap > 0.f) l = cap * tanhf(l / cap);
+    row[i] = l;
+  }
+}
+
+extern "C" int dn_logits_post(float* logits, int ld, int R, int V, float scale, float cap, hipStream_t stream) {
+  if (R <= 0 || V <= 0) return 0;
+  if (ld < V || R > 65535) return DN_ERR_SHAPE;
+  hipLaunchKernelGGL(logits_post_kernel, dim3((V + 1023) / 1024 > 64 ? 64 : (V + 1023) / 1024, R), dim3(256), 0, stream,
+                     logits, ld, V, scale, cap);
   return dn_launch_status();
 }

@@ -85,7 +85,8 @@ def _declare(name, lib):
     P, I, F = c_void_p, c_int, c_float
     sigs = {
         "elementwise": {
-            "dn_embed": [P, P, P, P, P, I, I, I, I, I, P],
+            "dn_embed": [P, P, P, P, P, I, I, I, I, I, F, P],
+            "dn_logits_post": [P, I, I, I, F, F, P],
             "dn_layernorm": [P, P, P, P, P, I, I, F, I, I, P],
             "dn_kv_write": [P, I, I, I, P, P, P, I, I, I, I, I, P],
             "dn_cast": [P, P, c_longlong, I, I, P],
@@ -164,8 +165,8 @@ _FLOATS = (torch.float32, torch.bfloat16)
 _I32 = (torch.int32,)
 
 
-def embed(tokens, positions, wte, wpe, out):
-    """out[t,:] = wte[tokens[t],:] + wpe[positions[t],:]; wpe may be None.  out is 32-bit."""
+def embed(tokens, positions, wte, wpe, out, token_scale=1.0):
+    """out[t,:] = wte[tokens[t],:] * token_scale + wpe[positions[t],:]; wpe may be None.  out is 32-bit."""
     T = tokens.shape[0]
     _dev(tokens, "tokens", _I32, 1), _dev(positions, "positions", _I32, 1)
     _dev(wte, "wte", _FLOATS, 2), _dev(out, "out", (torch.float32,), 2)
@@ -178,9 +179,18 @@ def embed(tokens, positions, wte, wpe, out):
         _need(wpe.is_contiguous() and wpe.shape[1] == E, "embed: wpe shape")
         n_pos = wpe.shape[0]
     _ok(_lib("elementwise").dn_embed(tokens.data_ptr(), positions.data_ptr(), wte.data_ptr(), _ptr(wpe),
-                                     out.data_ptr(), T, E, wte.shape[0], n_pos, _CODE[wte.dtype], _stream()),
-        "embed")
+                                     out.data_ptr(), T, E, wte.shape[0], n_pos, _CODE[wte.dtype], float(token_scale),
+                                     _stream()), "embed")
     return out
+
+
+def logits_post(logits, scale=1.0, softcap=0.0):
+    """In place on 32-bit logits [R, V]: times `scale`, then, if softcap > 0, softcap * tanh(l / softcap)."""
+    _dev(logits, "logits", (torch.float32,), 2)
+    R, V = logits.shape
+    _ok(_lib("elementwise").dn_logits_post(logits.data_ptr(), _rows(logits, "logits"), R, V, float(scale),
+                                           float(softcap), _stream()), "logits_post")
+    return logits
 
 
 class PackedMatrix:

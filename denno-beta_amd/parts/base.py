@@ -11,7 +11,8 @@ Kinds of part and their registries:
   feed-forward     FEED_FORWARDS   forward(h, ctx, accumulate_into)
   norm             NORMS           forward(x, out_dtype, rows=None) -> tensor
   position code    POSITIONS       table() for the embedding stage, rotate(q, k, ctx) for mixers
-  arrangement      ARRANGEMENTS    forward(x, ctx, cache): how norms, mixer and feed-forward stand in a block
+  arrangement      ARRANGEMENTS    SLOTS names its parts and their kinds; forward(x, ctx, caches, runtime): how
+                                   norms, mixers and feed-forwards stand in a block
 
 `h` is [T, width] in the activation dtype; `x` and `accumulate_into` are the 32-bit residual
 stream [T, width], which mixers and feed-forwards add their result to in place (the sum is
@@ -29,10 +30,12 @@ from ..weights.spec import ParamSpec
 
 @dataclass(frozen=True)
 class PagedKV:
-    """A mixer that keeps keys and values of `window` last positions (0: all) in pages."""
+    """A mixer that keeps keys and values of `window` last positions (0: all) in pages.
+    dtype: what the pages hold ("bfloat16", "float32"); None: the engine's activation dtype."""
     n_kv_heads: int
     head_dim: int
     window: int = 0
+    dtype: Optional[str] = None
 
 
 @dataclass(frozen=True)
@@ -46,8 +49,9 @@ class FixedState:
 @dataclass
 class Runtime:
     """What parts need to know about the engine they are bound into.  `position` is the model's
-    position encoding (set by the model before it binds its parts): a mixer asks it to turn its
-    queries and keys if it is of the kind that does (`rotates`)."""
+    position encoding (set by the model before it binds its parts): a mixer that names no position
+    encoding of its own asks this one to turn its queries and keys, if it is of the kind that does
+    (`rotates`)."""
     act_dtype: torch.dtype
     device: torch.device
     position: Optional["Part"] = None
@@ -148,3 +152,5 @@ FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
 POSITIONS = Registry("position encoding")
 ARRANGEMENTS = Registry("block arrangement")
+# the kinds that an arrangement's SLOTS may name
+KINDS = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS}

@@ -1,4 +1,10 @@
-"""Block arrangements: where the norms stand around a mixer and a feed-forward."""
+"""Block arrangements: where the norms stand around mixers and feed-forwards.
+
+An arrangement names its parts itself: SLOTS maps each part's name in the block to its kind ("norm",
+"mixer", "feed_forward").  A layer's description gives a part for every slot; the model builds them
+from the parts' registries and hands them to the arrangement's constructor by those names.  The
+arrangement says which of them keep caches (`mixers()`, in the order in which a LayerCall lists their
+caches) and runs them (`forward(x, ctx, caches, runtime)`, `caches` in that same order)."""
 from __future__ import annotations
 
 from ..kernels import ops
@@ -9,11 +15,16 @@ from .base import ARRANGEMENTS, LazyNorm, StreamStats
 class PreNormBlock:
     """x += mixer(norm1(x)); x += ffn(norm2(x))     (crates/denno-engine/src/model/gpt2.rs:152-220)"""
 
+    SLOTS = {"norm1": "norm", "mixer": "mixer", "norm2": "norm", "ffn": "feed_forward"}
+
     def __init__(self, norm1, mixer, norm2, ffn):
         self.norm1, self.mixer, self.norm2, self.ffn = norm1, mixer, norm2, ffn
 
     def parts(self):
         return [self.norm1, self.mixer, self.norm2, self.ffn]
+
+    def mixers(self):
+        return [self.mixer]
 
     def first_norm(self):
         """The norm that reads the residual stream first in this block."""
@@ -23,7 +34,8 @@ class PreNormBlock:
         self.mixer.prepare_lazy_norm(self.norm1)
         self.ffn.prepare_lazy_norm(self.norm2)
 
-    def forward(self, x, ctx, cache, runtime):
+    def forward(self, x, ctx, caches, runtime):
+        cache = caches[0]
         # A norm is a kernel of its own, or, where the parts on both sides of it can (steps of few
         # rows), it runs inside them: the part before leaves what the norm needs as it adds into the
         # stream, the part after applies it in its own kernel (parts.base.StreamStats, LazyNorm).

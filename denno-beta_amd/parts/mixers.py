@@ -4,7 +4,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import MIXERS, PagedKV, Part
+from .base import MIXERS, POSITIONS, PagedKV, Part
 from .linear import Linear
 
 
@@ -16,12 +16,14 @@ class CausalSelfAttention(Part):
 
     n_kv_heads < n_heads: query head h reads key head h // (n_heads // n_kv_heads).
     window > 0: a query at position p reads keys p - window + 1 .. p only.
-    scale multiplies the scores before the softmax."""
+    scale multiplies the scores before the softmax.
+    position: a position encoding of this layer's own, as (kind name, arguments), of the kind that
+    turns queries and keys; None: the model's."""
     graph_safe = True
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                  qkv_weight: str, qkv_bias, out_weight: str, out_bias, stored_in_out: bool = False,
-                 window: int = 0, out_init_std: float = 0.02):
+                 window: int = 0, out_init_std: float = 0.02, position=None):
         self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
         self.scale, self.window = float(scale), int(window)
         if n_heads % n_kv_heads != 0:
@@ -32,9 +34,13 @@ class CausalSelfAttention(Part):
         self.kv_width = n_kv_heads * head_dim
         self.qkv = Linear(width, self.q_width + 2 * self.kv_width, qkv_weight, qkv_bias, stored_in_out)
         self.out = Linear(self.q_width, width, out_weight, out_bias, stored_in_out, out_init_std)
+        self.position = POSITIONS.make(position) if position is not None else None
+        if self.position is not None:
+            self.graph_safe = getattr(self.position, "graph_safe", False)
 
     def param_specs(self):
-        return self.qkv.param_specs() + self.out.param_specs()
+        own = self.position.param_specs() if self.position is not None else []
+        return self.qkv.param_specs() + self.out.param_specs() + own
 
     def cache_spec(self):
         return PagedKV(self.n_kv_heads, self.head_dim, self.window)
@@ -43,6 +49,8 @@ class CausalSelfAttention(Part):
         super().bind(tensors, runtime)
         self.qkv.bind(tensors)
         self.out.bind(tensors)
+        if self.position is not None:
+            self.position.bind(tensors, runtime)
 
     def packed_input(self, n_rows):
         return self.qkv.packed_input(n_rows)
@@ -59,7 +67,7 @@ class CausalSelfAttention(Part):
     def forward(self, h, ctx, cache, accumulate_into, stats=None):
         act = self.runtime.act_dtype
         g = ctx.groups[cache.group]
-        position = self.runtime.position
+        position = self.position if self.position is not None else self.runtime.position
         if position is not None and getattr(position, "rotates", False):
             # queries and keys are turned by their positions before the keys go to the cache: the
             # product, the turn and the cache write are three steps here, not one kernel

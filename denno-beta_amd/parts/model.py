@@ -1,20 +1,24 @@
 """A decoder described as data, and the model built from the description.
 
-DecoderSpec names, layer by layer, the arrangement and the parts of each layer (a kind name
-and its arguments, looked up in the parts' registries), and the order in which layers run:
-a list of LayerCall, which may name a layer twice (its weights are shared; each call has a
-cache of its own) or let a call read the cache that another call writes.
+DecoderSpec names, layer by layer, the arrangement and the parts of each layer (for every slot
+that the arrangement declares, a kind name and its arguments, looked up in the parts'
+registries), and the order in which layers run: a list of LayerCall, which may name a layer
+twice (its weights are shared; each call has caches of its own) or let a call read the cache
+that another call writes.  What stands around the layers is described too: the token table
+and a multiplier for its rows, the position encoding, the final norm, the head (tied to the token
+table or a matrix of its own, with or without a bias) and what happens to its logits (a scale, a
+soft cap).
 """
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Dict, List, Optional, Sequence, Tuple, Union
 
 import torch
 
 from ..kernels import ops
 from ..weights.spec import ParamSpec
-from .base import ARRANGEMENTS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, FixedState, PagedKV, Runtime
+from .base import ARRANGEMENTS, KINDS, NORMS, POSITIONS, FixedState, PagedKV, Runtime
 from .linear import Linear
 from .positions import TokenEmbedding
 
@@ -23,18 +27,18 @@ PartSpec = Tuple[str, dict]   # (kind name in its registry, constructor argument
 
 @dataclass
 class LayerSpec:
-    arrangement: str
-    norm1: PartSpec
-    mixer: PartSpec
-    norm2: PartSpec
-    ffn: PartSpec
+    arrangement: str              # name in ARRANGEMENTS
+    parts: Dict[str, PartSpec]    # a part for every slot that the arrangement declares (its SLOTS)
 
 
 @dataclass
 class LayerCall:
     layer: int                    # index into DecoderSpec.layers
-    cache: int                    # index of the cache this call uses
+    cache: Union[int, Tuple[int, ...]]   # the cache this call uses; a tuple: one for each mixer of the layer
     writes_cache: bool = True     # False: it only reads what another call wrote
+
+    def caches(self) -> Tuple[int, ...]:
+        return (self.cache,) if isinstance(self.cache, int) else tuple(self.cache)
 
 
 @dataclass
@@ -48,6 +52,10 @@ class DecoderSpec:
     run_order: List[LayerCall]
     final_norm: PartSpec
     head_weight: Optional[str] = None     # None: the head is the token table, transposed
+    head_bias: Optional[str] = None       # a bias added to the logits
+    logit_scale: float = 1.0              # the logits times this
+    logit_softcap: float = 0.0            # > 0: then cap * tanh(logit / cap)
+    embedding_scale: float = 1.0          # the token table's rows times this, before the position table's
     eos_token_ids: Tuple[int, ...] = ()
     # how checkpoints of this architecture name things
     name_prefixes: Tuple[str, ...] = ("",)
@@ -77,13 +85,17 @@ class DecoderModel:
         self.embedding = TokenEmbedding(spec.vocab, spec.width, spec.token_table)
         self.position = POSITIONS.make(spec.position)
         self.blocks = []
-        for ls in spec.layers:
+        for i, ls in enumerate(spec.layers):
             if ls.arrangement not in ARRANGEMENTS:
                 raise KeyError(f"no block arrangement named {ls.arrangement!r}; known: {sorted(ARRANGEMENTS)}")
-            self.blocks.append(ARRANGEMENTS[ls.arrangement](
-                NORMS.make(ls.norm1), MIXERS.make(ls.mixer), NORMS.make(ls.norm2), FEED_FORWARDS.make(ls.ffn)))
+            cls = ARRANGEMENTS[ls.arrangement]
+            if set(ls.parts) != set(cls.SLOTS):
+                raise ValueError(f"layer {i}: arrangement {ls.arrangement!r} has the parts {sorted(cls.SLOTS)}, "
+                                 f"the description gives {sorted(ls.parts)}")
+            self.blocks.append(cls(**{slot: KINDS[kind].make(ls.parts[slot]) for slot, kind in cls.SLOTS.items()}))
         self.final_norm = NORMS.make(spec.final_norm)
-        self.head = None if spec.head_weight is None else Linear(spec.width, spec.vocab, spec.head_weight, None)
+        # the head: a matrix of its own, or the token table, transposed
+        self.head = Linear(spec.width, spec.vocab, spec.head_weight or spec.token_table, spec.head_bias)
         self._check_run_order()
         self.runtime = None
         self.graph_safe = all(getattr(p, "graph_safe", False) for p in self.all_parts())
@@ -93,25 +105,31 @@ class DecoderModel:
         spec = self.spec
         if not spec.run_order:
             raise ValueError("run_order is empty")
-        n_caches = max(c.cache for c in spec.run_order) + 1
-        writer = [None] * n_caches
+        n_caches = max(max(c.caches()) for c in spec.run_order) + 1
+        writer = [None] * n_caches        # cache -> (call, the cache's need) of the call that writes it
         for i, c in enumerate(spec.run_order):
             if not 0 <= c.layer < len(spec.layers):
                 raise ValueError(f"run_order[{i}] names layer {c.layer}; there are {len(spec.layers)}")
-            cs = self.blocks[c.layer].mixer.cache_spec()
-            if c.writes_cache:
-                if writer[c.cache] is not None:
-                    raise ValueError(f"run_order[{i}] writes cache {c.cache}, which run_order[{writer[c.cache]}] writes")
-                writer[c.cache] = i
-            else:
-                if writer[c.cache] is None:
-                    raise ValueError(f"run_order[{i}] reads cache {c.cache} before any call has written it")
-                if self.blocks[spec.run_order[writer[c.cache]].layer].mixer.cache_spec() != cs:
-                    raise ValueError(f"run_order[{i}] reads cache {c.cache}, whose writer keeps another kind of cache")
+            mixers = self.blocks[c.layer].mixers()
+            if len(c.caches()) != len(mixers):
+                raise ValueError(f"run_order[{i}] names {len(c.caches())} caches; layer {c.layer} has {len(mixers)} mixers")
+            for cache, mixer in zip(c.caches(), mixers):
+                cs = mixer.cache_spec()
+                if cache < 0:
+                    raise ValueError(f"run_order[{i}] names cache {cache}")
+                if c.writes_cache:
+                    if writer[cache] is not None:
+                        raise ValueError(f"run_order[{i}] writes cache {cache}, which run_order[{writer[cache][0]}] writes")
+                    writer[cache] = (i, cs)
+                else:
+                    if writer[cache] is None:
+                        raise ValueError(f"run_order[{i}] reads cache {cache} before any call has written it")
+                    if writer[cache][1] != cs:
+                        raise ValueError(f"run_order[{i}] reads cache {cache}, whose writer keeps another kind of cache")
         if any(w is None for w in writer):
             raise ValueError("a cache index is never written")
         self.n_caches = n_caches
-        self.cache_specs = [self.blocks[spec.run_order[w].layer].mixer.cache_spec() for w in writer]
+        self.cache_specs = [w[1] for w in writer]
 
     def all_parts(self):
         parts = [self.embedding, self.position]
@@ -128,8 +146,7 @@ class DecoderModel:
                     raise ValueError(f"two parts claim the tensor {s.name!r}")
                 seen.add(s.name)
                 specs.append(s)
-        if self.head is not None:
-            specs += self.head.param_specs()
+        specs += [s for s in self.head.param_specs() if s.name not in seen]     # (a tied head's weight is the table's)
         return specs
 
     # -- binding -------------------------------------------------------------------------
@@ -138,11 +155,7 @@ class DecoderModel:
         runtime.position = self.position          # mixers ask it to turn their queries and keys, if it does that
         for p in self.all_parts():
             p.bind(tensors, runtime)
-        if self.head is not None:
-            self.head.bind(tensors)
-        else:
-            self.head = Linear(self.spec.width, self.spec.vocab, self.spec.token_table, None)
-            self.head.bind(tensors)
+        self.head.bind(tensors)
         for b in self.blocks:
             after = getattr(b, "after_bind", None)     # an arrangement may make its parts ready for each other
             if after is not None:
@@ -174,15 +187,19 @@ class DecoderModel:
         -> 32-bit logits [R, vocab] at ctx.logit_rows."""
         rt = self.runtime
         x = torch.empty((ctx.T, self.spec.width), dtype=torch.float32, device=rt.device)
-        ops.embed(ctx.tokens, ctx.positions, self.embedding.weight, self.position.table(), x)
+        ops.embed(ctx.tokens, ctx.positions, self.embedding.weight, self.position.table(), x,
+                  token_scale=self.spec.embedding_scale)
         rt.stream_stats = None      # nobody has left anything for a norm of these rows yet
         order = self.spec.run_order
         for i, call in enumerate(order):
             nxt = self.blocks[order[i + 1].layer] if i + 1 < len(order) else None
             rt.next_norm = nxt.first_norm() if nxt is not None and hasattr(nxt, "first_norm") else None
-            self.blocks[call.layer].forward(x, ctx, cache.view(call.cache, call.writes_cache), rt)
+            self.blocks[call.layer].forward(x, ctx, [cache.view(c, call.writes_cache) for c in call.caches()], rt)
         rt.stream_stats = rt.next_norm = None
         if ctx.R == 0:
             return torch.empty((0, self.spec.vocab), dtype=torch.float32, device=rt.device)
         h = self.final_norm.forward(x, rt.act_dtype, rows=ctx.logit_rows, packed=self.head.packed_input(ctx.R))
-        return self.head(h, out_dtype=torch.float32)
+        logits = self.head(h, out_dtype=torch.float32)
+        if self.spec.logit_scale != 1.0 or self.spec.logit_softcap > 0:
+            ops.logits_post(logits, self.spec.logit_scale, self.spec.logit_softcap)
+        return logits

@@ -13,12 +13,21 @@ import math
 import torch
 
 
-def embed(tokens, positions, wte, wpe, out):
+def embed(tokens, positions, wte, wpe, out, token_scale=1.0):
     x = wte[tokens.long()].float()
+    if token_scale != 1.0:
+        x = x * torch.tensor(token_scale, dtype=torch.float32)
     if wpe is not None:
         x = x + wpe[positions.long()].float()
     out.copy_(x)
     return out
+
+
+def logits_post(logits, scale=1.0, softcap=0.0):
+    logits.mul_(torch.tensor(scale, dtype=torch.float32))
+    if softcap > 0:
+        logits.copy_(softcap * torch.tanh(logits / softcap))
+    return logits
 
 
 def layernorm(x, gamma, beta, eps, out, rows=None):

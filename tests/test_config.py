@@ -3,8 +3,9 @@ import json
 import pytest
 
 from conftest import TINY_A, TINY_B
-from denno_beta_amd.config import (ConfigError, EngineOptions, GPT2Config, known_architectures, load_config,
+from denno_beta_amd.config import (ConfigError, EngineOptions, known_architectures, load_config,
                                    resolve_architecture)
+from denno_beta_amd.models.gpt2 import GPT2Config
 
 
 def test_reads_every_key():
@@ -60,8 +61,8 @@ def test_load_config_from_folder(tmp_path):
     spec = arch.build(cfg)
     assert len(spec.layers) == 3 and spec.vocab == 1000 and spec.max_positions == 256
     # every size of the spec comes from the config
-    assert spec.layers[2].mixer[1]["scale"] == pytest.approx(1 / (48 ** 0.5) / 3)
-    assert spec.layers[0].ffn[1]["inner"] == 320 and spec.layers[0].norm1[1]["eps"] == 1e-6
+    assert spec.layers[2].parts["mixer"][1]["scale"] == pytest.approx(1 / (48 ** 0.5) / 3)
+    assert spec.layers[0].parts["ffn"][1]["inner"] == 320 and spec.layers[0].parts["norm1"][1]["eps"] == 1e-6
     with pytest.raises(ConfigError, match="config.json"):
         load_config(str(tmp_path / "nowhere"))
 

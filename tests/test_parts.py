@@ -19,8 +19,7 @@ def options(device, dtype="float32", **kw):
 
 
 def gpt2_spec(name, **changes):
-    from denno_beta_amd.config import GPT2Config
-    from denno_beta_amd.models.gpt2 import build_gpt2
+    from denno_beta_amd.models.gpt2 import GPT2Config, build_gpt2
     cfg = dict(TINY[name][0])
     cfg.update(changes)
     return cfg, build_gpt2(GPT2Config.from_dict(cfg))
@@ -133,6 +132,18 @@ def test_attention_mixer_part(backend, heads, kv_heads, dh, window):
     assert torch.allclose(got.cpu(), want, atol=2e-5)
 
 
+def test_a_cache_group_holds_the_dtype_that_its_mixers_ask_for():
+    """Pages hold the engine's activation dtype unless the mixer's PagedKV names one; caches that differ
+    in it are groups of their own."""
+    from denno_beta_amd.cache import CacheStorage
+    from denno_beta_amd.parts import PagedKV
+    c = CacheStorage([PagedKV(2, 16), PagedKV(2, 16, dtype="float32"), PagedKV(2, 16)], kv_dtype=torch.bfloat16,
+                     page_size=16, cache_tokens=64, max_live=2, device=torch.device("cpu"))
+    assert c.n_groups == 2 and c.k[0].dtype == torch.bfloat16 and c.k[1].dtype == torch.float32
+    assert c.k[0].shape[0] == 2 and c.v[1].shape == (1, 4, 2, 16, 16)
+    assert c.bytes_per_token() == 2 * 2 * 2 * 16 * 2 + 2 * 2 * 16 * 4
+
+
 # -- the order in which layers run is data -----------------------------------------------------
 def test_a_layer_named_twice(backend):
     from denno_beta_amd.engine import ModelRunner
@@ -205,11 +216,11 @@ def toy_model(device, mixers):
         mixer = ("toy_decay", dict(width=E, decay=0.5 + 0.1 * i, weight_name=p + "mix.w")) if kind == "toy_decay" else \
             ("causal_attention", dict(width=E, n_heads=2, n_kv_heads=2, head_dim=16, scale=0.25, qkv_weight=p + "qkv.w",
                                       qkv_bias=None, out_weight=p + "o.w", out_bias=None))
-        layers.append(LayerSpec(
-            "pre_norm", ("layernorm", dict(width=E, eps=1e-5, weight_name=p + "n1.g", bias_name=None)), mixer,
-            ("layernorm", dict(width=E, eps=1e-5, weight_name=p + "n2.g", bias_name=None)),
-            ("dense_mlp", dict(width=E, inner=64, activation="gelu_tanh", up_weight=p + "up.w", up_bias=None,
-                               down_weight=p + "down.w", down_bias=None))))
+        layers.append(LayerSpec("pre_norm", dict(
+            norm1=("layernorm", dict(width=E, eps=1e-5, weight_name=p + "n1.g", bias_name=None)), mixer=mixer,
+            norm2=("layernorm", dict(width=E, eps=1e-5, weight_name=p + "n2.g", bias_name=None)),
+            ffn=("dense_mlp", dict(width=E, inner=64, activation="gelu_tanh", up_weight=p + "up.w", up_bias=None,
+                                   down_weight=p + "down.w", down_bias=None)))))
     return DecoderSpec(vocab=50, width=E, max_positions=128, token_table="tok", position=("none", {}), layers=layers,
                        run_order=[LayerCall(i, i) for i in range(len(layers))],
                        final_norm=("layernorm", dict(width=E, eps=1e-5, weight_name="nf.g", bias_name=None)))
@@ -254,10 +265,10 @@ def toy_plain(spec, st, seq):
     for i, ls in enumerate(spec.layers):
         p = f"L{i}."
         h = P.layer_norm(x, st[p + "n1.g"], 0.0, 1e-5)
-        if ls.mixer[0] == "toy_decay":
+        if ls.parts["mixer"][0] == "toy_decay":
             s, out = torch.zeros(x.shape[1]), []
             for t in range(len(seq)):
-                s = ls.mixer[1]["decay"] * s + h[t]
+                s = ls.parts["mixer"][1]["decay"] * s + h[t]
                 out.append(s @ st[p + "mix.w"].t())
             x = x + torch.stack(out)
         else:
@@ -358,23 +369,25 @@ def turn_pairs(t, positions, head_dim, base):
     t.copy_(torch.stack([a * c - b * s, a * s + b * c], dim=-1).reshape(T, W).to(t.dtype))
 
 
+ROTATION_BASES = (50.0, 50.0, 7.0)     # the third layer turns by a base of its own, the others by the model's
+
+
 def rotation_model():
+    """Three layers; the model's position encoding turns queries and keys by a base of 50, the third
+    layer names one of its own with a base of 7."""
     from denno_beta_amd.parts import DecoderSpec, LayerCall, LayerSpec
     E = 32
     layers = []
-    for i, (heads, kv_heads) in enumerate(((2, 2), (4, 2))):
+    for i, (heads, kv_heads) in enumerate(((2, 2), (4, 2), (2, 1))):
         p = f"L{i}."
-        dh = E // heads
-        layers.append(LayerSpec(
-            "pre_norm", ("layernorm", dict(width=E, eps=1e-5, weight_name=p + "n1.g", bias_name=None)),
-            ("causal_attention", dict(width=E, n_heads=heads, n_kv_heads=kv_heads, head_dim=16, scale=0.25,
-                                      qkv_weight=p + "qkv.w", qkv_bias=None, out_weight=p + "o.w", out_bias=None))
-            if heads == 2 else
-            ("causal_attention", dict(width=E, n_heads=heads, n_kv_heads=kv_heads, head_dim=16, scale=0.25,
-                                      qkv_weight=p + "qkv.w", qkv_bias=None, out_weight=p + "o.w", out_bias=None)),
-            ("layernorm", dict(width=E, eps=1e-5, weight_name=p + "n2.g", bias_name=None)),
-            ("toy_experts", dict(width=E, inner=48, n_experts=3, prefix=p + "ffn."))))
-        assert dh in (16, 8)
+        own = dict(position=("toy_rotation", dict(head_dim=16, base=ROTATION_BASES[i]))) if i == 2 else {}
+        layers.append(LayerSpec("pre_norm", dict(
+            norm1=("layernorm", dict(width=E, eps=1e-5, weight_name=p + "n1.g", bias_name=None)),
+            mixer=("causal_attention", dict(width=E, n_heads=heads, n_kv_heads=kv_heads, head_dim=16, scale=0.25,
+                                            qkv_weight=p + "qkv.w", qkv_bias=None, out_weight=p + "o.w", out_bias=None,
+                                            **own)),
+            norm2=("layernorm", dict(width=E, eps=1e-5, weight_name=p + "n2.g", bias_name=None)),
+            ffn=("toy_experts", dict(width=E, inner=48, n_experts=3, prefix=p + "ffn.")))))
     return DecoderSpec(vocab=50, width=E, max_positions=128, token_table="tok",
                        position=("toy_rotation", dict(head_dim=16, base=50.0)), layers=layers,
                        run_order=[LayerCall(i, i) for i in range(len(layers))],
@@ -389,18 +402,18 @@ def rotation_plain(spec, st, seq, positions=None):
     x = st["tok"][torch.tensor(seq)]
     for i, ls in enumerate(spec.layers):
         p = f"L{i}."
-        a = ls.mixer[1]
+        a = ls.parts["mixer"][1]
         H, Hkv, dh = a["n_heads"], a["n_kv_heads"], a["head_dim"]
         h = P.layer_norm(x, st[p + "n1.g"], 0.0, 1e-5)
         qkv = h @ st[p + "qkv.w"].t()
         q, k, v = qkv[:, :H * dh].clone(), qkv[:, H * dh:(H + Hkv) * dh].clone(), qkv[:, (H + Hkv) * dh:]
-        turn_pairs(q, pos, dh, 50.0)
-        turn_pairs(k, pos, dh, 50.0)
+        turn_pairs(q, pos, dh, ROTATION_BASES[i])
+        turn_pairs(k, pos, dh, ROTATION_BASES[i])
         # query head hd reads key head hd // (H / Hkv): spread keys and values out to H heads
         spread = lambda t: t.reshape(T, Hkv, 1, dh).expand(T, Hkv, H // Hkv, dh).reshape(T, H * dh)   # noqa: E731
         x = x + P.causal_attention(q, spread(k), spread(v), H, a["scale"]) @ st[p + "o.w"].t()
         h = P.layer_norm(x, st[p + "n2.g"], 0.0, 1e-5)
-        f = ls.ffn[1]
+        f = ls.parts["ffn"][1]
         choice = first_max(h @ st[f["prefix"] + "router"].t())
         out = torch.zeros_like(x)
         for t in range(T):
@@ -438,6 +451,112 @@ def test_toy_rotation_and_toy_experts_are_registered_built_and_stepped(backend):
     assert torch.allclose(shifted, want[0], atol=2e-4)
     still = rotation_plain(spec, st, seqs[0], positions=torch.zeros(len(seqs[0])))
     assert (still - want[0]).abs().max() > 0.05
+    # the third layer's own base acts: with the model's base there too the logits differ
+    global ROTATION_BASES
+    kept, ROTATION_BASES = ROTATION_BASES, (50.0, 50.0, 50.0)
+    try:
+        assert (rotation_plain(spec, st, seqs[0]) - want[0]).abs().max() > 0.05
+    finally:
+        ROTATION_BASES = kept
+
+
+# -- an arrangement with four norms, a head with a bias and a scale -------------------------------
+def register_sandwich_arrangement():
+    from denno_beta_amd.parts import ARRANGEMENTS
+    if "toy_sandwich" in ARRANGEMENTS:
+        return
+
+    @ARRANGEMENTS.register("toy_sandwich")
+    class SandwichBlock:
+        """x += post1(mixer(pre1(x))); x += post2(ffn(pre2(x))): a norm before and a norm after each part, so
+        the parts' results pass through a norm before they are added.  The parts add into a stream of zeros
+        that stands in for the residual stream."""
+        SLOTS = {"pre1": "norm", "mixer": "mixer", "post1": "norm", "pre2": "norm", "ffn": "feed_forward",
+                 "post2": "norm"}
+
+        def __init__(self, pre1, mixer, post1, pre2, ffn, post2):
+            self.pre1, self.mixer, self.post1, self.pre2, self.ffn, self.post2 = pre1, mixer, post1, pre2, ffn, post2
+
+        def parts(self):
+            return [self.pre1, self.mixer, self.post1, self.pre2, self.ffn, self.post2]
+
+        def mixers(self):
+            return [self.mixer]
+
+        def forward(self, x, ctx, caches, runtime):
+            runtime.stream_stats = None            # nothing is left for a norm of these rows
+            out = torch.zeros_like(x)
+            self.mixer.forward(self.pre1.forward(x, runtime.act_dtype), ctx, caches[0], accumulate_into=out)
+            x += self.post1.forward(out, torch.float32)
+            out.zero_()
+            self.ffn.forward(self.pre2.forward(x, runtime.act_dtype), ctx, accumulate_into=out)
+            x += self.post2.forward(out, torch.float32)
+
+
+def sandwich_model():
+    from denno_beta_amd.parts import DecoderSpec, LayerCall, LayerSpec
+    E = 32
+    norm = lambda name, eps: ("layernorm", dict(width=E, eps=eps, weight_name=name + ".g", bias_name=name + ".b"))   # noqa: E731
+    layers = []
+    for i in range(2):
+        p = f"L{i}."
+        layers.append(LayerSpec("toy_sandwich", dict(
+            pre1=norm(p + "pre1", 1e-5), post1=norm(p + "post1", 1e-3), pre2=norm(p + "pre2", 1e-5),
+            post2=norm(p + "post2", 1e-2),
+            mixer=("causal_attention", dict(width=E, n_heads=2, n_kv_heads=2, head_dim=16, scale=0.25,
+                                            qkv_weight=p + "qkv.w", qkv_bias=None, out_weight=p + "o.w", out_bias=None)),
+            ffn=("dense_mlp", dict(width=E, inner=64, activation="gelu_tanh", up_weight=p + "up.w", up_bias=None,
+                                   down_weight=p + "down.w", down_bias=None)))))
+    return DecoderSpec(vocab=50, width=E, max_positions=128, token_table="tok",
+                       position=("learned_absolute", dict(n_positions=128, width=E, name="pos")), layers=layers,
+                       run_order=[LayerCall(i, i) for i in range(2)], final_norm=norm("nf", 1e-5),
+                       head_weight="head.w", head_bias="head.b", logit_scale=0.5, logit_softcap=3.0,
+                       embedding_scale=E ** 0.5)
+
+
+def sandwich_plain(st, seq):
+    E = 32
+    ln = lambda x, name, eps: P.layer_norm(x, st[name + ".g"], st[name + ".b"], eps)   # noqa: E731
+    x = st["tok"][torch.tensor(seq)] * E ** 0.5 + st["pos"][:len(seq)]
+    for i in range(2):
+        p = f"L{i}."
+        qkv = ln(x, p + "pre1", 1e-5) @ st[p + "qkv.w"].t()
+        a = P.causal_attention(qkv[:, :E], qkv[:, E:2 * E], qkv[:, 2 * E:], 2, 0.25) @ st[p + "o.w"].t()
+        x = x + ln(a, p + "post1", 1e-3)
+        f = P.gelu_tanh(ln(x, p + "pre2", 1e-5) @ st[p + "up.w"].t()) @ st[p + "down.w"].t()
+        x = x + ln(f, p + "post2", 1e-2)
+    logits = (ln(x, "nf", 1e-5) @ st["head.w"].t() + st["head.b"]) * 0.5
+    return 3.0 * torch.tanh(logits / 3.0)
+
+
+def test_a_four_norm_arrangement_and_a_head_with_bias_scale_and_cap(backend):
+    """An arrangement with other parts than the framework's own (four norms around a mixer and a
+    feed-forward) is registered here and described by name; the head is a matrix of its own with a
+    bias, its logits are scaled and capped, the token rows are multiplied.  The framework's files do not
+    change."""
+    from denno_beta_amd.engine import ModelRunner
+    from denno_beta_amd.parts import LayerSpec
+    register_sandwich_arrangement()
+    spec = sandwich_model()
+    names = {s.name for s in spec.param_specs()}
+    assert {"head.w", "head.b", "L1.post2.g", "L0.pre1.b"} <= names
+    tensors = draw(spec, backend)
+    tensors["head.w"] *= 40.0          # logits large enough for the cap to bend them
+    r = ModelRunner(spec, tensors, options(backend, cache_tokens=192))
+    st = {k: v.float().cpu() for k, v in tensors.items()}
+    seqs = [seeded_tokens(i, n, 50) for i, n in enumerate((30, 11, 47, 25))]
+    want = [sandwich_plain(st, s) for s in seqs]
+    assert max(w.abs().max().item() for w in want) > 2.0
+    for kind, steps in (("whole", U.whole_trace(seqs)), ("tail", U.tail_decode_trace(seqs, 8)),
+                        ("mixed", U.mixed_trace(seqs, seed=3))):
+        got = U.replay(r, steps)
+        for i in range(len(seqs)):
+            U.assert_close(got[f"r{i}"], want[i], "float32", f"four norms, {kind}, request {i}")
+    # a description that does not give the arrangement's parts is refused with their names
+    bad = sandwich_model()
+    bad.layers[0] = LayerSpec("toy_sandwich", {k: v for k, v in bad.layers[0].parts.items() if k != "post2"})
+    with pytest.raises(ValueError, match="post2"):
+        bad.instantiate()
 
 
 @pytest.mark.gpu

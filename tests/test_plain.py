@@ -193,6 +193,33 @@ def test_tiny_b_uses_its_options():
         assert not torch.allclose(m2.logits(toks), base, atol=1e-7), key
 
 
+def test_score_scale_options_are_a_scaling_of_the_queries():
+    """The two score options are not in the reference (it fixes 1/sqrt(head), gpt2.rs:174); their meaning
+    here is the architecture's config keys': scores divided by (layer index + 1), counted from 0, and no
+    1/sqrt(head) at all.  Parity unpinned by any vector of the reference; what pins the plain model is the
+    invariant that both are a scaling of a layer's query columns: a model with an option set equals the
+    model without it whose query weights and biases of layer l are multiplied by that layer's factor
+    (a wrong layer count, a factor applied twice or to the keys as well, would fail this)."""
+    cfg, m = tiny("B")
+    E, dh = cfg["n_embd"], cfg["n_embd"] // cfg["n_head"]
+    toks = seeded_tokens(6, 14, cfg["vocab_size"])
+    for option, factor in (("scale_attn_by_inverse_layer_idx", lambda l: 1.0 / (l + 1)),
+                           ("scale_attn_weights", lambda l: math.sqrt(dh))):
+        on = dict(cfg, scale_attn_by_inverse_layer_idx=False, scale_attn_weights=True)
+        on[option] = option == "scale_attn_by_inverse_layer_idx"
+        off = dict(cfg, scale_attn_by_inverse_layer_idx=False, scale_attn_weights=True)
+        scaled = dict(m.t)
+        for l in range(cfg["n_layer"]):
+            w, b = scaled[f"h.{l}.attn.c_attn.weight"].clone(), scaled[f"h.{l}.attn.c_attn.bias"].clone()
+            w[:, :E] *= factor(l)
+            b[:E] *= factor(l)
+            scaled[f"h.{l}.attn.c_attn.weight"], scaled[f"h.{l}.attn.c_attn.bias"] = w, b
+        want = P.PlainGPT2(off, scaled).logits(toks)
+        got = P.PlainGPT2(on, m.t).logits(toks)
+        assert torch.allclose(got, want, atol=2e-6), option
+        assert not torch.allclose(got, P.PlainGPT2(off, m.t).logits(toks), atol=1e-5), option
+
+
 def test_float64_agrees_with_float32():
     cfg, m32 = tiny("B")
     _, m64 = tiny("B", torch.float64)

@@ -22,6 +22,14 @@ int dn_attention(const void* q, int ldq, void* out, int ldo, const void* k_pool,
                  const int32_t* tile_nrows, const int32_t* tile_pos0, int n_tiles, int H, int Hkv, int dh,
                  int page_size, float scale, int window, int dtype, hipStream_t stream);
 
+// the same kernels' arithmetic for a step of single rows (tile s = request s = row s), every tile of keys a
+// workgroup of its own; part: n_tiles * H * ceil(max_context / dn_attention_rows_tile(dh)) * (dh + 2) floats
+int dn_attention_rows_tile(int dh);
+int dn_attention_rows(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
+                      const int32_t* block_tables, int max_blocks, const int32_t* tile_seq, const int32_t* tile_pos0,
+                      int n_tiles, float* part, int max_context, int H, int Hkv, int dh, int page_size, float scale,
+                      int window, int dtype, hipStream_t stream);
+
 // bfloat16, matrix cores: tiles of up to 128 rows
 int dn_attention_flash(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
                        const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,

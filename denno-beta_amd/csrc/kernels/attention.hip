@@ -21,6 +21,166 @@ namespace plain {
 constexpr int BQ = 16;
 constexpr int THREADS = 256;
 
+// One order of summation for every row, whichever kernel runs it and however its step was cut.  Keys
+// go in tiles of BK that start at absolute multiples of BK.  A tile alone gives, for a row, its largest
+// score m_T, the sum l_T of exp(score - m_T) and the values weighted with those, a_T; tiles are joined
+// in ascending order: the first as it is, a later one by
+//     m' = max(m, m_T),  l' = l exp(m - m') + l_T exp(m_T - m'),  a' = a exp(m - m') + a_T exp(m_T - m').
+// Inside a tile 16 threads share a row: thread g has the keys g, g + 16, ... (each score summed over
+// the dims in ascending order) and the dims g, g + 16, ... (each summed over the tile's keys in
+// ascending order); the 16 partial sums of l_T meet in the order of group_reduce<16>.
+
+// q . k over the dims in ascending order, one fused multiply-add a dim (16 dims' operands are read at a
+// time, so that the reads do not wait for one another; the sums keep their order)
+__device__ __forceinline__ float key_dot(const float* qr, const float* kr, int dh) {
+  float dot = 0.f;
+  for (int d0 = 0; d0 < dh; d0 += 16) {
+    float a[16], b[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a[i] = qr[d0 + i], b[i] = kr[d0 + i];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dot = fmaf(a[i], b[i], dot);
+  }
+  return dot;
+}
+
+// sum over the tile's keys, in ascending order, of p[j] times one dim of the values (vs: that dim of key 0)
+__device__ __forceinline__ float dim_sum(const float* ps, const float* vs, int dh, int BK) {
+  float a = 0.f;
+  for (int j0 = 0; j0 < BK; j0 += 16) {
+    float p[16], v[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) p[i] = ps[j0 + i], v[i] = vs[(j0 + i) * (dh + 1)];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a = fmaf(p[i], v[i], a);
+  }
+  return a;
+}
+
+// the scores of one row against the tile in Ks: p[j] to Ps (this row's BK entries), -> m_T, l_T
+__device__ __forceinline__ void tile_scores(const float* qr, const float* Ks, float* ps, int g, int nc, int dh, int kt,
+                                            int lo, int pos, bool row_ok, float scale, float& m_t, float& l_t) {
+  const float NEG_INF = -INFINITY;
+  float s[4];
+  float tmax = NEG_INF;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    s[c] = NEG_INF;
+    if (c < nc) {
+      const int j = g + 16 * c;
+      const int key = kt + j;
+      const float dot = key_dot(qr, Ks + j * (dh + 1), dh);
+      const bool ok = row_ok && key >= lo && key <= pos;
+      s[c] = ok ? dot * scale : NEG_INF;
+      tmax = fmaxf(tmax, s[c]);
+    }
+  }
+  tmax = group_reduce<16>(tmax, MaxOp());
+  float psum = 0.f;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    if (c < nc) {
+      const float p = s[c] > NEG_INF ? expf(s[c] - tmax) : 0.f;     // (a tile without a key: zeros)
+      ps[g + 16 * c] = p;
+      psum += p;
+    }
+  }
+  m_t = tmax;
+  l_t = group_reduce<16>(psum, SumOp());
+}
+
+// a_T[i] for the dims g + 16 i, from the row's p in ps and the tile's values in Vs
+__device__ __forceinline__ void tile_values(const float* ps, const float* Vs, int g, int nd, int dh, int BK,
+                                            float* a_t) {
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    a_t[i] = 0.f;
+    if (i < nd) {
+      a_t[i] = dim_sum(ps, Vs + g + 16 * i, dh, BK);
+    }
+  }
+}
+
+// joins a tile (m_t > -inf) to what the tiles before it gave
+__device__ __forceinline__ void join_tile(float& m, float& l, float* acc, float m_t, float l_t, const float* a_t,
+                                          int nd) {
+  if (!(m > -INFINITY)) {
+    m = m_t;
+    l = l_t;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (i < nd) acc[i] = a_t[i];
+    return;
+  }
+  const float m_new = fmaxf(m, m_t);
+  const float alpha = expf(m - m_new), beta = expf(m_t - m_new);
+  l = fmaf(l_t, beta, l * alpha);
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+    if (i < nd) acc[i] = fmaf(a_t[i], beta, acc[i] * alpha);
+  m = m_new;
+}
+
+// the tile of BK keys from kt of one request and key head into LDS (keys beyond last_pos and pages
+// given back: zeros).  Where each key's dims and each key's values start in the pools is worked out
+// first (Kb, Vb: BK entries each, -1 without a page), so that the loads of the keys and values
+// themselves wait for nothing, go out many at a time and need no division (BK is a power of two;
+// a thread's place in a key's dims moves on by carrying).  Every thread of the workgroup calls it; it
+// ends with a barrier.
+template <typename T>
+__device__ __forceinline__ void load_tile(float* Ks, float* Vs, long long* Kb, long long* Vb, const T* k_pool,
+                                          const T* v_pool, const int32_t* bt, int kt, int last_pos, int BK, int dh,
+                                          int page_size, int Hkv, int hk) {
+  for (int j = threadIdx.x; j < BK; j += THREADS) {
+    const int key = kt + j;
+    const int page = key <= last_pos ? bt[key / page_size] : -1;
+    const int off = key % page_size;
+    const long long head = static_cast<long long>(max(page, 0)) * Hkv + hk;
+    Kb[j] = page >= 0 ? (head * page_size + off) * dh : -1;
+    Vb[j] = page >= 0 ? head * dh * page_size + off : -1;
+  }
+  __syncthreads();
+  // BK * dh is at most 4,096 (tile_keys): 16 elements of the keys and 16 of the values per thread, all asked
+  // for before the first is put into LDS
+  constexpr int PER = 4096 / THREADS;
+  const int n = BK * dh;
+  float kv[PER], vv[PER];
+  const int shift = 31 - __clz(BK);
+  {
+    int j = threadIdx.x / dh, d = threadIdx.x % dh;      // keys: consecutive threads along a key's dims
+    const int dj = THREADS / dh, dd = THREADS % dh;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int e = threadIdx.x + i * THREADS;
+      kv[i] = vv[i] = 0.f;
+      if (e < n) {
+        const long long at = Kb[j];
+        if (at >= 0) kv[i] = to_float(k_pool[at + d]);
+        // values: consecutive threads along the keys of a dim (a page holds a dim's values side by side)
+        const long long av = Vb[e & (BK - 1)];
+        if (av >= 0) vv[i] = to_float(v_pool[av + static_cast<long long>(e >> shift) * page_size]);
+      }
+      j += dj, d += dd;
+      if (d >= dh) d -= dh, j += 1;
+    }
+  }
+  {
+    int j = threadIdx.x / dh, d = threadIdx.x % dh;
+    const int dj = THREADS / dh, dd = THREADS % dh;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int e = threadIdx.x + i * THREADS;
+      if (e < n) {
+        Ks[j * (dh + 1) + d] = kv[i];
+        Vs[(e & (BK - 1)) * (dh + 1) + (e >> shift)] = vv[i];
+      }
+      j += dj, d += dd;
+      if (d >= dh) d -= dh, j += 1;
+    }
+  }
+  __syncthreads();
+}
+
 template <typename T>
 __global__ __launch_bounds__(THREADS) void attention_kernel(
     const T* __restrict__ q, int ldq, T* __restrict__ out, int ldo, const T* __restrict__ k_pool,
@@ -31,8 +191,10 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
   extern __shared__ float smem[];
   float* Qs = smem;                    // [BQ][dh]
   float* Ks = Qs + BQ * dh;            // [BK][dh + 1]
-  float* Vs = Ks + BK * (dh + 1);      // [BK][dh]
-  float* Ps = Vs + BK * dh;            // [BQ][BK]
+  float* Vs = Ks + BK * (dh + 1);      // [BK][dh + 1]
+  float* Ps = Vs + BK * (dh + 1);      // [BQ][BK]
+  long long* Kb = reinterpret_cast<long long*>(Ps + BQ * BK);   // [BK], [BK]
+  long long* Vb = Kb + BK;
 
   const int tile = blockIdx.x, h = blockIdx.y;
   const int seq = tile_seq[tile];
@@ -61,74 +223,13 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
 
   for (int kt = (first_lo / BK) * BK; kt <= last_pos; kt += BK) {
     __syncthreads();
-    for (int e = t; e < BK * dh; e += THREADS) {
-      int j = e / dh, d = e % dh;
-      int key = kt + j;
-      float kv = 0.f, vv = 0.f;
-      if (key <= last_pos) {
-        int page = bt[key / page_size];
-        if (page >= 0) {
-          size_t base = (static_cast<size_t>(page) * Hkv + hk) * page_size * dh;
-          int off = key % page_size;
-          kv = to_float(k_pool[base + static_cast<size_t>(off) * dh + d]);
-          vv = to_float(v_pool[base + static_cast<size_t>(d) * page_size + off]);
-        }
-      }
-      Ks[j * (dh + 1) + d] = kv;
-      Vs[j * dh + d] = vv;
-    }
+    load_tile(Ks, Vs, Kb, Vb, k_pool, v_pool, bt, kt, last_pos, BK, dh, page_size, Hkv, hk);
+    float m_t, l_t, a_t[16];
+    tile_scores(Qs + qi * dh, Ks, Ps + qi * BK, g, nc, dh, kt, my_lo, my_pos, row_ok, scale, m_t, l_t);
     __syncthreads();
-
-    float s[4];
-    float tmax = NEG_INF;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      s[c] = NEG_INF;
-      if (c < nc) {
-        int j = g + 16 * c;
-        int key = kt + j;
-        float dot = 0.f;
-        const float* qr = Qs + qi * dh;
-        const float* kr = Ks + j * (dh + 1);
-        for (int d = 0; d < dh; ++d) dot = fmaf(qr[d], kr[d], dot);
-        bool ok = row_ok && key >= my_lo && key <= my_pos;
-        s[c] = ok ? dot * scale : NEG_INF;
-        tmax = fmaxf(tmax, s[c]);
-      }
-    }
-    tmax = group_reduce<16>(tmax, MaxOp());
-
-    float alpha = 1.f, psum = 0.f;
-    if (tmax > NEG_INF) {
-      float m_new = fmaxf(m, tmax);
-      alpha = m > NEG_INF ? expf(m - m_new) : 0.f;
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        if (c < nc) {
-          float p = s[c] > NEG_INF ? expf(s[c] - m_new) : 0.f;
-          Ps[qi * BK + g + 16 * c] = p;
-          psum += p;
-        }
-      }
-      m = m_new;
-    } else {
-#pragma unroll
-      for (int c = 0; c < 4; ++c)
-        if (c < nc) Ps[qi * BK + g + 16 * c] = 0.f;
-    }
-    psum = group_reduce<16>(psum, SumOp());
-    l = l * alpha + psum;
-    __syncthreads();
-
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      if (i < nd) {
-        int d = g + 16 * i;
-        float a = acc[i] * alpha;
-        const float* pr = Ps + qi * BK;
-        for (int j = 0; j < BK; ++j) a = fmaf(pr[j], Vs[j * dh + d], a);
-        acc[i] = a;
-      }
+    if (m_t > NEG_INF) {                // the same for the 16 threads of a row
+      tile_values(Ps + qi * BK, Vs, g, nd, dh, BK, a_t);
+      join_tile(m, l, acc, m_t, l_t, a_t, nd);
     }
   }
   if (row_ok) {
@@ -139,6 +240,99 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
       if (i < nd) o[g + 16 * i] = from_float<T>(acc[i] * inv);
   }
 }
+
+// A step of single rows (request s = tile s = row s): every tile of keys is a workgroup of its own, so
+// that a context of a thousand keys is sixteen workgroups side by side and not sixteen steps of one.  It
+// leaves (m_T, l_T, a_T) in part[((tile * H + h) * n_key_tiles + key tile) * (dh + 2)]; m_T = -inf: the
+// tile holds no key of this row.  row_join_kernel joins them in ascending order.
+template <typename T>
+__global__ __launch_bounds__(THREADS) void row_tiles_kernel(
+    const T* __restrict__ q, int ldq, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
+    const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ tile_seq,
+    const int32_t* __restrict__ tile_pos0, float* __restrict__ part, int n_key_tiles, int H, int Hkv, int dh,
+    int page_size, int BK, float scale, int window) {
+  extern __shared__ float smem[];
+  float* Qs = smem;                    // [dh]
+  float* Ks = Qs + dh;                 // [BK][dh + 1]
+  float* Vs = Ks + BK * (dh + 1);      // [BK][dh + 1]
+  float* Ps = Vs + BK * (dh + 1);      // [BK]
+  long long* Kb = reinterpret_cast<long long*>(Ps + BK);   // [BK], [BK]
+  long long* Vb = Kb + BK;
+  const int ktile = blockIdx.x, h = blockIdx.y, tile = blockIdx.z;
+  const int seq = tile_seq[tile];
+  if (seq < 0) return;
+  const int pos = tile_pos0[tile];
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int kt = ktile * BK;
+  const int t = threadIdx.x, g = t % 16;
+  float* mine = part + ((static_cast<size_t>(tile) * H + h) * n_key_tiles + ktile) * (dh + 2);
+  if (kt > pos || kt + BK <= lo) {
+    if (t == 0) mine[0] = -INFINITY;
+    return;
+  }
+  const int hk = h / (H / Hkv);
+  const int32_t* bt = block_tables + static_cast<size_t>(seq) * max_blocks;
+  for (int d = t; d < dh; d += THREADS) Qs[d] = to_float(q[static_cast<size_t>(tile) * ldq + h * dh + d]);
+  load_tile(Ks, Vs, Kb, Vb, k_pool, v_pool, bt, kt, pos, BK, dh, page_size, Hkv, hk);
+  // One row.  The same sums in the same order as 16 threads of the kernel above make them, spread wider:
+  // a thread per key for the scores, 16 threads for the sum of p as there, a thread per dim for the values.
+  const float NEG_INF = -INFINITY;
+  __shared__ float ml[2];
+  if (t < 64) {
+    float s = NEG_INF;
+    if (t < BK) {
+      const int key = kt + t;
+      const float dot = key_dot(Qs, Ks + t * (dh + 1), dh);
+      s = (key >= lo && key <= pos) ? dot * scale : NEG_INF;
+    }
+    const float tmax = wave_max(s);
+    if (t < BK) Ps[t] = s > NEG_INF ? expf(s - tmax) : 0.f;
+    // (the lanes of one wave: what they wrote to Ps is there for their reads)
+    float psum = 0.f;
+    if (t < 16)
+      for (int c = 0; c < BK / 16; ++c) psum += Ps[t + 16 * c];
+    psum = group_reduce<16>(psum, SumOp());
+    if (t == 0) {
+      ml[0] = tmax;
+      ml[1] = psum;
+      mine[0] = tmax;
+      mine[1] = psum;
+    }
+  }
+  __syncthreads();
+  if (!(ml[0] > NEG_INF)) return;
+  for (int d = t; d < dh; d += THREADS) mine[2 + d] = dim_sum(Ps, Vs + d, dh, BK);
+}
+
+template <typename T>
+__global__ void row_join_kernel(const float* __restrict__ part, T* __restrict__ out, int ldo,
+                                const int32_t* __restrict__ tile_seq, int n_key_tiles, int H, int dh) {
+  const int tile = blockIdx.x, h = blockIdx.y;
+  if (tile_seq[tile] < 0) return;
+  const int g = threadIdx.x;           // 16 threads, the dims g + 16 i each, as in the kernels above
+  const int nd = dh / 16;
+  const float* base = part + (static_cast<size_t>(tile) * H + h) * n_key_tiles * (dh + 2);
+  float m = -INFINITY, l = 0.f;
+  float acc[16], a_t[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+  for (int kt = 0; kt < n_key_tiles; ++kt) {
+    const float* p = base + static_cast<size_t>(kt) * (dh + 2);
+    const float m_t = p[0];
+    if (!(m_t > -INFINITY)) continue;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a_t[i] = i < nd ? p[2 + g + 16 * i] : 0.f;
+    join_tile(m, l, acc, m_t, p[1], a_t, nd);
+  }
+  const float inv = 1.0f / l;
+  T* o = out + static_cast<size_t>(tile) * ldo + h * dh;
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+    if (i < nd) o[g + 16 * i] = from_float<T>(acc[i] * inv);
+}
+
+// keys in a tile: a power of two, and at most 4,096 / dh (load_tile)
+static int tile_keys(int dh) { return dh <= 64 ? 64 : (dh <= 128 ? 32 : 16); }
 }  // namespace plain
 
 extern "C" int dn_attention(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
@@ -149,9 +343,9 @@ extern "C" int dn_attention(const void* q, int ldq, void* out, int ldo, const vo
   if (n_tiles <= 0) return 0;
   if (dh < 16 || dh > 256 || dh % 16 != 0 || Hkv < 1 || H % Hkv != 0 || page_size < 1 || max_blocks < 1)
     return DN_ERR_SHAPE;
-  int BK = dh <= 64 ? 64 : (dh <= 128 ? 32 : 16);
-  size_t lds = sizeof(float) * (static_cast<size_t>(plain::BQ) * dh + static_cast<size_t>(BK) * (dh + 1) +
-                                static_cast<size_t>(BK) * dh + static_cast<size_t>(plain::BQ) * BK);
+  int BK = plain::tile_keys(dh);
+  size_t lds = sizeof(float) * (static_cast<size_t>(plain::BQ) * dh + 2 * static_cast<size_t>(BK) * (dh + 1) +
+                                static_cast<size_t>(plain::BQ) * BK + 4 * BK);
   dim3 grid(n_tiles, H), block(plain::THREADS);
   if (dtype == DN_F32)
     hipLaunchKernelGGL(plain::attention_kernel<float>, grid, block, lds, stream, static_cast<const float*>(q), ldq,
@@ -165,6 +359,40 @@ extern "C" int dn_attention(const void* q, int ldq, void* out, int ldo, const vo
                        tile_nrows, tile_pos0, H, Hkv, dh, page_size, BK, scale, window);
   else
     return DN_ERR_DTYPE;
+  return dn_launch_status();
+}
+
+// A step of single rows with the plain kernels, every tile of keys a workgroup of its own: the same bits as
+// dn_attention gives (one order of summation).  max_context: the longest context of the step; part:
+// n_tiles * H * ceil(max_context / tile) * (dh + 2) floats, the tile being dn_attention_rows_tile(dh) keys.
+extern "C" int dn_attention_rows_tile(int dh) { return plain::tile_keys(dh); }
+
+extern "C" int dn_attention_rows(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
+                                 const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
+                                 const int32_t* tile_pos0, int n_tiles, float* part, int max_context, int H, int Hkv,
+                                 int dh, int page_size, float scale, int window, int dtype, hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (dh < 16 || dh > 256 || dh % 16 != 0 || Hkv < 1 || H % Hkv != 0 || page_size < 1 || max_blocks < 1 ||
+      max_context < 1 || !part || n_tiles > 65535 || H > 65535)
+    return DN_ERR_SHAPE;
+  const int BK = plain::tile_keys(dh);
+  const int n_key_tiles = (max_context + BK - 1) / BK;
+  const size_t lds = sizeof(float) * (static_cast<size_t>(dh) + 2 * static_cast<size_t>(BK) * (dh + 1) + 5 * BK);
+  dim3 grid(n_key_tiles, H, n_tiles), block(plain::THREADS);
+#define DN_ROWS(T)                                                                                                   \
+  hipLaunchKernelGGL(plain::row_tiles_kernel<T>, grid, block, lds, stream, static_cast<const T*>(q), ldq,            \
+                     static_cast<const T*>(k_pool), static_cast<const T*>(v_pool), block_tables, max_blocks, tile_seq, \
+                     tile_pos0, part, n_key_tiles, H, Hkv, dh, page_size, BK, scale, window);                         \
+  hipLaunchKernelGGL(plain::row_join_kernel<T>, dim3(n_tiles, H), dim3(16), 0, stream, part, static_cast<T*>(out), ldo, \
+                     tile_seq, n_key_tiles, H, dh)
+  if (dtype == DN_F32) {
+    DN_ROWS(float);
+  } else if (dtype == DN_BF16) {
+    DN_ROWS(bf16_t);
+  } else {
+    return DN_ERR_DTYPE;
+  }
+#undef DN_ROWS
   return dn_launch_status();
 }
 

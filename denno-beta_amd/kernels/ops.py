@@ -81,6 +81,16 @@ def _lib(name):
     return lib
 
 
+def _lib_quiet(name):
+    """The library for a call that launches nothing (not counted, not timed)."""
+    lib = _libs.get(name)
+    if lib is None:
+        global launches
+        lib = _lib(name)
+        launches -= 1
+    return lib
+
+
 def _declare(name, lib):
     P, I, F = c_void_p, c_int, c_float
     sigs = {
@@ -92,7 +102,7 @@ def _declare(name, lib):
             "dn_cast": [P, P, c_longlong, I, I, P],
         },
         "gemm": {
-            "dn_gemm": [P, I, P, P, P, I, P, I, I, I, I, I, I, I, I, P],
+            "dn_gemm": [P, I, P, P, P, I, P, I, I, I, I, I, I, I, I, P, c_longlong, P],
             "dn_pack_matrix": [P, P, I, I, P],
             "dn_gemm_norm_out": [P, I, P, P, P, I, I, I, I, P, P, I, P, P],
             "dn_gemm_norm_in": [P, I, P, P, P, F, P, P, I, I, I, I, I, P, P, P, I, I, I, I, I, P],
@@ -100,6 +110,8 @@ def _declare(name, lib):
         },
         "attention": {
             "dn_attention": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, I, P],
+            "dn_attention_rows": [P, I, P, I, P, P, P, I, P, P, I, P, I, I, I, I, I, F, I, I, P],
+            "dn_attention_rows_tile": [I],
             "dn_attention_flash": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, P],
             "dn_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, I, F, I, P],
         },
@@ -114,6 +126,9 @@ def _declare(name, lib):
         f = getattr(lib, fn)
         f.argtypes = args
         f.restype = c_int
+    if name == "gemm":
+        lib.dn_gemm_work_floats.argtypes = [I, I, I, I]
+        lib.dn_gemm_work_floats.restype = c_longlong
 
 
 def _stream():
@@ -341,12 +356,18 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
         _dev(bias, "bias", (torch.float32,), 1)
         _need(bias.is_contiguous() and bias.shape[0] == N, "linear: bias")
     epi = EPILOGUES[epilogue]
+    work, work_floats = None, 0
+    if not packed & PACKED_W and M <= 64:
+        # the plain product of few rows leaves the sums of K's segments in a workspace
+        work_floats = _lib_quiet("gemm").dn_gemm_work_floats(M, N, K, packed)
+        if work_floats:
+            work = torch.empty(work_floats, dtype=torch.float32, device=a.device)
     if residual is not None:
         _dev(residual, "residual", (torch.float32,), 2)
         _need(tuple(residual.shape) == (M, N) and epi == 0 and out is None, "linear: residual")
         ldr = _rows(residual, "residual")
         _ok(_lib("gemm").dn_gemm(a.data_ptr(), lda, wp, _ptr(bias), 0, 0, residual.data_ptr(), ldr,
-                                 M, N, K, _CODE[a.dtype], F32, 0, packed, _stream()),
+                                 M, N, K, _CODE[a.dtype], F32, 0, packed, _ptr(work), work_floats, _stream()),
             "linear" if _timed is None else f"linear {K} -> {N}, added into the stream")
         return residual
     if isinstance(out, PackedMatrix):
@@ -358,7 +379,7 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
         ldc = _rows(out, "out")
     _need(tuple(out.shape) == (M, N), "linear: out shape")
     _ok(_lib("gemm").dn_gemm(a.data_ptr(), lda, wp, _ptr(bias), out.data_ptr(), ldc, 0, 0, M, N, K,
-                             _CODE[a.dtype], _CODE[out.dtype], epi, packed, _stream()),
+                             _CODE[a.dtype], _CODE[out.dtype], epi, packed, _ptr(work), work_floats, _stream()),
         "linear" if _timed is None else f"linear {K} -> {N}" + (f", {epilogue}" if epi else ""))
     return out
 
@@ -487,6 +508,18 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
         return out
     n_tiles = tiles.shape[1]
     base = tiles.data_ptr()
+    if single_rows and max_context > 0:
+        # a step of single rows in the plain kernels: every tile of keys a workgroup of its own, the
+        # tiles' results joined in order by a second kernel; the same bits as the kernel below gives
+        _need(max_context <= block_tables.shape[1] * ps, "attention: max_context exceeds the block tables")
+        _need(n_tiles == T, "attention: a step of single rows has a tile for every row")
+        key_tiles = -(-max_context // lib.dn_attention_rows_tile(dh))
+        part = torch.empty(n_tiles * n_heads * key_tiles * (dh + 2), dtype=torch.float32, device=q.device)
+        _ok(lib.dn_attention_rows(
+            q.data_ptr(), ldq, out.data_ptr(), ldo, k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(),
+            block_tables.shape[1], base, base + 12 * n_tiles, n_tiles, part.data_ptr(), int(max_context), n_heads, Hkv,
+            dh, ps, float(scale), int(window), _CODE[q.dtype], _stream()), "attention (single rows)")
+        return out
     _ok(lib.dn_attention(
         q.data_ptr(), ldq, out.data_ptr(), ldo, k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(),
         block_tables.shape[1], base, base + 4 * n_tiles, base + 8 * n_tiles, base + 12 * n_tiles, n_tiles,

@@ -401,6 +401,29 @@ def test_linear_rows_do_not_depend_on_the_batch():
         assert torch.equal(sub, full[rows])
 
 
+@pytest.mark.parametrize("N,K", [(1600, 1600), (1600, 6400), (50257, 320), (100, 96), (333, 200), (4800, 1608)])
+def test_plain_linear_has_one_order_of_summation_whatever_the_rows(N, K):
+    """The 32-bit product has two kernels (up to 64 rows, where K's segments may be workgroups of their
+    own with a second kernel that adds their sums; more rows) and four row tiles: a row's result is the
+    same bits in all of them, alone or among 200 rows, with bias, GELU or the residual sum."""
+    a, w, bias = rnd(200, K, seed=1), rnd(N, K, seed=2, scale=0.1), rnd(N, seed=3)
+    full = {}
+    for epi in ("none", "gelu_erf"):
+        full[epi] = ops().linear(a, w, bias, out=torch.empty(200, N, device=DEV), epilogue=epi)
+    res0 = rnd(200, N, seed=4)
+    full["residual"] = ops().linear(a, w, bias, residual=res0.clone())
+    want = R.linear(a.double(), w.double(), bias.double(), out=torch.empty(200, N, dtype=torch.float64, device=DEV)).float()
+    assert torch.allclose(full["none"], want, atol=4e-6 * math.sqrt(K), rtol=2e-5)
+    for rows in ([0], [199], [5, 6], list(range(3, 11)), list(range(40, 49)), list(range(16)), list(range(100, 133)),
+                 list(range(64)), list(range(65))):
+        sub = a[rows].contiguous()
+        for epi in ("none", "gelu_erf"):
+            got = ops().linear(sub, w, bias, out=torch.empty(len(rows), N, device=DEV), epilogue=epi)
+            assert torch.equal(got, full[epi][rows]), (len(rows), epi)
+        got = ops().linear(sub, w, bias, residual=res0[rows].contiguous())
+        assert torch.equal(got, full["residual"][rows]), (len(rows), "residual")
+
+
 def test_linear_refuses_what_it_cannot_take():
     o = ops()
     with pytest.raises(o.KernelError, match="multiple of 8"):
@@ -600,10 +623,24 @@ def test_attention_rows_do_not_depend_on_the_batch():
     q, k, v, bt, tiles, T = paged_case([200, 90], [50, 90], H, H, dh, ps, torch.float32, seed=2)
     out = torch.zeros(T, H * dh, device=DEV)
     ops().attention(q[:, :H * dh], out, k, v, bt, tiles, H, 0.2)
-    # request 0's last row alone, as a decoded token
+    # request 0's last row alone, as a decoded token: in the kernel for portions, and in the kernels for steps of
+    # single rows, where every tile of keys is a workgroup of its own (launched for its context and for a longer one)
     one = torch.zeros(1, H * dh, device=DEV)
     ops().attention(q[49:50, :H * dh], one, k, v, bt, i32([[0], [0], [1], [199]]), H, 0.2)
     assert torch.equal(one[0], out[49])
+    for max_context in (200, 208):
+        one = torch.zeros(1, H * dh, device=DEV)
+        ops().attention(q[49:50, :H * dh], one, k, v, bt, i32([[0], [0], [1], [199]]), H, 0.2, single_rows=True,
+                        max_context=max_context)
+        assert torch.equal(one[0], out[49])
+    # both requests' last rows as one step of single rows, with a window
+    win = torch.zeros(T, H * dh, device=DEV)
+    ops().attention(q[:, :H * dh], win, k, v, bt, tiles, H, 0.2, 70)
+    two = torch.zeros(2, H * dh, device=DEV)
+    rows = torch.stack([q[49, :H * dh], q[139, :H * dh]]).contiguous()
+    ops().attention(rows, two, k, v, bt, i32([[0, 1], [0, 1], [1, 1], [199, 89]]), H, 0.2, 70, single_rows=True,
+                    max_context=200)
+    assert torch.equal(two[0], win[49]) and torch.equal(two[1], win[139])
 
 
 def test_sample_greedy_and_walk():

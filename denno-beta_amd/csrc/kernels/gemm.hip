@@ -446,6 +446,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int col = lane % 16, g = lane / 16;
   const int n0 = blockIdx.x * (16 * NB);
+  const int row0 = blockIdx.y * (MB * 16);     // the rows may be shared out among workgroups too (blockIdx.y)
   const int ksteps = (K + 31) / 32, nblocks = (N + 15) / 16;
   const bf16_t* wblk[NB];
 #pragma unroll
@@ -482,14 +483,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
       if constexpr (KV) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int m = mb * 16 + g * 4 + r;
+          const int m = row0 + mb * 16 + g * 4 + r;
           epi_slot[p][r] = m < M ? kv.slot_map[m] : -1;
         }
       }
       if (resid) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int m = min(mb * 16 + g * 4 + r, M - 1);
+          const int m = min(row0 + mb * 16 + g * 4 + r, M - 1);
           epi_x[p][r] = resid[static_cast<size_t>(m) * ldr + nn];
         }
       }
@@ -503,7 +504,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   if constexpr (NORM == NORM_IN) {
 #pragma unroll
     for (int t = 0; t < SR; ++t) {
-      const int row = min(wave + t * WAVES, M - 1);
+      const int row = min(row0 + wave + t * WAVES, M - 1);
 #pragma unroll
       for (int i = 0; i < SP; ++i)
         st[t][i] = *reinterpret_cast<const float2*>(nio.stats_in + (static_cast<size_t>(row) * nio.blocks_in + min(lane + 64 * i, nio.blocks_in - 1)) * 2);
@@ -528,11 +529,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   const int astep = (packed & PACKED_A) ? 512 : 32;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
-    int row = mb * 16 + col;
+    int row = row0 + mb * 16 + col;
     a_ok[mb] = row < M;
     // (a block of rows beyond M, where MB is more than the rows need, reads the last one again: packed
     // rows end with the block that holds row M - 1)
-    arow[mb] = (packed & PACKED_A) ? A + (static_cast<size_t>(min(mb, (M + 15) / 16 - 1)) * ksteps * 64 + lane) * 8
+    arow[mb] = (packed & PACKED_A) ? A + (static_cast<size_t>(min(static_cast<int>(blockIdx.y) * MB + mb, (M + 15) / 16 - 1)) * ksteps * 64 + lane) * 8
                                    : A + static_cast<size_t>(a_ok[mb] ? row : 0) * lda + g * 8;
   }
   // NORM_IN: the rows' means and 1 / sqrt(var + eps), joined while the first round of operands travels (a
@@ -557,8 +558,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
         }
       const float var = wave_sum(sq) / (16.f * blocks);
       if (lane == 0) {
-        rowstat[row][0] = row < M ? mean : 0.f;
-        rowstat[row][1] = row < M ? 1.0f / sqrtf(var + nio.eps) : 0.f;
+        rowstat[row][0] = row0 + row < M ? mean : 0.f;
+        rowstat[row][1] = row0 + row < M ? 1.0f / sqrtf(var + nio.eps) : 0.f;
       }
     }
   };
@@ -626,17 +627,17 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
         const float mean = group_reduce<16>(x, SumOp()) * (1.0f / 16.0f);
         const float d = x - mean;
         const float sq = group_reduce<16>(d * d, SumOp());
-        const int m = mb * 16 + g * 4 + r;
+        const int m = row0 + mb * 16 + g * 4 + r;
         if (col == 0 && m < M)
           *reinterpret_cast<float2*>(nio.stats_out + (static_cast<size_t>(m) * nblocks + blockIdx.x * NB + nb) * 2) = float2{mean, sq};
       }
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      int m = mb * 16 + g * 4 + r;
+      int m = row0 + mb * 16 + g * 4 + r;
       if (m >= M || nn >= N) continue;
       float v = s[r] + epi_bias[p];
-      if constexpr (NORM == NORM_IN) v = (s[r] - rowstat[m][0] * epi_norm[p]) * rowstat[m][1] + epi_bias[p];
+      if constexpr (NORM == NORM_IN) v = (s[r] - rowstat[m - row0][0] * epi_norm[p]) * rowstat[m - row0][1] + epi_bias[p];
       if (resid) {
         resid[static_cast<size_t>(m) * ldr + nn] = epi_x[p][r] + v;
         if constexpr (NORM == NORM_OUT)
@@ -831,7 +832,8 @@ struct Call {
 
 template <int MB, int NB, int WAVES, int U, typename TC, bool KV>
 static void launch_one(const Call& c, hipStream_t stream) {
-  dim3 grid((c.N + 16 * NB - 1) / (16 * NB)), block(WAVES * 64);
+  // (MB row blocks per workgroup: where the rows need more, the second grid dimension shares them out)
+  dim3 grid((c.N + 16 * NB - 1) / (16 * NB), ((c.M + 15) / 16 + MB - 1) / MB), block(WAVES * 64);
   KVScatter kv = c.kv ? *c.kv : KVScatter{};
   hipLaunchKernelGGL((gemm_kernel<MB, NB, WAVES, U, TC, KV>), grid, block, 0, stream,
                      static_cast<const bf16_t*>(c.A), c.lda, static_cast<const bf16_t*>(c.W), c.bias,
@@ -842,7 +844,7 @@ static void launch_one(const Call& c, hipStream_t stream) {
 // residual stream), for 17 to 64 rows
 template <int MB, int NB, int WAVES, int U>
 static void launch_norm(const Call& c, const NormIO& nio, int norm, hipStream_t stream) {
-  dim3 grid((c.N + 16 * NB - 1) / (16 * NB)), block(WAVES * 64);
+  dim3 grid((c.N + 16 * NB - 1) / (16 * NB), ((c.M + 15) / 16 + MB - 1) / MB), block(WAVES * 64);
   KVScatter kv = c.kv ? *c.kv : KVScatter{};
 #define DN_LN(TC, KV, NORM)                                                                                        \
   hipLaunchKernelGGL((gemm_kernel<MB, NB, WAVES, U, TC, KV, NORM>), grid, block, 0, stream,                       \
@@ -867,11 +869,8 @@ static void launch_mb_norm(const Call& c, const NormIO& nio, int norm, hipStream
       default: return launch_norm<4, 2, 8, 4>(c, nio, norm, stream);
     }
   }
-  switch (mb) {
-    case 2: return launch_norm<2, 1, 8, 8>(c, nio, norm, stream);
-    case 3: return launch_norm<3, 1, 8, 8>(c, nio, norm, stream);
-    default: return launch_norm<4, 1, 8, 8>(c, nio, norm, stream);
-  }
+  // (few columns: the rows in two halves, so that there are workgroups for all CUs)
+  return launch_norm<2, 1, 8, 8>(c, nio, norm, stream);
 }
 
 template <int MB, int NB, int WAVES, int U>
@@ -946,11 +945,8 @@ static void launch_mb(const Call& c, hipStream_t stream) {
       default: return launch<4, 2, WAVES, 4>(c, stream);
     }
   }
-  switch (mb) {
-    case 2: return launch<2, 1, WAVES, 8>(c, stream);
-    case 3: return launch<3, 1, WAVES, 8>(c, stream);
-    default: return launch<4, 1, WAVES, 8>(c, stream);
-  }
+  // (few columns: the rows in two halves, so that there are workgroups for all CUs)
+  return launch<2, 1, WAVES, 8>(c, stream);
 }
 
 static void run(const Call& c, hipStream_t stream) {

@@ -61,6 +61,10 @@ def host_library():
             "dn_cache_commit": (I, [P, L, I]), "dn_cache_length": (I, [P, L]), "dn_cache_slot": (I, [P, L]),
             "dn_cache_state": (I, [P, L, c_void_p]), "dn_cache_set_rng": (I, [P, L, ctypes.c_uint64, ctypes.c_uint64]),
             "dn_cache_note_sampled": (I, [P, L, I]),
+            "dn_cache_note_drawn_step": (None, [P, c_void_p, I]),
+            "dn_cache_note_tokens_step": (None, [P, c_void_p, c_void_p, I]),
+            "dn_sched_steps_done": (I, [P, c_void_p, c_void_p, I, IP]),
+            "dn_sched_tokens_sampled": (I, [P, c_void_p, I, c_void_p, IP]),
             "dn_cache_rng_states": (I, [P, c_void_p, I, c_void_p, c_void_p, IP]),
             "dn_cache_generation": (L, [P, I]), "dn_cache_block_table": (I, [P, L, I, c_void_p, I]),
             "dn_cache_blocks": (I, [P, L, I]), "dn_cache_free_pages": (I, [P, I]),
@@ -162,6 +166,14 @@ class CacheManager:
     def note_sampled(self, rid: int, token: int):
         """One number was drawn from the request's generator and gave `token`."""
         self._chk(self._lib.dn_cache_note_sampled(self._h, rid, token), f"sampled token of request {rid}")
+
+    def note_drawn_step(self, rids: np.ndarray):
+        """A number was drawn from the generator of each of these requests (ids that are no longer live are skipped)."""
+        self._lib.dn_cache_note_drawn_step(self._h, rids.ctypes.data, len(rids))
+
+    def note_tokens_step(self, rids: np.ndarray, tokens: np.ndarray):
+        """The tokens that those draws gave (int32), once they are known."""
+        self._lib.dn_cache_note_tokens_step(self._h, rids.ctypes.data, tokens.ctypes.data, len(rids))
 
     def rng_states(self, rids: np.ndarray):
         """-> (seeds, numbers drawn so far) of the requests, uint64 arrays."""

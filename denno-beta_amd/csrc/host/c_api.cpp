@@ -50,6 +50,12 @@ int dn_cache_set_rng(void* c, int64_t rid, uint64_t seed, uint64_t drawn) {
 int dn_cache_note_sampled(void* c, int64_t rid, int token) {
   return static_cast<CacheManager*>(c)->note_sampled(rid, token);
 }
+void dn_cache_note_drawn_step(void* c, const int64_t* rids, int n) {
+  static_cast<CacheManager*>(c)->note_drawn_step(rids, n);
+}
+void dn_cache_note_tokens_step(void* c, const int64_t* rids, const int32_t* tokens, int n) {
+  static_cast<CacheManager*>(c)->note_tokens_step(rids, tokens, n);
+}
 int dn_cache_rng_states(void* c, const int64_t* rids, int n, uint64_t* seeds, uint64_t* drawn, int* failed) {
   return static_cast<CacheManager*>(c)->rng_states(rids, n, seeds, drawn, failed);
 }
@@ -117,6 +123,12 @@ int dn_sched_schedule(void* s, int64_t* rid, int* start, int* count, int* sample
 }
 int dn_sched_step_done(void* s, int64_t rid, int count) { return static_cast<Scheduler*>(s)->step_done(rid, count); }
 int dn_sched_token_sampled(void* s, int64_t rid) { return static_cast<Scheduler*>(s)->token_sampled(rid); }
+int dn_sched_steps_done(void* s, const int64_t* rids, const int* counts, int n, int* failed) {
+  return static_cast<Scheduler*>(s)->steps_done(rids, counts, n, failed);
+}
+int dn_sched_tokens_sampled(void* s, const int64_t* rids, int n, int* last, int* failed) {
+  return static_cast<Scheduler*>(s)->tokens_sampled(rids, n, last, failed);
+}
 int dn_sched_finish(void* s, int64_t rid) { return static_cast<Scheduler*>(s)->finish(rid); }
 int dn_sched_n_waiting(void* s) { return static_cast<Scheduler*>(s)->n_waiting(); }
 int dn_sched_n_running(void* s) { return static_cast<Scheduler*>(s)->n_running(); }

@@ -232,6 +232,20 @@ int CacheManager::note_sampled(int64_t rid, int32_t token) {
   return kOk;
 }
 
+void CacheManager::note_drawn_step(const int64_t* rids, int n) {
+  for (int i = 0; i < n; ++i) {
+    auto it = by_rid_.find(rids[i]);
+    if (it != by_rid_.end()) slot_state_[it->second.slot].rng_drawn += 1;
+  }
+}
+
+void CacheManager::note_tokens_step(const int64_t* rids, const int32_t* tokens, int n) {
+  for (int i = 0; i < n; ++i) {
+    auto it = by_rid_.find(rids[i]);
+    if (it != by_rid_.end()) slot_state_[it->second.slot].last_token = tokens[i];
+  }
+}
+
 int CacheManager::rng_states(const int64_t* rids, int n, uint64_t* seeds, uint64_t* drawn, int* failed) const {
   for (int i = 0; i < n; ++i) {
     auto it = by_rid_.find(rids[i]);

@@ -60,6 +60,10 @@ class CacheManager {
   const SlotState* state(int64_t rid) const;
   int set_rng(int64_t rid, uint64_t seed, uint64_t drawn);
   int note_sampled(int64_t rid, int32_t token);
+  // the same in two halves, for a step's requests at once: a number was drawn for each (when the sampling
+  // kernel is launched), and later the tokens that it gave are known; ids that are no longer live are skipped
+  void note_drawn_step(const int64_t* rids, int n);
+  void note_tokens_step(const int64_t* rids, const int32_t* tokens, int n);
   // seeds and counts of a step's requests in one call; on a failure *failed is the entry's index
   int rng_states(const int64_t* rids, int n, uint64_t* seeds, uint64_t* drawn, int* failed) const;
   int64_t generation(int slot) const;         // bumped each time the slot is given out

@@ -171,6 +171,29 @@ int Scheduler::token_sampled(int64_t rid) {
   return r.generated >= r.max_new ? 1 : 0;
 }
 
+int Scheduler::steps_done(const int64_t* rids, const int* counts, int n, int* failed) {
+  for (int i = 0; i < n; ++i) {
+    int rc = step_done(rids[i], counts[i]);
+    if (rc < 0) {
+      *failed = i;
+      return rc;
+    }
+  }
+  return kSchedOk;
+}
+
+int Scheduler::tokens_sampled(const int64_t* rids, int n, int* last, int* failed) {
+  for (int i = 0; i < n; ++i) {
+    int rc = token_sampled(rids[i]);
+    if (rc < 0) {
+      *failed = i;
+      return rc;
+    }
+    last[i] = rc;
+  }
+  return kSchedOk;
+}
+
 int Scheduler::finish(int64_t rid) {
   auto it = reqs_.find(rid);
   if (it == reqs_.end()) return kSchedUnknown;

@@ -58,6 +58,10 @@ class Scheduler {
   int schedule(std::vector<StepEntry>* out, std::vector<int64_t>* preempted);
   int step_done(int64_t rid, int count);   // the step ran: count more tokens are in the cache
   int token_sampled(int64_t rid);          // -> 1 if that token was the request's last (length), else 0
+  // the same for all entries of a step in one call each; last[i] as token_sampled returns it.  On a failure
+  // *failed is the entry's index and the entries before it have been done.
+  int steps_done(const int64_t* rids, const int* counts, int n, int* failed);
+  int tokens_sampled(const int64_t* rids, int n, int* last, int* failed);
   int finish(int64_t rid);                 // pages and slot go back (running or waiting)
   int abort_step(const std::vector<int64_t>& rids);   // a failed step: its requests are dropped, pages back
 

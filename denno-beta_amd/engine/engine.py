@@ -33,6 +33,7 @@ class Request:
     finished: bool = False
     finish_reason: Optional[str] = None                 # "eos", "length", "error"
     preemptions: int = 0
+    n_sampled: int = 0     # tokens sampled for it so far, the one that the host has not read yet among them
 
     @property
     def generated(self) -> List[int]:
@@ -55,7 +56,19 @@ class StepRecord:
     prefill_rows: int
     requests: int
     preempted: int
-    host_ms: float = 0.0     # wall time of Engine.step on the host (it ends with the read of the sampled tokens)
+    ran_ahead: bool = False  # launched before the step before it had given its tokens to the host
+    host_ms: float = 0.0     # wall time of the step's two halves on the host (the second ends with the read of the tokens)
+
+
+@dataclass
+class _Launched:
+    """A step whose kernels are issued and whose sampled tokens are not read yet."""
+    plan: list
+    sampled: List[Request]           # the requests that are sampled, in the order of the logits' rows
+    last: Dict[int, bool]            # request id -> the token being sampled is its last (length)
+    alive: List[Request]             # the sampled requests that go on after this step
+    pending: object                  # sampling.sampler.Pending
+    record: StepRecord
 
 
 class Engine:
@@ -72,6 +85,8 @@ class Engine:
         self._next_rid = 0
         self.records: List[StepRecord] = []
         self.fail_next_step = False    # test hook: the next step raises after its pages were taken
+        self._ahead: Optional[_Launched] = None      # the step that was launched before the last one was read
+        self._failed_ahead: Optional[Exception] = None
 
     @classmethod
     def from_folder(cls, model_dir: str, options: Optional[EngineOptions] = None, cast_matrices=False):
@@ -101,26 +116,71 @@ class Engine:
         return rid
 
     def has_unfinished(self) -> bool:
-        return self.scheduler.n_waiting() + self.scheduler.n_running() > 0
+        """Requests are waiting or running, or a launched step's tokens have not been read yet."""
+        return self.scheduler.n_waiting() + self.scheduler.n_running() > 0 or self._ahead is not None
+
+    def _release(self, rid: int):
+        """The request's pages and slot go back, unless they have (its last token was already on its way)."""
+        if self.scheduler.known(rid) >= 0:
+            self.scheduler.finish(rid)
 
     def abort(self, rid: int):
         req = self.requests.get(rid)
         if req is None or req.finished:
             return
-        self.scheduler.finish(rid)
+        self._release(rid)
         req.finished, req.finish_reason = True, "aborted"
 
     # -- one step ------------------------------------------------------------------------
+    # A step has two halves: `_launch` plans it, issues its kernels and the sampling kernels and does the
+    # bookkeeping that needs counts only; `_complete` waits for the sampled tokens and does what needs the
+    # tokens themselves (the request's token list, the end-of-sequence check).  In steady decoding the next
+    # step is launched between the two, with its tokens taken from the device where the sampling kernel
+    # left them (`run_ahead`): the host's work on a step then hides behind the GPU's work on the next one,
+    # and a request that ends with an end-of-sequence token has run one step too many, whose token is
+    # thrown away.
     def step(self) -> List[StepOutput]:
+        if self._failed_ahead is not None:          # the step that was launched ahead could not run
+            exc, self._failed_ahead = self._failed_ahead, None
+            raise exc
+        launched, self._ahead = self._ahead, None
+        if launched is not None and all(r.finished for r in launched.sampled):
+            launched = None                         # launched ahead for requests that have all ended since
+        if launched is None:
+            launched = self._launch(None)
+        if launched is None:
+            return []
+        if self._may_run_ahead(launched):
+            try:
+                self._ahead = self._launch(launched)
+            except Exception as exc:     # its requests are dropped already; the caller hears of it at the next step
+                self._failed_ahead = exc
+        return self._complete(launched)
+
+    def _may_run_ahead(self, launched: "_Launched") -> bool:
+        """The next step can be planned and launched before this one's tokens are known on the host: it will
+        be single tokens of requests that were all sampled in this one, replayed from a graph, and nothing
+        about it depends on the tokens' values."""
+        if not (self.options.run_ahead and self.runner.runs_ahead() and launched.pending.final):
+            return False
+        if self.scheduler.n_waiting() > 0 or self.scheduler.n_running() == 0:
+            return False
+        if self.scheduler.n_running() != len(launched.alive):
+            return False                            # a running request that was not sampled in this step
+        return not any(r.params.has_penalties for r in launched.sampled)
+
+    def _launch(self, before: Optional["_Launched"]) -> Optional["_Launched"]:
+        """before: the step whose sampled tokens are still on the device only (then this step takes them
+        from there)."""
         t_begin = time.perf_counter()
         plan, preempted = self.scheduler.schedule()
         for rid in preempted:
             self.requests[rid].preemptions += 1
         if not plan:
-            if self.has_unfinished():
+            if self.has_unfinished() and before is None:
                 raise RuntimeError("scheduler: requests are waiting but none can run "
                                    "(a request larger than the cache should have been refused)")
-            return []
+            return None
         entries, sampled = [], []
         manager = self.runner.cache.manager
         for p in plan:
@@ -130,58 +190,89 @@ class Engine:
                 # request's slot record gets its generator (seed, numbers drawn so far: a request that
                 # comes back after preemption goes on where it was, so its samples do not change)
                 self.runner.cache.reset_states(manager.slot(p.rid))
-                manager.set_rng(p.rid, req.seed, len(req.generated))
-            wants = p.samples and len(req.generated) < req.max_new
-            entries.append(StepEntry(p.rid, req.tokens[p.start:p.start + p.count], [p.count - 1] if wants else []))
+                manager.set_rng(p.rid, req.seed, req.n_sampled)
+            wants = p.samples and req.n_sampled < req.max_new
+            tokens = req.tokens[p.start:p.start + p.count] if before is None else [0]     # ([0]: stands in for the token on the device)
+            entries.append(StepEntry(p.rid, tokens, [p.count - 1] if wants else []))
             if wants:
                 sampled.append(req)
         try:
             if self.fail_next_step:
                 self.fail_next_step = False
                 raise RuntimeError("step failed (injected)")
-            logits = self.runner.step(entries)
-            for p in plan:
-                self.scheduler.step_done(p.rid, p.count)
+            device_tokens = None
+            if before is not None:
+                place = {r.rid: i for i, r in enumerate(before.sampled)}
+                order = [place[p.rid] for p in plan]
+                device_tokens = before.pending.tokens
+                if order != list(range(len(before.sampled))):
+                    device_tokens = device_tokens[torch.tensor(order, dtype=torch.long, device=device_tokens.device)]
+            logits = self.runner.step(entries, device_tokens)
+            self.scheduler.steps_done(np.asarray([p.rid for p in plan], dtype=np.int64),
+                                      np.asarray([p.count for p in plan], dtype=np.int32))
             # each request's generator lives in its slot record: the seed and the count of numbers drawn
-            seeds, drawn = manager.rng_states(np.asarray([r.rid for r in sampled], dtype=np.int64))
-            tokens = self.sampler.sample(logits, [r.params for r in sampled], seeds.tolist(), drawn.tolist(),
-                                         [r.tokens for r in sampled])
-            for r, tok in zip(sampled, tokens):
-                manager.note_sampled(r.rid, int(tok))
+            rids = np.asarray([r.rid for r in sampled], dtype=np.int64)
+            seeds, drawn = manager.rng_states(rids)
+            pending = self.sampler.launch(logits, [r.params for r in sampled], seeds.tolist(), drawn.tolist(),
+                                          [r.tokens for r in sampled])
+            manager.note_drawn_step(rids)
+            last = self.scheduler.tokens_sampled(rids).tolist()
         except Exception:
             # the step's requests are dropped, their pages go back, the engine stays usable
             # (crates/denno-server/src/scheduler.rs:362-370, 457-469)
             for p in plan:
                 req = self.requests[p.rid]
-                self.scheduler.finish(p.rid)
-                req.finished, req.finish_reason = True, "error"
+                if not req.finished:
+                    self._release(p.rid)
+                    req.finished, req.finish_reason = True, "error"
             raise
+        alive = []
+        for r, is_last in zip(sampled, last):
+            r.n_sampled += 1
+            if is_last:
+                # the token that is being sampled is the request's last: nothing of it runs after this step
+                # (its pages go back now: whoever gets them writes after this step on the device)
+                self.scheduler.finish(r.rid)
+            else:
+                alive.append(r)
         self.records.append(StepRecord(
             rows=sum(p.count for p in plan), decode_rows=sum(1 for p in plan if p.count == 1 and p.start > 0),
             prefill_rows=sum(p.count for p in plan if not (p.count == 1 and p.start > 0)),
-            requests=len(plan), preempted=len(preempted)))
-        record = self.records[-1]
-        outputs = []
-        by_rid = {r.rid: t for r, t in zip(sampled, tokens)}
+            requests=len(plan), preempted=len(preempted), ran_ahead=before is not None,
+            host_ms=(time.perf_counter() - t_begin) * 1e3))
+        return _Launched(plan, sampled, dict(zip((r.rid for r in sampled), last)), alive, pending, self.records[-1])
+
+    def _complete(self, launched: "_Launched") -> List[StepOutput]:
+        t_begin = time.perf_counter()
+        tokens = self.sampler.read(launched.pending)
+        manager = self.runner.cache.manager
+        # (a request that ended meanwhile, by an end-of-sequence token of the step before, ran here for nothing)
+        told = [(r, int(t)) for r, t in zip(launched.sampled, tokens) if not r.finished]
+        manager.note_tokens_step(np.asarray([r.rid for r, _ in told], dtype=np.int64),
+                                 np.asarray([t for _, t in told], dtype=np.int32))
+        by_rid = {r.rid: t for r, t in told}
         eos = set(self.spec.eos_token_ids)
-        for p in plan:
+        outputs = []
+        for p in launched.plan:
             req = self.requests[p.rid]
+            if req.finished:
+                continue
             tok = by_rid.get(p.rid)
             if tok is not None:
-                req.tokens.append(int(tok))
-                last = self.scheduler.token_sampled(p.rid)
+                req.tokens.append(tok)
                 # the end-of-sequence token counts as generated (crates/denno-engine/src/engine.rs:1125-1129)
-                if int(tok) in eos and not req.params.ignore_eos:
+                if tok in eos and not req.params.ignore_eos:
                     req.finish_reason = "eos"
-                elif last:
+                    self._release(p.rid)
+                elif launched.last[p.rid]:
                     req.finish_reason = "length"
-            elif p.samples and len(req.generated) >= req.max_new:
+            elif p.samples and req.n_sampled >= req.max_new:
                 req.finish_reason = "length"      # max_tokens = 0: the prompt is computed, nothing is sampled
+                self._release(p.rid)
             if req.finish_reason is not None:
                 req.finished = True
-                self.scheduler.finish(p.rid)
-            outputs.append(StepOutput(p.rid, None if tok is None else int(tok), req.finished, req.finish_reason))
-        record.host_ms = (time.perf_counter() - t_begin) * 1e3
+            outputs.append(StepOutput(p.rid, tok, req.finished, req.finish_reason))
+        launched.record.host_ms += (time.perf_counter() - t_begin) * 1e3
         return outputs
 
     # -- whole generations ---------------------------------------------------------------

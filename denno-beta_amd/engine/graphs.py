@@ -116,7 +116,9 @@ class DecodeGraph:
             if bad >= 0:
                 raise BatchError(f"request {int(rids[bad])}: a token's page was given back already")
 
-    def run(self, rids, tokens, starts, slots) -> torch.Tensor:
+    def run(self, rids, tokens, starts, slots, device_tokens=None) -> torch.Tensor:
+        """device_tokens: the step's tokens as an int32 tensor on the device (a sampling that the host has
+        not read yet), in place of `tokens`."""
         i = self.turn
         self.turn ^= 1
         if self.copied[i] is not None:
@@ -126,6 +128,8 @@ class DecodeGraph:
         ev = torch.cuda.Event()
         ev.record()
         self.copied[i] = ev
+        if device_tokens is not None:
+            self._view("tokens")[:len(rids)].copy_(device_tokens)
         self.graph.replay()
         return self.logits
 
@@ -140,13 +144,18 @@ class DecodeGraphs:
     def takes(self, entries: Sequence[StepEntry]) -> bool:
         return self.runner.model.graph_safe and all(len(e.tokens) == 1 for e in entries)
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        """Runs a pure decode step; -> logits [R, vocab] at the wanted places (a copy)."""
+    def step(self, entries: Sequence[StepEntry], device_tokens=None) -> torch.Tensor:
+        """Runs a pure decode step; -> logits [R, vocab] at the wanted places (a copy).
+        device_tokens: int32 [entries] on the device: the entries' tokens, which the host does not know yet
+        (the entries then hold any token of the vocabulary in their place)."""
         runner = self.runner
         mgr, spec = runner.cache.manager, runner.spec
         n = len(entries)
         rids = np.asarray([e.rid for e in entries], dtype=np.int64)
         tokens = np.asarray([e.tokens[0] for e in entries], dtype=np.int64)
+        if device_tokens is not None and (device_tokens.dtype != torch.int32 or tuple(device_tokens.shape) != (n,)
+                                          or device_tokens.device != runner.device):
+            raise BatchError("device_tokens must be int32, one per entry, on the runner's device")
         starts = mgr.lengths(rids)
         if len(set(rids.tolist())) != n:
             raise BatchError("a request appears twice in one step")
@@ -172,7 +181,7 @@ class DecodeGraphs:
         g = self.graphs.get(key)
         if g is None:
             g = self.graphs[key] = DecodeGraph(runner, B, ctx_bucket)
-        logits = g.run(rids, tokens.astype(np.int32), starts, slots)
+        logits = g.run(rids, tokens.astype(np.int32), starts, slots, device_tokens)
         if len(rows) == n:
             out = logits[:n].clone()
         else:

@@ -91,6 +91,22 @@ class Scheduler:
         """One more token is known; -> True if it was the request's last (length)."""
         return bool(self._chk(self._lib.dn_sched_token_sampled(self._h, rid), f"token for request {rid}"))
 
+    def steps_done(self, rids: np.ndarray, counts: np.ndarray):
+        """step_done for all entries of a step (rids int64, counts int32)."""
+        failed = c_int(0)
+        rc = self._lib.dn_sched_steps_done(self._h, rids.ctypes.data, counts.ctypes.data, len(rids), ctypes.byref(failed))
+        if rc < 0:
+            raise SchedulerError(rc, f"step done for request {int(rids[failed.value])}")
+
+    def tokens_sampled(self, rids: np.ndarray) -> np.ndarray:
+        """token_sampled for all of them; -> int32 array, 1 where the token was the request's last."""
+        last = np.zeros(len(rids), dtype=np.int32)
+        failed = c_int(0)
+        rc = self._lib.dn_sched_tokens_sampled(self._h, rids.ctypes.data, len(rids), last.ctypes.data, ctypes.byref(failed))
+        if rc < 0:
+            raise SchedulerError(rc, f"token for request {int(rids[failed.value])}")
+        return last
+
     def finish(self, rid: int):
         self._chk(self._lib.dn_sched_finish(self._h, rid), f"finish request {rid}")
 

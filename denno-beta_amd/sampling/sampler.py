@@ -20,14 +20,20 @@ class Sampler:
         self.device = device
         self._zeros = {}      # rows -> [2, rows] of zeros on the device: temperatures and uniforms of all-greedy steps
 
-    def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
-               counters: Sequence[int], contexts: Sequence[Sequence[int]]) -> List[int]:
-        """logits: [R, V] 32-bit (changed in place by penalties); row r belongs to a request
+    def sample(self, logits, params, seeds, counters, contexts) -> List[int]:
+        """launch and read at once."""
+        return self.read(self.launch(logits, params, seeds, counters, contexts))
+
+    def launch(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
+               counters: Sequence[int], contexts: Sequence[Sequence[int]]) -> "Pending":
+        """Starts the sampling of a step's rows and does not wait for it.
+        logits: [R, V] 32-bit (changed in place by penalties); row r belongs to a request
         with params[r], the seed seeds[r], counters[r] tokens sampled so far and the tokens
-        contexts[r] (prompt + generated)."""
+        contexts[r] (prompt + generated).  `read` gives the tokens; `Pending.tokens` holds them on the
+        device as soon as the kernels have run, and is final if `Pending.final`."""
         R = logits.shape[0]
         if R == 0:
-            return []
+            return Pending(None, 0, None)
         dev = self.device
         if any(p.has_penalties for p in params):
             starts, flat = [0], []
@@ -43,7 +49,13 @@ class Sampler:
                 f32([p.frequency_penalty or 0.0 for p in params]),
                 f32([p.presence_penalty or 0.0 for p in params]),
                 torch.tensor([p.no_repeat_ngram_size or 0 for p in params], dtype=torch.int32, device=dev))
-        out = torch.empty(R, dtype=torch.int32, device=dev)
+        # top_p = 1 without top_k restricts nothing: such a row takes the plain walk over the whole
+        # vocabulary (the reference sorts it first, crates/denno-engine/src/sampler.rs:387-435, which
+        # gives the same distribution)
+        restricted = [r for r, p in enumerate(params)
+                      if not p.greedy and (p.top_k is not None or (p.top_p is not None and p.top_p < 1.0))]
+        n = len(restricted)
+        both = torch.empty(R + n, dtype=torch.int32, device=dev)       # tokens, then which listed rows are undecided
         if all(p.greedy for p in params):
             # nothing to bring to the device: a step of greedy rows costs no copy
             tu = self._zeros.get(R)
@@ -51,29 +63,49 @@ class Sampler:
                 tu = self._zeros[R] = torch.zeros((2, R), dtype=torch.float32, device=dev)
         else:
             temps = [0.0 if p.greedy else p.effective_temperature for p in params]
-            us = [0.0 if p.greedy else uniform(s, n) for p, s, n in zip(params, seeds, counters)]
+            us = [0.0 if p.greedy else uniform(s, n_) for p, s, n_ in zip(params, seeds, counters)]
             tu = torch.tensor([temps, us], dtype=torch.float32, device=dev)      # one copy for both
         t_dev, u_dev = tu[0], tu[1]
-        # top_p = 1 without top_k restricts nothing: such a row takes the plain walk over the whole
-        # vocabulary (the reference sorts it first, crates/denno-engine/src/sampler.rs:387-435, which
-        # gives the same distribution)
-        restricted = [r for r, p in enumerate(params)
-                      if not p.greedy and (p.top_k is not None or (p.top_p is not None and p.top_p < 1.0))]
-        ops.sample(logits, t_dev, u_dev, out)
+        ops.sample(logits, t_dev, u_dev, both[:R])
         if not restricted:
-            return out.tolist()
-        n = len(restricted)
+            return Pending(both, R, None)
         top_p = [params[r].top_p if params[r].top_p is not None else 1.0 for r in restricted]
         ints = torch.tensor([restricted, [params[r].top_k or 0 for r in restricted]], dtype=torch.int32, device=dev)
         ps = torch.tensor(top_p, dtype=torch.float32, device=dev)
-        both = torch.empty(R + n, dtype=torch.int32, device=dev)       # tokens, then which listed rows are undecided
-        both[:R].copy_(out)
         ops.sample_top(logits, ints[0], t_dev, u_dev, ints[1], ps, both[:R], both[R:])
-        host = both.tolist()
-        tokens, undecided = host[:R], [j for j in range(n) if host[R + j]]
+        return Pending(both, R, (logits, restricted, top_p, t_dev, u_dev))
+
+    def read(self, pending: "Pending") -> List[int]:
+        """Waits for a launched sampling; -> the rows' tokens."""
+        if pending.rows == 0:
+            return []
+        R = pending.rows
+        host = pending.both.tolist()
+        tokens = host[:R]
+        if pending.more is None:
+            return tokens
+        logits, restricted, top_p, t_dev, u_dev = pending.more
+        undecided = [j for j in range(len(restricted)) if host[R + j]]
         if undecided:
             # top-p alone whose cut lies beyond the 2,048 largest: the whole vocabulary, sorted
+            dev = self.device
             rows = torch.tensor([restricted[j] for j in undecided], dtype=torch.int32, device=dev)
             ps = torch.tensor([top_p[j] for j in undecided], dtype=torch.float32, device=dev)
-            tokens = ops.sample_full(logits, rows, t_dev, u_dev, ps, both[:R]).tolist()
+            tokens = ops.sample_full(logits, rows, t_dev, u_dev, ps, pending.both[:R]).tolist()
         return tokens
+
+
+class Pending:
+    """A launched sampling: `both[:rows]` are the tokens on the device.  final: no row can still change
+    (rows with top-k or top-p may, when `read` finds their cut beyond the candidates)."""
+
+    def __init__(self, both, rows, more):
+        self.both, self.rows, self.more = both, rows, more
+
+    @property
+    def tokens(self):
+        return self.both[:self.rows]
+
+    @property
+    def final(self):
+        return self.more is None

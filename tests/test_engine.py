@@ -207,7 +207,8 @@ def test_the_slot_record_holds_position_and_generator(backend, model_folders):
     zero for the next request that gets the slot, and carries a preempted request's generator on."""
     from denno_beta_amd.engine import SamplingParams
     from denno_beta_amd.sampling import uniform
-    e = engine_for(model_folders("A", "float32"), "float32", backend, cache_tokens=256, max_live=1)
+    e = engine_for(model_folders("A", "float32"), "float32", backend, cache_tokens=256, max_live=1,
+                   run_ahead=False)      # (step by step: nothing is launched before the last step's tokens are read)
     m = e.runner.cache.manager
     prompt = seeded_tokens(3, 11, 512)
     rid = e.add_request(prompt, SamplingParams(max_tokens=3, temperature=0.7, seed=99))
@@ -225,6 +226,45 @@ def test_the_slot_record_holds_position_and_generator(backend, model_folders):
     st = m.state(other)
     assert m.slot(other) == 0 and (st.num_computed, st.rng_seed, st.rng_drawn) == (4, 5, 1)
     assert uniform(99, 0) != uniform(99, 1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_running_ahead_changes_no_token(model_folders, tmp_path, dtype):
+    """In steady decoding the next step is launched before the host has read this step's tokens, which it takes
+    from the device.  Greedy and seeded temperature sampling, requests of different lengths that end by length
+    and by an end-of-sequence token, so few pages that requests are put back, more requests than may live at
+    once: every token is what the engine gives without running ahead."""
+    from denno_beta_amd.engine import SamplingParams
+    from denno_beta_amd.weights import write_model_folder
+    cfg, seed = TINY["B"]
+    prompts = [seeded_tokens(80 + i, n, 1000) for i, n in enumerate((5, 40, 9, 75, 21, 33, 2))]
+    greedy = [SamplingParams(max_tokens=m, temperature=0.0) for m in (30, 7, 45, 12, 1, 60, 25)]
+    # an end-of-sequence token that greedy decoding does meet: what request 0 generates tenth
+    first = engine_for(model_folders("B", dtype), dtype, "cuda:0", run_ahead=False).generate(prompts[:1], greedy[:1])[0]
+    folder = write_model_folder(str(tmp_path / "eos"), dict(cfg, eos_token_id=first[9]), seed, dtype)
+    warm = [SamplingParams(max_tokens=m, temperature=0.9, seed=5 + i) for i, m in enumerate((30, 7, 45, 12, 1, 60, 25))]
+    for params in (greedy, warm):
+        for kw in (dict(cache_tokens=1024, max_live=8), dict(cache_tokens=192, max_live=3)):
+            want_engine = engine_for(folder, dtype, "cuda:0", run_ahead=False, **kw)
+            want = want_engine.generate(prompts, params)
+            e = engine_for(folder, dtype, "cuda:0", run_ahead=True, **kw)
+            got = e.generate(prompts, params)
+            assert got == want, (params is greedy, kw)
+            assert [e.finish_reason(i) for i in range(7)] == [want_engine.finish_reason(i) for i in range(7)]
+            assert sum(r.ran_ahead for r in e.records) > 10 and not any(r.ran_ahead for r in want_engine.records)
+            m = e.runner.cache.manager
+            assert m.live() == 0 and not e.has_unfinished()
+            m.check()
+    assert "eos" in [e.finish_reason(i) for i in range(7)]
+    # one request alone, step by step: every step but the first of its decoding runs ahead
+    e = engine_for(folder, dtype, "cuda:0", run_ahead=True)
+    rid = e.add_request(prompts[3], SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True))
+    outs = []
+    while e.has_unfinished():
+        outs += [o.token for o in e.step() if o.token is not None]
+    assert outs == e.requests[rid].generated and len(outs) == 12
+    assert [r.ran_ahead for r in e.records] == [False] + [True] * 11
 
 
 @pytest.mark.gpu

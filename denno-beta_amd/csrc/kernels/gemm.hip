@@ -659,8 +659,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
 // (wave w: steps 2w, 2w + 1, then 2 (w + WAVES), ...), so that a row's share of a pair is one cache
 // line of 128 bytes; it loads A eight lanes to a row, turns each pair round through a piece of LDS
 // of its own (no barrier: a wave's LDS operations keep their order) and reads the operands from
-// there.  16 columns per workgroup, sums joined through LDS in wave order, as in gemm_kernel.
-template <int WAVES, typename TC, bool KV, int NORM = NORM_NONE>
+// there, two pairs at a time through two such pieces, so that the way into LDS and out of it is
+// waited for once per two pairs.  16 columns per workgroup, sums joined through LDS in wave order, as in gemm_kernel.
+template <int WAVES, typename TC, bool KV, int NORM, bool TWO>
 __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __restrict__ A, int lda,
                                                              const bf16_t* __restrict__ W,
                                                              const float* __restrict__ bias, TC* __restrict__ C,
@@ -670,13 +671,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
   constexpr int U = 4;                                     // pairs of steps in flight per wave
   constexpr int ROW = 9 * 8;                               // elements per row of a wave's piece: 8 chunks and one of padding
   __shared__ floatx4 red[WAVES][64];
-  __shared__ __attribute__((aligned(16))) bf16_t turn[WAVES][16 * ROW];
+  constexpr int PIECES = 2;                                // pairs turned round at a time
+  static_assert(U % PIECES == 0, "pairs in flight come in whole groups");
+  __shared__ __attribute__((aligned(16))) bf16_t turn[WAVES][PIECES][16 * ROW];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int col = lane % 16, g = lane / 16;
   const int n0 = blockIdx.x * 16;
   const int ksteps = (K + 31) / 32, npairs = (ksteps + 1) / 2, nblocks = (N + 15) / 16;
   const bf16_t* wblk = W + (static_cast<size_t>(min(static_cast<int>(blockIdx.x), nblocks - 1)) * ksteps * 64 + lane) * 8;
-  const bool two = M > 8;                                  // rows 8 .. 15 need a second load per pair
+  // (TWO: rows 8 .. 15 need a second load per pair)
   // NORM_IN: the rows' pairs of statistics are asked for before the operands (loads come back in the
   // order asked): wave w joins rows w, w + WAVES, ...; a lane holds up to SP pairs of a row
   constexpr int SP = 4, SR = 16 / WAVES;
@@ -715,7 +718,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
   const int lrow = lane / 8, lch = lane % 8;               // as loader: row and 16-byte chunk of the pair's 128 bytes
   const bf16_t* a0 = A + static_cast<size_t>(min(lrow, M - 1)) * lda + lch * 8;
   const bf16_t* a1 = A + static_cast<size_t>(min(lrow + 8, M - 1)) * lda + lch * 8;
-  bf16_t* mine = turn[wave];
+  bf16_t* mine = turn[wave][0];
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
   floatx4 acc = {0.f, 0.f, 0.f, 0.f};
   // a round: U pairs of steps per wave, all its loads issued at once (asking for the next round
@@ -732,21 +735,33 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
       const int p = p0 + u * WAVES;
       const bool ok = p * 64 + lch * 8 < K;
       al[u][0] = *reinterpret_cast<const u32x4*>(ok ? a0 + p * 64 : a0);
-      al[u][1] = *reinterpret_cast<const u32x4*>(ok && two ? a1 + p * 64 : a0);
+      if constexpr (TWO) al[u][1] = *reinterpret_cast<const u32x4*>(ok ? a1 + p * 64 : a0);
     }
   };
   auto use = [&](int p0, const bf16x8 (*b)[2], const u32x4 (*al)[2]) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int p = p0 + u * WAVES;
-      const bool ok = p < npairs && p * 64 + lch * 8 < K;
-      *reinterpret_cast<u32x4*>(mine + lrow * ROW + lch * 8) = ok ? al[u][0] : zero4;
-      if (two) *reinterpret_cast<u32x4*>(mine + (lrow + 8) * ROW + lch * 8) = ok ? al[u][1] : zero4;
-      // as operand: lane (row col, chunk g) of each of the pair's two steps
-      const bf16x8 f0 = *reinterpret_cast<const bf16x8*>(mine + col * ROW + g * 8);
-      const bf16x8 f1 = *reinterpret_cast<const bf16x8*>(mine + col * ROW + (4 + g) * 8);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, b[u][0], acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1, b[u][1], acc, 0, 0, 0);
+    for (int u0 = 0; u0 < U; u0 += PIECES) {
+#pragma unroll
+      for (int i = 0; i < PIECES; ++i) {
+        const int p = p0 + (u0 + i) * WAVES;
+        const bool ok = p < npairs && p * 64 + lch * 8 < K;
+        bf16_t* piece = mine + i * 16 * ROW;
+        *reinterpret_cast<u32x4*>(piece + lrow * ROW + lch * 8) = ok ? al[u0 + i][0] : zero4;
+        if constexpr (TWO) *reinterpret_cast<u32x4*>(piece + (lrow + 8) * ROW + lch * 8) = ok ? al[u0 + i][1] : zero4;
+      }
+      // as operand: lane (row col, chunk g) of each of a pair's two steps
+      bf16x8 f[PIECES][2];
+#pragma unroll
+      for (int i = 0; i < PIECES; ++i) {
+        const bf16_t* piece = mine + i * 16 * ROW;
+        f[i][0] = *reinterpret_cast<const bf16x8*>(piece + col * ROW + g * 8);
+        f[i][1] = *reinterpret_cast<const bf16x8*>(piece + col * ROW + (4 + g) * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < PIECES; ++i) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[i][0], b[u0 + i][0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[i][1], b[u0 + i][1], acc, 0, 0, 0);
+      }
     }
   };
   bf16x8 b0[U][2];
@@ -883,9 +898,14 @@ static void launch(const Call& c, hipStream_t stream) {
 template <int WAVES, typename TC, bool KV>
 static void launch16_one(const Call& c, hipStream_t stream) {
   KVScatter kv = c.kv ? *c.kv : KVScatter{};
-  hipLaunchKernelGGL((gemm16_kernel<WAVES, TC, KV>), dim3((c.N + 15) / 16), dim3(WAVES * 64), 0, stream,
-                     static_cast<const bf16_t*>(c.A), c.lda, static_cast<const bf16_t*>(c.W), c.bias,
-                     static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N, c.K, c.epi, kv, NormIO{});
+  if (c.M > 8)
+    hipLaunchKernelGGL((gemm16_kernel<WAVES, TC, KV, NORM_NONE, true>), dim3((c.N + 15) / 16), dim3(WAVES * 64), 0, stream,
+                       static_cast<const bf16_t*>(c.A), c.lda, static_cast<const bf16_t*>(c.W), c.bias,
+                       static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N, c.K, c.epi, kv, NormIO{});
+  else
+    hipLaunchKernelGGL((gemm16_kernel<WAVES, TC, KV, NORM_NONE, false>), dim3((c.N + 15) / 16), dim3(WAVES * 64), 0, stream,
+                       static_cast<const bf16_t*>(c.A), c.lda, static_cast<const bf16_t*>(c.W), c.bias,
+                       static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr, c.M, c.N, c.K, c.epi, kv, NormIO{});
 }
 
 // the same with the norm before the product (NORM_IN: bfloat16 out) or after it (NORM_OUT: into the residual stream)
@@ -893,10 +913,17 @@ template <int WAVES>
 static void launch16_norm(const Call& c, const NormIO& nio, int norm, hipStream_t stream) {
   KVScatter kv = c.kv ? *c.kv : KVScatter{};
   const dim3 grid((c.N + 15) / 16), block(WAVES * 64);
-#define DN_L16(TC, KV, NORM)                                                                                        \
-  hipLaunchKernelGGL((gemm16_kernel<WAVES, TC, KV, NORM>), grid, block, 0, stream, static_cast<const bf16_t*>(c.A), \
-                     c.lda, static_cast<const bf16_t*>(c.W), c.bias, static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr,  \
+#define DN_L16_ROWS(TC, KV, NORM, TWO)                                                                                   \
+  hipLaunchKernelGGL((gemm16_kernel<WAVES, TC, KV, NORM, TWO>), grid, block, 0, stream, static_cast<const bf16_t*>(c.A), \
+                     c.lda, static_cast<const bf16_t*>(c.W), c.bias, static_cast<TC*>(c.C), c.ldc, c.resid, c.ldr,       \
                      c.M, c.N, c.K, c.epi, kv, nio)
+#define DN_L16(TC, KV, NORM)                 \
+  do {                                       \
+    if (c.M > 8)                             \
+      DN_L16_ROWS(TC, KV, NORM, true);       \
+    else                                     \
+      DN_L16_ROWS(TC, KV, NORM, false);      \
+  } while (0)
   if (norm == NORM_OUT)
     DN_L16(float, false, NORM_OUT);
   else if (c.kv)
@@ -904,6 +931,7 @@ static void launch16_norm(const Call& c, const NormIO& nio, int norm, hipStream_
   else
     DN_L16(bf16_t, false, NORM_IN);
 #undef DN_L16
+#undef DN_L16_ROWS
 }
 
 template <int WAVES>

@@ -618,8 +618,10 @@ def test_attention_window_edges_in_every_kernel(H, dh, window, n):
                 assert (out[0].float() - want[p]).abs().max().item() < 0.2 / window, ("single row", p)
 
 
-def test_attention_rows_do_not_depend_on_the_batch():
-    H, dh, ps = 4, 32, 16
+@pytest.mark.parametrize("dh,ps", [(32, 16), (64, 16), (64, 4), (64, 6), (64, 64)])
+def test_attention_rows_do_not_depend_on_the_batch(dh, ps):
+    # (heads of 64 on pages of a multiple of 4 keys have a kernel of their own for steps of single rows)
+    H = 4
     q, k, v, bt, tiles, T = paged_case([200, 90], [50, 90], H, H, dh, ps, torch.float32, seed=2)
     out = torch.zeros(T, H * dh, device=DEV)
     ops().attention(q[:, :H * dh], out, k, v, bt, tiles, H, 0.2)
@@ -628,7 +630,7 @@ def test_attention_rows_do_not_depend_on_the_batch():
     one = torch.zeros(1, H * dh, device=DEV)
     ops().attention(q[49:50, :H * dh], one, k, v, bt, i32([[0], [0], [1], [199]]), H, 0.2)
     assert torch.equal(one[0], out[49])
-    for max_context in (200, 208):
+    for max_context in (200, min(264, bt.shape[1] * ps)):
         one = torch.zeros(1, H * dh, device=DEV)
         ops().attention(q[49:50, :H * dh], one, k, v, bt, i32([[0], [0], [1], [199]]), H, 0.2, single_rows=True,
                         max_context=max_context)

@@ -1328,7 +1328,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
                                                            const bf16_t* __restrict__ W, const float* __restrict__ bias,
                                                            TC* __restrict__ C, int ldc, float* __restrict__ resid, int ldr,
                                                            int M, int N, int K, int epi, int packed, int tiles_m,
-                                                           int tiles_n, KVScatter kv) {
+                                                           int tiles_n, KVScatter kv, float* __restrict__ part,
+                                                           int split_slabs) {
   constexpr int NW = WM * WN;
   constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
   constexpr int AB = BM / 16, WB = BN / 16;              // 1 KB blocks per slab
@@ -1344,7 +1345,11 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
   const int lane = threadIdx.x % 64;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
   const int wmb = (wave / WN) * TM, wnb = (wave % WN) * TN;     // in blocks
-  const int ksteps = K / 32, nblocks = (N + 15) / 16;
+  // part: K is shared out among the workgroups of blockIdx.y, split_slabs slabs each; a workgroup leaves
+  // its sums in part[blockIdx.y][m][n] and a second kernel adds them in order and ends with the epilogue
+  const int kall = K / 32, nblocks = (N + 15) / 16;
+  const int first = part ? blockIdx.y * split_slabs : 0;
+  const int ksteps = part ? min(split_slabs, kall - first) : kall;
   // where the 16 bytes of row lane % 16, columns 8 (lane / 16) .. of a block of A lie in its 1 KB
   // (see the loads below): any 8 and any 16 consecutive lanes read all banks once
   // (a packed A is in the operand's order already: lane l reads at 16 l)
@@ -1368,16 +1373,17 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
       // four cache lines, where a lane per row would touch sixteen
       const int g = lane / 16, h = (lane % 16) / 4, piece = (lane % 4) ^ g;
       if (packed & PACKED_A) {      // a block of packed rows is 1 KB as it lies, like a block of W
-        src[u] = A + static_cast<size_t>(min(m0 / 16 + b, (M + 15) / 16 - 1)) * ksteps * 512 + lane * 8;
+        src[u] = A + static_cast<size_t>(min(m0 / 16 + b, (M + 15) / 16 - 1)) * kall * 512 + lane * 8;
         step[u] = 512;
       } else {
         src[u] = A + static_cast<size_t>(min(m0 + b * 16 + 4 * h + g, M - 1)) * lda + piece * 8;
         step[u] = 32;
       }
     } else {
-      src[u] = W + static_cast<size_t>(min(n0 / 16 + b - AB, nblocks - 1)) * ksteps * 512 + lane * 8;
+      src[u] = W + static_cast<size_t>(min(n0 / 16 + b - AB, nblocks - 1)) * kall * 512 + lane * 8;
       step[u] = 512;
     }
+    src[u] += static_cast<size_t>(first) * step[u];
   }
   auto issue = [&](int kt) {
     u32x4* slab = lds + (kt % STAGES) * SLAB;
@@ -1438,6 +1444,19 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
       vpage[i] = run ? sq[0] / kv.page_size : -1;
       voff[i] = run ? sq[0] % kv.page_size : 0;
     }
+  }
+  if (part) {
+#pragma clang loop unroll(full)
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + (wnb + j) * 16 + (lane / 16) * 4;
+      if (n >= N) continue;
+#pragma clang loop unroll(full)
+      for (int i = 0; i < TM; ++i) {
+        const int m = m0 + (wmb + i) * 16 + lane % 16;
+        if (m < M) *reinterpret_cast<floatx4*>(part + (static_cast<size_t>(blockIdx.y) * M + m) * N + n) = acc[i][j];
+      }
+    }
+    return;
   }
   // every load of the epilogue before its first store: a wait for a load is a wait for the stores
   // issued before it as well (one counter), and a load per column block made the blocks take turns
@@ -1530,6 +1549,7 @@ static bool takes(const void* A, int lda, const void* W, const float* bias, cons
 struct Args {
   const void* A; int lda; const void* W; const float* bias; void* C; int ldc; float* resid; int ldr;
   int M, N, K, out_dtype, epi, packed; const KVScatter* kv;
+  float* part = nullptr; int splits = 1;       // part: K in `splits` shares, their sums in part[share][m][n]
 };
 
 template <typename TC, int WM, int WN, int TM, int TN, int STAGES, bool KV>
@@ -1544,10 +1564,11 @@ static int launch(const Args& a, hipStream_t stream) {
     if (e != hipSuccess) return static_cast<int>(e);
     raised = true;
   }
-  hipLaunchKernelGGL((gemm_kernel<TC, WM, WN, TM, TN, STAGES, KV>), dim3(tiles_m * tiles_n), dim3(WM * WN * 64), lds,
-                     stream, static_cast<const bf16_t*>(a.A), a.lda, static_cast<const bf16_t*>(a.W), a.bias,
-                     static_cast<TC*>(a.C), a.ldc, a.resid, a.ldr, a.M, a.N, a.K, a.epi, a.packed, tiles_m, tiles_n,
-                     a.kv ? *a.kv : KVScatter{});
+  const int split_slabs = (a.K / 32 + a.splits - 1) / a.splits;
+  hipLaunchKernelGGL((gemm_kernel<TC, WM, WN, TM, TN, STAGES, KV>), dim3(tiles_m * tiles_n, a.part ? a.splits : 1),
+                     dim3(WM * WN * 64), lds, stream, static_cast<const bf16_t*>(a.A), a.lda,
+                     static_cast<const bf16_t*>(a.W), a.bias, static_cast<TC*>(a.C), a.ldc, a.resid, a.ldr, a.M, a.N, a.K,
+                     a.epi, a.packed, tiles_m, tiles_n, a.kv ? *a.kv : KVScatter{}, a.part, split_slabs);
   return 0;
 }
 
@@ -1587,15 +1608,25 @@ static int pick(int M, int N, int K) {
 }
 
 // Up to 256 rows the few-rows kernel takes the product too (both read and write packed rows).
-// This one is the faster from 129 rows on where the product has 4,096 columns or more; with fewer
-// columns its 64-row tiles leave most CUs idle and the few-rows kernel stays ahead at every size.
+// This one is the faster from 105 rows on where the product has 4,096 columns or more; with fewer
+// columns its tiles leave most CUs idle and the few-rows kernel stays ahead, or level, at every size.
 static bool beats_few_rows(int M, int N, int K) {
   (void)K;
-  return M > 128 && N >= 4096;
+  return M > 104 && N >= 4096;
+}
+
+// A long K beside few columns and few rows: the tiles are few and each walks all of K, a slab at a time,
+// so K is shared out among several workgroups per tile (measured at 1,600 columns and K = 6,400: 42 us
+// whatever the rows up to 256, where a quarter of K takes 12).  The number of shares, 0 for none: 8 where
+// the tiles of 32 x 64 are at most 96, else 4 (65 rows: 26.2, 18.6, 17.5 us with 2, 4, 8 shares; 256 rows:
+// 27.8, 25.3, 26.1).
+static int shares_of_k(int M, int N, int K, int packed, bool kv) {
+  if (kv || (packed & PACKED_C) || M <= 64 || M > 512 || N >= 4096 || K < 4096) return 0;
+  return ((M + 31) / 32) * ((N + 63) / 64) <= 96 ? 8 : 4;
 }
 
 static int run(const Args& a, hipStream_t stream) {
-  switch (pick(a.M, a.N, a.K)) {
+  switch (pick(a.M, a.N, a.part ? a.K / a.splits : a.K)) {
     case 0: return launch_as<2, 2, 2, 4, 4>(a, stream);
     case 1: return launch_as<4, 2, 2, 4, 4>(a, stream);
     case 2: return launch_as<4, 2, 4, 4, 4>(a, stream);
@@ -1633,6 +1664,18 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
     if (in_dtype != DN_BF16) return DN_ERR_DTYPE;
     const bool few = skinny::takes(A, lda, W, M, K, packed);
     const bool many = direct::takes(A, lda, W, bias, C, ldc, resid, ldr, N, K, out_dtype, packed);
+    // (products that add into the residual stream only: the others keep one order of summation whether
+    // their result goes to rows or to packed rows)
+    const int shares = many && resid ? direct::shares_of_k(M, N, K, packed, false) : 0;
+    if (shares > 0 && work != nullptr && work_floats >= static_cast<long>(shares) * M * N) {
+      direct::Args a{A, lda, W, nullptr, nullptr, 0, nullptr, 0, M, N, K, DN_F32, EPI_NONE, packed & ~PACKED_C, nullptr};
+      a.part = work, a.splits = shares;
+      int rc = direct::run(a, stream);
+      if (rc != 0) return rc;
+      hipLaunchKernelGGL((plain::join_kernel<float>), dim3((N + 255) / 256, M), dim3(256), 0, stream, work, shares, bias,
+                         static_cast<float*>(nullptr), 0, resid, ldr, M, N, EPI_NONE);
+      return dn_launch_status();
+    }
     if (many && (!few || direct::beats_few_rows(M, N, K))) {
       int rc = direct::run(direct::Args{A, lda, W, bias, C, ldc, resid, ldr, M, N, K, out_dtype, epilogue, packed, nullptr}, stream);
       return rc != 0 ? rc : dn_launch_status();
@@ -1665,9 +1708,11 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
 }
 
 // floats of workspace that dn_gemm wants for these sizes (`work`; 0: none): the plain product of few rows
-// leaves the sums of K's segments there
+// leaves the sums of K's segments there, and the MFMA product of a long K beside few rows and columns that
+// adds into the residual stream the sums of K's shares (without the workspace it runs in the kernels that
+// need none; packed: the flags of a product that has a residual)
 extern "C" long dn_gemm_work_floats(int M, int N, int K, int packed) {
-  if (packed & PACKED_W) return 0;
+  if (packed & PACKED_W) return static_cast<long>(direct::shares_of_k(M, N, K, packed, false)) * M * N;
   return plain::work_floats(M, N, K);
 }
 

@@ -356,9 +356,12 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
         _dev(bias, "bias", (torch.float32,), 1)
         _need(bias.is_contiguous() and bias.shape[0] == N, "linear: bias")
     epi = EPILOGUES[epilogue]
+    if isinstance(out, PackedMatrix):
+        packed |= PACKED_C
     work, work_floats = None, 0
-    if not packed & PACKED_W and M <= 64:
-        # the plain product of few rows leaves the sums of K's segments in a workspace
+    if M <= 64 if not packed & PACKED_W else (64 < M <= 512 and residual is not None):
+        # products that share K out among workgroups leave the shares' sums in a workspace: the plain one
+        # of few rows, and the MFMA one of a long K beside few rows and columns that adds into the stream
         work_floats = _lib_quiet("gemm").dn_gemm_work_floats(M, N, K, packed)
         if work_floats:
             work = torch.empty(work_floats, dtype=torch.float32, device=a.device)
@@ -373,7 +376,7 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
     if isinstance(out, PackedMatrix):
         _need((packed & PACKED_W) and M <= PACKED_ROWS_MAX and N % 32 == 0 and out.device == a.device,
               f"linear: packed rows as out need a packed w, at most {PACKED_ROWS_MAX} rows and N a multiple of 32")
-        ldc, packed = 0, packed | PACKED_C
+        ldc = 0
     else:
         _dev(out, "out", _FLOATS, 2)
         ldc = _rows(out, "out")

@@ -376,6 +376,28 @@ def test_linear_with_packed_rows(M, N, K):
     assert torch.equal(o.layernorm(x, g, b, 1e-5, o.packed_rows(M, K, DEV), pick).rows(), rows.flip(0))
 
 
+@pytest.mark.parametrize("M", [65, 96, 100, 129, 256, 300, 512, 513])
+@pytest.mark.parametrize("N,K", [(1600, 6400), (1032, 4128), (96, 4096)])
+def test_linear_into_the_stream_with_a_long_inner_size(M, N, K):
+    """65 to 512 rows, fewer than 4,096 columns, K from 4,096 on, added into the residual stream: K is shared
+    out among workgroups and a second kernel adds the shares in order.  Against 64-bit sums; from rows and from
+    packed rows alike; the same bits on a second call."""
+    o = ops()
+    a, w, bias = rnd(M, K, seed=M, dtype=torch.bfloat16), rnd(N, K, seed=N, dtype=torch.bfloat16, scale=0.05), rnd(N, seed=3)
+    wp = o.pack_matrix(w)
+    x0 = rnd(M, N, seed=4)
+    want = (x0.double() + a.double() @ w.double().t() + bias.double()).float()
+    got = o.linear(a, wp, bias, residual=x0.clone())
+    assert torch.allclose(got, want, atol=2e-3, rtol=1e-4), (got - want).abs().max().item()
+    assert torch.equal(o.linear(a, wp, bias, residual=x0.clone()), got)
+    if M <= 256:
+        assert torch.equal(o.linear(o.pack_matrix(a), wp, bias, residual=x0.clone()), got)
+    # one request's rows do not depend on the rows beside them (other kernels below 65 rows: not the same bits)
+    if M >= 130:
+        part = o.linear(a[:M - 30].contiguous(), wp, bias, residual=x0[:M - 30].clone())
+        assert torch.allclose(part, got[:M - 30], atol=2e-3, rtol=1e-4)
+
+
 def test_packed_rows_are_refused_where_no_kernel_takes_them():
     o = ops()
     w = o.pack_matrix(rnd(64, 64, dtype=torch.bfloat16))

@@ -877,7 +877,7 @@ static void launch_norm(const Call& c, const NormIO& nio, int norm, hipStream_t 
 // 17 to 64 rows with a norm inside: the shapes that launch_mb picks for these rows (8 waves: K >= 1024)
 static void launch_mb_norm(const Call& c, const NormIO& nio, int norm, hipStream_t stream) {
   const int mb = (c.M + 15) / 16;
-  if (c.N >= 4096) {
+  if (c.N >= 2560) {
     switch (mb) {
       case 2: return launch_norm<2, 2, 8, 4>(c, nio, norm, stream);
       case 3: return launch_norm<3, 2, 8, 4>(c, nio, norm, stream);
@@ -943,8 +943,8 @@ static void launch16(const Call& c, hipStream_t stream) {
 
 // With more than 16 rows every workgroup reads all of A (16 cache lines per load and 16 lanes,
 // as A lies in rows), so wider workgroups read less in total, as long as enough of them remain
-// to keep the memory system busy: 2 column blocks per workgroup from 4,096 columns on, 4 from
-// 32,768 on, else 1.
+// to keep the memory system busy: 2 column blocks per workgroup from 2,560 columns on (3,072 columns at
+// 64 rows: 6.7 -> 5.6 us; 2,304 columns are slower that way), 4 from 32,768 on, else 1.
 template <int WAVES>
 static void launch_mb(const Call& c, hipStream_t stream) {
   const int mb = (c.M + 15) / 16;
@@ -966,7 +966,7 @@ static void launch_mb(const Call& c, hipStream_t stream) {
       default: return launch<4, 4, WAVES, 4>(c, stream);
     }
   }
-  if (c.N >= 4096) {
+  if (c.N >= 2560) {
     switch (mb) {
       case 2: return launch<2, 2, WAVES, 4>(c, stream);
       case 3: return launch<3, 2, WAVES, 4>(c, stream);
@@ -1608,11 +1608,12 @@ static int pick(int M, int N, int K) {
 }
 
 // Up to 256 rows the few-rows kernel takes the product too (both read and write packed rows).
-// This one is the faster from 105 rows on where the product has 4,096 columns or more; with fewer
-// columns its tiles leave most CUs idle and the few-rows kernel stays ahead, or level, at every size.
+// This one is the faster from 105 rows on where the product has 4,096 columns or more, and from 209 rows
+// on from 2,048 columns (2,304 columns at 224 rows: 8.3 against 10.6 us); with fewer columns its tiles
+// leave most CUs idle and the few-rows kernel stays ahead, or level, at every size.
 static bool beats_few_rows(int M, int N, int K) {
   (void)K;
-  return M > 104 && N >= 4096;
+  return (M > 104 && N >= 4096) || (M > 208 && N >= 2048);
 }
 
 // A long K beside few columns and few rows: the tiles are few and each walks all of K, a slab at a time,

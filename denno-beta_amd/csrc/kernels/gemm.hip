@@ -53,7 +53,26 @@ struct KVScatter {
   bf16_t* v_pool;
   int q_width, kv_width, dh, page_size, Hkv;
   int c_cols;     // columns of C that are stored: all of them, or q_width (nobody reads keys and values from C)
+  int page_shift; // log2(page_size) where that is a power of two, else -1 (kv_scatter_for sets it)
 };
+
+static int page_shift_of(int page_size) {
+  int s = 0;
+  while ((1 << s) < page_size) ++s;
+  return (1 << s) == page_size ? s : -1;
+}
+
+// a slot's page and offset: a shift and a mask where the page size allows it (a division by a number known
+// only at run time is some forty instructions, and the kernels' epilogues do two per token or per value)
+__device__ __forceinline__ void page_and_offset(const KVScatter& kv, int slot, int& page, int& off) {
+  if (kv.page_shift >= 0) {
+    page = slot >> kv.page_shift;
+    off = slot & (kv.page_size - 1);
+  } else {
+    page = slot / kv.page_size;
+    off = slot % kv.page_size;
+  }
+}
 
 
 // The same for four columns nn .. nn + 3 (nn a multiple of 4, so they are one head's): a key's
@@ -65,7 +84,8 @@ __device__ __forceinline__ void scatter_kv4(const KVScatter& kv, int m, int nn, 
   if (is_value) c -= kv.kv_width;
   const int slot = kv.slot_map[m];
   if (slot < 0) return;
-  const int page = slot / kv.page_size, off = slot % kv.page_size;
+  int page, off;
+  page_and_offset(kv, slot, page, off);
   const int hh = c / kv.dh, d = c % kv.dh;
   const size_t base = (static_cast<size_t>(page) * kv.Hkv + hh) * kv.page_size * kv.dh;
   if (is_value) {
@@ -84,7 +104,8 @@ __device__ __forceinline__ void scatter_kv_at(const KVScatter& kv, int slot, int
   const bool is_value = c >= kv.kv_width;
   if (is_value) c -= kv.kv_width;
   if (slot < 0) return;
-  const int page = slot / kv.page_size, off = slot % kv.page_size;
+  int page, off;
+  page_and_offset(kv, slot, page, off);
   const int hh = c / kv.dh, d = c % kv.dh;
   const size_t base = (static_cast<size_t>(page) * kv.Hkv + hh) * kv.page_size * kv.dh;
   if (is_value)
@@ -1157,14 +1178,16 @@ __global__ __launch_bounds__(WM * 128) __attribute__((amdgpu_waves_per_eu(2))) v
               const bool run = kv.page_size % 4 == 0 && slot[0] >= 0 && slot[0] % 4 == 0 && slot[1] == slot[0] + 1 && slot[2] == slot[0] + 2 &&
                                slot[3] == slot[0] + 3;
               if (run) {
-                const int page = slot[0] / kv.page_size, off = slot[0] % kv.page_size;
+                int page, off;
+                page_and_offset(kv, slot[0], page, off);
                 *reinterpret_cast<uint2*>(kv.v_pool + ((static_cast<size_t>(page) * kv.Hkv + hh) * kv.dh + d) * kv.page_size +
                                           off) = *reinterpret_cast<const uint2*>(cv);
               } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                   if (slot[e] < 0) continue;
-                  const int page = slot[e] / kv.page_size, off = slot[e] % kv.page_size;
+                  int page, off;
+                  page_and_offset(kv, slot[e], page, off);
                   kv.v_pool[((static_cast<size_t>(page) * kv.Hkv + hh) * kv.dh + d) * kv.page_size + off] = cv[e];
                 }
               }
@@ -1434,15 +1457,15 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
     for (int i = 0; i < TM; ++i) {
       const int m = m0 + (wmb + i) * 16 + lane % 16, mq = m - lane % 4;
       const int slot = m < M ? kv.slot_map[m] : -1;
-      kpage[i] = slot >= 0 ? slot / kv.page_size : -1;
-      koff[i] = slot >= 0 ? slot % kv.page_size : 0;
+      page_and_offset(kv, max(slot, 0), kpage[i], koff[i]);
+      if (slot < 0) kpage[i] = -1, koff[i] = 0;
       int sq[4];
 #pragma clang loop unroll(full)
       for (int e = 0; e < 4; ++e) sq[e] = mq + e < M ? kv.slot_map[mq + e] : -1;
       const bool run = kv.page_size % 4 == 0 && sq[0] >= 0 && sq[0] % 4 == 0 && sq[1] == sq[0] + 1 && sq[2] == sq[0] + 2 &&
                        sq[3] == sq[0] + 3;
-      vpage[i] = run ? sq[0] / kv.page_size : -1;
-      voff[i] = run ? sq[0] % kv.page_size : 0;
+      page_and_offset(kv, max(sq[0], 0), vpage[i], voff[i]);
+      if (!run) vpage[i] = -1, voff[i] = 0;
     }
   }
   if (part) {
@@ -1524,7 +1547,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
             for (int e = 0; e < 4; ++e) {
               const int slot = mq + e < M ? kv.slot_map[mq + e] : -1;
               if (slot < 0) continue;
-              const int page = slot / kv.page_size, off = slot % kv.page_size;
+              int page, off;
+              page_and_offset(kv, slot, page, off);
               kv.v_pool[((static_cast<size_t>(page) * kv.Hkv + hh) * kv.dh + d + q) * kv.page_size + off] =
                   from_float<bf16_t>(e == 0 ? t0 : e == 1 ? t1 : e == 2 ? t2 : t3);
             }
@@ -1764,7 +1788,7 @@ extern "C" int dn_gemm_norm_in(const void* A, int lda, const float* stats, const
       return DN_ERR_SHAPE;
     if ((c_cols != N && c_cols != q_width) || ldc < c_cols) return DN_ERR_SHAPE;
     kv = KVScatter{slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_width, Hkv * dh, dh,
-                   page_size, Hkv, c_cols};
+                   page_size, Hkv, c_cols, page_shift_of(page_size)};
   } else if (ldc == 0 ? (M <= 16 || N % 32 != 0) : ldc < N) {      // ldc == 0: C in packed rows (17 rows and more)
     return DN_ERR_SHAPE;
   }
@@ -1796,7 +1820,7 @@ extern "C" int dn_gemm_qkv(const void* A, int lda, const void* W, const float* b
   if (q_width < 0 || q_width + 2 * Hkv * dh != N || page_size < 1 || dh % 4 != 0) return DN_ERR_SHAPE;
   if ((c_cols != N && c_cols != q_width) || ldc < c_cols) return DN_ERR_SHAPE;
   KVScatter kv{slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_width, Hkv * dh, dh,
-               page_size, Hkv, c_cols};
+               page_size, Hkv, c_cols, page_shift_of(page_size)};
   if (many && (!few || direct::beats_few_rows(M, N, K))) {
     int rc = direct::run(direct::Args{A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, DN_BF16, EPI_NONE, packed, &kv}, stream);
     return rc != 0 ? rc : dn_launch_status();

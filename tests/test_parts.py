@@ -277,7 +277,7 @@ def toy_plain(spec, st, seq):
             x = x + a @ st[p + "o.w"].t()
         h = P.layer_norm(x, st[p + "n2.g"], 0.0, 1e-5)
         x = x + P.gelu_tanh(h @ st[p + "up.w"].t()) @ st[p + "down.w"].t()
-    return P.layer_norm(x, st["nf.g"], 0.0, 1e-5) @ st["tok"].t()
+    return P.layer_norm(x, st["nf.g"], 0.0, spec.final_norm[1]["eps"]) @ st["tok"].t()
 
 
 def test_a_toy_mixer_with_state_is_registered_built_and_stepped(backend):
@@ -404,7 +404,7 @@ def rotation_plain(spec, st, seq, positions=None):
         p = f"L{i}."
         a = ls.parts["mixer"][1]
         H, Hkv, dh = a["n_heads"], a["n_kv_heads"], a["head_dim"]
-        h = P.layer_norm(x, st[p + "n1.g"], 0.0, 1e-5)
+        h = P.layer_norm(x, st[p + "n1.g"], 0.0, ls.parts["norm1"][1]["eps"])
         qkv = h @ st[p + "qkv.w"].t()
         q, k, v = qkv[:, :H * dh].clone(), qkv[:, H * dh:(H + Hkv) * dh].clone(), qkv[:, (H + Hkv) * dh:]
         turn_pairs(q, pos, dh, ROTATION_BASES[i])
@@ -412,7 +412,7 @@ def rotation_plain(spec, st, seq, positions=None):
         # query head hd reads key head hd // (H / Hkv): spread keys and values out to H heads
         spread = lambda t: t.reshape(T, Hkv, 1, dh).expand(T, Hkv, H // Hkv, dh).reshape(T, H * dh)   # noqa: E731
         x = x + P.causal_attention(q, spread(k), spread(v), H, a["scale"]) @ st[p + "o.w"].t()
-        h = P.layer_norm(x, st[p + "n2.g"], 0.0, 1e-5)
+        h = P.layer_norm(x, st[p + "n2.g"], 0.0, ls.parts["norm2"][1]["eps"])
         f = ls.parts["ffn"][1]
         choice = first_max(h @ st[f["prefix"] + "router"].t())
         out = torch.zeros_like(x)
@@ -420,7 +420,7 @@ def rotation_plain(spec, st, seq, positions=None):
             e = int(choice[t])
             out[t] = P.gelu_tanh(h[t] @ st[f"{f['prefix']}e{e}.up"].t()) @ st[f"{f['prefix']}e{e}.down"].t()
         x = x + out
-    return P.layer_norm(x, st["nf.g"], 0.0, 1e-5) @ st["tok"].t()
+    return P.layer_norm(x, st["nf.g"], 0.0, spec.final_norm[1]["eps"]) @ st["tok"].t()
 
 
 def test_toy_rotation_and_toy_experts_are_registered_built_and_stepped(backend):
@@ -458,6 +458,118 @@ def test_toy_rotation_and_toy_experts_are_registered_built_and_stepped(backend):
         assert (rotation_plain(spec, st, seqs[0]) - want[0]).abs().max() > 0.05
     finally:
         ROTATION_BASES = kept
+
+
+# -- a whole toy architecture: its own config.json keys, registered here, written, loaded, served -----------
+def register_toy_architecture():
+    """`ToyTurnLM`: the toy rotation and the toy experts as an architecture of their own, with a configuration
+    class that reads its own keys from config.json.  Nothing of the framework's files changes."""
+    from dataclasses import asdict, dataclass
+    from denno_beta_amd.config import ConfigError, known_architectures, register_architecture
+    from denno_beta_amd.parts import DecoderSpec, LayerCall, LayerSpec
+    register_toy_rotation_and_experts()
+    if "ToyTurnLM" in known_architectures():
+        return
+
+    @dataclass(frozen=True)
+    class ToyTurnConfig:
+        toy_width: int
+        toy_heads: tuple          # per layer: (query heads, key heads)
+        toy_head_size: int
+        toy_inner: int
+        toy_experts: int
+        toy_vocab: int
+        toy_positions: int
+        toy_base: float
+        toy_last_base: float      # the last layer turns by a base of its own
+        toy_eps: float
+        toy_end: int              # the token that ends a request
+
+        @classmethod
+        def from_dict(cls, d):
+            missing = [k for k in cls.__dataclass_fields__ if k not in d]
+            if missing:
+                raise ConfigError(f"config.json of a ToyTurnLM lacks {missing}")
+            c = cls(**{k: d[k] for k in cls.__dataclass_fields__})
+            if c.toy_head_size % 16 != 0:
+                raise ConfigError(f"toy_head_size {c.toy_head_size}: heads come in steps of 16")
+            return cls(**{**asdict(c), "toy_heads": tuple(tuple(h) for h in c.toy_heads)})
+
+        def to_dict(self):
+            return {**asdict(self), "toy_heads": [list(h) for h in self.toy_heads]}
+
+    def build(cfg):
+        E, dh, layers = cfg.toy_width, cfg.toy_head_size, []
+        for i, (heads, kv_heads) in enumerate(cfg.toy_heads):
+            p = f"L{i}."
+            last = i == len(cfg.toy_heads) - 1
+            own = dict(position=("toy_rotation", dict(head_dim=dh, base=cfg.toy_last_base))) if last else {}
+            layers.append(LayerSpec("pre_norm", dict(
+                norm1=("layernorm", dict(width=E, eps=cfg.toy_eps, weight_name=p + "n1.g", bias_name=None)),
+                mixer=("causal_attention", dict(width=E, n_heads=heads, n_kv_heads=kv_heads, head_dim=dh, scale=dh ** -0.5,
+                                                qkv_weight=p + "qkv.w", qkv_bias=None, out_weight=p + "o.w", out_bias=None,
+                                                **own)),
+                norm2=("layernorm", dict(width=E, eps=cfg.toy_eps, weight_name=p + "n2.g", bias_name=None)),
+                ffn=("toy_experts", dict(width=E, inner=cfg.toy_inner, n_experts=cfg.toy_experts, prefix=p + "ffn.")))))
+        return DecoderSpec(vocab=cfg.toy_vocab, width=E, max_positions=cfg.toy_positions, token_table="tok",
+                           position=("toy_rotation", dict(head_dim=dh, base=cfg.toy_base)), layers=layers,
+                           run_order=[LayerCall(i, i) for i in range(len(layers))],
+                           final_norm=("layernorm", dict(width=E, eps=cfg.toy_eps, weight_name="nf.g", bias_name=None)),
+                           eos_token_ids=(cfg.toy_end,))
+
+    register_architecture(["ToyTurnLM", "toy_turn"], ToyTurnConfig, build)
+
+
+TOY_TURN = dict(architectures=["ToyTurnLM"], toy_width=48, toy_heads=[[3, 3], [3, 1]], toy_head_size=16, toy_inner=40,
+                toy_experts=2, toy_vocab=61, toy_positions=96, toy_base=30.0, toy_last_base=5.0, toy_eps=1e-6, toy_end=60)
+
+
+def test_a_whole_architecture_is_registered_written_loaded_and_served(backend, tmp_path):
+    """An architecture that the framework does not know: its configuration class, its builder and its parts are
+    defined in this file and registered by name; a model folder is written from a configuration and a seed,
+    read back through the registry by what its config.json says, and served by the engine (scheduler, portions,
+    sampling): every request's greedy tokens equal those of its run alone, and the logits of every way of cutting
+    the work agree with the plain functions of this file."""
+    from denno_beta_amd.config import ConfigError, load_config
+    from denno_beta_amd.engine import Engine, ModelRunner, SamplingParams
+    from denno_beta_amd.weights import write_model_folder
+    register_toy_architecture()
+    folder = write_model_folder(str(tmp_path / "toy"), TOY_TURN, seed=4, dtype="float32")
+    arch, cfg = load_config(folder)
+    assert arch.name == "ToyTurnLM" and cfg.toy_heads == ((3, 3), (3, 1)) and cfg.to_dict()["toy_inner"] == 40
+    with pytest.raises(ConfigError, match="toy_experts"):
+        arch.config_cls.from_dict({k: v for k, v in TOY_TURN.items() if k != "toy_experts"})
+    # the replay: whole, the tail token by token, portions, mixed with pages used again
+    r = ModelRunner.from_folder(folder, options(backend, cache_tokens=160))
+    seqs = [seeded_tokens(20 + i, n, 60) for i, n in enumerate((33, 9, 50, 21))]
+    # against the plain functions of this file (the toy parts multiply with the library, whose sums depend on
+    # the rows beside them: close, not equal)
+    from denno_beta_amd.weights.safetensors_io import SafetensorsFile
+    sf = SafetensorsFile(folder + "/model.safetensors")
+    st = {k: sf.tensor(k).float().clone() for k in sf.entries}
+    sf.close()
+    global ROTATION_BASES
+    kept, ROTATION_BASES = ROTATION_BASES, (30.0, 5.0)
+    try:
+        want = [rotation_plain(r.spec, st, s) for s in seqs]
+    finally:
+        ROTATION_BASES = kept
+    for kind, steps in (("whole", U.whole_trace(seqs)), ("tail", U.tail_decode_trace(seqs, 8)),
+                        ("portions", U.chunk_trace(seqs)), ("mixed", U.mixed_trace(seqs, seed=9))):
+        got = U.replay(r, steps)
+        for i in range(len(seqs)):
+            U.assert_close(got[f"r{i}"], want[i], "float32", f"the toy architecture, {kind}, request {i}")
+    r.cache.manager.check()
+    assert r.cache.manager.reuse_count(0) > 0
+    # served: six requests through the scheduler, portions of 16 tokens, three live at a time
+    def engine():
+        return Engine.from_folder(folder, options(backend, max_live=3, prefill_chunk=16, max_batch_tokens=40))
+    prompts = [seeded_tokens(40 + i, n, 60) for i, n in enumerate((5, 37, 18, 2, 44, 11))]
+    params = SamplingParams(temperature=0.0, max_tokens=12)
+    together = engine().generate(prompts, params)
+    for p, toks in zip(prompts, together):
+        assert engine().generate([p], params)[0] == toks
+        assert len(toks) == 12 or toks[-1] == 60
 
 
 # -- an arrangement with four norms, a head with a bias and a scale -------------------------------

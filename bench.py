@@ -97,28 +97,30 @@ class Workloads:
         return {"ms": t * 1e3, "tok_s": batch / t, "bytes": nbytes, "frac": nbytes / t / 1e9 / HBM_PEAK_GBS,
                 "mean_context": mean_ctx, "steps": steps}
 
-    def prefill(self, reps=3):
-        """-> {value, tokens, ms, frac}: two prompts of 1,024 tokens in one step, the median of `reps`."""
+    def prefill(self, reps=3, prompts=2):
+        """-> {value, tokens, ms, frac}: `prompts` prompts of 1,024 tokens in one step (two: the 2,048 tokens
+        of the contract), the median of `reps`."""
         from denno_beta_amd.engine import StepEntry
         runner, sync = self.runner, self.torch.cuda.synchronize
         times = []
         for i in range(reps + 1):
-            seqs = [self.prompt(1024), self.prompt(1024)]
-            for j in range(2):
+            seqs = [self.prompt(1024) for _ in range(prompts)]
+            for j in range(prompts):
                 runner.start_request(1000 + j)
             sync()
             t0 = time.perf_counter()
-            runner.step([StepEntry(1000 + j, seqs[j], [1023]) for j in range(2)])
+            runner.step([StepEntry(1000 + j, seqs[j], [1023]) for j in range(prompts)])
             sync()
             times.append(time.perf_counter() - t0)
-            for j in range(2):
+            for j in range(prompts):
                 runner.end_request(1000 + j)
         t = statistics.median(times[1:])
         cfg = self.cfg
         V, E = cfg["vocab_size"], cfg["n_embd"]
         mat = sum(w.numel() for w in _layer_matrices(runner))
-        flops = 2.0 * 2048 * mat + 2.0 * 2 * V * E + cfg["n_layer"] * 2 * (4.0 * E * 1024 * 1025 / 2)
-        return {"value": 2048 / t, "tokens": 2048, "ms": t * 1e3, "frac": flops / t / MFMA_PEAK[SHORT[self.dtype]]}
+        tokens = 1024 * prompts
+        flops = 2.0 * tokens * mat + 2.0 * prompts * V * E + cfg["n_layer"] * prompts * (4.0 * E * 1024 * 1025 / 2)
+        return {"value": tokens / t, "tokens": tokens, "ms": t * 1e3, "frac": flops / t / MFMA_PEAK[SHORT[self.dtype]]}
 
 
 def _layer_matrices(runner):
@@ -159,6 +161,7 @@ def main():
                     help="with --only decode or prefill: every launch between two HIP events (no graphs), and a "
                          "table of each kernel's share")
     ap.add_argument("--sequences", type=int, default=8, help="--only replay: how many of the eight sequences")
+    ap.add_argument("--prompts", type=int, default=2, help="--only prefill: prompts of 1,024 tokens in the one step")
     ap.add_argument("--only", choices=["decode", "prefill", "serving", "replay"], default=None,
                     help="run one workload and print a short line (decode, prefill: for profiling; serving: "
                          "BASELINE.json's configs[3], GPT-2 Large shape, 64 requests through the scheduler; replay: "
@@ -176,11 +179,11 @@ def main():
     if a.only in ("prefill", "decode"):
         from denno_beta_amd.kernels import ops
         if a.only == "prefill":
-            w.prefill(1)
+            w.prefill(1, a.prompts)
             if a.kernel_times:
                 ops.time_launches(True)
-            r = w.prefill(1 if a.kernel_times else 3)
-            print(json.dumps({"prefill_ms": r["ms"], "tokens": 2048, "frac": r["frac"]}))
+            r = w.prefill(1 if a.kernel_times else 3, a.prompts)
+            print(json.dumps({"prefill_ms": r["ms"], "tokens": r["tokens"], "tok_s": r["value"], "frac": r["frac"]}))
         else:
             if a.kernel_times:
                 w.decode(a.batch, 2, 2, blocks=1)

@@ -405,6 +405,18 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
 __device__ __forceinline__ __bf16 to_bf16(float f) { return static_cast<__bf16>(f); }
 
+// eight values rounded to bfloat16, two per conversion (v_cvt_pk_bf16_f32 takes a pair)
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float floatx2;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+__device__ __forceinline__ bf16x8 to_bf16x8(const float* v) {
+  typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+  u32x4 w;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{v[2 * i], v[2 * i + 1]}, bf16x2));
+  return __builtin_bit_cast(bf16x8, w);
+}
+
 // ---------------------------------------------------------------------------------------
 // flash: portions of prompts.  A workgroup takes up to 128 consecutive rows of one request
 // and one head.  It has GROUPS x 4 waves: wave w owns the 32 rows 32 (w % 4), and the groups
@@ -577,48 +589,48 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
     }
     if (any) {
       const bf16_t* Tb = tiles_lds + (buf * GROUPS + grp) * TPS * TSZ;
+      // (the first product of a tile starts from a constant zero: no registers to clear)
+      const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       floatx16 s[TPS];
 #pragma unroll
       for (int c = 0; c < TPS; ++c) {
+        if (!act[c]) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[c][i] = 0.f;
-        if (!act[c]) continue;
+          for (int i = 0; i < 16; ++i) s[c][i] = NEG_INF;
+          continue;
+        }
         const bf16_t* Kb = Tb + c * TSZ;
 #pragma unroll
         for (int cc = 0; cc < DH16; ++cc) {
           const bf16x8 kf = *reinterpret_cast<const bf16x8*>(Kb + qcol * KROW + (2 * cc + g) * 8);
-          s[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[cc], s[c], 0, 0, 0);
+          s[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[cc], cc == 0 ? zero16 : s[c], 0, 0, 0);
         }
       }
-      // s[c][i]: key kw + 8*(i/4) + 4*g + i%4, query = this lane's column.  Scores are kept times
-      // log2(e), so that each probability is one multiply-add and one v_exp_f32.  Only a tile that
-      // touches the causal edge (or the window's) of one of the wave's rows needs the mask; the
+      // s[c][i]: key kw + 8*(i/4) + 4*g + i%4, query = this lane's column.  The running maximum is kept
+      // times scale * log2(e) (the scale is positive: the largest score is the largest product), so that
+      // each probability is one multiply-add and one v_exp_f32 on the product as the MFMA left it.  Only a
+      // tile that touches the causal edge (or the window's) of one of the wave's rows needs the mask; the
       // others skip it, the same for the whole wave.
       float tmax = NEG_INF;
 #pragma unroll
       for (int c = 0; c < TPS; ++c) {
         const int kw = kw0 + 32 * c;
         const bool edge = kw + 31 > pos0 + wrow0 || (window > 0 && kw < hi_w - window + 1);
-        if (!act[c]) {
-#pragma unroll
-          for (int i = 0; i < 16; ++i) s[c][i] = NEG_INF;
-        } else if (edge) {
+        if (!act[c]) continue;
+        if (edge) {
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
             int key = kw + 8 * (i / 4) + 4 * g + (i % 4);
             bool ok = key >= my_lo && key <= my_pos;
-            s[c][i] = ok ? s[c][i] * scale2 : NEG_INF;
+            s[c][i] = ok ? s[c][i] : NEG_INF;
             tmax = fmaxf(tmax, s[c][i]);
           }
         } else {
 #pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            s[c][i] *= scale2;
-            tmax = fmaxf(tmax, s[c][i]);
-          }
+          for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s[c][i]);
         }
       }
-      tmax = fmaxf(tmax, other_half(tmax));
+      tmax = fmaxf(tmax, other_half(tmax)) * scale2;      // (-inf stays -inf)
       float p[TPS][16];
       float psum = 0.f, alpha = 1.f;
       if (tmax > NEG_INF) {
@@ -628,7 +640,7 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
         for (int c = 0; c < TPS; ++c)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-            p[c][i] = __builtin_amdgcn_exp2f(s[c][i] - m_new);  // a masked score is -inf: 0
+            p[c][i] = __builtin_amdgcn_exp2f(fmaf(s[c][i], scale2, -m_new));  // a masked score is -inf: 0
             psum += p[c][i];
           }
         m = m_new;
@@ -644,9 +656,7 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
       for (int c = 0; c < TPS; ++c)
 #pragma unroll
-        for (int a0 = 0; a0 < 2; ++a0)
-#pragma unroll
-          for (int j = 0; j < 8; ++j) pb[c][a0][j] = to_bf16(p[c][8 * a0 + j]);
+        for (int a0 = 0; a0 < 2; ++a0) pb[c][a0] = to_bf16x8(&p[c][8 * a0]);
       // alpha belongs to the lane's query, and so do all of the lane's accumulators; once the running
       // maxima have settled it is 1 for the whole wave, tile after tile
       if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
@@ -727,7 +737,9 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
                                   int n_tiles, int H, int Hkv, int dh, int page_size, float scale, int window,
                                   hipStream_t stream) {
   if (n_tiles <= 0) return 0;
-  // ldo == 0: out is a packed matrix of H * dh columns (a multiple of 32)
+  // ldo == 0: out is a packed matrix of H * dh columns (a multiple of 32); the kernel takes the largest score
+  // for the largest product of a query and a key, so the scale is positive
+  if (!(scale > 0.f)) return DN_ERR_SHAPE;
   if (Hkv < 1 || H % Hkv != 0 || page_size % 16 != 0 || max_blocks < 1 || ldq % 8 != 0 || ldo % 4 != 0 || ldo < 0 ||
       (ldo == 0 && (H * dh) % 32 != 0) || reinterpret_cast<uintptr_t>(q) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(out) % 8 != 0)

@@ -472,7 +472,8 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
     _need(n_heads % Hkv == 0, f"attention: {n_heads} heads over {Hkv} key heads")
     ldq, ldo = _rows(q, "q"), (0 if out_packed else _rows(out, "out"))
     lib = _lib("attention")
-    fast = q.dtype == torch.bfloat16 and ps % 16 == 0 and ldq % 8 == 0 and q.data_ptr() % 16 == 0
+    # (the kernel for portions takes the largest score for the largest product: a scale that is not positive goes the plain way)
+    fast = q.dtype == torch.bfloat16 and ps % 16 == 0 and ldq % 8 == 0 and q.data_ptr() % 16 == 0 and scale > 0
     decode = fast and decode_attention_applies(q.dtype, ps, dh, single_rows, max_context)
     _need(not out_packed or (fast and attention_writes_packed(q.dtype, ps, dh, single_rows, max_context, tiles_wide)),
           "attention: packed rows as out are written by the bfloat16 kernels only")

@@ -444,15 +444,20 @@ namespace flash {
 constexpr int ROWS = 128;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
 
-template <int DH16, int GROUPS, int TPS>     // head size / 16; groups of 4 waves; tiles a wave takes per step
+// POW2: the page size is a power of two (page_size = 1 << page_shift), so that a key's page and its place in
+// the page are a shift and a mask: a tile's keys need four such pairs a step, and a division by a number
+// known only at run time is some twenty-five vector instructions.
+template <int DH16, int GROUPS, int TPS, bool POW2>     // head size / 16; groups of 4 waves; tiles a wave takes per step
 __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2))) void kernel(
     const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_row0,
     const int32_t* __restrict__ tile_nrows, const int32_t* __restrict__ tile_pos0, int H, int Hkv, int page_size,
-    float scale, int window) {
+    int page_shift, float scale, int window) {
   constexpr int DH = DH16 * 16;
   constexpr int DB = (DH + 31) / 32;
+  auto page_index = [&](int key) { return POW2 ? key >> page_shift : key / page_size; };
+  auto page_offset = [&](int key) { return POW2 ? key & (page_size - 1) : key % page_size; };
   constexpr int CH = DH / 8;                 // 16-byte chunks in a key
   constexpr int KROW = (CH + 1) * 8;         // a key's row in LDS, one chunk of padding: 16 rows, 16 bank groups
   constexpr int VROW = 40;                   // a dim's row of 32 keys in LDS, 16 bytes of padding
@@ -507,7 +512,7 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
   // kt .. kt+15, pg[1] for kt+16 .. kt+31; -1 beyond the rows' last key.
   struct Pages { int a, b; };
   auto pages_of = [&](int kt_) {
-    return Pages{kt_ <= hi_g ? bt[kt_ / page_size] : -1, kt_ + 16 <= hi_g ? bt[(kt_ + 16) / page_size] : -1};
+    return Pages{kt_ <= hi_g ? bt[page_index(kt_)] : -1, kt_ + 16 <= hi_g ? bt[page_index(kt_ + 16)] : -1};
   };
   // Thread t's share of its tile: chunk t (+ 256 u) of the keys, counted along a key's dims and
   // then from key to key, and of the values, counted along a dim's 16 keys of a page, then from
@@ -515,7 +520,7 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
   // pool's start and is stored as zeros.
   u32x4 kregs[TPS][KU], vregs[TPS][VU];
   auto fetch = [&](int kt_, const Pages pg, u32x4* kreg, u32x4* vreg) {
-    const int off0 = kt_ % page_size, off1 = (kt_ + 16) % page_size;
+    const int off0 = page_offset(kt_), off1 = page_offset(kt_ + 16);
 #pragma unroll
     for (int u = 0; u < KU; ++u) {
       const int idx = min(t + 256 * u, KCH - 1), key = idx / CH, ch = idx % CH;
@@ -751,16 +756,25 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
   if (n_tiles > 65535) return DN_ERR_SHAPE;      // the grid's second dimension
   dim3 grid(H, n_tiles);
   const bool two = static_cast<long>(n_tiles) * H <= 256;
-#define DN_FLASH_G(D, G, T)                                                                                        \
-  hipLaunchKernelGGL((flash::kernel<D, G, T>), grid, dim3(256 * G), 0, stream, static_cast<const bf16_t*>(q), ldq, \
-                     static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),                          \
-                     static_cast<const bf16_t*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0, tile_nrows, \
-                     tile_pos0, H, Hkv, page_size, scale, window)
-#define DN_FLASH(D, G)    \
-  if (G == 2 && two)      \
-    DN_FLASH_G(D, G, 1);  \
-  else                    \
-    DN_FLASH_G(D, 1, (D <= 6 ? 2 : 1))
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
+  const bool pow2 = (1 << page_shift) == page_size;
+#define DN_FLASH_P(D, G, T, P)                                                                                        \
+  hipLaunchKernelGGL((flash::kernel<D, G, T, P>), grid, dim3(256 * G), 0, stream, static_cast<const bf16_t*>(q), ldq, \
+                     static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),                             \
+                     static_cast<const bf16_t*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0, tile_nrows,   \
+                     tile_pos0, H, Hkv, page_size, page_shift, scale, window)
+#define DN_FLASH_G(D, G, T)    \
+  if (pow2)                    \
+    DN_FLASH_P(D, G, T, true); \
+  else                         \
+    DN_FLASH_P(D, G, T, false)
+#define DN_FLASH(D, G)                  \
+  if (G == 2 && two) {                  \
+    DN_FLASH_G(D, G, 1);                \
+  } else {                              \
+    DN_FLASH_G(D, 1, (D <= 6 ? 2 : 1)); \
+  }
   switch (dh) {
     case 16: DN_FLASH(1, 2); break;
     case 32: DN_FLASH(2, 2); break;
@@ -772,6 +786,7 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
   }
 #undef DN_FLASH
 #undef DN_FLASH_G
+#undef DN_FLASH_P
   return dn_launch_status();
 }
 

@@ -499,7 +499,8 @@ def test_attention(dtype, H, Hkv, dh, ps, window):
 
 @pytest.mark.parametrize("H,Hkv,dh,ps,window", [(4, 4, 16, 16, 0), (25, 25, 64, 16, 0), (6, 2, 48, 32, 0),
                                                 (2, 1, 128, 64, 0), (3, 3, 96, 16, 0), (4, 2, 32, 16, 20),
-                                                (5, 5, 64, 32, 7), (2, 2, 64, 16, 150)])
+                                                (5, 5, 64, 32, 7), (2, 2, 64, 16, 150), (4, 2, 64, 48, 0),
+                                                (3, 3, 32, 80, 30)])
 def test_attention_mfma_kernel_for_portions(H, Hkv, dh, ps, window):
     """The bfloat16 kernel for portions of prompts (tiles of up to 128 rows): a long portion deep
     in a context, a whole prompt, a short portion, single rows."""
@@ -521,7 +522,7 @@ def test_attention_mfma_kernel_for_portions(H, Hkv, dh, ps, window):
         assert T2 == 200 and torch.equal(packed.rows(), rows)
 
 
-@pytest.mark.parametrize("H,Hkv,dh,ps,window", [(8, 8, 64, 16, 0), (8, 2, 32, 32, 40)])
+@pytest.mark.parametrize("H,Hkv,dh,ps,window", [(8, 8, 64, 16, 0), (8, 2, 32, 32, 40), (8, 4, 64, 48, 0)])
 def test_attention_mfma_kernel_with_many_workgroups(H, Hkv, dh, ps, window):
     """More workgroups than CUs: the kernel then runs one group of waves per workgroup, not two."""
     g = torch.Generator().manual_seed(3)

@@ -805,7 +805,10 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
 // exchanges inside the loop.
 // ---------------------------------------------------------------------------------------
 namespace decode {
-template <int LPK, int WAVES>   // lanes per key = dh / 8; waves per workgroup
+// POW2: page_size = 1 << page_shift; a key's page and its place in the page are then a shift and a mask (a lane
+// works out a dozen such pairs per 64 keys before it can ask for the keys and values: as divisions by a number
+// known only at run time they were some six hundred instructions in front of the loads)
+template <int LPK, int WAVES, bool POW2>   // lanes per key = dh / 8; waves per workgroup
 __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out,
                                                        int ldo, const bf16_t* __restrict__ k_pool,
                                                        const bf16_t* __restrict__ v_pool,
@@ -814,8 +817,11 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
                                                        const int32_t* __restrict__ tile_row0,
                                                        const int32_t* __restrict__ tile_pos0,
                                                        float* __restrict__ part, int n_splits, int chunks, int H,
-                                                       int Hkv, int page_size, float scale, int window) {
+                                                       int Hkv, int page_size, int page_shift, float scale,
+                                                       int window) {
   constexpr int DH = LPK * 8;
+  auto page_index = [&](int key) { return POW2 ? key >> page_shift : key / page_size; };
+  auto page_offset = [&](int key) { return POW2 ? key & (page_size - 1) : key % page_size; };
   constexpr int KPI = 64 / LPK;          // keys per load instruction
   constexpr int DPL = (DH + 63) / 64;    // dims per lane in the second product
   constexpr int GROUP = LPK < 8 ? LPK : 8;   // load instructions issued together
@@ -864,9 +870,9 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
       const int kb = kbase + blk * 16;
       live[blk] = kb <= pos && kb + 16 > lo;
       const int kk = live[blk] ? kb : (pos / 16) * 16;
-      const int page = bt[kk / page_size];
+      const int page = bt[page_index(kk)];
       live[blk] = live[blk] && page >= 0;
-      const bf16_t* vb = v_pool + (static_cast<size_t>(max(page, 0)) * Hkv + hk) * DH * page_size + kk % page_size;
+      const bf16_t* vb = v_pool + (static_cast<size_t>(max(page, 0)) * Hkv + hk) * DH * page_size + page_offset(kk);
 #pragma unroll
       for (int i = 0; i < DPL; ++i) {
         const int d = min(lane + 64 * i, DH - 1);
@@ -884,9 +890,9 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
       for (int u = 0; u < GROUP; ++u) {
         const int key = kbase + (it0 + u) * KPI + grp;
         const int kk = (key >= lo && key <= pos) ? key : pos;     // a key that surely has a page
-        const int page = bt[kk / page_size];
+        const int page = bt[page_index(kk)];
         kv[u] = *reinterpret_cast<const bf16x8*>(
-            k_pool + ((static_cast<size_t>(page) * Hkv + hk) * page_size + kk % page_size) * DH + sub * 8);
+            k_pool + ((static_cast<size_t>(page) * Hkv + hk) * page_size + page_offset(kk)) * DH + sub * 8);
       }
 #pragma unroll
       for (int u = 0; u < GROUP; ++u) {
@@ -1004,11 +1010,21 @@ extern "C" int dn_attention_decode(const void* q, int ldq, void* out, int ldo, c
     return DN_ERR_SHAPE;
   if (waves != 4 && !(waves == 8 && dh <= 128) && !(waves == 16 && dh <= 64)) return DN_ERR_SHAPE;
   dim3 grid(n_splits, H, n_tiles), block(waves * 64);
-#define DN_DECODE_W(L, W)                                                                                          \
-  hipLaunchKernelGGL((decode::partial_kernel<L, W>), grid, block, 0, stream, static_cast<const bf16_t*>(q), ldq,   \
-                     static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),                           \
-                     static_cast<const bf16_t*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0, tile_pos0, \
-                     part, n_splits, chunks, H, Hkv, page_size, scale, window)
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
+  const bool pow2 = (1 << page_shift) == page_size;
+#define DN_DECODE_P(L, W, P)                                                                                          \
+  hipLaunchKernelGGL((decode::partial_kernel<L, W, P>), grid, block, 0, stream, static_cast<const bf16_t*>(q), ldq,   \
+                     static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),                              \
+                     static_cast<const bf16_t*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0, tile_pos0,    \
+                     part, n_splits, chunks, H, Hkv, page_size, page_shift, scale, window)
+#define DN_DECODE_W(L, W)    \
+  do {                       \
+    if (pow2)                \
+      DN_DECODE_P(L, W, true);  \
+    else                     \
+      DN_DECODE_P(L, W, false); \
+  } while (0)
 #define DN_DECODE(L)                  \
   if (waves == 16) {                  \
     if constexpr (L <= 8) DN_DECODE_W(L, 16); \
@@ -1026,6 +1042,7 @@ extern "C" int dn_attention_decode(const void* q, int ldq, void* out, int ldo, c
   }
 #undef DN_DECODE
 #undef DN_DECODE_W
+#undef DN_DECODE_P
   if (n_splits > 1)
     hipLaunchKernelGGL(decode::join_kernel, dim3(n_tiles, H), dim3(64), 0, stream, part, static_cast<bf16_t*>(out),
                        ldo, tile_seq, tile_row0, n_splits, H, dh);

@@ -539,7 +539,7 @@ def test_attention_mfma_kernel_with_many_workgroups(H, Hkv, dh, ps, window):
 
 @pytest.mark.parametrize("H,Hkv,dh,ps,window", [(4, 4, 16, 16, 0), (25, 25, 64, 16, 0), (6, 2, 32, 32, 0),
                                                 (2, 1, 128, 64, 0), (3, 3, 256, 16, 0), (5, 5, 64, 16, 100),
-                                                (2, 2, 64, 32, 300)])
+                                                (2, 2, 64, 32, 300), (4, 2, 64, 48, 0), (3, 3, 32, 80, 90)])
 def test_attention_split_kernel_for_decoding(H, Hkv, dh, ps, window):
     """The bfloat16 kernel for steps in which every request brings one row: contexts on both sides
     of a split's edge (256 keys) and of a page's."""

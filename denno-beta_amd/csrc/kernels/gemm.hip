@@ -1452,6 +1452,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
   // multiple of 4 are 8 bytes side by side for one dim: the four lanes of a quad, which hold four
   // tokens x four dims, exchange them (a 4 x 4 turn), and each stores four tokens of one dim.
   int kpage[KV ? TM : 1], koff[KV ? TM : 1], vpage[KV ? TM : 1], voff[KV ? TM : 1];
+  int vslot[KV ? TM : 1][4];      // the quad's four tokens' slots, for values that do not lie side by side (decoded tokens)
   if constexpr (KV) {
 #pragma clang loop unroll(full)
     for (int i = 0; i < TM; ++i) {
@@ -1466,6 +1467,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
                        sq[3] == sq[0] + 3;
       page_and_offset(kv, max(sq[0], 0), vpage[i], voff[i]);
       if (!run) vpage[i] = -1, voff[i] = 0;
+#pragma clang loop unroll(full)
+      for (int e = 0; e < 4; ++e) vslot[i][e] = sq[e];
     }
   }
   if (part) {
@@ -1545,7 +1548,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
           } else {
 #pragma clang loop unroll(full)
             for (int e = 0; e < 4; ++e) {
-              const int slot = mq + e < M ? kv.slot_map[mq + e] : -1;
+              const int slot = vslot[i][e];
               if (slot < 0) continue;
               int page, off;
               page_and_offset(kv, slot, page, off);

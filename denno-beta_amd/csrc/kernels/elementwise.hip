@@ -7,17 +7,55 @@
 // x[t,:] = wte[token_t,:] * token_scale + wpe[pos_t,:]   (crates/denno-engine/src/model/gpt2.rs:142-150,
 // where the scale is 1).  wpe may be null (an architecture whose positions enter elsewhere).
 // ---------------------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t words4;
+// element i of the 16 bytes w as a table of TW holds them
+template <typename TW>
+__device__ __forceinline__ float element(const words4& w, int i);
+template <>
+__device__ __forceinline__ float element<float>(const words4& w, int i) { return __uint_as_float(w[i]); }
+template <>
+__device__ __forceinline__ float element<bf16_t>(const words4& w, int i) {
+  return __uint_as_float(i % 2 == 0 ? w[i / 2] << 16 : w[i / 2] & 0xffff0000u);
+}
+
 template <typename TW>
 __global__ void embed_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ positions,
                              const TW* __restrict__ wte, const TW* __restrict__ wpe, float* __restrict__ x,
-                             int T, int E, int vocab, int n_pos, float token_scale) {
+                             int T, int E, int vocab, int n_pos, float token_scale, int wide) {
   int t = blockIdx.x;
   if (t >= T) return;
   int tok = tokens[t];
   int pos = positions[t];
   bool ok = tok >= 0 && tok < vocab && (wpe == nullptr || (pos >= 0 && pos < n_pos));
+  const float nan = __uint_as_float(0x7fc00000u);   // an id outside the table: NaN, never a neighbour's row
+  if (wide) {
+    // 16 bytes of each table per thread and step (E a multiple of that many elements, the tables aligned):
+    // a row of 1,600 is one step, all its loads on their way at once
+    constexpr int VEC = 16 / sizeof(TW);
+    for (int e = threadIdx.x * VEC; e < E; e += blockDim.x * VEC) {
+      float v[VEC];
+      if (ok) {
+        const words4 a = *reinterpret_cast<const words4*>(wte + static_cast<size_t>(tok) * E + e);
+        words4 b = {0u, 0u, 0u, 0u};
+        if (wpe != nullptr) b = *reinterpret_cast<const words4*>(wpe + static_cast<size_t>(pos) * E + e);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          v[i] = element<TW>(a, i);
+          if (token_scale != 1.0f) v[i] *= token_scale;
+          if (wpe != nullptr) v[i] += element<TW>(b, i);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = nan;
+      }
+      float* dst = x + static_cast<size_t>(t) * E + e;
+#pragma unroll
+      for (int i = 0; i < VEC; i += 4) *reinterpret_cast<float4*>(dst + i) = float4{v[i], v[i + 1], v[i + 2], v[i + 3]};
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < E; e += blockDim.x) {
-    float v = __uint_as_float(0x7fc00000u);   // an id outside the table: NaN, never a neighbour's row
+    float v = nan;
     if (ok) {
       v = to_float(wte[static_cast<size_t>(tok) * E + e]);
       if (token_scale != 1.0f) v *= token_scale;
@@ -32,14 +70,17 @@ extern "C" int dn_embed(const int32_t* tokens, const int32_t* positions, const v
                         hipStream_t stream) {
   if (T <= 0) return 0;
   dim3 grid(T), block(256);
+  const int vec = table_dtype == DN_F32 ? 4 : 8;
+  const int wide = E % vec == 0 && reinterpret_cast<uintptr_t>(wte) % 16 == 0 && reinterpret_cast<uintptr_t>(wpe) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(x) % 16 == 0;
   if (table_dtype == DN_F32)
     hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, tokens, positions,
                        static_cast<const float*>(wte), static_cast<const float*>(wpe), x, T, E, vocab, n_pos,
-                       token_scale);
+                       token_scale, wide);
   else if (table_dtype == DN_BF16)
     hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, tokens, positions,
                        static_cast<const bf16_t*>(wte), static_cast<const bf16_t*>(wpe), x, T, E, vocab, n_pos,
-                       token_scale);
+                       token_scale, wide);
   else
     return DN_ERR_DTYPE;
   return dn_launch_status();

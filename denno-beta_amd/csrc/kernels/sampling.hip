@@ -65,10 +65,15 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
   const float T = temperature[r];
 
   if (!(T > 0.f)) {
+    // (eight loads asked for at a time: one after the other they were most of the kernel's time)
     Best b{-INFINITY, 0x7fffffff};
-    for (int i = t; i < V; i += THREADS) {
-      float v = row[i];
-      if (v > b.v) b = Best{v, i};
+    for (int i0 = t; i0 < V; i0 += 8 * THREADS) {
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = row[min(i0 + j * THREADS, V - 1)];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (i0 + j * THREADS < V && v[j] > b.v) b = Best{v[j], i0 + j * THREADS};
     }
     b = block_best(b, best_scratch);
     if (t == 0) out[r] = b.i == 0x7fffffff ? 0 : b.i;
@@ -79,13 +84,26 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
   const int seg = (V + THREADS - 1) / THREADS;
   const int lo = min(V, t * seg), hi = min(V, lo + seg);
   float mx = -INFINITY;
-  for (int i = lo; i < hi; ++i) {
-    float z = row[i] / T;
-    if (z > mx) mx = z;
+  for (int i0 = lo; i0 < hi; i0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = row[min(i0 + j, V - 1)];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float z = v[j] / T;
+      if (i0 + j < hi && z > mx) mx = z;
+    }
   }
   mx = block_max(mx, f_scratch);
   float s = 0.f;
-  for (int i = lo; i < hi; ++i) s += expf(row[i] / T - mx);
+  for (int i0 = lo; i0 < hi; i0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = row[min(i0 + j, V - 1)];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (i0 + j < hi) s += expf(v[j] / T - mx);
+  }
   seg_sum[t] = s;
   __syncthreads();
   if (t == 0) {

@@ -14,8 +14,8 @@ in its download cache, main.rs:555-565; there is no network here).  Option names
 are the reference's: max-tokens 128, temperature unset = 1.0 and 0 = greedy, seed unset =
 entropy.  `--quant` names the precision: the reference's fp32 (default there) and this
 engine's bf16; its int8 and q4 modes are not built.  Beyond the reference: `--prompt-ids`
-for token ids where the folder has no tokenizer.json, `--top-k`, `--top-p` (the reference's
-request parameters, crates/denno-engine/src/engine.rs:42-43), `--ignore-eos`; `--prompt-file` with
+for token ids where the folder has no tokenizer.json, `--top-k`, `--top-p`, `--stop` (the reference's
+request parameters, crates/denno-engine/src/engine.rs:42-44), `--ignore-eos`; `--prompt-file` with
 one prompt a line (token ids separated by commas or blanks), which all go through the scheduler
 together, one line of output each in the file's order; and the engine's own options (`--max-live`,
 `--page-size`, `--cache-tokens`, `--prefill-chunk`, `--max-batch-tokens`, `--kv-policy`,
@@ -64,6 +64,8 @@ def parser():
     g.add_argument("--top-k", type=int, default=None)
     g.add_argument("--top-p", type=float, default=None)
     g.add_argument("--seed", type=int, default=None)
+    g.add_argument("--stop", action="append", default=None,
+                   help="a text that ends the generation where it first appears (needs tokenizer.json); may be given more than once")
     g.add_argument("--repetition-penalty", type=float, default=None)
     g.add_argument("--frequency-penalty", type=float, default=None)
     g.add_argument("--presence-penalty", type=float, default=None)
@@ -121,20 +123,24 @@ def cmd_generate(a):
         max_tokens=a.max_tokens, temperature=a.temperature, top_k=a.top_k, top_p=a.top_p, seed=a.seed,
         repetition_penalty=a.repetition_penalty, frequency_penalty=a.frequency_penalty,
         presence_penalty=a.presence_penalty, no_repeat_ngram_size=a.no_repeat_ngram_size,
-        ignore_eos=a.ignore_eos)
+        ignore_eos=a.ignore_eos, stop_sequences=tuple(a.stop or ()))
+    if a.stop and tok is None:
+        raise SystemExit(f"--stop is a text: {a.model} has no tokenizer.json (or the tokenizers package is missing)")
     max_live = a.max_live if a.max_live is not None else min(len(prompts), 64)
     eng = Engine.from_folder(a.model, EngineOptions(
         dtype=quant, max_live=max_live, seed=a.seed, page_size=a.page_size, cache_tokens=a.cache_tokens,
         prefill_chunk=a.prefill_chunk, max_batch_tokens=a.max_batch_tokens, kv_policy=a.kv_policy,
-        use_graphs=not a.no_graphs), a.cast_weights)
-    for out in eng.generate(prompts, params):
+        use_graphs=not a.no_graphs), a.cast_weights,
+        detokenize=(lambda ids: tok.decode(list(ids))) if tok is not None else None)
+    for rid, out in enumerate(eng.generate(prompts, params)):
         if a.raw or tok is None:
             # the raw path stops at the end-of-sequence token without keeping it (main.rs:708-710)
             eos = set(eng.spec.eos_token_ids)
             if out and out[-1] in eos and not a.ignore_eos:
                 out = out[:-1]
         if tok is not None and a.prompt is not None:
-            print(tok.decode(out))
+            text = eng.requests[rid].text      # cut at a stop sequence, where one ended it
+            print(text if text is not None else tok.decode(out))
         else:
             print(",".join(str(t) for t in out))
     return 0

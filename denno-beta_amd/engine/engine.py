@@ -31,7 +31,9 @@ class Request:
     max_new: int
     tokens: List[int] = field(default_factory=list)    # prompt + generated
     finished: bool = False
-    finish_reason: Optional[str] = None                 # "eos", "length", "error"
+    finish_reason: Optional[str] = None                 # "eos", "length", "stop_sequence", "error", "aborted"
+    text: Optional[str] = None                          # the generated text, where the engine has a detokenizer
+    stop_sequence: Optional[str] = None                 # the stop sequence that ended it
     preemptions: int = 0
     n_sampled: int = 0     # tokens sampled for it so far, the one that the host has not read yet among them
 
@@ -72,8 +74,10 @@ class _Launched:
 
 
 class Engine:
-    def __init__(self, runner: ModelRunner, options: Optional[EngineOptions] = None):
+    def __init__(self, runner: ModelRunner, options: Optional[EngineOptions] = None, detokenize=None):
+        """detokenize: token ids -> text, for requests with stop sequences (and for `Request.text`)."""
         self.runner = runner
+        self.detokenize = detokenize
         self.options = options or runner.options
         self.spec = runner.spec
         self.scheduler = Scheduler(
@@ -89,9 +93,10 @@ class Engine:
         self._failed_ahead: Optional[Exception] = None
 
     @classmethod
-    def from_folder(cls, model_dir: str, options: Optional[EngineOptions] = None, cast_matrices=False):
+    def from_folder(cls, model_dir: str, options: Optional[EngineOptions] = None, cast_matrices=False,
+                    detokenize=None):
         options = options or EngineOptions()
-        return cls(ModelRunner.from_folder(model_dir, options, cast_matrices), options)
+        return cls(ModelRunner.from_folder(model_dir, options, cast_matrices), options, detokenize)
 
     @classmethod
     def from_random(cls, config: dict, seed: int, options: Optional[EngineOptions] = None, stored=None):
@@ -103,6 +108,8 @@ class Engine:
         """Queues a request; raises on an empty prompt, a prompt that fills the context, a token
         outside the vocabulary, or a request that could never fit the cache."""
         params = (params or SamplingParams()).validate()
+        if any(params.stop_sequences) and self.detokenize is None:
+            raise ValueError("stop_sequences are texts: the engine needs a detokenizer for them (Engine(..., detokenize=))")
         prompt = [int(t) for t in prompt]
         for t in prompt:
             if not 0 <= t < self.spec.vocab:
@@ -264,6 +271,9 @@ class Engine:
                 if tok in eos and not req.params.ignore_eos:
                     req.finish_reason = "eos"
                     self._release(p.rid)
+                elif any(req.params.stop_sequences) and self._stops(req):
+                    req.finish_reason = "stop_sequence"
+                    self._release(p.rid)
                 elif launched.last[p.rid]:
                     req.finish_reason = "length"
             elif p.samples and req.n_sampled >= req.max_new:
@@ -271,9 +281,35 @@ class Engine:
                 self._release(p.rid)
             if req.finish_reason is not None:
                 req.finished = True
+                if self.detokenize is not None and req.text is None:
+                    out = req.generated
+                    if out and out[-1] in eos and req.finish_reason == "eos":
+                        out = out[:-1]               # the end-of-sequence token is no text
+                    req.text = self._text_of(out)
             outputs.append(StepOutput(p.rid, tok, req.finished, req.finish_reason))
         launched.record.host_ms += (time.perf_counter() - t_begin) * 1e3
         return outputs
+
+    def _text_of(self, tokens: List[int]) -> str:
+        """The text of the tokens; tokens at the end that leave a character unfinished (the detokenizer
+        puts U+FFFD there) wait for the tokens that finish it (engine.rs:1209-1218)."""
+        n = len(tokens)
+        text = self.detokenize(tokens[:n])
+        while n > 0 and text.endswith("\ufffd"):
+            n -= 1
+            text = self.detokenize(tokens[:n])
+        return text
+
+    def _stops(self, req: Request) -> bool:
+        """Whether one of the request's stop sequences has appeared in its generated text: the text is cut
+        where the earliest of them begins (engine.rs:1241-1257)."""
+        text = self._text_of(req.generated)
+        found = [(text.find(s), s) for s in req.params.stop_sequences if s and s in text]
+        if not found:
+            return False
+        at, seq = min(found, key=lambda f: f[0])
+        req.text, req.stop_sequence = text[:at], seq
+        return True
 
     # -- whole generations ---------------------------------------------------------------
     def generate(self, prompts: Iterable[Sequence[int]], params=None) -> List[List[int]]:

@@ -1,10 +1,10 @@
 """SamplingParams: the reference's generation parameters under their own names
 (crates/denno-engine/src/engine.rs:40-77): max_tokens 256, temperature 1.0 when unset
-(0 or less: greedy), top_k, top_p, seed, and the four repetition controls."""
+(0 or less: greedy), top_k, top_p, stop_sequences, seed, and the four repetition controls."""
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Optional
+from typing import Optional, Tuple
 
 
 # top-k / top-p work on the largest candidates only: the reference's own subset size for
@@ -24,6 +24,9 @@ class SamplingParams:
     presence_penalty: Optional[float] = None       # None or 0: off
     no_repeat_ngram_size: Optional[int] = None     # None or <= 1: off
     ignore_eos: bool = False                 # go on past an end-of-sequence token (benchmarks, random weights)
+    # texts that end the generation where the first of them appears in the generated text, which is cut there
+    # (engine.rs:44, 1241-1257); the engine needs a detokenizer for them
+    stop_sequences: Tuple[str, ...] = ()
 
     def validate(self):
         if self.max_tokens < 0:
@@ -42,6 +45,9 @@ class SamplingParams:
             raise ValueError(f"top_k must be between 1 and {TOP_CANDIDATES}, got {self.top_k}")
         if self.top_p is not None and not 0.0 < self.top_p <= 1.0:
             raise ValueError("top_p must be in (0, 1]")
+        if isinstance(self.stop_sequences, str) or not all(isinstance(x, str) for x in self.stop_sequences):
+            raise ValueError("stop_sequences must be a list of strings")
+        self.stop_sequences = tuple(self.stop_sequences)
         return self
 
     @property

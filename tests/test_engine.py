@@ -13,12 +13,16 @@ from plain.gpt2_plain import PlainGPT2
 from plain import sampler_plain as SP
 
 
-def engine_for(folder, dtype, device, **kw):
+def options_for(dtype, device, **kw):
     from denno_beta_amd.config import EngineOptions
-    from denno_beta_amd.engine import Engine
     opts = dict(dtype=dtype, device=device, page_size=16, cache_tokens=1024, max_live=4)
     opts.update(kw)
-    return Engine.from_folder(folder, EngineOptions(**opts))
+    return EngineOptions(**opts)
+
+
+def engine_for(folder, dtype, device, **kw):
+    from denno_beta_amd.engine import Engine
+    return Engine.from_folder(folder, options_for(dtype, device, **kw))
 
 
 def test_greedy_generation_matches_plain(backend, model_folders):
@@ -125,6 +129,59 @@ def test_eos_and_max_tokens(backend, model_folders, tmp_path):
     assert len(e.generate([long_prompt], SamplingParams(max_tokens=50, temperature=0.0))[0]) == 8
     assert e.generate([prompt], SamplingParams(max_tokens=0))[0] == [] and e.finish_reason(1) == "length"
     assert e.runner.cache.manager.live() == 0
+
+
+def test_stop_sequences(backend, model_folders):
+    """crates/denno-engine/src/engine.rs:2214-2236 (stop_sequence_truncates_at_first_occurrence): the text is cut
+    where the first stop sequence begins and does not hold it, the reason and the sequence are told; a sequence
+    that never appears changes nothing.  The detokenizer is the caller's: here token t reads "t<t>"."""
+    from denno_beta_amd.engine import Engine, ModelRunner, SamplingParams
+    folder = model_folders("A", "float32")
+    words = lambda ids: " ".join(f"t{t}" for t in ids)                          # noqa: E731
+
+    def engine(**kw):
+        return Engine(ModelRunner.from_folder(folder, options_for("float32", backend, **kw)), detokenize=words)
+    prompts = [seeded_tokens(i, n, 512) for i, n in enumerate((9, 30, 4))]
+    free = SamplingParams(max_tokens=20, temperature=0.0, ignore_eos=True)
+    e = engine()
+    full = e.generate(prompts, free)
+    assert [e.requests[i].text for i in range(3)] == [words(t) for t in full] and e.finish_reason(0) == "length"
+    # each request stops at its own seventh token's text, or at its twelfth's if that comes first in the text
+    for i, toks in enumerate(full):
+        stops = (f"t{toks[11]} ", f"t{toks[6]} ")
+        at = min(words(toks).find(x) for x in stops)
+        first = min(stops, key=lambda x: words(toks).find(x))
+        e = engine()
+        rid = e.add_request(prompts[i], SamplingParams(max_tokens=20, temperature=0.0, ignore_eos=True, stop_sequences=stops))
+        while e.has_unfinished():
+            e.step()
+        r = e.requests[rid]
+        assert r.finish_reason == "stop_sequence" and r.stop_sequence == first
+        assert r.text == words(toks)[:at] and first not in r.text and words(toks).startswith(r.text)
+        assert r.generated == toks[:len(r.generated)] and len(r.generated) < 20
+        assert e.runner.cache.manager.live() == 0
+    # a sequence that never appears, and an empty one: nothing changes
+    e = engine()
+    same = e.generate(prompts, SamplingParams(max_tokens=20, temperature=0.0, ignore_eos=True, stop_sequences=("t9999", "")))
+    assert same == full and e.finish_reason(1) == "length"
+    # all three together, each with its own sequence, beside each other in the batch
+    e = engine()
+    rids = [e.add_request(p, SamplingParams(max_tokens=20, temperature=0.0, ignore_eos=True,
+                                            stop_sequences=(f"t{toks[8]} ",))) for p, toks in zip(prompts, full)]
+    while e.has_unfinished():
+        e.step()
+    for rid, toks in zip(rids, full):
+        assert e.requests[rid].text == words(toks)[:words(toks).find(f"t{toks[8]} ")]
+    # an unfinished character at the end of the text waits for the token that finishes it
+    halves = lambda ids: "".join("\u00e9" if t % 2 else "x" for t in ids[:len(ids) - len(ids) % 2]) + ("\ufffd" if len(ids) % 2 else "")   # noqa: E731
+    e = Engine(ModelRunner.from_folder(folder, options_for("float32", backend)), detokenize=halves)
+    e.generate([prompts[0]], SamplingParams(max_tokens=5, temperature=0.0, ignore_eos=True))
+    assert "\ufffd" not in e.requests[0].text and len(e.requests[0].text) == 4
+    # texts need a detokenizer
+    with pytest.raises(ValueError, match="detokenizer"):
+        Engine(ModelRunner.from_folder(folder, options_for("float32", backend))).add_request([1], SamplingParams(stop_sequences=("a",)))
+    with pytest.raises(ValueError, match="list of strings"):
+        SamplingParams(stop_sequences="ab").validate()
 
 
 def test_refused_requests(backend, model_folders):
@@ -360,5 +417,11 @@ def test_command_line_with_text(backend, model_folders, tmp_path):
         assert out.returncode == 0, out.stderr
         ids = tok.encode(text).ids
         assert out.stdout.strip() == tok.decode(plain.greedy(ids, 5)), extra
+    # --stop: the text ends where the stop sequence begins
+    whole = tok.decode(plain.greedy(tok.encode("hello world").ids, 5))
+    third = whole.split()[2]
+    out = run("--raw", "--stop", third, "--stop", "never")
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.strip() == whole[:whole.find(third)].strip() and third not in out.stdout
     assert fallback_template(None, "hello") == "user: hello\n\nassistant:"          # tokenizer.rs:319-324
     assert fallback_template("be nice", "hi") == "system: be nice\n\nuser: hi\n\nassistant:"

@@ -54,7 +54,7 @@ class Workloads:
         from denno_beta_amd.config import EngineOptions
         from denno_beta_amd.engine import ModelRunner
         self.torch, self.a, self.dtype = torch, a, dtype
-        self.cfg, self.full_layers = baseline_config(2, a.layers)
+        self.cfg, self.full_layers = baseline_config({"xl": 2, "large": 3, "medium": 4}[a.shape], a.layers)
         P = self.cfg["n_positions"]
         live = max(64, a.batch)
         self.opts = EngineOptions(dtype=dtype, page_size=16, cache_tokens=live * P, max_live=live, max_batch_tokens=4096,
@@ -162,6 +162,8 @@ def main():
                          "table of each kernel's share")
     ap.add_argument("--sequences", type=int, default=8, help="--only replay: how many of the eight sequences")
     ap.add_argument("--prompts", type=int, default=2, help="--only prefill: prompts of 1,024 tokens in the one step")
+    ap.add_argument("--shape", choices=["xl", "large", "medium"], default="xl",
+                    help="--only decode / prefill: the layer sizes of BASELINE.json's configs[2], [3] or [4]")
     ap.add_argument("--only", choices=["decode", "prefill", "serving", "replay"], default=None,
                     help="run one workload and print a short line (decode, prefill: for profiling; serving: "
                          "BASELINE.json's configs[3], GPT-2 Large shape, 64 requests through the scheduler; replay: "
@@ -201,7 +203,7 @@ def main():
         "metric": "GPT-2 XL decode tokens/s (batch 8, context 512)", "value": main_point["tok_s"], "unit": "tokens/s",
         "n_gpus": 1, "steps": main_point["steps"], "warmup": a.warmup, "ms_per_step": main_point["ms"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": short, "data": "synthetic",
-        "config": {"model": "gpt2-xl-shape", "n_layer": cfg["n_layer"], "n_layer_full": w.full_layers,
+        "config": {"model": f"gpt2-{a.shape}-shape", "n_layer": cfg["n_layer"], "n_layer_full": w.full_layers,
                    "n_embd": cfg["n_embd"], "n_head": cfg["n_head"], "n_inner": cfg["n_inner"],
                    "vocab_size": cfg["vocab_size"], "n_positions": cfg["n_positions"], "global_batch": a.batch,
                    "seq_len": a.context, "page_size": w.opts.page_size, "weights": "random N(0,0.02)",

@@ -78,7 +78,11 @@ def test_kv_write(dtype):
 @pytest.mark.parametrize("in_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", [(1, 1001, 72), (5, 64, 8), (130, 200, 320), (64, 1600, 1600), (33, 50257, 96),
                                    (200, 333, 72), (300, 1600, 1600), (257, 129, 200), (2048, 256, 6400),
-                                   (48, 4800, 1600), (17, 4104, 72), (40, 33000, 40)])
+                                   (48, 4800, 1600), (17, 4104, 72), (40, 33000, 40),
+                                   # on both sides of the borders between the bfloat16 kernels: columns (2,560; 4,096),
+                                   # rows (104 / 105, 208 / 209), a long inner size into the stream (65 .. 512 rows)
+                                   (48, 2552, 256), (64, 2568, 1280), (104, 4104, 1024), (105, 4104, 1024),
+                                   (208, 2304, 768), (209, 2304, 768), (65, 1032, 4128), (512, 1000, 4096)])
 def test_linear(in_dtype, M, N, K):
     a, w, bias = rnd(M, K, seed=7, dtype=in_dtype), rnd(N, K, seed=8, dtype=in_dtype, scale=0.2), rnd(N, seed=9)
     if in_dtype == torch.bfloat16:      # the MFMA kernels take the packed matrix; rows go to the plain kernel

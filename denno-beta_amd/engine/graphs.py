@@ -12,6 +12,7 @@ replay.
 """
 from __future__ import annotations
 
+import gc
 from typing import Dict, List, Sequence, Tuple
 
 import numpy as np
@@ -79,8 +80,19 @@ class DecodeGraph:
         torch.cuda.current_stream(dev).wait_stream(side)
         torch.cuda.synchronize(dev)
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
-            self.logits = runner.model.forward(self.ctx, cache)
+        # The collector is run now and stays off while the stream records: a finalizer that gives device or
+        # pinned memory back, or destroys another graph (a runner and its graphs refer to each other, so
+        # only the collector frees them, whenever its turn comes), is an error during a capture, raised
+        # inside a destructor, which ends the process.
+        gc.collect()
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(self.graph):
+                self.logits = runner.model.forward(self.ctx, cache)
+        finally:
+            if collecting:
+                gc.enable()
 
     def _view(self, name):
         b, n = self.off[name]

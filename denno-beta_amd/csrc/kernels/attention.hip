@@ -749,13 +749,13 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
       (ldo == 0 && (H * dh) % 32 != 0) || reinterpret_cast<uintptr_t>(q) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(out) % 8 != 0)
     return DN_ERR_SHAPE;
-  // Two groups of waves where the workgroups are fewer than the CUs (a wave's chain of dependent
-  // steps per tile then bounds the time, and two groups halve the tiles a wave walks); with more
-  // workgroups the SIMDs are busy and the second group's share of carrying tiles only adds work.  Up to a head
-  // size of 64: beyond, the tiles of two groups do not fit 64 KB of LDS.
+  // Two groups of waves up to a head size of 64 (a wave's chain of dependent steps per tile bounds a
+  // workgroup's time, and two groups halve the tiles a wave walks; measured at head sizes 16 to 64 with
+  // 400 to 3,200 workgroups: 2 x 1,024 rows 38 -> 30 us, 8 x 1,024 rows 82 -> 74 us, never more than a
+  // twentieth slower).  Beyond, one group: with heads of 96 and 128 two were slower by a fifth wherever
+  // the workgroups outnumber the CUs.
   if (n_tiles > 65535) return DN_ERR_SHAPE;      // the grid's second dimension
   dim3 grid(H, n_tiles);
-  const bool two = static_cast<long>(n_tiles) * H <= 256;
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
   const bool pow2 = (1 << page_shift) == page_size;
@@ -770,8 +770,8 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
   else                         \
     DN_FLASH_P(D, G, T, false)
 #define DN_FLASH(D, G)                  \
-  if (G == 2 && two) {                  \
-    DN_FLASH_G(D, G, 1);                \
+  if (G == 2) {                         \
+    DN_FLASH_G(D, 2, 1);                \
   } else {                              \
     DN_FLASH_G(D, 1, (D <= 6 ? 2 : 1)); \
   }

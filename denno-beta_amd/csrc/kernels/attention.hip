@@ -475,9 +475,12 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2)
   const int seq = tile_seq[tile];
   if (seq < 0) return;                       // the whole workgroup
   const int row0 = tile_row0[tile], nrows = tile_nrows[tile], pos0 = tile_pos0[tile];
-  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  // (the wave's number through readfirstlane: what follows from it, the wave's rows and keys, which tiles it
+  // carries and whether a tile touches an edge, is then worked out once per wave by the scalar unit, and its
+  // page numbers come by scalar loads)
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), lane = threadIdx.x % 64;
   const int grp = wave / 4;                  // which tiles this wave multiplies
-  const int t = threadIdx.x % 256, ti = threadIdx.x / 256;   // this thread carries chunk t of the step's tiles ti TPS ..
+  const int t = threadIdx.x % 256, ti = wave / 4;   // this thread carries chunk t of the step's tiles ti TPS ..
   const int wrow0 = (wave % 4) * 32;
   const bool has_rows = wrow0 < nrows;       // a wave without rows still carries tiles into LDS
   const int qcol = lane % 32, g = lane / 32;

@@ -836,7 +836,7 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
   const int split = blockIdx.x, h = blockIdx.y, tile = blockIdx.z;
   const int row = tile;
   const int32_t* bt = block_tables + static_cast<size_t>(tile) * max_blocks;
-  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int lane = threadIdx.x % 64, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);   // (a scalar)
   const int sub = lane % LPK, grp = lane / LPK;
   const bf16x8 qv = *reinterpret_cast<const bf16x8*>(q + static_cast<size_t>(row) * ldq + h * DH + sub * 8);
   if (tile_seq[tile] < 0) return;

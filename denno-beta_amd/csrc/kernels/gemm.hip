@@ -464,7 +464,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
   constexpr int BLOCKS = MB * NB;                          // 16 x 16 blocks of C in this workgroup
   constexpr int PASSES = (BLOCKS + WAVES - 1) / WAVES;     // wave w finishes blocks w, w + WAVES, ...
   __shared__ floatx4 red[WAVES][BLOCKS][64];
-  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), lane = threadIdx.x % 64;   // (a scalar: what follows from it is the scalar unit's work)
   const int col = lane % 16, g = lane / 16;
   const int n0 = blockIdx.x * (16 * NB);
   const int row0 = blockIdx.y * (MB * 16);     // the rows may be shared out among workgroups too (blockIdx.y)

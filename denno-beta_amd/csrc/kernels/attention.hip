@@ -304,6 +304,114 @@ __global__ __launch_bounds__(THREADS) void row_tiles_kernel(
   for (int d = t; d < dh; d += THREADS) mine[2 + d] = dim_sum(Ps, Vs + d, dh, BK);
 }
 
+// four consecutive elements in one load
+__device__ __forceinline__ void load4(const float* p, float* v) {
+  const float4 x = *reinterpret_cast<const float4*>(p);
+  v[0] = x.x, v[1] = x.y, v[2] = x.z, v[3] = x.w;
+}
+__device__ __forceinline__ void load4(const bf16_t* p, float* v) {
+  const uint2 x = *reinterpret_cast<const uint2*>(p);
+  v[0] = __uint_as_float(x.x << 16), v[1] = __uint_as_float(x.x & 0xffff0000u);
+  v[2] = __uint_as_float(x.y << 16), v[3] = __uint_as_float(x.y & 0xffff0000u);
+}
+
+// row_tiles_kernel for heads of 64 and pages that hold a multiple of 4 keys: the same sums in the same
+// order, a workgroup being one wave.  Four keys from a multiple of 4 lie in one page, so a page is looked
+// up once per four keys, by the wave and not by the lane.  The keys come 16 lanes to a key's 64 dims,
+// 16 bytes each, are laid down in LDS as they came (keys 68 floats apart: no bank shared by the 16-byte
+// stores or reads) and are read back a lane per key; the values come a lane per dim, four keys' values
+// of that dim in one load (a page holds a dim's values side by side), and stay in registers.  All loads
+// are asked for before the first is used, and none depends on another's result but for the page table's.
+template <typename T>
+__global__ __launch_bounds__(64) void row_tile64_kernel(
+    const T* __restrict__ q, int ldq, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
+    const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ tile_seq,
+    const int32_t* __restrict__ tile_pos0, float* __restrict__ part, int n_key_tiles, int H, int Hkv, int page_size,
+    float scale, int window) {
+  constexpr int DH = 64, BK = 64, LD = DH + 4, QUADS = BK / 4;
+  __shared__ __attribute__((aligned(16))) float Ks[BK * LD];
+  __shared__ __attribute__((aligned(16))) float Qs[DH];
+  __shared__ __attribute__((aligned(16))) float Ps[BK];
+  const int ktile = blockIdx.x, h = blockIdx.y, tile = blockIdx.z;
+  const int seq = tile_seq[tile];
+  if (seq < 0) return;
+  const int pos = tile_pos0[tile];
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int kt = ktile * BK;
+  const int lane = threadIdx.x;
+  float* mine = part + ((static_cast<size_t>(tile) * H + h) * n_key_tiles + ktile) * (DH + 2);
+  if (kt > pos || kt + BK <= lo) {
+    if (lane == 0) mine[0] = -INFINITY;
+    return;
+  }
+  const int hk = h / (H / Hkv);
+  const int32_t* bt = block_tables + static_cast<size_t>(seq) * max_blocks;
+  // the page of each four keys (-1: beyond the row's position, or given back)
+  int page[QUADS];
+#pragma unroll
+  for (int i = 0; i < QUADS; ++i) page[i] = kt + 4 * i <= pos ? bt[(kt + 4 * i) / page_size] : -1;
+  const float qd = to_float(q[static_cast<size_t>(tile) * ldq + h * DH + lane]);
+  const int r = lane / 16, c = lane % 16;
+  float kv[QUADS][4], vv[QUADS][4];
+#pragma unroll
+  for (int i = 0; i < QUADS; ++i) {
+    const size_t head = static_cast<size_t>(max(page[i], 0)) * Hkv + hk;
+    const int off = (kt + 4 * i) % page_size;
+    load4(k_pool + (head * page_size + off + r) * DH + 4 * c, kv[i]);
+    load4(v_pool + (head * DH + lane) * page_size + off, vv[i]);
+  }
+  Qs[lane] = qd;
+  // keys beyond the row's position and pages given back: zeros, as in load_tile
+#pragma unroll
+  for (int i = 0; i < QUADS; ++i) {
+    const bool k_in = page[i] >= 0 && kt + 4 * i + r <= pos;
+    *reinterpret_cast<float4*>(&Ks[(4 * i + r) * LD + 4 * c]) =
+        k_in ? float4{kv[i][0], kv[i][1], kv[i][2], kv[i][3]} : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (!(page[i] >= 0 && kt + 4 * i + e <= pos)) vv[i][e] = 0.f;
+  }
+  __syncthreads();
+  const float NEG_INF = -INFINITY;
+  // a lane per key: the score over the dims in ascending order, as key_dot sums it
+  float dot = 0.f;
+#pragma unroll
+  for (int d4 = 0; d4 < DH / 4; ++d4) {
+    const float4 a = *reinterpret_cast<const float4*>(&Qs[4 * d4]);
+    const float4 b = *reinterpret_cast<const float4*>(&Ks[lane * LD + 4 * d4]);
+    dot = fmaf(a.x, b.x, dot);
+    dot = fmaf(a.y, b.y, dot);
+    dot = fmaf(a.z, b.z, dot);
+    dot = fmaf(a.w, b.w, dot);
+  }
+  const int key = kt + lane;
+  const float sc = (key >= lo && key <= pos) ? dot * scale : NEG_INF;
+  const float tmax = wave_max(sc);
+  Ps[lane] = sc > NEG_INF ? expf(sc - tmax) : 0.f;
+  __syncthreads();
+  // the sum of p as 16 threads of a row make it in the kernels above
+  float psum = 0.f;
+  if (lane < 16)
+    for (int cc = 0; cc < BK / 16; ++cc) psum += Ps[lane + 16 * cc];
+  psum = group_reduce<16>(psum, SumOp());
+  if (lane == 0) {
+    mine[0] = tmax;
+    mine[1] = psum;
+  }
+  if (!(tmax > NEG_INF)) return;
+  // a lane per dim: the tile's keys in ascending order, as dim_sum sums them
+  float a = 0.f;
+#pragma unroll
+  for (int i = 0; i < QUADS; ++i) {
+    const float4 p4 = *reinterpret_cast<const float4*>(&Ps[4 * i]);
+    a = fmaf(p4.x, vv[i][0], a);
+    a = fmaf(p4.y, vv[i][1], a);
+    a = fmaf(p4.z, vv[i][2], a);
+    a = fmaf(p4.w, vv[i][3], a);
+  }
+  mine[2 + lane] = a;
+}
+
 template <typename T>
 __global__ void row_join_kernel(const float* __restrict__ part, T* __restrict__ out, int ldo,
                                 const int32_t* __restrict__ tile_seq, int n_key_tiles, int H, int dh) {
@@ -316,13 +424,25 @@ __global__ void row_join_kernel(const float* __restrict__ part, T* __restrict__ 
   float acc[16], a_t[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-  for (int kt = 0; kt < n_key_tiles; ++kt) {
-    const float* p = base + static_cast<size_t>(kt) * (dh + 2);
-    const float m_t = p[0];
-    if (!(m_t > -INFINITY)) continue;
+  // four tiles' results are asked for at a time (a tile without a key left only its first number: the rest
+  // of its entry is read and not used); they are joined one after the other, in order
+  for (int kt0 = 0; kt0 < n_key_tiles; kt0 += 4) {
+    float m_t[4], l_t[4], a4[4][16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) a_t[i] = i < nd ? p[2 + g + 16 * i] : 0.f;
-    join_tile(m, l, acc, m_t, p[1], a_t, nd);
+    for (int u = 0; u < 4; ++u) {
+      const float* p = base + static_cast<size_t>(min(kt0 + u, n_key_tiles - 1)) * (dh + 2);
+      m_t[u] = p[0];
+      l_t[u] = p[1];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) a4[u][i] = i < nd ? p[2 + g + 16 * i] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (kt0 + u >= n_key_tiles || !(m_t[u] > -INFINITY)) continue;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) a_t[i] = a4[u][i];
+      join_tile(m, l, acc, m_t[u], l_t[u], a_t, nd);
+    }
   }
   const float inv = 1.0f / l;
   T* o = out + static_cast<size_t>(tile) * ldo + h * dh;
@@ -379,10 +499,17 @@ extern "C" int dn_attention_rows(const void* q, int ldq, void* out, int ldo, con
   const int n_key_tiles = (max_context + BK - 1) / BK;
   const size_t lds = sizeof(float) * (static_cast<size_t>(dh) + 2 * static_cast<size_t>(BK) * (dh + 1) + 5 * BK);
   dim3 grid(n_key_tiles, H, n_tiles), block(plain::THREADS);
+  const bool wave_tiles = dh == 64 && page_size % 4 == 0 && reinterpret_cast<uintptr_t>(k_pool) % 16 == 0 &&
+                          reinterpret_cast<uintptr_t>(v_pool) % 16 == 0;
 #define DN_ROWS(T)                                                                                                   \
-  hipLaunchKernelGGL(plain::row_tiles_kernel<T>, grid, block, lds, stream, static_cast<const T*>(q), ldq,            \
-                     static_cast<const T*>(k_pool), static_cast<const T*>(v_pool), block_tables, max_blocks, tile_seq, \
-                     tile_pos0, part, n_key_tiles, H, Hkv, dh, page_size, BK, scale, window);                         \
+  if (wave_tiles)                                                                                                    \
+    hipLaunchKernelGGL(plain::row_tile64_kernel<T>, grid, dim3(64), 0, stream, static_cast<const T*>(q), ldq,        \
+                       static_cast<const T*>(k_pool), static_cast<const T*>(v_pool), block_tables, max_blocks,       \
+                       tile_seq, tile_pos0, part, n_key_tiles, H, Hkv, page_size, scale, window);                    \
+  else                                                                                                               \
+    hipLaunchKernelGGL(plain::row_tiles_kernel<T>, grid, block, lds, stream, static_cast<const T*>(q), ldq,          \
+                       static_cast<const T*>(k_pool), static_cast<const T*>(v_pool), block_tables, max_blocks,       \
+                       tile_seq, tile_pos0, part, n_key_tiles, H, Hkv, dh, page_size, BK, scale, window);            \
   hipLaunchKernelGGL(plain::row_join_kernel<T>, dim3(n_tiles, H), dim3(16), 0, stream, part, static_cast<T*>(out), ldo, \
                      tile_seq, n_key_tiles, H, dh)
   if (dtype == DN_F32) {

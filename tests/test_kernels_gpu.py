@@ -647,7 +647,8 @@ def test_attention_window_edges_in_every_kernel(H, dh, window, n):
 
 @pytest.mark.parametrize("dh,ps", [(32, 16), (64, 16), (64, 4), (64, 6), (64, 64)])
 def test_attention_rows_do_not_depend_on_the_batch(dh, ps):
-    # (several head sizes and page sizes, a page of 6 keys among them)
+    # (heads of 64 on pages of a multiple of 4 keys have a kernel of their own for steps of single rows; a page of
+    # 6 keys and heads of 32 take the general one)
     H = 4
     q, k, v, bt, tiles, T = paged_case([200, 90], [50, 90], H, H, dh, ps, torch.float32, seed=2)
     out = torch.zeros(T, H * dh, device=DEV)

@@ -879,11 +879,10 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
       (ldo == 0 && (H * dh) % 32 != 0) || reinterpret_cast<uintptr_t>(q) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(out) % 8 != 0)
     return DN_ERR_SHAPE;
-  // Two groups of waves up to a head size of 64 (a wave's chain of dependent steps per tile bounds a
-  // workgroup's time, and two groups halve the tiles a wave walks; measured at head sizes 16 to 64 with
-  // 400 to 3,200 workgroups: 2 x 1,024 rows 38 -> 30 us, 8 x 1,024 rows 82 -> 74 us, never more than a
-  // twentieth slower).  Beyond, one group: with heads of 96 and 128 two were slower by a fifth wherever
-  // the workgroups outnumber the CUs.
+  // Two groups of waves up to a head size of 64: a wave's chain of dependent steps per tile bounds a
+  // workgroup's time, and two groups halve the tiles a wave walks (the faster, or level, at every grid
+  // size measured).  Beyond, one group: with heads of 96 and 128 two were the slower wherever the
+  // workgroups outnumber the CUs.
   if (n_tiles > 65535) return DN_ERR_SHAPE;      // the grid's second dimension
   dim3 grid(H, n_tiles);
   int page_shift = 0;

@@ -964,8 +964,8 @@ static void launch16(const Call& c, hipStream_t stream) {
 
 // With more than 16 rows every workgroup reads all of A (16 cache lines per load and 16 lanes,
 // as A lies in rows), so wider workgroups read less in total, as long as enough of them remain
-// to keep the memory system busy: 2 column blocks per workgroup from 2,560 columns on (3,072 columns at
-// 64 rows: 6.7 -> 5.6 us; 2,304 columns are slower that way), 4 from 32,768 on, else 1.
+// to keep the memory system busy: 2 column blocks per workgroup from 2,560 columns on (with 2,304 columns
+// that way was the slower), 4 from 32,768 on, else 1.
 template <int WAVES>
 static void launch_mb(const Call& c, hipStream_t stream) {
   const int mb = (c.M + 15) / 16;
@@ -1608,8 +1608,7 @@ static int launch_as(const Args& a, hipStream_t stream) {
 
 // The tiles on offer: rows x columns, slabs in flight.  256 rows: 8 waves as 4 x 2, one workgroup
 // per CU; the small ones leave room for several workgroups per CU.  64 x 64 and 32 x 64 (4 waves) are
-// for products with few rows and a long K, whose larger tiles would leave most CUs idle (512 x 1600 x
-// 6400: 50 -> 39 us; 300 rows: 50 -> 37 us).
+// for products with few rows and a long K, whose larger tiles would leave most CUs idle.
 struct Shape { int bm, bn, stages; };
 constexpr Shape SHAPES[] = {{64, 128, 4}, {128, 128, 4}, {256, 128, 4}, {256, 160, 4}, {256, 192, 4},
                             {256, 224, 4}, {256, 256, 4}, {256, 320, 3}, {64, 64, 4}, {32, 64, 4}};
@@ -1636,7 +1635,7 @@ static int pick(int M, int N, int K) {
 
 // Up to 256 rows the few-rows kernel takes the product too (both read and write packed rows).
 // This one is the faster from 105 rows on where the product has 4,096 columns or more, and from 209 rows
-// on from 2,048 columns (2,304 columns at 224 rows: 8.3 against 10.6 us); with fewer columns its tiles
+// on from 2,048 columns (both borders as measured); with fewer columns its tiles
 // leave most CUs idle and the few-rows kernel stays ahead, or level, at every size.
 static bool beats_few_rows(int M, int N, int K) {
   (void)K;
@@ -1644,10 +1643,9 @@ static bool beats_few_rows(int M, int N, int K) {
 }
 
 // A long K beside few columns and few rows: the tiles are few and each walks all of K, a slab at a time,
-// so K is shared out among several workgroups per tile (measured at 1,600 columns and K = 6,400: 42 us
-// whatever the rows up to 256, where a quarter of K takes 12).  The number of shares, 0 for none: 8 where
-// the tiles of 32 x 64 are at most 96, else 4 (65 rows: 26.2, 18.6, 17.5 us with 2, 4, 8 shares; 256 rows:
-// 27.8, 25.3, 26.1).
+// so K is shared out among several workgroups per tile (whole, such a product takes the same time whatever
+// its rows up to 256, and a quarter of K less than a third of it).  The number of shares, 0 for none: 8
+// where the tiles of 32 x 64 are at most 96, else 4 (with more rows 8 shares gain nothing over 4).
 static int shares_of_k(int M, int N, int K, int packed, bool kv) {
   if (kv || (packed & PACKED_C) || M <= 64 || M > 512 || N >= 4096 || K < 4096) return 0;
   return ((M + 31) / 32) * ((N + 63) / 64) <= 96 ? 8 : 4;

@@ -483,8 +483,6 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
         # chunk (every load issued at once), within what the head size leaves registers for
         # (where the batch alone gives two workgroups or more per CU the chip is busy anyway, and
         # the smallest workgroups were measured fastest)
-        # (measured at heads of 64 and a context of 560, 4 / 8 / 16 waves: 64 rows 46.0 / 44.7 / 49.2 us, 32 rows
-        # 27.7 / 28.5 / 30.2, 16 rows 18.7 / 17.0 / 18.3, 8 rows 14.0 / 12.0 / 10.8)
         groups = n_tiles * n_heads
         waves = (4 if max_context <= 256 else 8 if groups >= 1024 else 4 if groups >= 512 else
                  8 if groups >= 300 or max_context <= 512 else 16)

@@ -57,7 +57,7 @@ class Workloads:
         self.cfg, self.full_layers = baseline_config({"xl": 2, "large": 3, "medium": 4}[a.shape], a.layers)
         P = self.cfg["n_positions"]
         live = max(64, a.batch)
-        self.opts = EngineOptions(dtype=dtype, page_size=16, cache_tokens=live * P, max_live=live, max_batch_tokens=4096,
+        self.opts = EngineOptions(dtype=dtype, page_size=a.page_size, cache_tokens=live * P, max_live=live, max_batch_tokens=4096,
                                   prefill_chunk=1024, use_graphs=not (a.no_graphs or a.kernel_times), seed=0,
                                   norms_inside_products=not a.norm_kernels)
         self.runner = ModelRunner.from_random(self.cfg, seed=0, options=self.opts, stored=dtype)
@@ -161,6 +161,7 @@ def main():
                     help="with --only decode or prefill: every launch between two HIP events (no graphs), and a "
                          "table of each kernel's share")
     ap.add_argument("--sequences", type=int, default=8, help="--only replay: how many of the eight sequences")
+    ap.add_argument("--page-size", type=int, default=16, help="tokens in a page of the cache (decode and prefill)")
     ap.add_argument("--prompts", type=int, default=2, help="--only prefill: prompts of 1,024 tokens in the one step")
     ap.add_argument("--shape", choices=["xl", "large", "medium"], default="xl",
                     help="--only decode / prefill: the layer sizes of BASELINE.json's configs[2], [3] or [4]")

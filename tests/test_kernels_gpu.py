@@ -526,9 +526,11 @@ def test_attention_mfma_kernel_for_portions(H, Hkv, dh, ps, window):
         assert T2 == 200 and torch.equal(packed.rows(), rows)
 
 
-@pytest.mark.parametrize("H,Hkv,dh,ps,window", [(8, 8, 64, 16, 0), (8, 2, 32, 32, 40), (8, 4, 64, 48, 0)])
+@pytest.mark.parametrize("H,Hkv,dh,ps,window", [(8, 8, 64, 16, 0), (8, 2, 32, 32, 40), (8, 4, 64, 48, 0),
+                                                (8, 8, 96, 16, 0), (8, 2, 128, 32, 60)])
 def test_attention_mfma_kernel_with_many_workgroups(H, Hkv, dh, ps, window):
-    """More workgroups than CUs: the kernel then runs one group of waves per workgroup, not two."""
+    """More workgroups than CUs, so that they follow one another on a CU: two groups of waves a workgroup up to
+    heads of 64, one group beyond (two tiles of keys a step for heads of 96, one for 128)."""
     g = torch.Generator().manual_seed(3)
     new_rows = [int(n) for n in torch.randint(1, 200, (36,), generator=g)]
     seq_lens = [n + int(x) for n, x in zip(new_rows, torch.randint(0, 150, (36,), generator=g))]

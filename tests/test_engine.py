@@ -325,6 +325,43 @@ def test_running_ahead_changes_no_token(model_folders, tmp_path, dtype):
 
 
 @pytest.mark.gpu
+def test_no_collection_runs_while_a_step_is_captured(model_folders):
+    """A runner and its captured steps refer to each other, so only Python's cyclic collector frees an engine that
+    is let go; its finalizers give pinned and device memory back and destroy graphs, which must not happen while
+    another engine's stream records a step.  With the collector made eager (a collection at every allocation
+    or so), engines are let go one after the other and the next one captures its steps: no collection may
+    start during a capture, every engine gives the same tokens, and the collector is left as it was found."""
+    import gc
+    from denno_beta_amd.engine import SamplingParams
+    folder = model_folders("A", "bfloat16")
+    prompts = [seeded_tokens(300 + i, n, TINY["A"][0]["vocab_size"]) for i, n in enumerate((9, 30))]
+    params = [SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True)] * 2
+    during = []
+
+    def watch(phase, info):
+        if phase == "start" and torch.cuda.is_current_stream_capturing():
+            during.append(info)
+    old = gc.get_threshold()
+    gc.callbacks.append(watch)
+    gc.set_threshold(20, 3, 3)
+    try:
+        assert gc.isenabled()
+        first = None
+        for _ in range(3):
+            e = engine_for(folder, "bfloat16", "cuda:0")      # graphs are on by default
+            got = e.generate(prompts, params)
+            assert len(e.runner.graphs.graphs) > 0, "no step was captured"
+            first = first or got
+            assert got == first
+            del e      # garbage now: the next engine's captures run while it waits for the collector
+        assert gc.isenabled()
+    finally:
+        gc.set_threshold(*old)
+        gc.callbacks.remove(watch)
+    assert during == []
+
+
+@pytest.mark.gpu
 def test_serving_at_large_layer_sizes_gives_each_request_its_solo_tokens(tmp_path):
     """Two layers of GPT-2 Large's sizes, 24 requests with prompts of 16 to 300 tokens admitted into a
     running batch, portions of 64, 200 tokens a step, so few pages that requests are put back: in 32-bit

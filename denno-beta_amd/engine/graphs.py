@@ -13,6 +13,7 @@ replay.
 from __future__ import annotations
 
 import gc
+import weakref
 from typing import Dict, List, Sequence, Tuple
 
 import numpy as np
@@ -33,7 +34,7 @@ def batch_bucket(n: int, limit: int):
 
 class DecodeGraph:
     def __init__(self, runner, batch: int, max_context: int):
-        self.runner, self.B, self.max_context = runner, batch, max_context
+        self.manager, self.B, self.max_context = runner.cache.manager, batch, max_context      # (no way back to the runner: no cycle)
         cache, dev = runner.cache, runner.device
         self.layouts = cache.layouts
         B = batch
@@ -81,8 +82,8 @@ class DecodeGraph:
         torch.cuda.synchronize(dev)
         self.graph = torch.cuda.CUDAGraph()
         # The collector is run now and stays off while the stream records: a finalizer that gives device or
-        # pinned memory back, or destroys another graph (a runner and its graphs refer to each other, so
-        # only the collector frees them, whenever its turn comes), is an error during a capture, raised
+        # pinned memory back, or destroys another graph (whatever of an engine let go earlier sits in a cycle of
+        # references waits for the collector, whenever its turn comes), is an error during a capture, raised
         # inside a destructor, which ends the process.
         gc.collect()
         collecting = gc.isenabled()
@@ -101,7 +102,7 @@ class DecodeGraph:
     def _fill(self, hv, rids, tokens, starts, slots):
         """The step's tables into a host buffer: rids int64 [n], tokens, starts, slots int32 [n]."""
         B, n = self.B, len(rids)
-        mgr = self.runner.cache.manager
+        mgr = self.manager
 
         def put(name, vals, fill):
             b, ln = self.off[name]
@@ -150,8 +151,15 @@ class DecodeGraphs:
     """The graphs of one runner, captured on demand."""
 
     def __init__(self, runner):
-        self.runner = runner
+        self._runner = weakref.ref(runner)      # the runner owns these graphs; a reference back would be a cycle
         self.graphs: Dict[Tuple[int, int], DecodeGraph] = {}
+
+    @property
+    def runner(self):
+        runner = self._runner()
+        if runner is None:
+            raise BatchError("the runner of these graphs is gone")
+        return runner
 
     def takes(self, entries: Sequence[StepEntry]) -> bool:
         return self.runner.model.graph_safe and all(len(e.tokens) == 1 for e in entries)

@@ -326,8 +326,8 @@ def test_running_ahead_changes_no_token(model_folders, tmp_path, dtype):
 
 @pytest.mark.gpu
 def test_no_collection_runs_while_a_step_is_captured(model_folders):
-    """A runner and its captured steps refer to each other, so only Python's cyclic collector frees an engine that
-    is let go; its finalizers give pinned and device memory back and destroy graphs, which must not happen while
+    """What of an engine sits in a cycle of references is freed by Python's cyclic collector, whenever its turn
+    comes; the finalizers give pinned and device memory back and destroy graphs, which must not happen while
     another engine's stream records a step.  With the collector made eager (a collection at every allocation
     or so), engines are let go one after the other and the next one captures its steps: no collection may
     start during a capture, every engine gives the same tokens, and the collector is left as it was found."""

@@ -67,20 +67,37 @@ class Sampler:
             tu = torch.tensor([temps, us], dtype=torch.float32, device=dev)      # one copy for both
         t_dev, u_dev = tu[0], tu[1]
         ops.sample(logits, t_dev, u_dev, both[:R])
-        if not restricted:
-            return Pending(both, R, None)
-        top_p = [params[r].top_p if params[r].top_p is not None else 1.0 for r in restricted]
-        ints = torch.tensor([restricted, [params[r].top_k or 0 for r in restricted]], dtype=torch.int32, device=dev)
-        ps = torch.tensor(top_p, dtype=torch.float32, device=dev)
-        ops.sample_top(logits, ints[0], t_dev, u_dev, ints[1], ps, both[:R], both[R:])
-        return Pending(both, R, (logits, restricted, top_p, t_dev, u_dev))
+        more = None
+        if restricted:
+            top_p = [params[r].top_p if params[r].top_p is not None else 1.0 for r in restricted]
+            ints = torch.tensor([restricted, [params[r].top_k or 0 for r in restricted]], dtype=torch.int32, device=dev)
+            ps = torch.tensor(top_p, dtype=torch.float32, device=dev)
+            ops.sample_top(logits, ints[0], t_dev, u_dev, ints[1], ps, both[:R], both[R:])
+            more = (logits, restricted, top_p, t_dev, u_dev)
+        return Pending(both, R, more, *self._bring_home(both))
+
+    @staticmethod
+    def _bring_home(both):
+        """The copy of a step's tokens to the host is asked for here, behind the sampling kernels, and not when
+        they are read: a copy asked for at the read would queue behind whatever was launched meanwhile (the
+        whole next step, where the engine runs ahead), and the read would wait for all of that.  -> (the
+        pinned host tensor, the event that says it is filled)."""
+        if both.device.type != "cuda":
+            return both, None
+        host = torch.empty(both.shape, dtype=both.dtype, pin_memory=True)
+        host.copy_(both, non_blocking=True)
+        filled = torch.cuda.Event()
+        filled.record()
+        return host, filled
 
     def read(self, pending: "Pending") -> List[int]:
         """Waits for a launched sampling; -> the rows' tokens."""
         if pending.rows == 0:
             return []
         R = pending.rows
-        host = pending.both.tolist()
+        if pending.filled is not None:
+            pending.filled.synchronize()
+        host = pending.host.tolist()
         tokens = host[:R]
         if pending.more is None:
             return tokens
@@ -99,8 +116,9 @@ class Pending:
     """A launched sampling: `both[:rows]` are the tokens on the device.  final: no row can still change
     (rows with top-k or top-p may, when `read` finds their cut beyond the candidates)."""
 
-    def __init__(self, both, rows, more):
+    def __init__(self, both, rows, more, host=None, filled=None):
         self.both, self.rows, self.more = both, rows, more
+        self.host, self.filled = host, filled      # both on the host, and the event that says so (None: no wait)
 
     @property
     def tokens(self):

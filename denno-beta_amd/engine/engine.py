@@ -214,7 +214,8 @@ class Engine:
                 device_tokens = before.pending.tokens
                 if order != list(range(len(before.sampled))):
                     device_tokens = device_tokens[torch.tensor(order, dtype=torch.long, device=device_tokens.device)]
-            logits = self.runner.step(entries, device_tokens)
+            # (the sampling below is this stream's next work: the logits need not outlive the next step)
+            logits = self.runner.step(entries, device_tokens, borrow=True)
             self.scheduler.steps_done(np.asarray([p.rid for p in plan], dtype=np.int64),
                                       np.asarray([p.count for p in plan], dtype=np.int32))
             # each request's generator lives in its slot record: the seed and the count of numbers drawn

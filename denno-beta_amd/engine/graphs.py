@@ -164,8 +164,10 @@ class DecodeGraphs:
     def takes(self, entries: Sequence[StepEntry]) -> bool:
         return self.runner.model.graph_safe and all(len(e.tokens) == 1 for e in entries)
 
-    def step(self, entries: Sequence[StepEntry], device_tokens=None) -> torch.Tensor:
-        """Runs a pure decode step; -> logits [R, vocab] at the wanted places (a copy).
+    def step(self, entries: Sequence[StepEntry], device_tokens=None, borrow=False) -> torch.Tensor:
+        """Runs a pure decode step; -> logits [R, vocab] at the wanted places: a copy, or with `borrow`, where every
+        entry wants its logits, the graph's own buffer, which holds them until the same graph is replayed (enough
+        for a caller that samples from them on this stream before its next step).
         device_tokens: int32 [entries] on the device: the entries' tokens, which the host does not know yet
         (the entries then hold any token of the vocabulary in their place)."""
         runner = self.runner
@@ -203,7 +205,7 @@ class DecodeGraphs:
             g = self.graphs[key] = DecodeGraph(runner, B, ctx_bucket)
         logits = g.run(rids, tokens.astype(np.int32), starts, slots, device_tokens)
         if len(rows) == n:
-            out = logits[:n].clone()
+            out = logits[:n] if borrow else logits[:n].clone()
         else:
             out = logits[torch.tensor(rows, dtype=torch.long, device=logits.device)] if rows else logits[:0].clone()
         mgr.commit_step(rids, new_lens)

@@ -80,17 +80,19 @@ class ModelRunner:
         return self.graphs is not None and self.model.graph_safe
 
     # -- the step ------------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry], device_tokens=None) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], device_tokens=None, borrow=False) -> torch.Tensor:
         """-> logits [R, vocab], 32-bit, on the device: the wanted places in the order of the
         entries and of each entry's `want`.  On return the cache holds the entries' tokens.
         device_tokens: for a step of single tokens that captured graphs run (`runs_ahead`): the tokens as
-        an int32 tensor on the device, where the host does not know them yet."""
+        an int32 tensor on the device, where the host does not know them yet.
+        borrow: the logits may be a buffer that a later step overwrites (a replayed graph's own output): for a
+        caller that is done with them, on this stream, before its next step."""
         entries = list(entries)
         if not entries:
             return torch.empty((0, self.spec.vocab), dtype=torch.float32, device=self.device)
         if self.graphs is not None and self.graphs.takes(entries):
             self.steps_run += 1
-            return self.graphs.step(entries, device_tokens)
+            return self.graphs.step(entries, device_tokens, borrow)
         if device_tokens is not None:
             raise ValueError("device_tokens: only a step of single tokens that captured graphs run takes them")
         ctx = build_context(entries, self.cache, self.spec.vocab, self.spec.max_positions, self.device)

@@ -117,7 +117,9 @@ class Scheduler:
         return self._lib.dn_sched_n_running(self._h)
 
     def known(self, rid: int) -> int:
-        return self._chk(self._lib.dn_sched_known(self._h, rid), f"request {rid}")
+        """The tokens the scheduler knows of the request; -1 if it has no such request (any more)."""
+        rc = self._lib.dn_sched_known(self._h, rid)
+        return -1 if rc == UNKNOWN else self._chk(rc, f"request {rid}")
 
     def computed(self, rid: int) -> int:
         return self._chk(self._lib.dn_sched_computed(self._h, rid), f"request {rid}")

@@ -129,6 +129,23 @@ def test_eos_and_max_tokens(backend, model_folders, tmp_path):
     assert len(e.generate([long_prompt], SamplingParams(max_tokens=50, temperature=0.0))[0]) == 8
     assert e.generate([prompt], SamplingParams(max_tokens=0))[0] == [] and e.finish_reason(1) == "length"
     assert e.runner.cache.manager.live() == 0
+    # the end-of-sequence token as the very last token that max_tokens allows: the scheduler has let the
+    # request go when its last token was launched, and the end-of-sequence rule finds nothing left to give back
+    e = engine_for(d, "float32", backend)
+    out = e.generate([prompt], SamplingParams(max_tokens=stop + 1, temperature=0.0))[0]
+    assert out == first[:stop + 1] and e.finish_reason(0) == "eos" and e.runner.cache.manager.live() == 0
+    e.runner.cache.manager.check()
+    # a request given up while its last token is on its way (steps are launched ahead where they can be)
+    e = engine_for(folder, "float32", backend)
+    rid = e.add_request(prompt, SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True))
+    while len(e.requests[rid].generated) < 5:
+        e.step()
+    e.abort(rid)
+    assert e.finish_reason(rid) == "aborted"
+    while e.has_unfinished():
+        e.step()
+    assert e.runner.cache.manager.live() == 0
+    e.runner.cache.manager.check()
 
 
 def test_stop_sequences(backend, model_folders):

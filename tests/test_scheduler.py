@@ -132,6 +132,7 @@ def test_finish_of_a_waiting_request_and_unknown():
     assert s.n_waiting() == 0
     with pytest.raises(SchedulerError, match="unknown"):
         s.finish(1)
+    assert s.known(1) == -1 and s.known(0) == 10      # asking is no error
     s.finish(0)
     assert cache.live() == 0 and cache.free_pages(0) == 64
 

@@ -81,11 +81,11 @@ class DecodeGraph:
         torch.cuda.current_stream(dev).wait_stream(side)
         torch.cuda.synchronize(dev)
         self.graph = torch.cuda.CUDAGraph()
-        # The collector is run now and stays off while the stream records: a finalizer that gives device or
-        # pinned memory back, or destroys another graph (whatever of an engine let go earlier sits in a cycle of
-        # references waits for the collector, whenever its turn comes), is an error during a capture, raised
-        # inside a destructor, which ends the process.
-        gc.collect()
+        # The collector stays off while the stream records: a finalizer that gives device or pinned memory
+        # back, or destroys another graph (whatever of an engine let go earlier sits in a cycle of references
+        # waits for the collector, whenever its turn comes), is an error during a capture, raised inside a
+        # destructor, which ends the process.  (It is not run first either: a full collection costs
+        # milliseconds, and a serving run captures a graph per batch and context bucket as it goes.)
         collecting = gc.isenabled()
         gc.disable()
         try:

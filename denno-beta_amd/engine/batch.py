@@ -64,6 +64,7 @@ def plan_rows(entries: Sequence[StepEntry], starts: Sequence[int], vocab: int, m
     """Host arrays of the batch: tokens, positions, logit rows, row starts, tiles (narrow and wide)."""
     tokens, positions, logit_rows, row_start, tiles, wide = [], [], [], [0], [], []
     seen = set()
+    rows = 0
     for s, (e, start) in enumerate(zip(entries, starts)):
         n = len(e.tokens)
         if n == 0:
@@ -74,12 +75,16 @@ def plan_rows(entries: Sequence[StepEntry], starts: Sequence[int], vocab: int, m
         if start + n > max_positions:
             raise BatchError(f"request {e.rid}: {start} tokens in the cache + {n} exceed the model's "
                              f"{max_positions} positions")
-        row0 = len(tokens)
-        for t in e.tokens:
-            if not 0 <= int(t) < vocab:
-                raise BatchError(f"request {e.rid}: token id {t} is outside the vocabulary of {vocab}")
-        tokens.extend(int(t) for t in e.tokens)
-        positions.extend(range(start, start + n))
+        row0 = rows
+        rows += n
+        # (arrays, not loops over tokens: a prompt's portion is a thousand of them)
+        ids = np.asarray(e.tokens, dtype=np.int64)
+        bad = (ids < 0) | (ids >= vocab)
+        if ids.ndim != 1 or bad.any():
+            t = e.tokens[int(np.argmax(bad))] if ids.ndim == 1 else e.tokens
+            raise BatchError(f"request {e.rid}: token id {t} is outside the vocabulary of {vocab}")
+        tokens.append(ids)
+        positions.append(np.arange(start, start + n, dtype=np.int64))
         for w in e.want:
             if not 0 <= w < n:
                 raise BatchError(f"request {e.rid}: wanted place {w} is not among its {n} tokens")
@@ -92,7 +97,9 @@ def plan_rows(entries: Sequence[StepEntry], starts: Sequence[int], vocab: int, m
     # a tile's work grows with the keys before its last row: the kernel starts workgroups in this
     # order, the longest first (with the shortest last, the chip runs empty evenly)
     wide.sort(key=lambda t: -(t[3] + t[2]))
-    return tokens, positions, logit_rows, row_start, tiles, wide
+    none = np.empty(0, dtype=np.int64)
+    return (np.concatenate(tokens) if tokens else none, np.concatenate(positions) if positions else none, logit_rows,
+            row_start, tiles, wide)
 
 
 def build_context(entries: Sequence[StepEntry], cache, vocab: int, max_positions: int, device) -> StepContext:

@@ -131,7 +131,14 @@ def _declare(name, lib):
         lib.dn_gemm_work_floats.restype = c_longlong
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    """The current stream's handle, asked for before every launch: through torch's own short way where it has
+    one (building a Stream object costs several microseconds, as much as the launch itself)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -151,24 +158,27 @@ def _ok(rc, what):
 
 
 def _need(cond, msg):
+    """msg: the text, or what makes it (a message that has to be put together is made only when it is needed:
+    these checks stand in front of every launch)."""
     if not cond:
-        raise KernelError(msg)
+        raise KernelError(msg() if callable(msg) else msg)
 
 
 def _dev(t, name, dtypes=None, dims=None):
-    _need(isinstance(t, torch.Tensor) and t.is_cuda, f"{name}: must be a tensor on the GPU")
-    if dtypes is not None:
-        _need(t.dtype in dtypes, f"{name}: dtype {t.dtype}, wanted one of {dtypes}")
-    if dims is not None:
-        _need(t.dim() == dims, f"{name}: {t.dim()} dimensions, wanted {dims}")
+    if not (isinstance(t, torch.Tensor) and t.is_cuda):
+        raise KernelError(f"{name}: must be a tensor on the GPU")
+    if dtypes is not None and t.dtype not in dtypes:
+        raise KernelError(f"{name}: dtype {t.dtype}, wanted one of {dtypes}")
+    if dims is not None and t.dim() != dims:
+        raise KernelError(f"{name}: {t.dim()} dimensions, wanted {dims}")
     return t
 
 
 def _rows(t, name):
     """A 2-D tensor whose rows are contiguous; returns its leading dimension."""
-    _need(t.dim() == 2 and (t.shape[1] == 1 or t.stride(1) == 1), f"{name}: rows must be contiguous")
+    _need(t.dim() == 2 and (t.shape[1] == 1 or t.stride(1) == 1), lambda: f"{name}: rows must be contiguous")
     ld = t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
-    _need(ld >= t.shape[1], f"{name}: rows overlap")
+    _need(ld >= t.shape[1], lambda: f"{name}: rows overlap")
     return ld
 
 
@@ -249,7 +259,7 @@ PACKED_ROWS_MIN = 17     # up to 16 rows the few-rows product turns ordinary row
 def packed_rows(n_rows, width, device) -> PackedMatrix:
     """An empty packed matrix for n_rows <= 256 rows of activations."""
     _need(n_rows <= PACKED_ROWS_MAX and width % 32 == 0,
-          f"packed rows: at most {PACKED_ROWS_MAX} rows of a width that is a multiple of 32, not {n_rows} x {width}")
+          lambda: f"packed rows: at most {PACKED_ROWS_MAX} rows of a width that is a multiple of 32, not {n_rows} x {width}")
     data = torch.empty(-(-n_rows // 16) * (width // 32) * 512, dtype=torch.bfloat16, device=device)
     return PackedMatrix(data, (n_rows, width))
 
@@ -259,7 +269,7 @@ def pack_matrix(w) -> PackedMatrix:
     _dev(w, "w", (torch.bfloat16,), 2)
     N, K = w.shape
     _need(w.is_contiguous(), "pack_matrix: w must be contiguous")
-    _need(K % 8 == 0, f"pack_matrix: the inner size {K} must be a multiple of 8")
+    _need(K % 8 == 0, lambda: f"pack_matrix: the inner size {K} must be a multiple of 8")
     data = torch.empty(-(-N // 16) * -(-K // 32) * 512, dtype=torch.bfloat16, device=w.device)
     _ok(_lib("gemm").dn_pack_matrix(w.data_ptr(), data.data_ptr(), N, K, _stream()), "pack_matrix")
     return PackedMatrix(data, (N, K))
@@ -327,19 +337,19 @@ def _operands(a, w, what):
     """(leading dimension of a, N, packed flags) of the product a [M, K] . w [N, K]^T."""
     M, K = a.shape
     if isinstance(a, PackedMatrix):
-        _need(isinstance(w, PackedMatrix), f"{what}: packed rows need a packed matrix")
-        _need(M <= PACKED_ROWS_MAX and K % 32 == 0, f"{what}: packed rows {a.shape}")
+        _need(isinstance(w, PackedMatrix), lambda: f"{what}: packed rows need a packed matrix")
+        _need(M <= PACKED_ROWS_MAX and K % 32 == 0, lambda: f"{what}: packed rows {a.shape}")
         lda, flags = 0, PACKED_A
     else:
         _dev(a, "a", _FLOATS, 2)
         lda, flags = _rows(a, "a"), 0
     if isinstance(w, PackedMatrix):
-        _need(a.dtype == torch.bfloat16, f"{what}: a packed matrix needs bfloat16 rows, not {a.dtype}")
-        _need(w.device == a.device and w.shape[1] == K, f"{what}: w {w.shape} does not fit a {tuple(a.shape)}")
-        _need(a.data_ptr() % 16 == 0 and lda % 8 == 0, f"{what}: the rows of a must be aligned to 16 bytes")
+        _need(a.dtype == torch.bfloat16, lambda: f"{what}: a packed matrix needs bfloat16 rows, not {a.dtype}")
+        _need(w.device == a.device and w.shape[1] == K, lambda: f"{what}: w {w.shape} does not fit a {tuple(a.shape)}")
+        _need(a.data_ptr() % 16 == 0 and lda % 8 == 0, lambda: f"{what}: the rows of a must be aligned to 16 bytes")
         return lda, w.shape[0], flags | PACKED_W
     _dev(w, "w", (a.dtype,), 2)
-    _need(w.is_contiguous() and w.shape[1] == K, f"{what}: w {tuple(w.shape)} does not fit a {tuple(a.shape)}")
+    _need(w.is_contiguous() and w.shape[1] == K, lambda: f"{what}: w {tuple(w.shape)} does not fit a {tuple(a.shape)}")
     return lda, w.shape[0], flags
 
 
@@ -349,7 +359,7 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
     reference for bfloat16) or a PackedMatrix (the MFMA kernels); bias: 32-bit [N].  With a packed
     w and at most 256 rows, a and a bfloat16 out may be packed rows."""
     M, K = a.shape
-    _need(K % 8 == 0, f"linear: the inner size {K} must be a multiple of 8")
+    _need(K % 8 == 0, lambda: f"linear: the inner size {K} must be a multiple of 8")
     lda, N, packed = _operands(a, w, "linear")
     wp = w.data_ptr()
     if bias is not None:
@@ -375,7 +385,7 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
         return residual
     if isinstance(out, PackedMatrix):
         _need((packed & PACKED_W) and M <= PACKED_ROWS_MAX and N % 32 == 0 and out.device == a.device,
-              f"linear: packed rows as out need a packed w, at most {PACKED_ROWS_MAX} rows and N a multiple of 32")
+              lambda: f"linear: packed rows as out need a packed w, at most {PACKED_ROWS_MAX} rows and N a multiple of 32")
         ldc = 0
     else:
         _dev(out, "out", _FLOATS, 2)
@@ -399,7 +409,7 @@ def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
     N = w.shape[0]
     _need(N == q_width + 2 * kvw, "linear_qkv: columns are not q | k | v")
     _need(not isinstance(out, PackedMatrix) and out.dim() == 2 and out.shape[0] == M and out.shape[1] in (N, q_width),
-          f"linear_qkv: out must be [{M}, {N}] or [{M}, {q_width}]")
+          lambda: f"linear_qkv: out must be [{M}, {N}] or [{M}, {q_width}]")
     if isinstance(w, PackedMatrix) and out.dtype == torch.bfloat16:
         _dev(out, "out", None, 2)
         _dev(slot_map, "slot_map", _I32, 1), _dev(k_pool, "k_pool", (torch.bfloat16,), 4)
@@ -468,8 +478,8 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
           "attention: pools")
     _need(q.shape[1] >= n_heads * dh and tuple(out.shape) == (T, n_heads * dh), "attention: q/out shapes")
     _need(block_tables.is_contiguous() and tiles.is_contiguous() and tiles.shape[0] == 4, "attention: tables")
-    _need(dh % 16 == 0 and 16 <= dh <= 256, f"attention: head size {dh} must be a multiple of 16 up to 256")
-    _need(n_heads % Hkv == 0, f"attention: {n_heads} heads over {Hkv} key heads")
+    _need(dh % 16 == 0 and 16 <= dh <= 256, lambda: f"attention: head size {dh} must be a multiple of 16 up to 256")
+    _need(n_heads % Hkv == 0, lambda: f"attention: {n_heads} heads over {Hkv} key heads")
     ldq, ldo = _rows(q, "q"), (0 if out_packed else _rows(out, "out"))
     lib = _lib("attention")
     # (the kernel for portions takes the largest score for the largest product: a scale that is not positive goes the plain way)
@@ -599,7 +609,7 @@ def penalties(logits, ctx, ctx_start, repetition, frequency, presence, ngram):
     _need(ctx_start.shape[0] == R + 1, "penalties: ctx_start")
     for t, n in ((repetition, "repetition"), (frequency, "frequency"), (presence, "presence")):
         _dev(t, n, (torch.float32,), 1)
-        _need(t.shape[0] == R, f"penalties: {n}")
+        _need(t.shape[0] == R, lambda: f"penalties: {n}")
     _dev(ngram, "ngram", _I32, 1)
     _need(ngram.shape[0] == R, "penalties: ngram")
     _ok(_lib("sampling").dn_penalties(logits.data_ptr(), ld, R, V, ctx.data_ptr(), ctx_start.data_ptr(),
@@ -653,10 +663,10 @@ def norm_folded(w_rows, bias, gamma, beta):
 def _rows_or_packed(t, name, M, width):
     """The leading dimension of a bfloat16 [M, width] tensor in rows, or 0 for packed rows."""
     if isinstance(t, PackedMatrix):
-        _need(tuple(t.shape) == (M, width) and width % 32 == 0, f"{name}: packed rows of another shape")
+        _need(tuple(t.shape) == (M, width) and width % 32 == 0, lambda: f"{name}: packed rows of another shape")
         return 0
     _dev(t, name, (torch.bfloat16,), 2)
-    _need(tuple(t.shape) == (M, width), f"{name}: shape")
+    _need(tuple(t.shape) == (M, width), lambda: f"{name}: shape")
     return _rows(t, name)
 
 
@@ -676,7 +686,7 @@ def linear_norm_out(a, w, bias, residual, gamma, copy, stats):
     for v, name in ((bias, "bias"), (gamma, "gamma")):
         if v is not None:
             _dev(v, name, (torch.float32,), 1)
-            _need(v.is_contiguous() and v.shape[0] == N, f"linear_norm_out: {name}")
+            _need(v.is_contiguous() and v.shape[0] == N, lambda: f"linear_norm_out: {name}")
     _need(gamma is not None, "linear_norm_out: gamma")
     _ok(_lib("gemm").dn_gemm_norm_out(a.data_ptr(), lda, w.data_ptr(), _ptr(bias), residual.data_ptr(),
                                       _rows(residual, "residual"), M, N, K, gamma.data_ptr(), copy.data_ptr(),
@@ -705,7 +715,7 @@ def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None):
           "linear_norm_in: stats")
     for v, name in ((c1, "c1"), (c2, "c2")):
         _dev(v, name, (torch.float32,), 1)
-        _need(v.is_contiguous() and v.shape[0] == N, f"linear_norm_in: {name}")
+        _need(v.is_contiguous() and v.shape[0] == N, lambda: f"linear_norm_in: {name}")
     if kv is None:
         _need(tuple(out.shape) == (M, N), "linear_norm_in: out shape")
         args = (0, 0, 0, 0, 0, 0, 0, 0)

@@ -57,9 +57,6 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
                                                           int32_t* __restrict__ out) {
   __shared__ Best best_scratch[WAVES];
   __shared__ float f_scratch[WAVES];
-  __shared__ float seg_sum[THREADS];
-  __shared__ int winner;
-  __shared__ float winner_base, target_s;
   const int r = blockIdx.x, t = threadIdx.x;
   const float* row = logits + static_cast<size_t>(r) * ld;
   const float T = temperature[r];
@@ -80,67 +77,112 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
     return;
   }
 
-  // contiguous segments, so that the walk goes upwards through the vocabulary
-  const int seg = (V + THREADS - 1) / THREADS;
-  const int lo = min(V, t * seg), hi = min(V, lo + seg);
+  // The walk goes upwards through the vocabulary: the token is the first whose running sum of exp(z - max)
+  // reaches uniform x total.  The sums are made block by block (a block: BLK consecutive tokens, BLK a multiple
+  // of 64 such that there are at most MAXB blocks), a wave per block, 64 consecutive tokens per load; the first
+  // wave then finds the block in which the running sum reaches the target (each lane a run of consecutive
+  // blocks, a scan over the lanes, the lane whose run it is walks it), and walks that block 64 tokens at a time
+  // (a scan over the lanes again).  Every sum is taken in the order of the tokens.
+  constexpr int MAXB = 4096;
+  __shared__ float block_sum[MAXB];
+  const int wave = t / DN_WAVE, lane = t % DN_WAVE;
+  const int per64 = (V + 64 * MAXB - 1) / (64 * MAXB);      // loads of 64 tokens per block
+  const int BLK = 64 * per64;
+  const int NB = (V + BLK - 1) / BLK;
+  const float inv_T = 1.0f / T;
   float mx = -INFINITY;
-  for (int i0 = lo; i0 < hi; i0 += 8) {
+  for (int i0 = t; i0 < V; i0 += 8 * THREADS) {
     float v[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = row[min(i0 + j, V - 1)];
+    for (int j = 0; j < 8; ++j) v[j] = row[min(i0 + j * THREADS, V - 1)];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      float z = v[j] / T;
-      if (i0 + j < hi && z > mx) mx = z;
+      const float z = v[j] * inv_T;
+      if (i0 + j * THREADS < V && z > mx) mx = z;
     }
   }
   mx = block_max(mx, f_scratch);
-  float s = 0.f;
-  for (int i0 = lo; i0 < hi; i0 += 8) {
-    float v[8];
+  // (a multiplication by 1 / T and the hardware's exponential: one workgroup has a row's whole vocabulary to get
+  // through, and a division and a full-precision exp per token were most of its time)
+  auto weight = [&](int i) { return i < V ? __expf(fmaf(row[i], inv_T, -mx)) : 0.f; };
+  // an inclusive scan over the wave's lanes, in lane order
+  auto scan = [&](float x) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = row[min(i0 + j, V - 1)];
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-      if (i0 + j < hi) s += expf(v[j] / T - mx);
-  }
-  seg_sum[t] = s;
-  __syncthreads();
-  if (t == 0) {
-    float total = 0.f;
-    for (int k = 0; k < THREADS; ++k) total += seg_sum[k];
-    float target = uniform[r] * total;
-    float run = 0.f;
-    int w = -1;
-    float base = 0.f;
-    for (int k = 0; k < THREADS; ++k) {
-      float next = run + seg_sum[k];
-      if (w < 0 && next >= target && min(V, k * seg) < V) {
-        w = k;
-        base = run;
-      }
-      run = next;
+    for (int d = 1; d < DN_WAVE; d <<= 1) {
+      const float o = __shfl_up(x, d, DN_WAVE);
+      if (lane >= d) x += o;
     }
-    winner = w;
-    winner_base = base;
-    target_s = target;
+    return x;
+  };
+  for (int b0 = wave; b0 < NB; b0 += 4 * WAVES) {
+    float e[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int blk = b0 + u * WAVES;
+      e[u] = 0.f;
+      if (blk < NB)
+        for (int k = 0; k < per64; ++k) e[u] += weight(blk * BLK + k * 64 + lane);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int blk = b0 + u * WAVES;
+      const float sum = wave_sum(e[u]);      // (one fixed order, whatever the batch)
+      if (blk < NB && lane == 0) block_sum[blk] = sum;
+    }
   }
   __syncthreads();
-  if (winner < 0) {
-    if (t == 0) out[r] = V - 1;
-    return;
-  }
-  if (t == winner) {
-    float u = target_s - winner_base;
-    int pick = hi - 1;
-    for (int i = lo; i < hi; ++i) {
-      u -= expf(row[i] / T - mx);
-      if (u <= 0.f) {
-        pick = i;
+  if (wave == 0) {
+    const int per = (NB + DN_WAVE - 1) / DN_WAVE;      // consecutive blocks per lane
+    float mine = 0.f;
+    for (int j = 0; j < per; ++j) {
+      const int blk = lane * per + j;
+      if (blk < NB) mine += block_sum[blk];
+    }
+    const float incl = scan(mine);
+    const float total = __shfl(incl, DN_WAVE - 1, DN_WAVE);
+    const float target = uniform[r] * total;
+    const unsigned long long reached = __ballot(incl >= target && lane * per < NB);
+    int found = -1;
+    float base = 0.f;
+    if (reached != 0ull) {
+      const int first = __ffsll(static_cast<long long>(reached)) - 1;
+      const float before = __shfl_up(incl, 1, DN_WAVE);      // the sum of the lanes before (lane 0: nothing)
+      if (lane == first) {
+        float run = lane == 0 ? 0.f : before;
+        for (int j = 0; j < per; ++j) {
+          const int blk = lane * per + j;
+          if (blk >= NB) break;
+          // (the run's last block, if rounding lets this walk end short of what the scan said)
+          found = blk;
+          base = run;
+          const float next = run + block_sum[blk];
+          if (next >= target) break;
+          run = next;
+        }
+      }
+    }
+    // the wave goes on alone: what lane `first` found comes to the others through the exchange below
+    const int src = reached != 0ull ? __ffsll(static_cast<long long>(reached)) - 1 : 0;
+    found = __shfl(found, src, DN_WAVE);
+    base = __shfl(base, src, DN_WAVE);
+    if (found < 0) {
+      if (lane == 0) out[r] = V - 1;
+      return;
+    }
+    float run = base;
+    int pick = min(V, (found + 1) * BLK) - 1;      // the block's last token, if rounding lets the walk run out
+    for (int k = 0; k < per64; ++k) {
+      const int i = found * BLK + k * 64 + lane;
+      const float x = weight(i);
+      const float cum = run + scan(x);
+      const unsigned long long hit = __ballot(cum >= target && i < V);
+      if (hit != 0ull) {
+        pick = found * BLK + k * 64 + __ffsll(static_cast<long long>(hit)) - 1;
         break;
       }
+      run = __shfl(cum, DN_WAVE - 1, DN_WAVE);
     }
-    out[r] = pick;
+    if (lane == 0) out[r] = pick;
   }
 }
 

@@ -64,17 +64,28 @@ class Sampler:
         else:
             temps = [0.0 if p.greedy else p.effective_temperature for p in params]
             us = [0.0 if p.greedy else uniform(s, n_) for p, s, n_ in zip(params, seeds, counters)]
-            tu = torch.tensor([temps, us], dtype=torch.float32, device=dev)      # one copy for both
+            tu = self._to_device([temps, us], torch.float32)      # one copy for both
         t_dev, u_dev = tu[0], tu[1]
         ops.sample(logits, t_dev, u_dev, both[:R])
         more = None
         if restricted:
             top_p = [params[r].top_p if params[r].top_p is not None else 1.0 for r in restricted]
-            ints = torch.tensor([restricted, [params[r].top_k or 0 for r in restricted]], dtype=torch.int32, device=dev)
-            ps = torch.tensor(top_p, dtype=torch.float32, device=dev)
+            ints = self._to_device([restricted, [params[r].top_k or 0 for r in restricted]], torch.int32)
+            ps = self._to_device(top_p, torch.float32)
             ops.sample_top(logits, ints[0], t_dev, u_dev, ints[1], ps, both[:R], both[R:])
             more = (logits, restricted, top_p, t_dev, u_dev)
         return Pending(both, R, more, *self._bring_home(both))
+
+    def _to_device(self, values, dtype):
+        """A small table for the sampling kernels.  Through pinned memory and without waiting: a copy from
+        ordinary host memory holds the host until the stream has run dry, and with it the step that the engine
+        launches ahead."""
+        host = torch.tensor(values, dtype=dtype)
+        if self.device.type != "cuda":
+            return host.to(self.device)
+        pinned = torch.empty(host.shape, dtype=dtype, pin_memory=True)
+        pinned.copy_(host)
+        return pinned.to(self.device, non_blocking=True)
 
     @staticmethod
     def _bring_home(both):

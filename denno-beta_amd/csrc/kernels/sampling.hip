@@ -429,12 +429,16 @@ __global__ __launch_bounds__(THREADS) void sample_full_kernel(const float* __res
                                                                const float* __restrict__ temperature,
                                                                const float* __restrict__ uniform,
                                                                const float* __restrict__ top_p,
+                                                               const int32_t* __restrict__ only,
                                                                uint32_t* __restrict__ work,
                                                                int32_t* __restrict__ out) {
   __shared__ float seg_sum[THREADS];
   __shared__ float seg_base[THREADS];
   __shared__ float total_s;
   __shared__ int first_s;
+  // only: a flag per listed row (none: all are meant); a row whose flag is 0 is left as it is, so that the
+  // caller can launch this behind sample_top_kernel without reading what that left undecided
+  if (only != nullptr && only[blockIdx.x] == 0) return;
   const int t = threadIdx.x;
   const int r = rows[blockIdx.x];
   const float* row = logits + static_cast<size_t>(r) * ld;
@@ -567,11 +571,11 @@ extern "C" int dn_sample_top(const float* logits, int ld, int n_rows, int V, con
 
 // work: 3 * n_pad 32-bit words per listed row, n_pad the power of two from V up
 extern "C" int dn_sample_full(const float* logits, int ld, int n_rows, int V, int n_pad, const int32_t* rows,
-                              const float* temperature, const float* uniform, const float* top_p, void* work,
-                              int32_t* out, hipStream_t stream) {
+                              const float* temperature, const float* uniform, const float* top_p,
+                              const int32_t* only, void* work, int32_t* out, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (V < 1 || ld < V || n_pad < V || n_pad < 2 || (n_pad & (n_pad - 1)) != 0) return DN_ERR_SHAPE;
   hipLaunchKernelGGL(sampling::sample_full_kernel, dim3(n_rows), dim3(sampling::THREADS), 0, stream, logits, ld, V,
-                     n_pad, rows, temperature, uniform, top_p, static_cast<uint32_t*>(work), out);
+                     n_pad, rows, temperature, uniform, top_p, only, static_cast<uint32_t*>(work), out);
   return dn_launch_status();
 }

@@ -119,7 +119,7 @@ def _declare(name, lib):
             "dn_sample": [P, I, I, I, P, P, P, P],
             "dn_penalties": [P, I, I, I, P, P, P, P, P, P, P],
             "dn_sample_top": [P, I, I, I, P, P, P, P, P, P, P, P],
-            "dn_sample_full": [P, I, I, I, I, P, P, P, P, P, P, P],
+            "dn_sample_full": [P, I, I, I, I, P, P, P, P, P, P, P, P],
         },
     }[name]
     for fn, args in sigs.items():
@@ -578,9 +578,11 @@ def sample_top(logits, rows, temperature, uniform, top_k, top_p, out, undecided)
     return out
 
 
-def sample_full(logits, rows, temperature, uniform, top_p, out):
+def sample_full(logits, rows, temperature, uniform, top_p, out, only=None):
     """top-p over the whole sorted vocabulary for the rows listed in `rows` (each with temperature
-    > 0), then the walk with uniform[row]: what `sample_top` leaves undecided."""
+    > 0), then the walk with uniform[row]: what `sample_top` leaves undecided.  only: int32, a flag per listed
+    row, on the device; a row whose flag is 0 keeps its token (`sample_top`'s `undecided`: launched behind it, the
+    rows that it left undecided are done without the host reading which they are)."""
     _dev(logits, "logits", (torch.float32,), 2), _dev(rows, "rows", _I32, 1)
     _dev(temperature, "temperature", (torch.float32,), 1), _dev(uniform, "uniform", (torch.float32,), 1)
     _dev(top_p, "top_p", (torch.float32,), 1), _dev(out, "out", _I32, 1)
@@ -588,14 +590,17 @@ def sample_full(logits, rows, temperature, uniform, top_p, out):
     ld = _rows(logits, "logits")
     n = rows.shape[0]
     _need(top_p.shape[0] == n, "sample_full: one top_p per listed row")
+    if only is not None:
+        _dev(only, "only", _I32, 1)
+        _need(only.shape[0] == n and only.is_contiguous(), "sample_full: one flag per listed row")
     _need(temperature.shape[0] == R and uniform.shape[0] == R and out.shape[0] == R, "sample_full: rows")
     n_pad = 2
     while n_pad < V:
         n_pad *= 2
     work = torch.empty(n * 3 * n_pad, dtype=torch.int32, device=logits.device)
     _ok(_lib("sampling").dn_sample_full(logits.data_ptr(), ld, n, V, n_pad, rows.data_ptr(), temperature.data_ptr(),
-                                        uniform.data_ptr(), top_p.data_ptr(), work.data_ptr(), out.data_ptr(),
-                                        _stream()), "sample_full")
+                                        uniform.data_ptr(), top_p.data_ptr(), _ptr(only), work.data_ptr(),
+                                        out.data_ptr(), _stream()), "sample_full")
     return out
 
 

@@ -11,7 +11,7 @@ from typing import List, Sequence
 import torch
 
 from ..kernels import ops
-from .params import SamplingParams
+from .params import TOP_CANDIDATES, SamplingParams
 from .rng import uniform
 
 
@@ -33,7 +33,7 @@ class Sampler:
         device as soon as the kernels have run, and is final if `Pending.final`."""
         R = logits.shape[0]
         if R == 0:
-            return Pending(None, 0, None)
+            return Pending(None, 0)
         dev = self.device
         if any(p.has_penalties for p in params):
             starts, flat = [0], []
@@ -67,14 +67,18 @@ class Sampler:
             tu = self._to_device([temps, us], torch.float32)      # one copy for both
         t_dev, u_dev = tu[0], tu[1]
         ops.sample(logits, t_dev, u_dev, both[:R])
-        more = None
         if restricted:
             top_p = [params[r].top_p if params[r].top_p is not None else 1.0 for r in restricted]
             ints = self._to_device([restricted, [params[r].top_k or 0 for r in restricted]], torch.int32)
             ps = self._to_device(top_p, torch.float32)
             ops.sample_top(logits, ints[0], t_dev, u_dev, ints[1], ps, both[:R], both[R:])
-            more = (logits, restricted, top_p, t_dev, u_dev)
-        return Pending(both, R, more, *self._bring_home(both))
+            if logits.shape[1] > TOP_CANDIDATES and any(params[r].top_k is None for r in restricted):
+                # top-p alone whose cut lies beyond the 2,048 largest: the whole vocabulary, sorted.  Launched
+                # behind the kernel that says which rows these are, and which it does not touch the others of:
+                # the host need not read the flags first, so the step's tokens are final once the kernels
+                # have run and the next step can be launched ahead
+                ops.sample_full(logits, ints[0], t_dev, u_dev, ps, both[:R], only=both[R:])
+        return Pending(both, R, *self._bring_home(both))
 
     def _to_device(self, values, dtype):
         """A small table for the sampling kernels.  Through pinned memory and without waiting: a copy from
@@ -105,30 +109,16 @@ class Sampler:
         """Waits for a launched sampling; -> the rows' tokens."""
         if pending.rows == 0:
             return []
-        R = pending.rows
         if pending.filled is not None:
             pending.filled.synchronize()
-        host = pending.host.tolist()
-        tokens = host[:R]
-        if pending.more is None:
-            return tokens
-        logits, restricted, top_p, t_dev, u_dev = pending.more
-        undecided = [j for j in range(len(restricted)) if host[R + j]]
-        if undecided:
-            # top-p alone whose cut lies beyond the 2,048 largest: the whole vocabulary, sorted
-            dev = self.device
-            rows = torch.tensor([restricted[j] for j in undecided], dtype=torch.int32, device=dev)
-            ps = torch.tensor([top_p[j] for j in undecided], dtype=torch.float32, device=dev)
-            tokens = ops.sample_full(logits, rows, t_dev, u_dev, ps, pending.both[:R]).tolist()
-        return tokens
+        return pending.host.tolist()[:pending.rows]
 
 
 class Pending:
-    """A launched sampling: `both[:rows]` are the tokens on the device.  final: no row can still change
-    (rows with top-k or top-p may, when `read` finds their cut beyond the candidates)."""
+    """A launched sampling: `both[:rows]` are the tokens on the device, final as soon as the kernels have run."""
 
-    def __init__(self, both, rows, more, host=None, filled=None):
-        self.both, self.rows, self.more = both, rows, more
+    def __init__(self, both, rows, host=None, filled=None):
+        self.both, self.rows = both, rows
         self.host, self.filled = host, filled      # both on the host, and the event that says so (None: no wait)
 
     @property
@@ -137,4 +127,4 @@ class Pending:
 
     @property
     def final(self):
-        return self.more is None
+        return True

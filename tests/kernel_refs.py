@@ -188,9 +188,11 @@ def sample_top(logits, rows, temperature, uniform, top_k, top_p, out, undecided)
     return out
 
 
-def sample_full(logits, rows, temperature, uniform, top_p, out):
+def sample_full(logits, rows, temperature, uniform, top_p, out, only=None):
     from plain import sampler_plain as sp
     for j, r in enumerate(rows.tolist()):
+        if only is not None and int(only[j]) == 0:
+            continue
         p = float(top_p[j])
         out[r] = sp.top_k_top_p(logits[r].tolist(), float(temperature[r]), None, None if p >= 1.0 else p,
                                 float(uniform[r]))

@@ -318,7 +318,11 @@ def test_running_ahead_changes_no_token(model_folders, tmp_path, dtype):
     first = engine_for(model_folders("B", dtype), dtype, "cuda:0", run_ahead=False).generate(prompts[:1], greedy[:1])[0]
     folder = write_model_folder(str(tmp_path / "eos"), dict(cfg, eos_token_id=first[9]), seed, dtype)
     warm = [SamplingParams(max_tokens=m, temperature=0.9, seed=5 + i) for i, m in enumerate((30, 7, 45, 12, 1, 60, 25))]
-    for params in (greedy, warm):
+    # top-k and top-p, among them top-p alone (whose rows a second kernel may have to finish: on the device, without
+    # the host in between, so that these steps run ahead as well)
+    cut = [SamplingParams(max_tokens=m, temperature=1.1, seed=9 + i, top_k=(None, 5, 40)[i % 3], top_p=(0.9, None, 0.7)[i % 3])
+           for i, m in enumerate((30, 7, 45, 12, 1, 60, 25))]
+    for params in (greedy, warm, cut):
         for kw in (dict(cache_tokens=1024, max_live=8), dict(cache_tokens=192, max_live=3)):
             want_engine = engine_for(folder, dtype, "cuda:0", run_ahead=False, **kw)
             want = want_engine.generate(prompts, params)

@@ -763,6 +763,13 @@ def test_top_p_beyond_the_2048_largest_takes_the_whole_vocabulary():
     for i in range(0, n - 1, 4):
         tok, whole = SP.top_p_alone(row.tolist(), 1.0, 0.9999, float(u[i]))
         assert whole and tok == got[i], i
+    # the second kernel launched behind the first with the first's own flags: the rows left undecided get the
+    # same tokens, and the row that was decided keeps its token (it is not even looked at)
+    again = torch.full((n,), -1, dtype=torch.int32, device=DEV)
+    flags = torch.full((n,), -1, dtype=torch.int32, device=DEV)
+    ops().sample_top(logits, rows, temp, u, i32([0] * n), ps, again, flags)
+    ops().sample_full(logits, rows, temp, u, ps, again, only=flags)
+    assert again.tolist() == got
     # the sampler does both steps, and with top_p = 1 takes the plain walk
     sp = SamplingParams(temperature=1.0, top_p=0.9999, seed=3)
     toks = Sampler(torch.device(DEV)).sample(logits[:4].clone(), [sp] * 4, [3] * 4, [0, 1, 2, 3], [[]] * 4)

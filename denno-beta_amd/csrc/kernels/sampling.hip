@@ -268,14 +268,24 @@ __global__ __launch_bounds__(THREADS) void sample_top_kernel(const float* __rest
                                                               const int32_t* __restrict__ top_k,
                                                               const float* __restrict__ top_p,
                                                               int32_t* __restrict__ out,
-                                                              int32_t* __restrict__ undecided) {
+                                                              int32_t* __restrict__ undecided,
+                                                              uint32_t* __restrict__ work) {
   __shared__ uint32_t cand_key[CAND];
   __shared__ int32_t cand_idx[CAND];
-  __shared__ float cand_e[CAND];
+  __shared__ __attribute__((aligned(16))) float cand_e[CAND];
+  __shared__ __attribute__((aligned(16))) float cand_q[CAND];
+  __shared__ float total_s;
+  // the 256 bins in eight copies, a lane's by its number, 257 apart (so that the copies lie in different
+  // banks): in the first pass nearly every key goes to one of two or three bins, and additions to one address
+  // wait for each other
+  constexpr int COPIES = 8, HSTRIDE = 257;
+  __shared__ int hist_copy[COPIES * HSTRIDE];
   __shared__ int hist[256];
-  __shared__ int cnt_gt[THREADS], cnt_eq[THREADS];
+  constexpr int EQ_LIST = 2048;
+  __shared__ int eq_idx[EQ_LIST];
+  __shared__ int cnt_eq[THREADS];
   __shared__ uint32_t sel_prefix;
-  __shared__ int sel_remaining, eq_quota;
+  __shared__ int sel_remaining, n_gt, n_eq;
   const int t = threadIdx.x;
   const int r = rows[blockIdx.x];
   const float* row = logits + static_cast<size_t>(r) * ld;
@@ -283,86 +293,157 @@ __global__ __launch_bounds__(THREADS) void sample_top_kernel(const float* __rest
   int k = top_k[blockIdx.x];
   const int m = min(min(k > 0 ? k : CAND, CAND), V);
 
+  // 0. every key once (one division per token), into `keys`; a thread writes the keys that it reads in the
+  // passes below, eight loads asked for at a time (one workgroup has a row's whole vocabulary to get through on
+  // one CU, several times: it counts instructions)
+  uint32_t* keys = work + static_cast<size_t>(blockIdx.x) * V;
+  for (int i0 = t; i0 < V; i0 += 8 * THREADS) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = row[min(i0 + j * THREADS, V - 1)];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (i0 + j * THREADS < V) keys[i0 + j * THREADS] = order_key(v[j] / T);
+  }
   // 1. the m-th largest key, by four passes over 8 bits each
   if (t == 0) {
     sel_prefix = 0u;
     sel_remaining = m;
+    n_gt = 0;
+    n_eq = 0;
   }
   for (int pass = 0; pass < 4; ++pass) {
     const int shift = 24 - 8 * pass;
-    if (t < 256) hist[t] = 0;
+    for (int i = t; i < COPIES * HSTRIDE; i += THREADS) hist_copy[i] = 0;
     __syncthreads();
     const uint32_t prefix = sel_prefix;
     const uint32_t mask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
-    for (int i = t; i < V; i += THREADS) {
-      uint32_t key = order_key(row[i] / T);
-      if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 0xff], 1);
+    for (int i0 = t; i0 < V; i0 += 8 * THREADS) {
+      uint32_t key[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) key[j] = keys[min(i0 + j * THREADS, V - 1)];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (i0 + j * THREADS < V && (key[j] & mask) == prefix)
+          atomicAdd(&hist_copy[(t % COPIES) * HSTRIDE + ((key[j] >> shift) & 0xff)], 1);
     }
     __syncthreads();
-    if (t == 0) {
-      int remaining = sel_remaining;
-      int b = 255;
-      for (; b > 0; --b) {
-        if (hist[b] >= remaining) break;
-        remaining -= hist[b];
+    if (t < 256) {
+      int n = 0;
+#pragma unroll
+      for (int c = 0; c < COPIES; ++c) n += hist_copy[c * HSTRIDE + t];
+      hist[t] = n;
+    }
+    __syncthreads();
+    if (t < DN_WAVE) {
+      // the bin in which the count from the top reaches what remains: lane l holds bins 255 - 4 l .. 252 - 4 l,
+      // a scan over the lanes counts from the top, and the first lane that reaches the mark looks among its four
+      const int remaining = sel_remaining;
+      int own[4], mine = 0;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        own[q] = hist[255 - 4 * t - q];
+        mine += own[q];
       }
-      sel_prefix = prefix | (static_cast<uint32_t>(b) << shift);
-      sel_remaining = remaining;
+      int incl = mine;
+#pragma unroll
+      for (int d = 1; d < DN_WAVE; d <<= 1) {
+        const int o = __shfl_up(incl, d, DN_WAVE);
+        if (t >= d) incl += o;
+      }
+      const unsigned long long reached = __ballot(incl >= remaining);
+      // (the whole row counts at least `remaining` keys in this pass, so the last lane reaches the mark)
+      const int first = reached != 0ull ? __ffsll(static_cast<long long>(reached)) - 1 : DN_WAVE - 1;
+      if (t == first) {
+        int left = remaining - (incl - mine), b = 255 - 4 * t;
+#pragma unroll
+        for (int q = 0; q < 3; ++q) {
+          if (own[q] >= left) break;
+          left -= own[q];
+          b -= 1;
+        }
+        sel_prefix = prefix | (static_cast<uint32_t>(b) << shift);
+        sel_remaining = left;
+      }
     }
     __syncthreads();
   }
   const uint32_t thr = sel_prefix;
-  if (t == 0) eq_quota = sel_remaining;   // how many keys equal to thr belong to the m
-  // 2. the candidates, in order of their index
-  const int seg = (V + THREADS - 1) / THREADS;
-  const int lo = min(V, t * seg), hi = min(V, lo + seg);
-  int ngt = 0, neq = 0;
-  for (int i = lo; i < hi; ++i) {
-    uint32_t key = order_key(row[i] / T);
-    ngt += key > thr;
-    neq += key == thr;
-  }
-  cnt_gt[t] = ngt;
-  cnt_eq[t] = neq;
+  const int quota = sel_remaining;       // how many keys equal to thr belong to the m
+  const int greater = m - quota;         // and how many keys are greater
+  // 2. the candidates: every key above thr, in any place (the sort below puts them in order), and of the keys
+  // equal to thr the `quota` with the lowest indices: these are listed first and ranked among themselves
   for (int i = t; i < CAND; i += THREADS) {
     cand_key[i] = 0u;
     cand_idx[i] = 0x7fffffff;
   }
   __syncthreads();
-  if (t == 0) {
-    int a = 0, b = 0;
-    for (int i = 0; i < THREADS; ++i) {
-      int g = cnt_gt[i], e = cnt_eq[i];
-      cnt_gt[i] = a;
-      cnt_eq[i] = b;
-      a += g;
-      b += e;
-    }
-  }
-  __syncthreads();
-  {
-    const int quota = eq_quota;
-    int eq_rank = cnt_eq[t];
-    int dst = cnt_gt[t] + min(eq_rank, quota);
-    for (int i = lo; i < hi; ++i) {
-      uint32_t key = order_key(row[i] / T);
-      bool take = key > thr;
-      if (key == thr) {
-        take = eq_rank < quota;
-        eq_rank += 1;
-      }
-      if (take) {
-        cand_key[dst] = key;
-        cand_idx[dst] = i;
-        dst += 1;
+  for (int i0 = t; i0 < V; i0 += 8 * THREADS) {
+    uint32_t key[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) key[j] = keys[min(i0 + j * THREADS, V - 1)];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int i = i0 + j * THREADS;
+      if (i >= V) continue;
+      if (key[j] > thr) {
+        const int at = atomicAdd(&n_gt, 1);
+        cand_key[at] = key[j];
+        cand_idx[at] = i;
+      } else if (key[j] == thr) {
+        const int at = atomicAdd(&n_eq, 1);
+        if (at < EQ_LIST) eq_idx[at] = i;
       }
     }
   }
   __syncthreads();
-  // 3. bitonic sort: key descending, equal keys by ascending index
-  for (int size = 2; size <= CAND; size <<= 1) {
+  const int equals = n_eq;
+  if (equals <= EQ_LIST) {
+    for (int j = t; j < equals; j += THREADS) {
+      const int mine = eq_idx[j];
+      int rank = 0;
+      for (int o = 0; o < equals; ++o) rank += eq_idx[o] < mine;
+      if (rank < quota) {
+        cand_key[greater + rank] = thr;
+        cand_idx[greater + rank] = mine;
+      }
+    }
+  } else {
+    // more equal keys than the list holds (a row of nearly equal logits): in the order of their indices, a
+    // thread a stretch of the row, one thread the stretches' counts
+    __syncthreads();      // (every thread's keys are in memory)
+    const int seg = (V + THREADS - 1) / THREADS;
+    const int lo = min(V, t * seg), hi = min(V, lo + seg);
+    int mine = 0;
+    for (int i = lo; i < hi; ++i) mine += keys[i] == thr;
+    cnt_eq[t] = mine;
+    __syncthreads();
+    if (t == 0) {
+      int before = 0;
+      for (int i = 0; i < THREADS; ++i) {
+        const int e = cnt_eq[i];
+        cnt_eq[i] = before;
+        before += e;
+      }
+    }
+    __syncthreads();
+    int rank = cnt_eq[t];
+    for (int i = lo; i < hi && rank < quota; ++i) {
+      if (keys[i] == thr) {
+        cand_key[greater + rank] = thr;
+        cand_idx[greater + rank] = i;
+        rank += 1;
+      }
+    }
+  }
+  __syncthreads();
+  // 3. bitonic sort: key descending, equal keys by ascending index; of the first n_sort places (the others
+  // hold nothing)
+  int n_sort = 2;
+  while (n_sort < m) n_sort <<= 1;
+  for (int size = 2; size <= n_sort; size <<= 1) {
     for (int stride = size >> 1; stride > 0; stride >>= 1) {
-      for (int i = t; i < CAND / 2; i += THREADS) {
+      for (int i = t; i < n_sort / 2; i += THREADS) {
         int a = 2 * i - (i & (stride - 1));
         int b = a + stride;
         bool descending = (a & size) == 0;
@@ -379,21 +460,65 @@ __global__ __launch_bounds__(THREADS) void sample_top_kernel(const float* __rest
       __syncthreads();
     }
   }
-  // 4. softmax numerators, cut, walk: in the list's order, one thread, as the reference does it
+  // 4. softmax numerators, cut, walk: every sum in the list's order, one addition after the other as the
+  // reference makes them, by one thread.  It reads sixteen numbers at a time (four 16-byte reads, asked for
+  // together) and looks only after every sixteen additions whether the running sum has reached its mark (it
+  // never goes back: the numbers are not negative), then finds the place among those sixteen: a thread that
+  // fetched each number by itself and tested after each spent a hundred cycles per number, two thousand times
+  // a sum.
   const float z0 = key_value(cand_key[0]);
   for (int i = t; i < m; i += THREADS) cand_e[i] = expf(key_value(cand_key[i]) - z0);
   __syncthreads();
+  const float p = top_p[blockIdx.x];
+  // x[i0 .. i0 + 15], those from n on as zeros (adding 0 changes nothing)
+  auto sixteen = [](const float* x, int i0, int n, float* v) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float4 f = *reinterpret_cast<const float4*>(x + i0 + 4 * q);
+      v[4 * q] = f.x, v[4 * q + 1] = f.y, v[4 * q + 2] = f.z, v[4 * q + 3] = f.w;
+    }
+    if (i0 + 16 > n) {
+#pragma unroll
+      for (int j = 0; j < 16; ++j)
+        if (i0 + j >= n) v[j] = 0.f;
+    }
+  };
+  auto sum_of = [&](int n) {
+    float total = 0.f;
+    for (int i0 = 0; i0 < n; i0 += 16) {
+      float v[16];
+      sixteen(cand_e, i0, n, v);
+#pragma unroll
+      for (int j = 0; j < 16; ++j) total += v[j];
+    }
+    return total;
+  };
+  if (p < 1.0f) {
+    if (t == 0) total_s = sum_of(m);
+    __syncthreads();
+    const float total = total_s;
+    for (int i = t; i < m; i += THREADS) cand_q[i] = cand_e[i] / total;      // (each share by the same division)
+    __syncthreads();
+  }
   if (t == 0) {
     int keep = m;
-    const float p = top_p[blockIdx.x];
     if (p < 1.0f) {
-      float total = 0.f;
-      for (int i = 0; i < m; ++i) total += cand_e[i];
       float cum = 0.f;
-      for (int i = 0; i < m; ++i) {
-        cum += cand_e[i] / total;
+      for (int i0 = 0; i0 < m; i0 += 16) {
+        float v[16];
+        sixteen(cand_q, i0, m, v);
+        const float before = cum;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) cum += v[j];
         if (cum >= p) {
-          keep = i + 1;
+          float again = before;
+          for (int j = 0; j < 16; ++j) {
+            again += v[j];
+            if (again >= p) {
+              keep = i0 + j + 1;
+              break;
+            }
+          }
           break;
         }
       }
@@ -401,18 +526,27 @@ __global__ __launch_bounds__(THREADS) void sample_top_kernel(const float* __rest
     // top-p alone over a vocabulary larger than the subset: a cut that is not reached before the
     // subset's last member needs the tail (sampler.rs:425-433)
     undecided[blockIdx.x] = (k <= 0 && V > CAND && keep == m) ? 1 : 0;
-    float total = 0.f;
-    for (int i = 0; i < keep; ++i) total += cand_e[i];
-    float u = uniform[r] * total;
-    int pick = cand_idx[keep - 1];
-    for (int i = 0; i < keep; ++i) {
-      u -= cand_e[i];
+    float u = uniform[r] * sum_of(keep);
+    int place = keep - 1;
+    for (int i0 = 0; i0 < keep; i0 += 16) {
+      float v[16];
+      sixteen(cand_e, i0, keep, v);
+      const float before = u;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) u -= v[j];
       if (u <= 0.f) {
-        pick = cand_idx[i];
+        float again = before;
+        for (int j = 0; j < 16; ++j) {
+          again -= v[j];
+          if (again <= 0.f) {
+            place = min(i0 + j, keep - 1);
+            break;
+          }
+        }
         break;
       }
     }
-    out[r] = pick;
+    out[r] = cand_idx[place];
   }
 }
 
@@ -561,11 +695,12 @@ extern "C" int dn_penalties(float* logits, int ld, int R, int V, const int32_t* 
 
 extern "C" int dn_sample_top(const float* logits, int ld, int n_rows, int V, const int32_t* rows,
                              const float* temperature, const float* uniform, const int32_t* top_k,
-                             const float* top_p, int32_t* out, int32_t* undecided, hipStream_t stream) {
+                             const float* top_p, int32_t* out, int32_t* undecided, void* work,
+                             hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  if (V < 1 || ld < V) return DN_ERR_SHAPE;
+  if (V < 1 || ld < V || work == nullptr) return DN_ERR_SHAPE;      // work: V 32-bit words per listed row
   hipLaunchKernelGGL(sampling::sample_top_kernel, dim3(n_rows), dim3(sampling::THREADS), 0, stream, logits, ld, V,
-                     rows, temperature, uniform, top_k, top_p, out, undecided);
+                     rows, temperature, uniform, top_k, top_p, out, undecided, static_cast<uint32_t*>(work));
   return dn_launch_status();
 }
 

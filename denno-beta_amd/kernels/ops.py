@@ -118,7 +118,7 @@ def _declare(name, lib):
         "sampling": {
             "dn_sample": [P, I, I, I, P, P, P, P],
             "dn_penalties": [P, I, I, I, P, P, P, P, P, P, P],
-            "dn_sample_top": [P, I, I, I, P, P, P, P, P, P, P, P],
+            "dn_sample_top": [P, I, I, I, P, P, P, P, P, P, P, P, P],
             "dn_sample_full": [P, I, I, I, I, P, P, P, P, P, P, P, P],
         },
     }[name]
@@ -572,9 +572,10 @@ def sample_top(logits, rows, temperature, uniform, top_k, top_p, out, undecided)
     _need(top_k.shape[0] == n and top_p.shape[0] == n and undecided.shape[0] == n,
           "sample_top: one top_k, top_p and undecided per listed row")
     _need(temperature.shape[0] == R and uniform.shape[0] == R and out.shape[0] == R, "sample_top: rows")
+    work = torch.empty(max(1, n) * V, dtype=torch.int32, device=logits.device)      # every row's keys, made once
     _ok(_lib("sampling").dn_sample_top(logits.data_ptr(), ld, n, V, rows.data_ptr(), temperature.data_ptr(),
                                        uniform.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), out.data_ptr(),
-                                       undecided.data_ptr(), _stream()), "sample_top")
+                                       undecided.data_ptr(), work.data_ptr(), _stream()), "sample_top")
     return out
 
 

@@ -736,6 +736,42 @@ def test_sample_top_and_penalties():
     assert torch.allclose(l.cpu(), want, atol=1e-6) and l[2, 8].item() == float("-inf")
 
 
+@pytest.mark.parametrize("V,levels", [(6000, 3), (6000, 40), (50257, 7), (3000, 1), (2100, 2)])
+def test_sample_top_with_many_equal_logits(V, levels):
+    """Logits that take few different values, so that many keys are equal to the one at the cut: of these the
+    ones with the lowest indices belong to the candidates, as the plain sampler sorts (value descending, then
+    index ascending).  With 3 levels over 6,000 tokens some 2,000 tie at the cut, with 1 or 2 levels more than the
+    2,048 that the kernel lists before it ranks them (it then walks the row in stretches)."""
+    from denno_beta_amd.sampling import uniform
+    g = torch.Generator().manual_seed(V + levels)
+    logits = (torch.randint(0, levels, (6, V), generator=g).float() * 0.5).to(DEV).contiguous()
+    rows = i32([0, 1, 2, 3, 4, 5])
+    ks, ps = i32([1, 7, 300, 2048, 0, 0]), torch.tensor([1.0, 0.9, 1.0, 0.95, 0.5, 0.02], device=DEV)
+    temp = torch.full((6,), 0.9, device=DEV)
+    for trial in range(3):
+        u = torch.tensor([uniform(trial, i) for i in range(6)], device=DEV)
+        out = torch.full((6,), -1, dtype=torch.int32, device=DEV)
+        undecided = torch.full((6,), -1, dtype=torch.int32, device=DEV)
+        ops().sample_top(logits, rows, temp, u, ks, ps, out, undecided)
+        want_und = torch.zeros(6, dtype=torch.int32)
+        want = R.sample_top(logits.cpu(), rows.cpu(), temp.cpu(), u.cpu(), ks.cpu(), ps.cpu(),
+                            torch.full((6,), -1, dtype=torch.int32), want_und)
+        assert undecided.tolist() == want_und.tolist(), trial
+        for i in range(6):
+            if want_und[i] or out[i].item() == want[i].item():
+                continue
+            # The walk over hundreds of equal numbers in 32-bit may end one place from where the plain sampler's
+            # (in 64-bit) ends: a neighbour in the sorted list is right too, anything else is not
+            order = sorted(range(V), key=lambda j: (-float(logits[i, j]), j))
+            at = order.index(want[i].item())
+            assert out[i].item() in order[max(0, at - 1):at + 2], (trial, i, out[i].item(), want[i].item())
+    assert out[0].item() == int(logits[0].argmax())      # top_k 1: the first of the largest
+    # top_k 7 of a row whose largest value is taken by hundreds of tokens: one of the seven with the lowest indices
+    if levels <= 7:
+        first7 = [j for j in range(V) if float(logits[1, j]) == float(logits[1].max())][:7]
+        assert out[1].item() in first7
+
+
 def test_top_p_beyond_the_2048_largest_takes_the_whole_vocabulary():
     """Flat logits over a vocabulary of 50,257 with top-p 0.9999: among the 2,048 largest the cut falls on
     the last, so the subset kernel must leave the row undecided and the kernel over the whole sorted

@@ -695,6 +695,28 @@ def test_sample_greedy_and_walk():
     assert out[0].item() == 0
 
 
+@pytest.mark.parametrize("V", [1, 17, 64, 65, 1000, 4097, 50257, 300001])
+def test_temperature_walk_at_other_vocabulary_sizes(V):
+    """The walk's place against the running sums in 64-bit: for every row and its uniform number u the token
+    picked is the first whose running share of the probability reaches u, to within what 32-bit sums can tell
+    (the share before the token is at most u, the share with it at least u, both with a margin of 1e-5).  Sizes
+    below, at and above a wave's 64 tokens, a block's worth, and one that needs blocks of more than 64 tokens."""
+    from denno_beta_amd.sampling import uniform
+    n = 16
+    logits = rnd(n, V, seed=V % 1000, scale=3.0)
+    temp = torch.tensor([0.3, 0.7, 1.0, 1.9] * 4, device=DEV)
+    u = torch.tensor([uniform(11, i) for i in range(n - 2)] + [0.0, 0.9999999], device=DEV)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    ops().sample(logits, temp, u, out)
+    z = logits.double().cpu() / temp.double().cpu()[:, None]
+    cum = torch.softmax(z, dim=1).cumsum(dim=1)
+    for r, tok in enumerate(out.tolist()):
+        assert 0 <= tok < V
+        before = float(cum[r, tok - 1]) if tok > 0 else 0.0
+        assert before <= float(u[r]) + 1e-5 and float(cum[r, tok]) >= float(u[r]) - 1e-5, (r, tok, before, float(cum[r, tok]), float(u[r]))
+    assert out[n - 2].item() == 0
+
+
 def test_sample_frequencies():
     # [0, 4] at T = 1: index 1 with probability 0.982 (sampler.rs:686-704), here over a row padded with -inf
     from denno_beta_amd.sampling import uniform

@@ -186,59 +186,81 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
   }
 }
 
-// One workgroup per row.  ctx holds the rows' contexts (prompt + generated) one after the
-// other; row r's is ctx[ctx_start[r] .. ctx_start[r+1]).  Each distinct token is handled by
-// the thread that holds its first occurrence, so no two threads write one logit in a phase.
+constexpr int HELD = 8192;      // tokens of a context that the penalties keep in the workgroup's memory (32 KB)
+
+// One workgroup per row.  Row r's context (prompt + generated) is ctx[ctx_begin[r] .. + ctx_len[r]): the
+// contexts one after the other, or each in its request's row of a table of token histories that lives on the
+// device.  Each distinct token is handled by the thread that holds its first occurrence, so no two threads
+// write one logit in a phase.
 __global__ __launch_bounds__(THREADS) void penalties_kernel(float* __restrict__ logits, int ld, int V,
                                                              const int32_t* __restrict__ ctx,
-                                                             const int32_t* __restrict__ ctx_start,
+                                                             const int32_t* __restrict__ ctx_begin,
+                                                             const int32_t* __restrict__ ctx_len,
                                                              const float* __restrict__ repetition,
                                                              const float* __restrict__ frequency,
                                                              const float* __restrict__ presence,
                                                              const int32_t* __restrict__ ngram) {
   const int r = blockIdx.x;
   float* row = logits + static_cast<size_t>(r) * ld;
-  const int32_t* c = ctx + ctx_start[r];
-  const int n = ctx_start[r + 1] - ctx_start[r];
+  const int32_t* c = ctx + ctx_begin[r];
+  const int n = ctx_len[r];
   const float rep = repetition[r], fq = frequency[r], pr = presence[r];
   const int ng = ngram[r];
-  if (rep != 1.0f || fq != 0.f || pr != 0.f) {
-    for (int i = threadIdx.x; i < n; i += THREADS) {
-      int tok = c[i];
-      if (tok < 0 || tok >= V) continue;
-      bool first = true;
-      int count = 0;
-      for (int j = 0; j < n; ++j) {
-        if (c[j] == tok) {
-          if (j < i) {
-            first = false;
-            break;
-          }
-          count += 1;
+  const bool counts = rep != 1.0f || fq != 0.f || pr != 0.f;
+  if (!counts && !(ng > 1 && n >= ng)) return;      // (the same for the whole workgroup)
+  // Every thread compares its token with the whole context: a context of up to HELD tokens is brought into the
+  // workgroup's memory once, where all lanes of a wave read one word at a time; a longer one is read where it is.
+  __shared__ int32_t held[HELD];
+  auto run = [&](const int32_t* __restrict__ s) {
+    if (counts) {
+      for (int i = threadIdx.x; i < n; i += THREADS) {
+        const int tok = s[i];
+        if (tok < 0 || tok >= V) continue;
+        bool earlier = false;
+#pragma unroll 8
+        for (int j = 0; j < i; ++j) earlier |= s[j] == tok;
+        if (earlier) continue;
+        int count = 0;
+#pragma unroll 8
+        for (int j = i; j < n; ++j) count += s[j] == tok ? 1 : 0;
+        float l = row[tok];
+        if (rep != 1.0f) l = l > 0.f ? l / rep : l * rep;
+        float sub = 0.f;
+        if (fq != 0.f) sub += fq * static_cast<float>(count);
+        if (pr != 0.f) sub += pr;
+        if (sub != 0.f) l -= sub;
+        row[tok] = l;
+      }
+    }
+    __syncthreads();
+    if (ng > 1 && n >= ng) {
+      const int32_t* prefix = s + n - (ng - 1);
+      for (int i = threadIdx.x; i <= n - ng; i += THREADS) {
+        bool same = true;
+        for (int k = 0; k < ng - 1 && same; ++k) same = s[i + k] == prefix[k];
+        if (same) {
+          int f = s[i + ng - 1];
+          if (f >= 0 && f < V) row[f] = -INFINITY;
         }
       }
-      if (!first) continue;
-      float l = row[tok];
-      if (rep != 1.0f) l = l > 0.f ? l / rep : l * rep;
-      float sub = 0.f;
-      if (fq != 0.f) sub += fq * static_cast<float>(count);
-      if (pr != 0.f) sub += pr;
-      if (sub != 0.f) l -= sub;
-      row[tok] = l;
     }
+  };
+  if (n <= HELD) {
+    for (int i = threadIdx.x; i < n; i += THREADS) held[i] = c[i];
+    __syncthreads();
+    run(held);
+  } else {
+    run(c);
   }
-  __syncthreads();
-  if (ng > 1 && n >= ng) {
-    const int32_t* prefix = c + n - (ng - 1);
-    for (int i = threadIdx.x; i <= n - ng; i += THREADS) {
-      bool same = true;
-      for (int k = 0; k < ng - 1 && same; ++k) same = c[i + k] == prefix[k];
-      if (same) {
-        int f = c[i + ng - 1];
-        if (f >= 0 && f < V) row[f] = -INFINITY;
-      }
-    }
-  }
+}
+
+// The sampled tokens of the listed rows into their requests' histories: history[begin[j] + len[j]] =
+// tokens[rows[j]] (a history's next place), so that the next step's penalties find them without the host.
+__global__ void history_append_kernel(int32_t* __restrict__ history, const int32_t* __restrict__ begin,
+                                      const int32_t* __restrict__ len, const int32_t* __restrict__ rows,
+                                      const int32_t* __restrict__ tokens, int n) {
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j < n) history[begin[j] + len[j]] = tokens[rows[j]];
 }
 
 // ---------------------------------------------------------------------------------------
@@ -683,13 +705,22 @@ extern "C" int dn_sample(const float* logits, int ld, int R, int V, const float*
   return dn_launch_status();
 }
 
-extern "C" int dn_penalties(float* logits, int ld, int R, int V, const int32_t* ctx, const int32_t* ctx_start,
-                            const float* repetition, const float* frequency, const float* presence,
-                            const int32_t* ngram, hipStream_t stream) {
+extern "C" int dn_penalties(float* logits, int ld, int R, int V, const int32_t* ctx, const int32_t* ctx_begin,
+                            const int32_t* ctx_len, const float* repetition, const float* frequency,
+                            const float* presence, const int32_t* ngram, hipStream_t stream) {
   if (R <= 0) return 0;
   if (V < 1 || ld < V) return DN_ERR_SHAPE;
   hipLaunchKernelGGL(sampling::penalties_kernel, dim3(R), dim3(sampling::THREADS), 0, stream, logits, ld, V, ctx,
-                     ctx_start, repetition, frequency, presence, ngram);
+                     ctx_begin, ctx_len, repetition, frequency, presence, ngram);
+  return dn_launch_status();
+}
+
+// (the host has checked that every begin[j] + len[j] lies inside the history and every rows[j] inside tokens)
+extern "C" int dn_history_append(int32_t* history, const int32_t* begin, const int32_t* len, const int32_t* rows,
+                                 const int32_t* tokens, int n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(sampling::history_append_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, history, begin,
+                     len, rows, tokens, n);
   return dn_launch_status();
 }
 

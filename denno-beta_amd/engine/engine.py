@@ -84,7 +84,7 @@ class Engine:
             runner.cache.manager, max_live=self.options.max_live,
             max_batch_tokens=self.options.max_batch_tokens, prefill_chunk=self.options.prefill_chunk,
             policy=self.options.kv_policy, max_positions=self.spec.max_positions)
-        self.sampler = Sampler(runner.device)
+        self.sampler = Sampler(runner.device, self.options.max_live, self.spec.max_positions + 1)
         self.requests: Dict[int, Request] = {}
         self._next_rid = 0
         self.records: List[StepRecord] = []
@@ -172,9 +172,7 @@ class Engine:
             return False
         if self.scheduler.n_waiting() > 0 or self.scheduler.n_running() == 0:
             return False
-        if self.scheduler.n_running() != len(launched.alive):
-            return False                            # a running request that was not sampled in this step
-        return not any(r.params.has_penalties for r in launched.sampled)
+        return self.scheduler.n_running() == len(launched.alive)     # (else: a running request not sampled in this step)
 
     def _launch(self, before: Optional["_Launched"]) -> Optional["_Launched"]:
         """before: the step whose sampled tokens are still on the device only (then this step takes them
@@ -198,6 +196,8 @@ class Engine:
                 # comes back after preemption goes on where it was, so its samples do not change)
                 self.runner.cache.reset_states(manager.slot(p.rid))
                 manager.set_rng(p.rid, req.seed, req.n_sampled)
+                if req.params.has_penalties:      # what the penalties read lies on the device, beside the sampler
+                    self.sampler.remember(manager.slot(p.rid), req.tokens)
             wants = p.samples and req.n_sampled < req.max_new
             tokens = req.tokens[p.start:p.start + p.count] if before is None else [0]     # ([0]: stands in for the token on the device)
             entries.append(StepEntry(p.rid, tokens, [p.count - 1] if wants else []))
@@ -221,8 +221,11 @@ class Engine:
             # each request's generator lives in its slot record: the seed and the count of numbers drawn
             rids = np.asarray([r.rid for r in sampled], dtype=np.int64)
             seeds, drawn = manager.rng_states(rids)
-            pending = self.sampler.launch(logits, [r.params for r in sampled], seeds.tolist(), drawn.tolist(),
-                                          [r.tokens for r in sampled])
+            # (a request's history holds its known tokens and, where this step runs ahead, the one sampled
+            # in the step before, which only the device knows yet)
+            ahead = 0 if before is None else 1
+            places = [(manager.slot(r.rid), len(r.tokens) + ahead) for r in sampled]
+            pending = self.sampler.launch(logits, [r.params for r in sampled], seeds.tolist(), drawn.tolist(), places)
             manager.note_drawn_step(rids)
             last = self.scheduler.tokens_sampled(rids).tolist()
         except Exception:

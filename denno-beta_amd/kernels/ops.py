@@ -117,7 +117,8 @@ def _declare(name, lib):
         },
         "sampling": {
             "dn_sample": [P, I, I, I, P, P, P, P],
-            "dn_penalties": [P, I, I, I, P, P, P, P, P, P, P],
+            "dn_penalties": [P, I, I, I, P, P, P, P, P, P, P, P],
+            "dn_history_append": [P, P, P, P, P, I, P],
             "dn_sample_top": [P, I, I, I, P, P, P, P, P, P, P, P, P],
             "dn_sample_full": [P, I, I, I, I, P, P, P, P, P, P, P, P],
         },
@@ -605,23 +606,42 @@ def sample_full(logits, rows, temperature, uniform, top_p, out, only=None):
     return out
 
 
-def penalties(logits, ctx, ctx_start, repetition, frequency, presence, ngram):
+def penalties(logits, ctx, begin, length, repetition, frequency, presence, ngram, bounds=None):
     """In place on logits [R, V]: repetition, frequency, presence penalties and the n-gram ban,
-    each row over its own context ctx[ctx_start[r]:ctx_start[r+1]]."""
+    each row over its own context ctx[begin[r] : begin[r] + length[r]] (ctx: int32, one dimension: the
+    contexts one after the other, or a table of histories seen as one run).  bounds: the largest
+    begin + length, as the host knows it (the tables themselves are on the device)."""
     _dev(logits, "logits", (torch.float32,), 2)
     R, V = logits.shape
     ld = _rows(logits, "logits")
-    _dev(ctx, "ctx", _I32, 1), _dev(ctx_start, "ctx_start", _I32, 1)
-    _need(ctx_start.shape[0] == R + 1, "penalties: ctx_start")
+    _dev(ctx, "ctx", _I32, 1), _dev(begin, "begin", _I32, 1), _dev(length, "length", _I32, 1)
+    _need(ctx.is_contiguous() and begin.shape[0] == R and length.shape[0] == R, "penalties: one begin and one length per row")
+    _need(bounds is None or 0 <= bounds <= ctx.shape[0], "penalties: a context beyond the end of ctx")
     for t, n in ((repetition, "repetition"), (frequency, "frequency"), (presence, "presence")):
         _dev(t, n, (torch.float32,), 1)
         _need(t.shape[0] == R, lambda: f"penalties: {n}")
     _dev(ngram, "ngram", _I32, 1)
     _need(ngram.shape[0] == R, "penalties: ngram")
-    _ok(_lib("sampling").dn_penalties(logits.data_ptr(), ld, R, V, ctx.data_ptr(), ctx_start.data_ptr(),
+    _ok(_lib("sampling").dn_penalties(logits.data_ptr(), ld, R, V, ctx.data_ptr(), begin.data_ptr(), length.data_ptr(),
                                       repetition.data_ptr(), frequency.data_ptr(), presence.data_ptr(),
                                       ngram.data_ptr(), _stream()), "penalties")
     return logits
+
+
+def history_append(history, begin, length, rows, tokens, bounds=None):
+    """history[begin[j] + length[j]] = tokens[rows[j]] for every j: the tokens sampled for the listed rows, each
+    into its request's history (int32, one dimension) at the history's next place.  bounds: (the largest
+    begin + length, the largest row), as the host knows them."""
+    for t, n in ((history, "history"), (begin, "begin"), (length, "length"), (rows, "rows"), (tokens, "tokens")):
+        _dev(t, n, _I32, 1)
+        _need(t.is_contiguous(), lambda: f"history_append: {n}")
+    n = begin.shape[0]
+    _need(length.shape[0] == n and rows.shape[0] == n, "history_append: one length and one row per begin")
+    if bounds is not None:
+        _need(0 <= bounds[0] < history.shape[0] and 0 <= bounds[1] < tokens.shape[0], "history_append: beyond the history or the tokens")
+    _ok(_lib("sampling").dn_history_append(history.data_ptr(), begin.data_ptr(), length.data_ptr(), rows.data_ptr(),
+                                           tokens.data_ptr(), n, _stream()), "history_append")
+    return history
 
 
 # ---------------------------------------------------------------------------------------

@@ -16,39 +16,70 @@ from .rng import uniform
 
 
 class Sampler:
-    def __init__(self, device):
-        self.device = device
+    """slots, positions: the histories that the penalties read lie on the device, a row of `positions` tokens per
+    slot (a request's slot in the cache manager).  A request with penalties is written there when it is admitted
+    (`remember`), and every token sampled for it is added behind on the device, so that a step needs nothing of
+    the tokens from the host, not even those of the step before."""
+
+    def __init__(self, device, slots: int = 0, positions: int = 0):
+        self.device = torch.device(device)
         self._zeros = {}      # rows -> [2, rows] of zeros on the device: temperatures and uniforms of all-greedy steps
+        self.history = None
+        self._room(slots, positions)
+
+    def _room(self, slots, positions):
+        if slots > 0 and positions > 0 and (self.history is None or self.history.shape[0] < slots
+                                            or self.history.shape[1] < positions):
+            self.history = torch.zeros((slots, positions), dtype=torch.int32, device=self.device)
+
+    def remember(self, slot: int, tokens: Sequence[int]):
+        """The tokens of the request in `slot` so far (prompt + generated), from the start."""
+        n = len(tokens)
+        if self.history is None or not (0 <= slot < self.history.shape[0]) or n > self.history.shape[1]:
+            raise ValueError(f"sampler: no room for {n} tokens in slot {slot}")
+        if n:
+            self.history[slot, :n].copy_(self._to_device(list(tokens), torch.int32))
 
     def sample(self, logits, params, seeds, counters, contexts) -> List[int]:
-        """launch and read at once."""
-        return self.read(self.launch(logits, params, seeds, counters, contexts))
+        """launch and read at once, the rows' contexts (prompt + generated) given as lists."""
+        places = None
+        if any(p.has_penalties for p in params):
+            self._room(len(contexts), max(len(c) for c in contexts) + 1)
+            places = []
+            for r, (p, c) in enumerate(zip(params, contexts)):
+                if p.has_penalties:
+                    self.remember(r, c)
+                places.append((r, len(c)))
+        return self.read(self.launch(logits, params, seeds, counters, places))
 
     def launch(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
-               counters: Sequence[int], contexts: Sequence[Sequence[int]]) -> "Pending":
+               counters: Sequence[int], places: Sequence = None) -> "Pending":
         """Starts the sampling of a step's rows and does not wait for it.
         logits: [R, V] 32-bit (changed in place by penalties); row r belongs to a request
-        with params[r], the seed seeds[r], counters[r] tokens sampled so far and the tokens
-        contexts[r] (prompt + generated).  `read` gives the tokens; `Pending.tokens` holds them on the
-        device as soon as the kernels have run, and is final if `Pending.final`."""
+        with params[r], the seed seeds[r] and counters[r] tokens sampled so far; places[r] = (slot, n): its
+        history's slot and how many tokens it holds (needed for rows with penalties only).  `read` gives the
+        tokens; `Pending.tokens` holds them on the device as soon as the kernels have run."""
         R = logits.shape[0]
         if R == 0:
             return Pending(None, 0)
         dev = self.device
-        if any(p.has_penalties for p in params):
-            starts, flat = [0], []
-            for p, c in zip(params, contexts):
-                if p.has_penalties:
-                    flat.extend(int(t) for t in c)
-                starts.append(len(flat))
-            f32 = lambda vals: torch.tensor(vals, dtype=torch.float32, device=dev)   # noqa: E731
-            ops.penalties(
-                logits, torch.tensor(flat or [0], dtype=torch.int32, device=dev),
-                torch.tensor(starts, dtype=torch.int32, device=dev),
-                f32([p.repetition_penalty if p.repetition_penalty is not None else 1.0 for p in params]),
-                f32([p.frequency_penalty or 0.0 for p in params]),
-                f32([p.presence_penalty or 0.0 for p in params]),
-                torch.tensor([p.no_repeat_ngram_size or 0 for p in params], dtype=torch.int32, device=dev))
+        punished = [r for r, p in enumerate(params) if p.has_penalties]
+        if punished:
+            if places is None or self.history is None:
+                raise ValueError("sampler: rows with penalties need their histories' places")
+            width = self.history.shape[1]
+            for r in punished:
+                slot, n = places[r]
+                if not (0 <= slot < self.history.shape[0] and 0 <= n < width):
+                    raise ValueError(f"sampler: a history of {n} tokens in slot {slot} does not fit")
+            begin = [places[r][0] * width if p.has_penalties else 0 for r, p in enumerate(params)]
+            length = [places[r][1] if p.has_penalties else 0 for r, p in enumerate(params)]
+            where = self._to_device([begin, length, [p.no_repeat_ngram_size or 0 for p in params]], torch.int32)
+            f = self._to_device([[p.repetition_penalty if p.repetition_penalty is not None else 1.0 for p in params],
+                                 [p.frequency_penalty or 0.0 for p in params],
+                                 [p.presence_penalty or 0.0 for p in params]], torch.float32)
+            ops.penalties(logits, self.history.view(-1), where[0], where[1], f[0], f[1], f[2], where[2],
+                          bounds=max(b + n for b, n in zip(begin, length)))
         # top_p = 1 without top_k restricts nothing: such a row takes the plain walk over the whole
         # vocabulary (the reference sorts it first, crates/denno-engine/src/sampler.rs:387-435, which
         # gives the same distribution)
@@ -78,6 +109,11 @@ class Sampler:
                 # the host need not read the flags first, so the step's tokens are final once the kernels
                 # have run and the next step can be launched ahead
                 ops.sample_full(logits, ints[0], t_dev, u_dev, ps, both[:R], only=both[R:])
+        if punished:
+            # each sampled token behind its request's history, for the next step's penalties
+            t = self._to_device([[begin[r] for r in punished], [length[r] for r in punished], punished], torch.int32)
+            ops.history_append(self.history.view(-1), t[0], t[1], t[2], both,
+                               bounds=(max(begin[r] + length[r] for r in punished), max(punished)))
         return Pending(both, R, *self._bring_home(both))
 
     def _to_device(self, values, dtype):

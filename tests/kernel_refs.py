@@ -161,17 +161,22 @@ def sample(logits, temperature, uniform, out):
     return out
 
 
-def penalties(logits, ctx, ctx_start, repetition, frequency, presence, ngram):
+def penalties(logits, ctx, begin, length, repetition, frequency, presence, ngram, bounds=None):
     from plain import sampler_plain as sp
-    cs = ctx_start.tolist()
     for r in range(logits.shape[0]):
-        c = ctx[cs[r]:cs[r + 1]].tolist()
+        c = ctx[int(begin[r]):int(begin[r]) + int(length[r])].tolist()
         row = logits[r].tolist()
         row = sp.repetition_penalty(row, c, float(repetition[r]))
         row = sp.frequency_presence(row, c, float(frequency[r]), float(presence[r]))
         row = sp.no_repeat_ngram(row, c, int(ngram[r]))
         logits[r] = torch.tensor(row, dtype=torch.float32)
     return logits
+
+
+def history_append(history, begin, length, rows, tokens, bounds=None):
+    for b, n, r in zip(begin.tolist(), length.tolist(), rows.tolist()):
+        history[b + n] = tokens[r]
+    return history
 
 
 def sample_top(logits, rows, temperature, uniform, top_k, top_p, out, undecided):

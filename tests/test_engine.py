@@ -322,7 +322,13 @@ def test_running_ahead_changes_no_token(model_folders, tmp_path, dtype):
     # the host in between, so that these steps run ahead as well)
     cut = [SamplingParams(max_tokens=m, temperature=1.1, seed=9 + i, top_k=(None, 5, 40)[i % 3], top_p=(0.9, None, 0.7)[i % 3])
            for i, m in enumerate((30, 7, 45, 12, 1, 60, 25))]
-    for params in (greedy, warm, cut):
+    # penalties over the request's own tokens, which lie on the device beside the sampler: a step that runs ahead
+    # counts the token of the step before, which the host has not seen.  Some rows with, some without
+    punished = [SamplingParams(max_tokens=m, temperature=(0.0, 0.9, 1.2)[i % 3], seed=20 + i, top_k=(None, None, 30)[i % 3],
+                               repetition_penalty=(1.4, None, 1.1, None)[i % 4], frequency_penalty=(None, 0.3)[i % 2],
+                               presence_penalty=(0.2, None, None)[i % 3], no_repeat_ngram_size=(None, 2, 3, None)[i % 4])
+                for i, m in enumerate((30, 7, 45, 12, 1, 60, 25))]
+    for params in (greedy, warm, cut, punished):
         for kw in (dict(cache_tokens=1024, max_live=8), dict(cache_tokens=192, max_live=3)):
             want_engine = engine_for(folder, dtype, "cuda:0", run_ahead=False, **kw)
             want = want_engine.generate(prompts, params)

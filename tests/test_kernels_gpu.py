@@ -748,14 +748,65 @@ def test_sample_top_and_penalties():
         assert out.tolist() == want.tolist(), trial
         assert undecided.tolist() == [0] * 5          # a vocabulary within the 2,048 candidates is always decided
     assert out[2].item() == 10
-    ctx = i32([3, 4, 3, 9, 4, 3] + [7, 8, 7, 8, 7])
-    start = i32([0, 6, 6, 11])
+    # contexts as rows of a table of histories, with other tokens behind each row's length that must not count
+    ctx = i32([3, 4, 3, 9, 4, 3, 1, 1] + [5, 5, 5, 5, 5, 5, 5, 5] + [7, 8, 7, 8, 7, 2, 2, 2])
+    begin, length = i32([0, 8, 16]), i32([6, 0, 5])
     l = rnd(3, V, seed=5)
-    want = R.penalties(l.clone().cpu(), ctx.cpu(), start.cpu(), torch.tensor([1.5, 1.0, 1.0]), torch.tensor([0.3, 0.0, 0.0]),
-                       torch.tensor([0.2, 0.0, 0.5]), torch.tensor([0, 0, 2], dtype=torch.int32))
-    ops().penalties(l, ctx, start, torch.tensor([1.5, 1.0, 1.0], device=DEV), torch.tensor([0.3, 0.0, 0.0], device=DEV),
-                    torch.tensor([0.2, 0.0, 0.5], device=DEV), i32([0, 0, 2]))
+    want = R.penalties(l.clone().cpu(), ctx.cpu(), begin.cpu(), length.cpu(), torch.tensor([1.5, 1.0, 1.0]),
+                       torch.tensor([0.3, 0.0, 0.0]), torch.tensor([0.2, 0.0, 0.5]), torch.tensor([0, 0, 2], dtype=torch.int32))
+    before = l.clone()
+    ops().penalties(l, ctx, begin, length, torch.tensor([1.5, 1.0, 1.0], device=DEV), torch.tensor([0.3, 0.0, 0.0], device=DEV),
+                    torch.tensor([0.2, 0.0, 0.5], device=DEV), i32([0, 0, 2]), bounds=21)
     assert torch.allclose(l.cpu(), want, atol=1e-6) and l[2, 8].item() == float("-inf")
+    assert torch.equal(l[1], before[1]) and l[0, 1] == before[0, 1] and l[2, 2] == before[2, 2]
+    with pytest.raises(Exception):
+        ops().penalties(l, ctx, begin, length, torch.ones(3, device=DEV), torch.zeros(3, device=DEV),
+                        torch.zeros(3, device=DEV), i32([0, 0, 0]), bounds=25)
+
+
+def test_penalties_over_long_contexts():
+    """Contexts from nothing to more tokens than the kernel keeps in the workgroup's memory (8,192), few distinct
+    tokens so that each is counted often, every row with its own options; tokens outside the vocabulary count for
+    nothing."""
+    V = 517
+    lens = [0, 1, 2, 700, 1025, 8192, 8193, 9001]
+    g = torch.Generator().manual_seed(12)
+    width = 9100
+    table = torch.randint(0, V, (len(lens), width), generator=g, dtype=torch.int32)
+    table[3, 5] = V + 3
+    table[4, 0] = -1
+    for r, n in enumerate(lens):                    # what lies behind a context must not count: a token that
+        table[r, n:] = 77                           # would show at once
+    ctx = table.to(DEV).view(-1)
+    begin, length = i32([r * width for r in range(len(lens))]), i32(lens)
+    rep = torch.tensor([1.3, 1.3, 1.0, 1.2, 1.0, 1.5, 1.1, 1.0])
+    fq = torch.tensor([0.1, 0.0, 0.2, 0.05, 0.0, 0.01, 0.02, 0.0])
+    pr = torch.tensor([0.0, 0.4, 0.0, 0.3, 0.0, 0.2, 0.0, 0.0])
+    ng = torch.tensor([2, 2, 2, 3, 2, 0, 4, 2], dtype=torch.int32)
+    l = rnd(len(lens), V, seed=6, scale=2.0)
+    want = R.penalties(l.clone().cpu(), ctx.cpu(), begin.cpu(), length.cpu(), rep, fq, pr, ng)
+    ops().penalties(l, ctx, begin, length, rep.to(DEV), fq.to(DEV), pr.to(DEV), ng.to(DEV), bounds=7 * width + 9001)
+    assert torch.equal(torch.isinf(l.cpu()), torch.isinf(want))
+    fin = ~torch.isinf(want)
+    assert torch.allclose(l.cpu()[fin], want[fin], atol=1e-5, rtol=1e-6)
+    assert torch.equal(l[0].cpu(), want[0]) and (l[7].cpu() != rnd(len(lens), V, seed=6, scale=2.0)[7].cpu()).sum() > 0
+
+
+def test_history_append():
+    """Sampled tokens go behind their requests' histories, each at its own place, and nothing else changes."""
+    history = torch.arange(100, 140, dtype=torch.int32, device=DEV)        # 4 histories of 10 places
+    tokens = i32([11, 22, 33, 44, 55, -1, -1])                            # a step's tokens, and flags behind them
+    begin, length, rows = i32([30, 0, 10]), i32([9, 0, 4]), i32([4, 0, 2])
+    want = R.history_append(history.clone().cpu(), begin.cpu(), length.cpu(), rows.cpu(), tokens.cpu())
+    ops().history_append(history, begin, length, rows, tokens, bounds=(39, 4))
+    assert history.tolist() == want.tolist()
+    assert history[39].item() == 55 and history[0].item() == 11 and history[14].item() == 33
+    changed = (history.cpu() != torch.arange(100, 140, dtype=torch.int32)).nonzero().flatten().tolist()
+    assert changed == [0, 14, 39]
+    with pytest.raises(Exception):
+        ops().history_append(history, begin, length, rows, tokens, bounds=(40, 4))
+    with pytest.raises(Exception):
+        ops().history_append(history, begin, length, rows, tokens, bounds=(39, 7))
 
 
 @pytest.mark.parametrize("V,levels", [(6000, 3), (6000, 40), (50257, 7), (3000, 1), (2100, 2)])

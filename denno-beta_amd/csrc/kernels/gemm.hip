@@ -338,11 +338,22 @@ __global__ __launch_bounds__(256) void rows_kernel(const TI* __restrict__ A, int
   }
 }
 
-// the segments' sums of each element, added in ascending order from zero, then the epilogue
+// Where the key and value columns of a fused projection of few rows go besides C (slot_map == null: nowhere):
+// as KVScatter says it, with pools of C's own type.
+template <typename TC>
+struct KVRows {
+  const int32_t* slot_map;
+  TC* k_pool;
+  TC* v_pool;
+  int q_width, kv_width, dh, page_size, Hkv;
+};
+
+// the segments' sums of each element, added in ascending order from zero, then the epilogue; the keys and values
+// among the columns also go to their tokens' places in the cache, so that no kernel has to copy them there
 template <typename TC>
 __global__ __launch_bounds__(256) void join_kernel(const float* __restrict__ part, int nseg, const float* __restrict__ bias,
                                                     TC* __restrict__ C, int ldc, float* __restrict__ resid, int ldr,
-                                                    int M, int N, int epi) {
+                                                    int M, int N, int epi, KVRows<TC> kv) {
   const int n = blockIdx.x * 256 + threadIdx.x, m = blockIdx.y;
   if (n >= N) return;
   float tot = 0.f;
@@ -358,6 +369,21 @@ __global__ __launch_bounds__(256) void join_kernel(const float* __restrict__ par
   }
   for (; s < nseg; ++s) tot += p[s * step];
   finish<TC>(tot, m, n, bias, C, ldc, resid, ldr, epi);
+  if (kv.slot_map != nullptr && n >= kv.q_width) {
+    const int slot = kv.slot_map[m];
+    if (slot < 0) return;
+    int c = n - kv.q_width;
+    const bool is_value = c >= kv.kv_width;
+    if (is_value) c -= kv.kv_width;
+    const int page = slot / kv.page_size, off = slot % kv.page_size;
+    const int hh = c / kv.dh, d = c % kv.dh;
+    const size_t base = (static_cast<size_t>(page) * kv.Hkv + hh) * kv.page_size * kv.dh;
+    const TC x = from_float<TC>(apply_epilogue(bias ? tot + bias[n] : tot, epi));      // what finish stored in C
+    if (is_value)
+      kv.v_pool[base + static_cast<size_t>(d) * kv.page_size + off] = x;
+    else
+      kv.k_pool[base + static_cast<size_t>(off) * kv.dh + d] = x;
+  }
 }
 
 constexpr int FEW_ROWS = 64;
@@ -371,17 +397,25 @@ static long work_floats(int M, int N, int K) {
   return static_cast<long>(nseg) * M * N;
 }
 
+// whether the few-rows kernel takes these operands (it loads four elements at a time: rows that do not start
+// at multiples of that go the other way)
+template <typename TI>
+static bool few_rows_take(const void* A, int lda, const void* W, int M, int K) {
+  const size_t quad = 4 * sizeof(TI);
+  return M <= FEW_ROWS && reinterpret_cast<uintptr_t>(A) % quad == 0 && reinterpret_cast<uintptr_t>(W) % quad == 0 &&
+         lda % 4 == 0 && K % 4 == 0;
+}
+
+// kv: a fused projection's cache write, done by the kernel that joins the segments (so only where there is one:
+// few_rows_take and work_floats > 0)
 template <typename TI, typename TC>
 static int run(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, float* resid, int ldr, int M,
-               int N, int K, int epi, float* work, long have, hipStream_t stream) {
+               int N, int K, int epi, float* work, long have, hipStream_t stream, KVRows<TC> kv = KVRows<TC>{}) {
   const TI* a = static_cast<const TI*>(A);
   const TI* w = static_cast<const TI*>(W);
   TC* c = static_cast<TC*>(C);
-  // the few-rows kernel loads four elements at a time: rows that do not start at multiples of that go the other way
-  const size_t quad = 4 * sizeof(TI);
-  const bool aligned = reinterpret_cast<uintptr_t>(A) % quad == 0 && reinterpret_cast<uintptr_t>(W) % quad == 0 &&
-                       lda % 4 == 0 && K % 4 == 0;
-  if (M > FEW_ROWS || !aligned) {
+  if (!few_rows_take<TI>(A, lda, W, M, K)) {
+    if (kv.slot_map) return DN_ERR_SHAPE;
     dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
     hipLaunchKernelGGL((gemm_kernel<TI, TC>), grid, dim3(256), 0, stream, a, lda, w, bias, c, ldc, resid, ldr, M, N, K,
                        epi);
@@ -390,6 +424,7 @@ static int run(const void* A, int lda, const void* W, const float* bias, void* C
   const long need = work_floats(M, N, K);
   if (need > 0 && (work == nullptr || have < need)) return DN_ERR_SHAPE;     // dn_gemm_work_floats says how much
   float* part = need > 0 ? work : nullptr;
+  if (kv.slot_map && !part) return DN_ERR_SHAPE;
   const int nseg = (K + SEG - 1) / SEG;
   const int rm = M <= 8 ? 8 : M <= 16 ? 16 : M <= 32 ? 32 : 64;
   dim3 grid((N + BN - 1) / BN, (M + rm - 1) / rm, part ? nseg : 1);
@@ -403,7 +438,7 @@ static int run(const void* A, int lda, const void* W, const float* bias, void* C
 #undef DN_ROWS
   if (part)
     hipLaunchKernelGGL((join_kernel<TC>), dim3((N + 255) / 256, M), dim3(256), 0, stream, part, nseg, bias, c, ldc, resid,
-                       ldr, M, N, epi);
+                       ldr, M, N, epi, kv);
   return 0;
 }
 }  // namespace plain
@@ -1699,7 +1734,7 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
       int rc = direct::run(a, stream);
       if (rc != 0) return rc;
       hipLaunchKernelGGL((plain::join_kernel<float>), dim3((N + 255) / 256, M), dim3(256), 0, stream, work, shares, bias,
-                         static_cast<float*>(nullptr), 0, resid, ldr, M, N, EPI_NONE);
+                         static_cast<float*>(nullptr), 0, resid, ldr, M, N, EPI_NONE, plain::KVRows<float>{});
       return dn_launch_status();
     }
     if (many && (!few || direct::beats_few_rows(M, N, K))) {
@@ -1730,6 +1765,39 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
   else
     return DN_ERR_DTYPE;
 #undef DN_LAUNCH
+  return rc != 0 ? rc : dn_launch_status();
+}
+
+// The fused projection of few rows in the plain kernels (32-bit, or bfloat16 weights in rows): C [M, N] = A . W^T +
+// bias, and the key columns (q_width ..) and the value columns behind them also go to the slots slot_map[m] of the
+// pools (keys [page, Hkv, page_size, dh], values [page, Hkv, dh, page_size], of C's type), written by the kernel
+// that adds the segments' sums.  Only where the product has that kernel: dn_gemm_plain_qkv_takes.
+extern "C" int dn_gemm_plain_qkv_takes(const void* A, int lda, const void* W, int M, int N, int K, int dtype) {
+  if (plain::work_floats(M, N, K) <= 0) return 0;
+  return dtype == DN_F32 ? plain::few_rows_take<float>(A, lda, W, M, K)
+                         : dtype == DN_BF16 ? plain::few_rows_take<bf16_t>(A, lda, W, M, K) : 0;
+}
+
+extern "C" int dn_gemm_plain_qkv(const void* A, int lda, const void* W, const float* bias, void* C, int ldc, int M,
+                                 int N, int K, int dtype, const int32_t* slot_map, void* k_pool, void* v_pool,
+                                 int q_width, int Hkv, int dh, int page_size, float* work, long work_floats,
+                                 hipStream_t stream) {
+  if (M <= 0) return 0;
+  if (N < 1 || K < 1 || lda < K || ldc < N || !slot_map || !k_pool || !v_pool || Hkv < 1 || dh < 1 || page_size < 1 ||
+      q_width < 0 || q_width + 2 * Hkv * dh != N)
+    return DN_ERR_SHAPE;
+  int rc;
+  if (dtype == DN_F32) {
+    plain::KVRows<float> kv{slot_map, static_cast<float*>(k_pool), static_cast<float*>(v_pool), q_width, Hkv * dh, dh,
+                            page_size, Hkv};
+    rc = plain::run<float, float>(A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, EPI_NONE, work, work_floats, stream, kv);
+  } else if (dtype == DN_BF16) {
+    plain::KVRows<bf16_t> kv{slot_map, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), q_width, Hkv * dh,
+                             dh, page_size, Hkv};
+    rc = plain::run<bf16_t, bf16_t>(A, lda, W, bias, C, ldc, nullptr, 0, M, N, K, EPI_NONE, work, work_floats, stream, kv);
+  } else {
+    return DN_ERR_DTYPE;
+  }
   return rc != 0 ? rc : dn_launch_status();
 }
 

@@ -103,6 +103,8 @@ def _declare(name, lib):
         },
         "gemm": {
             "dn_gemm": [P, I, P, P, P, I, P, I, I, I, I, I, I, I, I, P, c_longlong, P],
+            "dn_gemm_plain_qkv_takes": [P, I, P, I, I, I, I],
+            "dn_gemm_plain_qkv": [P, I, P, P, P, I, I, I, I, I, P, P, P, I, I, I, I, P, c_longlong, P],
             "dn_pack_matrix": [P, P, I, I, P],
             "dn_gemm_norm_out": [P, I, P, P, P, I, I, I, I, P, P, I, P, P],
             "dn_gemm_norm_in": [P, I, P, P, P, F, P, P, I, I, I, I, I, P, P, P, I, I, I, I, I, P],
@@ -429,6 +431,28 @@ def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
             "linear_qkv" if _timed is None else f"linear {K} -> {N}, cache write")
         return out[:, :q_width]
     _need(out.shape[1] == N, "linear_qkv: without the fused kernel out must hold all columns")
+    if not isinstance(w, PackedMatrix) and not isinstance(a, PackedMatrix) and out.dtype == a.dtype and M <= 64:
+        # few rows in the plain kernels: where K is shared out among workgroups, the kernel that adds their sums
+        # writes the keys and values to the cache as well
+        _need(K % 8 == 0, lambda: f"linear_qkv: the inner size {K} must be a multiple of 8")
+        lda, _, _ = _operands(a, w, "linear_qkv")
+        _dev(out, "out", (a.dtype,), 2)
+        if _lib_quiet("gemm").dn_gemm_plain_qkv_takes(a.data_ptr(), lda, w.data_ptr(), M, N, K, _CODE[a.dtype]):
+            _dev(slot_map, "slot_map", _I32, 1), _dev(k_pool, "k_pool", (a.dtype,), 4), _dev(v_pool, "v_pool", (a.dtype,), 4)
+            _need(k_pool.is_contiguous() and v_pool.is_contiguous() and tuple(v_pool.shape) == (n_pages, Hkv, dh, ps),
+                  "linear_qkv: pools")
+            _need(slot_map.is_contiguous() and slot_map.shape[0] == M, "linear_qkv: slot_map")
+            if bias is not None:
+                _dev(bias, "bias", (torch.float32,), 1)
+                _need(bias.is_contiguous() and bias.shape[0] == N, "linear_qkv: bias")
+            work_floats = _lib_quiet("gemm").dn_gemm_work_floats(M, N, K, 0)
+            work = torch.empty(work_floats, dtype=torch.float32, device=a.device)
+            _ok(_lib("gemm").dn_gemm_plain_qkv(a.data_ptr(), lda, w.data_ptr(), _ptr(bias), out.data_ptr(), _rows(out, "out"),
+                                               M, N, K, _CODE[a.dtype], slot_map.data_ptr(), k_pool.data_ptr(),
+                                               v_pool.data_ptr(), q_width, Hkv, dh, ps, work.data_ptr(), work_floats,
+                                               _stream()),
+                "linear_qkv" if _timed is None else f"linear {K} -> {N}, cache write")
+            return out[:, :q_width]
     linear(a, w, bias, out=out)
     kv_write(out, q_width, q_width + kvw, slot_map, k_pool, v_pool)
     return out[:, :q_width]

@@ -185,6 +185,35 @@ def test_linear_qkv_writes_the_cache(M, slots_in, queries_only):
     assert pools[0].abs().sum() > 0 and pools[1].abs().sum() > 0
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,K,ps", [(1, 256, 16), (8, 1600, 16), (7, 264, 12), (33, 512, 8), (64, 384, 16), (65, 256, 16), (5, 96, 16)])
+def test_linear_qkv_in_the_plain_kernels(dtype, M, K, ps):
+    """The fused projection with weights in rows (the 32-bit engine's): with few rows and a K of several segments
+    the kernel that adds the segments' sums writes the cache too; with more rows, or one segment, a kernel of its
+    own does.  Either way against the product followed by the reference's write, bit for bit, a row without a slot
+    among them and a page size that is no power of two."""
+    H, Hkv, dh, n_pages = 5, 3, 16, 30
+    N = (H + 2 * Hkv) * dh
+    a, w, bias = rnd(M, K, seed=1, dtype=dtype), rnd(N, K, seed=2, dtype=dtype, scale=0.2), rnd(N, seed=3)
+    slots = torch.randperm(n_pages * ps, generator=torch.Generator().manual_seed(M))[:M].to(torch.int32)
+    if M > 2:
+        slots[2] = -1
+    slots = slots.to(DEV)
+    pools = [torch.zeros(n_pages, Hkv, ps, dh, dtype=dtype, device=DEV), torch.zeros(n_pages, Hkv, dh, ps, dtype=dtype, device=DEV)]
+    want_pools = [torch.zeros_like(p) for p in pools]
+    out = torch.full((M, N), 7.0, dtype=dtype, device=DEV)
+    before = ops().launches
+    queries = ops().linear_qkv(a, w, bias, out, slots, pools[0], pools[1], H * dh)
+    fused = M <= 64 and K > 128
+    assert ops().launches - before == (1 if fused else 2), (M, K)
+    want = torch.empty(M, N, dtype=dtype, device=DEV)
+    ops().linear(a, w, bias, out=want)
+    R.kv_write(want, H * dh, (H + Hkv) * dh, slots, want_pools[0], want_pools[1])
+    assert torch.equal(out, want) and torch.equal(queries, want[:, :H * dh])
+    assert torch.equal(pools[0], want_pools[0]) and torch.equal(pools[1], want_pools[1])
+    assert pools[0].abs().sum() > 0 and pools[1].abs().sum() > 0
+
+
 @pytest.mark.parametrize("M,E,I,epilogue", [(1, 64, 256, "gelu_tanh"), (8, 1600, 6400, "gelu_tanh"), (5, 96, 320, "gelu_erf"),
                                             (16, 1600, 4800, "none"), (13, 2560, 1024, "none"), (3, 4096, 4112, "gelu_tanh"),
                                             (9, 16, 16, "none"), (2, 336, 1000, "none")])

@@ -25,11 +25,7 @@ class Sampler:
         self.device = torch.device(device)
         self._zeros = {}      # rows -> [2, rows] of zeros on the device: temperatures and uniforms of all-greedy steps
         self.history = None
-        self._room(slots, positions)
-
-    def _room(self, slots, positions):
-        if slots > 0 and positions > 0 and (self.history is None or self.history.shape[0] < slots
-                                            or self.history.shape[1] < positions):
+        if slots > 0 and positions > 0:
             self.history = torch.zeros((slots, positions), dtype=torch.int32, device=self.device)
 
     def remember(self, slot: int, tokens: Sequence[int]):
@@ -41,10 +37,13 @@ class Sampler:
             self.history[slot, :n].copy_(self._to_device(list(tokens), torch.int32))
 
     def sample(self, logits, params, seeds, counters, contexts) -> List[int]:
-        """launch and read at once, the rows' contexts (prompt + generated) given as lists."""
+        """launch and read at once, the rows' contexts (prompt + generated) given as lists: for a sampler that
+        serves no engine, since the contexts are written over the histories of slots 0, 1, ..."""
         places = None
         if any(p.has_penalties for p in params):
-            self._room(len(contexts), max(len(c) for c in contexts) + 1)
+            if self.history is None:
+                self.history = torch.zeros((len(contexts), max(len(c) for c in contexts) + 1), dtype=torch.int32,
+                                           device=self.device)
             places = []
             for r, (p, c) in enumerate(zip(params, contexts)):
                 if p.has_penalties:

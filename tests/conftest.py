@@ -38,6 +38,14 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a GPU (run on the MI355X box)")
 
 
+@pytest.fixture(autouse=True)
+def _seeded(request):
+    """Every test starts from the same state of torch's default generators (CPU and device), derived from its
+    name, so that a test that draws without a generator of its own draws the same numbers in every run."""
+    import zlib
+    torch.manual_seed(zlib.crc32(request.node.nodeid.encode()))
+
+
 def pytest_collection_modifyitems(config, items):
     if torch.cuda.is_available():
         return

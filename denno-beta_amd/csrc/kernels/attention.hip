@@ -575,7 +575,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
 // the page are a shift and a mask: a tile's keys need four such pairs a step, and a division by a number
 // known only at run time is some twenty-five vector instructions.
 template <int DH16, int GROUPS, int TPS, bool POW2>     // head size / 16; groups of 4 waves; tiles a wave takes per step
-__global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(2))) void kernel(
+__global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(DH16 > 12 && GROUPS == 1 ? 1 : 2))) void kernel(
     const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_row0,
@@ -898,22 +898,29 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
     DN_FLASH_P(D, G, T, true); \
   else                         \
     DN_FLASH_P(D, G, T, false)
-#define DN_FLASH(D, G)                  \
-  if (G == 2) {                         \
-    DN_FLASH_G(D, 2, 1);                \
-  } else {                              \
-    DN_FLASH_G(D, 1, (D <= 6 ? 2 : 1)); \
-  }
+#define DN_FLASH2(D) DN_FLASH_G(D, 2, 1)                      /* two groups of waves, a tile each */
+#define DN_FLASH1(D) DN_FLASH_G(D, 1, (D <= 6 ? 2 : 1))       /* one group, two tiles a step where registers allow */
   switch (dh) {
-    case 16: DN_FLASH(1, 2); break;
-    case 32: DN_FLASH(2, 2); break;
-    case 48: DN_FLASH(3, 2); break;
-    case 64: DN_FLASH(4, 2); break;
-    case 96: DN_FLASH(6, 1); break;
-    case 128: DN_FLASH(8, 1); break;
+    case 16: DN_FLASH2(1); break;
+    case 32: DN_FLASH2(2); break;
+    case 48: DN_FLASH2(3); break;
+    case 64: DN_FLASH2(4); break;
+    case 80: DN_FLASH1(5); break;
+    case 96: DN_FLASH1(6); break;
+    case 112: DN_FLASH1(7); break;
+    case 128: DN_FLASH1(8); break;
+    case 144: DN_FLASH1(9); break;
+    case 160: DN_FLASH1(10); break;
+    case 176: DN_FLASH1(11); break;
+    case 192: DN_FLASH1(12); break;
+    case 208: DN_FLASH1(13); break;
+    case 224: DN_FLASH1(14); break;
+    case 240: DN_FLASH1(15); break;
+    case 256: DN_FLASH1(16); break;
     default: return DN_ERR_SHAPE;
   }
-#undef DN_FLASH
+#undef DN_FLASH1
+#undef DN_FLASH2
 #undef DN_FLASH_G
 #undef DN_FLASH_P
   return dn_launch_status();
@@ -937,7 +944,11 @@ namespace decode {
 // POW2: page_size = 1 << page_shift; a key's page and its place in the page are then a shift and a mask (a lane
 // works out a dozen such pairs per 64 keys before it can ask for the keys and values: as divisions by a number
 // known only at run time they were some six hundred instructions in front of the loads)
-template <int LPK, int WAVES, bool POW2>   // lanes per key = dh / 8; waves per workgroup
+// A key's 16-byte pieces lie on LPK lanes side by side, LPK the power of two that holds them: with a head size
+// that is no power of two (48, 80, 96, ...) the lanes beyond the key's last piece hold zeros.
+constexpr int lanes_per_key(int dh) { return dh <= 16 ? 2 : dh <= 32 ? 4 : dh <= 64 ? 8 : dh <= 128 ? 16 : 32; }
+
+template <int DH, int WAVES, bool POW2>   // head size (a multiple of 16 up to 256); waves per workgroup
 __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out,
                                                        int ldo, const bf16_t* __restrict__ k_pool,
                                                        const bf16_t* __restrict__ v_pool,
@@ -948,7 +959,9 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
                                                        float* __restrict__ part, int n_splits, int chunks, int H,
                                                        int Hkv, int page_size, int page_shift, float scale,
                                                        int window) {
-  constexpr int DH = LPK * 8;
+  static_assert(DH % 16 == 0 && DH >= 16 && DH <= 256, "head size");
+  constexpr int LPK = lanes_per_key(DH);
+  constexpr int PIECES = DH / 8;         // 16-byte pieces of a key: the lanes sub < PIECES of its LPK
   auto page_index = [&](int key) { return POW2 ? key >> page_shift : key / page_size; };
   auto page_offset = [&](int key) { return POW2 ? key & (page_size - 1) : key % page_size; };
   constexpr int KPI = 64 / LPK;          // keys per load instruction
@@ -964,7 +977,9 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
   const int32_t* bt = block_tables + static_cast<size_t>(tile) * max_blocks;
   const int lane = threadIdx.x % 64, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);   // (a scalar)
   const int sub = lane % LPK, grp = lane / LPK;
-  const bf16x8 qv = *reinterpret_cast<const bf16x8*>(q + static_cast<size_t>(row) * ldq + h * DH + sub * 8);
+  const bool holds = PIECES == LPK || sub < PIECES;     // (a lane without a piece: zeros, which add nothing to a score)
+  bf16x8 qv = {};
+  if (holds) qv = *reinterpret_cast<const bf16x8*>(q + static_cast<size_t>(row) * ldq + h * DH + sub * 8);
   if (tile_seq[tile] < 0) return;
   const int pos = tile_pos0[tile];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
@@ -1020,8 +1035,10 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
         const int key = kbase + (it0 + u) * KPI + grp;
         const int kk = (key >= lo && key <= pos) ? key : pos;     // a key that surely has a page
         const int page = bt[page_index(kk)];
-        kv[u] = *reinterpret_cast<const bf16x8*>(
-            k_pool + ((static_cast<size_t>(page) * Hkv + hk) * page_size + page_offset(kk)) * DH + sub * 8);
+        kv[u] = bf16x8{};
+        if (holds)
+          kv[u] = *reinterpret_cast<const bf16x8*>(
+              k_pool + ((static_cast<size_t>(page) * Hkv + hk) * page_size + page_offset(kk)) * DH + sub * 8);
       }
 #pragma unroll
       for (int u = 0; u < GROUP; ++u) {
@@ -1154,19 +1171,30 @@ extern "C" int dn_attention_decode(const void* q, int ldq, void* out, int ldo, c
     else                     \
       DN_DECODE_P(L, W, false); \
   } while (0)
-#define DN_DECODE(L)                  \
+#define DN_DECODE(D)                  \
   if (waves == 16) {                  \
-    if constexpr (L <= 8) DN_DECODE_W(L, 16); \
+    if constexpr (D <= 64) DN_DECODE_W(D, 16); \
   } else if (waves == 8) {            \
-    if constexpr (L <= 16) DN_DECODE_W(L, 8);  \
+    if constexpr (D <= 128) DN_DECODE_W(D, 8);  \
   } else                              \
-    DN_DECODE_W(L, 4)
+    DN_DECODE_W(D, 4)
   switch (dh) {
-    case 16: DN_DECODE(2); break;
-    case 32: DN_DECODE(4); break;
-    case 64: DN_DECODE(8); break;
-    case 128: DN_DECODE(16); break;
-    case 256: DN_DECODE(32); break;
+    case 16: DN_DECODE(16); break;
+    case 32: DN_DECODE(32); break;
+    case 48: DN_DECODE(48); break;
+    case 64: DN_DECODE(64); break;
+    case 80: DN_DECODE(80); break;
+    case 96: DN_DECODE(96); break;
+    case 112: DN_DECODE(112); break;
+    case 128: DN_DECODE(128); break;
+    case 144: DN_DECODE(144); break;
+    case 160: DN_DECODE(160); break;
+    case 176: DN_DECODE(176); break;
+    case 192: DN_DECODE(192); break;
+    case 208: DN_DECODE(208); break;
+    case 224: DN_DECODE(224); break;
+    case 240: DN_DECODE(240); break;
+    case 256: DN_DECODE(256); break;
     default: return DN_ERR_SHAPE;
   }
 #undef DN_DECODE

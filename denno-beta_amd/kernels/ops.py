@@ -458,8 +458,8 @@ def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
     return out[:, :q_width]
 
 
-FLASH_HEAD_DIMS = (16, 32, 48, 64, 96, 128)
-DECODE_HEAD_DIMS = (16, 32, 64, 128, 256)
+FLASH_HEAD_DIMS = tuple(range(16, 257, 16))
+DECODE_HEAD_DIMS = tuple(range(16, 257, 16))
 DECODE_SPLIT = 256     # the decode kernel's smallest chunk; captured decode steps round contexts up to it
 
 

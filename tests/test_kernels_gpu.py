@@ -533,7 +533,10 @@ def test_attention(dtype, H, Hkv, dh, ps, window):
 @pytest.mark.parametrize("H,Hkv,dh,ps,window", [(4, 4, 16, 16, 0), (25, 25, 64, 16, 0), (6, 2, 48, 32, 0),
                                                 (2, 1, 128, 64, 0), (3, 3, 96, 16, 0), (4, 2, 32, 16, 20),
                                                 (5, 5, 64, 32, 7), (2, 2, 64, 16, 150), (4, 2, 64, 48, 0),
-                                                (3, 3, 32, 80, 30)])
+                                                (3, 3, 32, 80, 30), (5, 5, 80, 16, 0), (2, 1, 112, 16, 25),
+                                                (2, 2, 144, 16, 0), (2, 1, 160, 32, 0), (3, 3, 176, 16, 0),
+                                                (2, 2, 192, 16, 90), (1, 1, 208, 16, 0), (2, 1, 224, 48, 0),
+                                                (1, 1, 240, 16, 0), (2, 2, 256, 16, 40)])
 def test_attention_mfma_kernel_for_portions(H, Hkv, dh, ps, window):
     """The bfloat16 kernel for portions of prompts (tiles of up to 128 rows): a long portion deep
     in a context, a whole prompt, a short portion, single rows."""
@@ -556,7 +559,8 @@ def test_attention_mfma_kernel_for_portions(H, Hkv, dh, ps, window):
 
 
 @pytest.mark.parametrize("H,Hkv,dh,ps,window", [(8, 8, 64, 16, 0), (8, 2, 32, 32, 40), (8, 4, 64, 48, 0),
-                                                (8, 8, 96, 16, 0), (8, 2, 128, 32, 60)])
+                                                (8, 8, 96, 16, 0), (8, 2, 128, 32, 60), (8, 8, 80, 16, 0),
+                                                (8, 4, 160, 16, 30), (8, 8, 256, 16, 0)])
 def test_attention_mfma_kernel_with_many_workgroups(H, Hkv, dh, ps, window):
     """More workgroups than CUs, so that they follow one another on a CU: two groups of waves a workgroup up to
     heads of 64, one group beyond (two tiles of keys a step for heads of 96, one for 128)."""
@@ -574,7 +578,11 @@ def test_attention_mfma_kernel_with_many_workgroups(H, Hkv, dh, ps, window):
 
 @pytest.mark.parametrize("H,Hkv,dh,ps,window", [(4, 4, 16, 16, 0), (25, 25, 64, 16, 0), (6, 2, 32, 32, 0),
                                                 (2, 1, 128, 64, 0), (3, 3, 256, 16, 0), (5, 5, 64, 16, 100),
-                                                (2, 2, 64, 32, 300), (4, 2, 64, 48, 0), (3, 3, 32, 80, 90)])
+                                                (2, 2, 64, 32, 300), (4, 2, 64, 48, 0), (3, 3, 32, 80, 90),
+                                                (6, 2, 48, 16, 0), (5, 5, 80, 32, 0), (3, 3, 96, 16, 0),
+                                                (2, 1, 112, 16, 50), (2, 2, 144, 16, 0), (2, 1, 160, 16, 0),
+                                                (1, 1, 176, 32, 0), (2, 2, 192, 16, 0), (1, 1, 208, 16, 70),
+                                                (2, 1, 224, 16, 0), (2, 2, 240, 16, 0)])
 def test_attention_split_kernel_for_decoding(H, Hkv, dh, ps, window):
     """The bfloat16 kernel for steps in which every request brings one row: contexts on both sides
     of a split's edge (256 keys) and of a page's."""
@@ -607,11 +615,13 @@ def test_attention_split_kernel_for_decoding(H, Hkv, dh, ps, window):
             ops().attention(one[0], packed, *one[1:])
 
 
+@pytest.mark.parametrize("dh", [64, 48, 96, 208])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_attention_finds_a_far_key(dtype):
+def test_attention_finds_a_far_key(dtype, dh):
     """One key among hundreds matches the query strongly: the output must be its value, whichever
-    page and tile it lies in (the first key, a page's edge, the last key of a tile, the newest)."""
-    H, dh, ps, n = 2, 64, 16, 700
+    page and tile it lies in (the first key, a page's edge, the last key of a tile, the newest).  Head sizes
+    that are a power of two and others (whose keys leave lanes of the decode kernel empty)."""
+    H, ps, n = 2, 16, 700
     for far in (0, 15, 16, 63, 64, 383, 699):
         q, k, v, bt, tiles, T = paged_case([n], [1], H, H, dh, ps, dtype, seed=far)
         page, off = int(bt[0, far // ps]), far % ps

@@ -26,6 +26,8 @@ class Sampler:
         self._zeros = {}      # rows -> [2, rows] of zeros on the device: temperatures and uniforms of all-greedy steps
         self.history = None
         if slots > 0 and positions > 0:
+            if slots * positions >= 2 ** 31:      # the kernels address the table with 32-bit offsets
+                raise ValueError(f"sampler: {slots} histories of {positions} tokens are more than the kernels address")
             self.history = torch.zeros((slots, positions), dtype=torch.int32, device=self.device)
 
     def remember(self, slot: int, tokens: Sequence[int]):

@@ -224,7 +224,8 @@ class Engine:
             # (a request's history holds its known tokens and, where this step runs ahead, the one sampled
             # in the step before, which only the device knows yet)
             ahead = 0 if before is None else 1
-            places = [(manager.slot(r.rid), len(r.tokens) + ahead) for r in sampled]
+            places = ([(manager.slot(r.rid), len(r.tokens) + ahead) for r in sampled]
+                      if any(r.params.has_penalties for r in sampled) else None)
             pending = self.sampler.launch(logits, [r.params for r in sampled], seeds.tolist(), drawn.tolist(), places)
             manager.note_drawn_step(rids)
             last = self.scheduler.tokens_sampled(rids).tolist()

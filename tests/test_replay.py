@@ -82,8 +82,9 @@ def _cfg(L, E, H, I, V, P, eps=1e-5, act="gelu_new", inv=False):
 
 
 OTHER_SIZES = {
-    "one head of 80": _cfg(1, 80, 1, 320, 101, 160, 1e-3),                        # no MFMA attention kernel takes 80
-    "three heads of 112": _cfg(2, 336, 3, 1000, 777, 200, 1e-6, "gelu", True),    # nor 112; widths no multiple of 32
+    "one head of 80": _cfg(1, 80, 1, 320, 101, 160, 1e-3),                        # a key on 10 of the decode kernel's 16 lanes
+    "three heads of 112": _cfg(2, 336, 3, 1000, 777, 200, 1e-6, "gelu", True),    # on 14 of 16; widths no multiple of 32
+    "two heads of 208": _cfg(1, 416, 2, 800, 500, 200),                           # on 26 of 32; the portions' kernel with a CU to itself
     "three heads of 16": _cfg(4, 48, 3, 64, 50, 130),                             # a feed-forward narrower than 4 E
     "two heads of 256": _cfg(1, 512, 2, 2048, 1000, 300),                         # the largest head size
     "five heads of 48": _cfg(2, 240, 5, 960, 333, 260, 1e-5, "gelu", True),
@@ -94,9 +95,9 @@ OTHER_SIZES = {
 @pytest.mark.parametrize("name", list(OTHER_SIZES))
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_other_head_sizes_and_widths(tmp_path, name, dtype):
-    """Every head size in steps of 16 has a kernel (the MFMA kernels for some, the plain one for the
-    rest), and widths need be no multiple of 32: four cuttings of four requests each, one of them
-    to the last position but two."""
+    """Every head size in steps of 16 has its kernels (in bfloat16 the MFMA kernel for portions and the split
+    kernel for decode steps, whose lanes a head size that is no power of two does not fill), and widths need be
+    no multiple of 32: four cuttings of four requests each, one of them to the last position but two."""
     from denno_beta_amd.weights import write_model_folder
     cfg = OTHER_SIZES[name]
     folder = str(tmp_path)

@@ -477,7 +477,7 @@ def attention_writes_packed(dtype, page_size, head_dim, single_rows, max_context
 
 
 def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, window=0, tiles_wide=None,
-              single_rows=False, max_context=0):
+              single_rows=False, max_context=0, decode_waves=None):
     """Causal attention of the batch's rows over the paged cache.
 
     q: [T, >= H*dh] rows contiguous, head h at columns h*dh..; out: [T, H*dh];
@@ -519,9 +519,16 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
         # (where the batch alone gives two workgroups or more per CU the chip is busy anyway, and
         # the smallest workgroups were measured fastest)
         groups = n_tiles * n_heads
-        waves = (4 if max_context <= 256 else 8 if groups >= 1024 else 4 if groups >= 512 else
+        # (a head size that is no power of two leaves lanes empty and needs more registers: from a thousand
+        # workgroups on its smallest ones are up to a third faster, where the others' sizes are level)
+        many = 8 if dh & (dh - 1) == 0 else 4
+        waves = (4 if max_context <= 256 else many if groups >= 1024 else 4 if groups >= 512 else
                  8 if groups >= 300 or max_context <= 512 else 16)
         waves = min(waves, 16 if dh <= 64 else 8 if dh <= 128 else 4)
+        if decode_waves is not None:       # (for measurements and tests: 4, 8 or 16 as far as the head size allows)
+            _need(decode_waves in (4, 8, 16) and decode_waves <= (16 if dh <= 64 else 8 if dh <= 128 else 4),
+                  lambda: f"attention: {decode_waves} waves with a head size of {dh}")
+            waves = decode_waves
         # the context is split over workgroups only where the batch alone does not give about one
         # workgroup per CU: a second kernel has to join the splits
         total_chunks = -(-max_context // (waves * 64))

@@ -116,7 +116,7 @@ def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None):
 
 
 def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, window=0, tiles_wide=None,
-              single_rows=False, max_context=0):
+              single_rows=False, max_context=0, decode_waves=None):
     n_pages, hkv, ps, dh = k_pool.shape
     group = n_heads // hkv
     tl = tiles.cpu().tolist()

@@ -597,6 +597,13 @@ def test_attention_split_kernel_for_decoding(H, Hkv, dh, ps, window):
         ops().attention(q[:, :H * dh], out, k, v, bt, tiles, H, scale, window, tiles_wide=paged_case.wide,
                         single_rows=True, max_context=max_context)
         assert torch.allclose(out.float(), want, **TOL[torch.bfloat16])
+        # every size of workgroup that the head size allows, not only the one that `attention` picks here
+        for waves in (4, 8, 16):
+            if waves <= (16 if dh <= 64 else 8 if dh <= 128 else 4):
+                other = torch.zeros(T, H * dh, dtype=torch.bfloat16, device=DEV)
+                ops().attention(q[:, :H * dh], other, k, v, bt, tiles, H, scale, window, single_rows=True,
+                                max_context=max_context, decode_waves=waves)
+                assert torch.allclose(other.float(), want, **TOL[torch.bfloat16]), waves
         if (H * dh) % 32 == 0:               # the same rows, packed for the product that follows
             packed = ops().packed_rows(T, H * dh, DEV)
             ops().attention(q[:, :H * dh], packed, k, v, bt, tiles, H, scale, window, single_rows=True,

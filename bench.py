@@ -72,7 +72,10 @@ class Workloads:
         a, P, sync = self.a, self.cfg["n_positions"], self.torch.cuda.synchronize
         steps = max(1, min(steps, (P - a.context - warmup - 2) // blocks))
         eng = Engine(self.runner, self.opts)
-        sp = SamplingParams(max_tokens=P, temperature=0.0, ignore_eos=True)
+        # greedy, unless --only decode names other sampling options (what the sampling kernels cost a step)
+        sp = SamplingParams(max_tokens=P, temperature=getattr(a, "temperature", 0.0), top_k=getattr(a, "top_k", None),
+                            top_p=getattr(a, "top_p", None), repetition_penalty=getattr(a, "repetition_penalty", None),
+                            seed=3, ignore_eos=True)
         rids = [eng.add_request(self.prompt(a.context), sp) for _ in range(batch)]
         while any(eng.scheduler.computed(r) < a.context for r in rids):
             eng.step()
@@ -163,6 +166,10 @@ def main():
     ap.add_argument("--sequences", type=int, default=8, help="--only replay: how many of the eight sequences")
     ap.add_argument("--page-size", type=int, default=16, help="tokens in a page of the cache (decode and prefill)")
     ap.add_argument("--prompts", type=int, default=2, help="--only prefill: prompts of 1,024 tokens in the one step")
+    ap.add_argument("--temperature", type=float, default=0.0, help="--only decode: sampling instead of greedy (0: greedy)")
+    ap.add_argument("--top-k", type=int, default=None, help="--only decode, with --temperature")
+    ap.add_argument("--top-p", type=float, default=None, help="--only decode, with --temperature")
+    ap.add_argument("--repetition-penalty", type=float, default=None, help="--only decode: penalties over each request's tokens")
     ap.add_argument("--shape", choices=["xl", "large", "medium"], default="xl",
                     help="--only decode / prefill: the layer sizes of BASELINE.json's configs[2], [3] or [4]")
     ap.add_argument("--only", choices=["decode", "prefill", "serving", "replay"], default=None,
@@ -178,6 +185,9 @@ def main():
     if a.only == "replay":
         return replay(a)
 
+    if a.only != "decode" and (a.temperature or a.top_k or a.top_p or a.repetition_penalty):
+        print("bench.py: sampling options go with --only decode (the contract's line is greedy)")
+        sys.exit(2)
     w = Workloads(a, a.dtype)
     if a.only in ("prefill", "decode"):
         from denno_beta_amd.kernels import ops

@@ -99,10 +99,10 @@ class Sampler:
             # (the first kernel takes the restricted rows as greedy ones, which costs it a third of the walk:
             # the kernel after it decides their tokens)
             later = set(restricted)
-            first = [0.0 if r in later else t for r, t in enumerate(temps)]
-            tu = self._to_device([temps, us, first], torch.float32)      # one copy for all
+            first = [[0.0 if r in later else t for r, t in enumerate(temps)]] if restricted else []
+            tu = self._to_device([temps, us] + first, torch.float32)      # one copy for all
         t_dev, u_dev = tu[0], tu[1]
-        ops.sample(logits, tu[2] if tu.shape[0] > 2 else t_dev, u_dev, both[:R])
+        ops.sample(logits, tu[2] if restricted else t_dev, u_dev, both[:R])
         if restricted:
             top_p = [params[r].top_p if params[r].top_p is not None else 1.0 for r in restricted]
             ints = self._to_device([restricted, [params[r].top_k or 0 for r in restricted]], torch.int32)

@@ -25,7 +25,10 @@ _CSRC = os.path.join(_PKG, "csrc")
 HIP_ARCH = "gfx950"
 HIP_FLAGS = ["--offload-arch=" + HIP_ARCH, "-O3", "-std=c++17", "-shared", "-fPIC",
              # hipcc -O3 must not form packed 32-bit float instructions on this target
-             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             # a kernel's first arguments arrive in scalar registers with the launch, where it would otherwise
+             # begin by loading them: a trip to memory less in front of every kernel of a decode step
+             "-mllvm", "-amdgpu-kernarg-preload-count=16"]
 HOST_FLAGS = ["-std=c++17", "-O2", "-shared", "-fPIC", "-Wall", "-Wextra"]
 
 # name -> (compiler kind, sources relative to csrc/, headers that the hash covers too)

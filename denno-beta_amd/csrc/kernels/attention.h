@@ -38,7 +38,10 @@ int dn_attention_flash(const void* q, int ldq, void* out, int ldo, const void* k
 
 // bfloat16, one row per request (tile s = request s = row s); the context is cut into n_splits runs of
 // `chunks` chunks of waves * 64 keys; part: device memory for n_tiles * H * n_splits * (dh + 2) floats
-// of split results (not touched when n_splits == 1)
+// of split results (not touched when n_splits == 1).  tile_row0 is not read: tile s is row s of q and
+// of out and row s of the block tables, whatever the table says (the kernels address them by the
+// workgroup's index, so that these loads do not wait for the table's); a caller whose tile s is
+// another row takes dn_attention_flash or dn_attention.
 int dn_attention_decode(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
                         const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
                         const int32_t* tile_row0, const int32_t* tile_pos0, int n_tiles, float* part, int n_splits,

@@ -456,6 +456,9 @@ static int run(const void* A, int lda, const void* W, const float* bias, void* C
 #define PACKED_A 2
 #define PACKED_C 4
 
+static int g_tune[8] = {-1, -1, 0, 0, 0, 0, 0, 0};   // [0] direct shape, [1] shares, [2] kernel (1 few, 2 many), [3] skinny MB*100+NB*10+U
+extern "C" void dn_gemm_tune(int i, int v) { g_tune[i] = v; }
+
 namespace skinny {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
@@ -1004,6 +1007,18 @@ static void launch16(const Call& c, hipStream_t stream) {
 template <int WAVES>
 static void launch_mb(const Call& c, hipStream_t stream) {
   const int mb = (c.M + 15) / 16;
+  if (g_tune[3] > 0 && mb > 1) {
+    switch (g_tune[3]) {
+      case 424: return launch<4, 2, WAVES, 4>(c, stream);
+      case 444: return launch<4, 4, WAVES, 4>(c, stream);
+      case 442: return launch<4, 4, WAVES, 2>(c, stream);
+      case 418: return launch<4, 1, WAVES, 8>(c, stream);
+      case 224: return launch<2, 2, WAVES, 4>(c, stream);
+      case 244: return launch<2, 4, WAVES, 4>(c, stream);
+      case 822: return launch<8, 2, WAVES, 2>(c, stream);
+      default: break;
+    }
+  }
   if (mb == 1 && !(c.packed & (PACKED_A | PACKED_C)) && c.M > 1) return launch16<WAVES>(c, stream);
   if (mb == 1) return launch<1, 1, WAVES, 8>(c, stream);
   if (mb > 4) {
@@ -1646,7 +1661,8 @@ static int launch_as(const Args& a, hipStream_t stream) {
 // for products with few rows and a long K, whose larger tiles would leave most CUs idle.
 struct Shape { int bm, bn, stages; };
 constexpr Shape SHAPES[] = {{64, 128, 4}, {128, 128, 4}, {256, 128, 4}, {256, 160, 4}, {256, 192, 4},
-                            {256, 224, 4}, {256, 256, 4}, {256, 320, 3}, {64, 64, 4}, {32, 64, 4}};
+                            {256, 224, 4}, {256, 256, 4}, {256, 320, 3}, {64, 64, 4}, {32, 64, 4},
+                            {64, 64, 8}, {32, 64, 8}, {64, 128, 6}, {32, 128, 8}, {128, 64, 6}, {64, 32, 8}};
 
 static double model_us(const Shape& s, int M, int N, int K) {
   const double tiles = static_cast<double>((M + s.bm - 1) / s.bm) * ((N + s.bn - 1) / s.bn);
@@ -1659,9 +1675,10 @@ static double model_us(const Shape& s, int M, int N, int K) {
 }
 
 static int pick(int M, int N, int K) {
+  if (g_tune[0] >= 0) return g_tune[0];
   int best = 0;
   double best_us = 1e30;
-  for (int i = 0; i < static_cast<int>(sizeof(SHAPES) / sizeof(SHAPES[0])); ++i) {
+  for (int i = 0; i < 10; ++i) {
     const double us = model_us(SHAPES[i], M, N, K);
     if (us < best_us) best_us = us, best = i;
   }
@@ -1674,6 +1691,7 @@ static int pick(int M, int N, int K) {
 // leave most CUs idle and the few-rows kernel stays ahead, or level, at every size.
 static bool beats_few_rows(int M, int N, int K) {
   (void)K;
+  if (g_tune[2] > 0) return g_tune[2] == 2;
   return (M > 104 && N >= 4096) || (M > 208 && N >= 2048);
 }
 
@@ -1682,6 +1700,7 @@ static bool beats_few_rows(int M, int N, int K) {
 // its rows up to 256, and a quarter of K less than a third of it).  The number of shares, 0 for none: 8
 // where the tiles of 32 x 64 are at most 96, else 4 (with more rows 8 shares gain nothing over 4).
 static int shares_of_k(int M, int N, int K, int packed, bool kv) {
+  if (g_tune[1] >= 0) return (kv || (packed & PACKED_C)) ? 0 : g_tune[1];
   if (kv || (packed & PACKED_C) || M <= 64 || M > 512 || N >= 4096 || K < 4096) return 0;
   return ((M + 31) / 32) * ((N + 63) / 64) <= 96 ? 8 : 4;
 }
@@ -1697,7 +1716,13 @@ static int run(const Args& a, hipStream_t stream) {
     case 6: return launch_as<4, 2, 4, 8, 4>(a, stream);
     case 7: return launch_as<4, 2, 4, 10, 3>(a, stream);
     case 8: return launch_as<2, 2, 2, 2, 4>(a, stream);
-    default: return launch_as<2, 2, 1, 2, 4>(a, stream);
+    case 9: return launch_as<2, 2, 1, 2, 4>(a, stream);
+    case 10: return launch_as<2, 2, 2, 2, 8>(a, stream);
+    case 11: return launch_as<2, 2, 1, 2, 8>(a, stream);
+    case 12: return launch_as<2, 2, 2, 4, 6>(a, stream);
+    case 13: return launch_as<2, 2, 1, 4, 8>(a, stream);
+    case 14: return launch_as<2, 2, 4, 2, 6>(a, stream);
+    default: return launch_as<2, 2, 2, 1, 8>(a, stream);
   }
 }
 }  // namespace direct

@@ -73,6 +73,14 @@ class _Launched:
     record: StepRecord
 
 
+class _AheadFailed(Exception):
+    """The step that was launched ahead could not run; its requests are not dropped yet (`plan`)."""
+
+    def __init__(self, plan):
+        super().__init__("the step launched ahead failed")
+        self.plan = plan
+
+
 class Engine:
     def __init__(self, runner: ModelRunner, options: Optional[EngineOptions] = None, detokenize=None):
         """detokenize: token ids -> text, for requests with stop sequences (and for `Request.text`)."""
@@ -123,8 +131,10 @@ class Engine:
         return rid
 
     def has_unfinished(self) -> bool:
-        """Requests are waiting or running, or a launched step's tokens have not been read yet."""
-        return self.scheduler.n_waiting() + self.scheduler.n_running() > 0 or self._ahead is not None
+        """Requests are waiting or running, a launched step's tokens have not been read yet, or the failure
+        of a step that was launched ahead has not been reported yet (the next `step` raises it)."""
+        return (self.scheduler.n_waiting() + self.scheduler.n_running() > 0 or self._ahead is not None
+                or self._failed_ahead is not None)
 
     def _release(self, rid: int):
         """The request's pages and slot go back, unless they have (its last token was already on its way)."""
@@ -157,12 +167,34 @@ class Engine:
             launched = self._launch(None)
         if launched is None:
             return []
+        failed_plan = None
         if self._may_run_ahead(launched):
             try:
                 self._ahead = self._launch(launched)
-            except Exception as exc:     # its requests are dropped already; the caller hears of it at the next step
-                self._failed_ahead = exc
-        return self._complete(launched)
+            except _AheadFailed as failure:
+                # This step's tokens are sampled already and are the requests' own: they are read and told first.
+                # Then the failed step's requests are dropped, and the caller hears the error from the next
+                # `step`, which `has_unfinished` keeps it calling for.
+                failed_plan, self._failed_ahead = failure.plan, failure.__cause__
+        outputs = self._complete(launched)
+        if failed_plan is not None:
+            dropped = self._drop(failed_plan)
+            for o in outputs:
+                if o.rid in dropped:
+                    o.finished, o.finish_reason = True, "error"
+        return outputs
+
+    def _drop(self, plan) -> set:
+        """A step that failed: its requests end with an error and their pages go back, so that the engine stays
+        usable (crates/denno-server/src/scheduler.rs:362-370, 457-469).  -> the requests dropped here."""
+        dropped = set()
+        for p in plan:
+            req = self.requests[p.rid]
+            if not req.finished:
+                self._release(p.rid)
+                req.finished, req.finish_reason = True, "error"
+                dropped.add(p.rid)
+        return dropped
 
     def _may_run_ahead(self, launched: "_Launched") -> bool:
         """The next step can be planned and launched before this one's tokens are known on the host: it will
@@ -229,14 +261,10 @@ class Engine:
             pending = self.sampler.launch(logits, [r.params for r in sampled], seeds.tolist(), drawn.tolist(), places)
             manager.note_drawn_step(rids)
             last = self.scheduler.tokens_sampled(rids).tolist()
-        except Exception:
-            # the step's requests are dropped, their pages go back, the engine stays usable
-            # (crates/denno-server/src/scheduler.rs:362-370, 457-469)
-            for p in plan:
-                req = self.requests[p.rid]
-                if not req.finished:
-                    self._release(p.rid)
-                    req.finished, req.finish_reason = True, "error"
+        except Exception as exc:
+            if before is not None:       # launched ahead: the step before is told first (see `step`)
+                raise _AheadFailed(plan) from exc
+            self._drop(plan)
             raise
         alive = []
         for r, is_last in zip(sampled, last):

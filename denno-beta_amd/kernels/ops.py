@@ -514,6 +514,8 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
           "attention: packed rows as out are written by the bfloat16 kernels only")
     if decode:
         n_tiles = tiles.shape[1]
+        # (the split kernel does not read the tiles' rows: tile s is row s)
+        _need(n_tiles == T, "attention: a step of single rows has a tile for every row, tile s for row s")
         # a workgroup's waves take 64 keys each at a time: as many waves as make the context one
         # chunk (every load issued at once), within what the head size leaves registers for
         # (where the batch alone gives two workgroups or more per CU the chip is busy anyway, and

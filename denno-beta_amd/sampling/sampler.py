@@ -43,9 +43,14 @@ class Sampler:
         serves no engine, since the contexts are written over the histories of slots 0, 1, ..."""
         places = None
         if any(p.has_penalties for p in params):
-            if self.history is None:
-                self.history = torch.zeros((len(contexts), max(len(c) for c in contexts) + 1), dtype=torch.int32,
-                                           device=self.device)
+            rows, width = len(contexts), max(len(c) for c in contexts) + 1
+            if self.history is None or self.history.shape[0] < rows or self.history.shape[1] < width:
+                # (every call writes its contexts anew, so a larger table need not keep the old one's rows)
+                rows = max(rows, 0 if self.history is None else self.history.shape[0])
+                width = max(width, 0 if self.history is None else self.history.shape[1])
+                if rows * width >= 2 ** 31:
+                    raise ValueError(f"sampler: {rows} histories of {width} tokens are more than the kernels address")
+                self.history = torch.zeros((rows, width), dtype=torch.int32, device=self.device)
             places = []
             for r, (p, c) in enumerate(zip(params, contexts)):
                 if p.has_penalties:

@@ -201,6 +201,25 @@ def test_stop_sequences(backend, model_folders):
         SamplingParams(stop_sequences="ab").validate()
 
 
+def test_a_sampler_alone_takes_any_contexts(backend):
+    """A Sampler that serves no engine keeps its own table of histories: a later call with more rows or longer
+    contexts than the first gets a larger one."""
+    from denno_beta_amd.sampling import Sampler, SamplingParams
+    dev = torch.device(backend)
+    s = Sampler(dev)
+    g = torch.Generator().manual_seed(5)
+    V = 97
+    sp = SamplingParams(temperature=0.0, repetition_penalty=1.5, presence_penalty=0.4)
+    for rows, n in ((2, 5), (3, 40), (1, 7), (5, 41)):
+        logits = torch.randn(rows, V, generator=g)
+        ctxs = [torch.randint(0, V, (n + r,), generator=g).tolist() for r in range(rows)]
+        got = s.sample(logits.clone().to(dev), [sp] * rows, [1] * rows, [0] * rows, ctxs)
+        for r in range(rows):
+            row = SP.repetition_penalty(logits[r].tolist(), ctxs[r], 1.5)
+            row = SP.frequency_presence(row, ctxs[r], 0.0, 0.4)
+            assert got[r] == SP.greedy(row), (rows, n, r)
+
+
 def test_refused_requests(backend, model_folders):
     from denno_beta_amd.engine import SamplingParams, SchedulerError
     e = engine_for(model_folders("A", "float32"), "float32", backend, cache_tokens=64)
@@ -349,6 +368,107 @@ def test_running_ahead_changes_no_token(model_folders, tmp_path, dtype):
         outs += [o.token for o in e.step() if o.token is not None]
     assert outs == e.requests[rid].generated and len(outs) == 12
     assert [r.ran_ahead for r in e.records] == [False] + [True] * 11
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("how", ["flag", "launch"])
+def test_a_step_launched_ahead_that_fails(model_folders, how):
+    """The step that is launched before the last one's tokens are read fails (in the engine, or at a kernel
+    launch of its sampling).  The step before is told whole: its tokens are the requests' own and its outputs say
+    that the requests ended with an error; the error reaches whoever calls `step` next, `generate` included
+    (`has_unfinished` stays true until then); nothing stale is raised later; pages and slots come back and the
+    next requests give a clean engine's tokens."""
+    from denno_beta_amd.engine import SamplingParams
+    from denno_beta_amd.kernels import ops
+    folder = model_folders("B", "float32")
+    prompts = [seeded_tokens(60 + i, n, 1000) for i, n in enumerate((12, 30, 5))]
+    sp = SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True)
+    mk = lambda: engine_for(folder, "float32", "cuda:0", cache_tokens=512, run_ahead=True)   # noqa: E731
+    clean = mk().generate(prompts, sp)
+
+    def fail(e):
+        if how == "flag":
+            e.fail_next_step = True
+        else:
+            ops.fail_after_launches(0)      # a replayed graph launches nothing through ops: the sampling kernel is next
+    e = mk()
+    rids = [e.add_request(p, sp) for p in prompts]
+    while not (e.records and e.records[-1].ran_ahead):
+        e.step()
+    n_before = [len(e.requests[r].generated) for r in rids]
+    fail(e)
+    outs = e.step()          # reads the step launched ahead; the step launched from here fails
+    ops.fail_after_launches(None)
+    assert sorted(o.rid for o in outs) == rids and all(o.finished and o.finish_reason == "error" for o in outs)
+    assert all(o.token == e.requests[o.rid].generated[-1] for o in outs)
+    assert [len(e.requests[r].generated) for r in rids] == [n + 1 for n in n_before]
+    assert [e.requests[r].generated for r in rids] == [c[:n + 1] for c, n in zip(clean, n_before)]
+    assert e.has_unfinished()
+    with pytest.raises((RuntimeError, ops.KernelError), match="injected"):
+        e.step()
+    assert not e.has_unfinished() and e.step() == []
+    m = e.runner.cache.manager
+    assert m.live() == 0 and m.free_pages(0) == 32
+    m.check()
+    assert e.generate(prompts, sp) == clean
+    # through generate: the error is the caller's, and the engine goes on afterwards
+    e = mk()
+    launch = e.sampler.launch
+
+    def failing(*a, **kw):
+        if sum(r.ran_ahead for r in e.records) >= 3:       # (the step that asks now is launched ahead as well)
+            raise RuntimeError("injected: the sampler")
+        return launch(*a, **kw)
+    e.sampler.launch = failing
+    with pytest.raises(RuntimeError, match="injected"):
+        e.generate(prompts, sp)
+    e.sampler.launch = launch
+    assert all(e.finish_reason(r) == "error" for r in range(3))
+    assert [e.requests[r].generated for r in range(3)] == [c[:len(e.requests[r].generated)] for r, c in enumerate(clean)]
+    assert all(len(e.requests[r].generated) >= 4 for r in range(3))
+    assert not e.has_unfinished() and e.runner.cache.manager.live() == 0
+    e.runner.cache.manager.check()
+    assert e.generate(prompts, sp) == clean
+
+
+@pytest.mark.gpu
+def test_abort_and_stop_sequence_while_a_step_is_ahead(model_folders):
+    """A request is aborted, and another ends by a stop sequence, while the step after is already launched with
+    them in it: their pages and slots go back behind that step on the stream, the other requests' tokens are what
+    they are without running ahead, and nothing is lost or held twice."""
+    from denno_beta_amd.engine import Engine, ModelRunner, SamplingParams
+    folder = model_folders("B", "float32")
+    words = lambda ids: " ".join(f"t{t}" for t in ids)                          # noqa: E731
+    prompts = [seeded_tokens(70 + i, n, 1000) for i, n in enumerate((9, 33, 17, 4))]
+    free = SamplingParams(max_tokens=24, temperature=0.0, ignore_eos=True)
+
+    def engine(run_ahead):
+        return Engine(ModelRunner.from_folder(folder, options_for("float32", "cuda:0", cache_tokens=512, run_ahead=run_ahead)),
+                      detokenize=words)
+    full = engine(False).generate(prompts, free)
+    stop = f"t{full[1][10]} "
+    k = full[1].index(full[1][10])          # the stop sequence's first appearance among the tokens
+    got = {}
+    for run_ahead in (False, True):
+        e = engine(run_ahead)
+        rids = [e.add_request(p, SamplingParams(max_tokens=24, temperature=0.0, ignore_eos=True,
+                                                stop_sequences=(stop,) if i == 1 else ())) for i, p in enumerate(prompts)]
+        while e.has_unfinished():
+            e.step()
+            if len(e.requests[rids[2]].generated) == 6 and not e.requests[rids[2]].finished:
+                e.abort(rids[2])            # (with run_ahead the step that holds its seventh token is in flight)
+        got[run_ahead] = [(e.requests[r].generated, e.requests[r].finish_reason, e.requests[r].text) for r in rids]
+        m = e.runner.cache.manager
+        m.check()
+        assert m.live() == 0 and m.free_pages(0) == 32
+        if run_ahead:
+            assert sum(r.ran_ahead for r in e.records) > 10
+        # the engine goes on: the same prompts again, nothing stopped, give the full tokens
+        assert e.generate(prompts, free) == full
+    assert got[True] == got[False]
+    assert got[True][1][1] == "stop_sequence" and got[True][1][0] == full[1][:k + 1] and k >= 1
+    assert got[True][2][1] == "aborted" and got[True][2][0] == full[2][:6]
+    assert got[True][0][0] == full[0] and got[True][3][0] == full[3]
 
 
 @pytest.mark.gpu

@@ -2,9 +2,9 @@
 
 Each cache that the model's run order names has a need (PagedKV or FixedState, from its
 mixer).  Caches with the same need form a group: a paged group has one pool of pages,
-[caches, n_pages, Hkv, page_size, dh] for keys and [caches, n_pages, Hkv, dh, page_size] for
-values (a page's values transposed, as attention's second product reads them), and one block table
-per request, shared by the group's caches; a state group has [caches, slots, *shape] and is
+[caches, n_pages, Hkv, page_size, dh] for keys and [caches, n_pages, Hkv, dv, page_size] for
+values (a page's values transposed, as attention's second product reads them; dv is dh unless
+the need names a width of its own for values), and one block table per request, shared by the group's caches; a state group has [caches, slots, *shape] and is
 indexed by the request's slot.  Groups with different needs (all keys, a window of them)
 draw from pools of their own.
 """
@@ -56,7 +56,7 @@ class CacheStorage:
             n = len(self.members[g])
             if isinstance(cs, PagedKV):
                 shape = (n, n_pages, cs.n_kv_heads, page_size, cs.head_dim)
-                vshape = (n, n_pages, cs.n_kv_heads, cs.head_dim, page_size)   # a page's values transposed
+                vshape = (n, n_pages, cs.n_kv_heads, cs.v_dim, page_size)   # a page's values transposed
                 dt = _TORCH[cs.dtype] if cs.dtype is not None else kv_dtype
                 if allocate:
                     # zeros, not empty: a page's unwritten tail is read (masked) by attention,
@@ -104,5 +104,5 @@ class CacheStorage:
         for g, cs in enumerate(self.group_specs):
             if isinstance(cs, PagedKV):
                 dt = _TORCH[cs.dtype] if cs.dtype is not None else self.kv_dtype
-                total += len(self.members[g]) * 2 * cs.n_kv_heads * cs.head_dim * torch.empty((), dtype=dt).element_size()
+                total += len(self.members[g]) * cs.n_kv_heads * (cs.head_dim + cs.v_dim) * torch.empty((), dtype=dt).element_size()
         return total

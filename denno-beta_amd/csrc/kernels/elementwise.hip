@@ -5,7 +5,7 @@
 
 // ---------------------------------------------------------------------------------------
 // x[t,:] = wte[token_t,:] * token_scale + wpe[pos_t,:]   (crates/denno-engine/src/model/gpt2.rs:142-150,
-// where the scale is 1).  wpe may be null (an architecture whose positions enter elsewhere).
+// where the scale is 1), as the first two entries of a list of tables that are added up.
 // ---------------------------------------------------------------------------------------
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t words4;
 // element i of the 16 bytes w as a table of TW holds them
@@ -18,16 +18,30 @@ __device__ __forceinline__ float element<bf16_t>(const words4& w, int i) {
   return __uint_as_float(i % 2 == 0 ? w[i / 2] << 16 : w[i / 2] & 0xffff0000u);
 }
 
+// x[t,:] = sum over the listed tables, in the list's order, of table_i[index_i[t],:] * scale_i: the token table
+// and the position table for this architecture; an architecture with a further table (a second one over the
+// tokens, one over another per-row integer) lists it behind them.
+constexpr int EMBED_TABLES_MAX = 4;
+struct EmbedTables {
+  const void* table[EMBED_TABLES_MAX];
+  const int32_t* index[EMBED_TABLES_MAX];
+  int rows[EMBED_TABLES_MAX];
+  float scale[EMBED_TABLES_MAX];
+  int n;
+};
+
 template <typename TW>
-__global__ void embed_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ positions,
-                             const TW* __restrict__ wte, const TW* __restrict__ wpe, float* __restrict__ x,
-                             int T, int E, int vocab, int n_pos, float token_scale, int wide) {
+__global__ void embed_kernel(EmbedTables tb, float* __restrict__ x, int T, int E, int wide) {
   int t = blockIdx.x;
   if (t >= T) return;
-  int tok = tokens[t];
-  int pos = positions[t];
-  bool ok = tok >= 0 && tok < vocab && (wpe == nullptr || (pos >= 0 && pos < n_pos));
-  const float nan = __uint_as_float(0x7fc00000u);   // an id outside the table: NaN, never a neighbour's row
+  int id[EMBED_TABLES_MAX];
+  bool ok = true;
+#pragma unroll
+  for (int i = 0; i < EMBED_TABLES_MAX; ++i) {
+    id[i] = i < tb.n ? tb.index[i][t] : 0;
+    ok = ok && (i >= tb.n || (id[i] >= 0 && id[i] < tb.rows[i]));
+  }
+  const float nan = __uint_as_float(0x7fc00000u);   // an id outside a table: NaN, never a neighbour's row
   if (wide) {
     // 16 bytes of each table per thread and step (E a multiple of that many elements, the tables aligned):
     // a row of 1,600 is one step, all its loads on their way at once
@@ -35,55 +49,84 @@ __global__ void embed_kernel(const int32_t* __restrict__ tokens, const int32_t* 
     for (int e = threadIdx.x * VEC; e < E; e += blockDim.x * VEC) {
       float v[VEC];
       if (ok) {
-        const words4 a = *reinterpret_cast<const words4*>(wte + static_cast<size_t>(tok) * E + e);
-        words4 b = {0u, 0u, 0u, 0u};
-        if (wpe != nullptr) b = *reinterpret_cast<const words4*>(wpe + static_cast<size_t>(pos) * E + e);
+        words4 w[EMBED_TABLES_MAX];
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-          v[i] = element<TW>(a, i);
-          if (token_scale != 1.0f) v[i] *= token_scale;
-          if (wpe != nullptr) v[i] += element<TW>(b, i);
+        for (int i = 0; i < EMBED_TABLES_MAX; ++i)
+          if (i < tb.n) w[i] = *reinterpret_cast<const words4*>(static_cast<const TW*>(tb.table[i]) + static_cast<size_t>(id[i]) * E + e);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+          v[k] = element<TW>(w[0], k);
+          if (tb.scale[0] != 1.0f) v[k] *= tb.scale[0];
         }
+#pragma unroll
+        for (int i = 1; i < EMBED_TABLES_MAX; ++i)
+          if (i < tb.n) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+              float a = element<TW>(w[i], k);
+              if (tb.scale[i] != 1.0f) a *= tb.scale[i];
+              v[k] += a;
+            }
+          }
       } else {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) v[i] = nan;
+        for (int k = 0; k < VEC; ++k) v[k] = nan;
       }
       float* dst = x + static_cast<size_t>(t) * E + e;
 #pragma unroll
-      for (int i = 0; i < VEC; i += 4) *reinterpret_cast<float4*>(dst + i) = float4{v[i], v[i + 1], v[i + 2], v[i + 3]};
+      for (int k = 0; k < VEC; k += 4) *reinterpret_cast<float4*>(dst + k) = float4{v[k], v[k + 1], v[k + 2], v[k + 3]};
     }
     return;
   }
   for (int e = threadIdx.x; e < E; e += blockDim.x) {
     float v = nan;
     if (ok) {
-      v = to_float(wte[static_cast<size_t>(tok) * E + e]);
-      if (token_scale != 1.0f) v *= token_scale;
-      if (wpe != nullptr) v += to_float(wpe[static_cast<size_t>(pos) * E + e]);
+      v = to_float(static_cast<const TW*>(tb.table[0])[static_cast<size_t>(id[0]) * E + e]);
+      if (tb.scale[0] != 1.0f) v *= tb.scale[0];
+      for (int i = 1; i < tb.n; ++i) {
+        float a = to_float(static_cast<const TW*>(tb.table[i])[static_cast<size_t>(id[i]) * E + e]);
+        if (tb.scale[i] != 1.0f) a *= tb.scale[i];
+        v += a;
+      }
     }
     x[static_cast<size_t>(t) * E + e] = v;
   }
 }
 
-extern "C" int dn_embed(const int32_t* tokens, const int32_t* positions, const void* wte, const void* wpe,
-                        float* x, int T, int E, int vocab, int n_pos, int table_dtype, float token_scale,
-                        hipStream_t stream) {
+// tables, indices, rows, scales: n <= 4 entries each (host arrays); every table [rows_i, E] of table_dtype
+extern "C" int dn_embed_sum(const void* const* tables, const int32_t* const* indices, const int* rows,
+                            const float* scales, int n, float* x, int T, int E, int table_dtype,
+                            hipStream_t stream) {
   if (T <= 0) return 0;
-  dim3 grid(T), block(256);
+  if (n < 1 || n > EMBED_TABLES_MAX || E < 1) return DN_ERR_SHAPE;
+  EmbedTables tb{};
+  tb.n = n;
   const int vec = table_dtype == DN_F32 ? 4 : 8;
-  const int wide = E % vec == 0 && reinterpret_cast<uintptr_t>(wte) % 16 == 0 && reinterpret_cast<uintptr_t>(wpe) % 16 == 0 &&
-                   reinterpret_cast<uintptr_t>(x) % 16 == 0;
+  int wide = E % vec == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0;
+  for (int i = 0; i < n; ++i) {
+    if (!tables[i] || !indices[i] || rows[i] < 1) return DN_ERR_SHAPE;
+    tb.table[i] = tables[i], tb.index[i] = indices[i], tb.rows[i] = rows[i], tb.scale[i] = scales[i];
+    wide = wide && reinterpret_cast<uintptr_t>(tables[i]) % 16 == 0;
+  }
+  dim3 grid(T), block(256);
   if (table_dtype == DN_F32)
-    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, tokens, positions,
-                       static_cast<const float*>(wte), static_cast<const float*>(wpe), x, T, E, vocab, n_pos,
-                       token_scale, wide);
+    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, tb, x, T, E, wide);
   else if (table_dtype == DN_BF16)
-    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, tokens, positions,
-                       static_cast<const bf16_t*>(wte), static_cast<const bf16_t*>(wpe), x, T, E, vocab, n_pos,
-                       token_scale, wide);
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, tb, x, T, E, wide);
   else
     return DN_ERR_DTYPE;
   return dn_launch_status();
+}
+
+// the token table and, unless it is null, the position table
+extern "C" int dn_embed(const int32_t* tokens, const int32_t* positions, const void* wte, const void* wpe,
+                        float* x, int T, int E, int vocab, int n_pos, int table_dtype, float token_scale,
+                        hipStream_t stream) {
+  const void* tables[2] = {wte, wpe};
+  const int32_t* indices[2] = {tokens, positions};
+  const int rows[2] = {vocab, n_pos};
+  const float scales[2] = {token_scale, 1.0f};
+  return dn_embed_sum(tables, indices, rows, scales, wpe ? 2 : 1, x, T, E, table_dtype, stream);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -456,9 +456,6 @@ static int run(const void* A, int lda, const void* W, const float* bias, void* C
 #define PACKED_A 2
 #define PACKED_C 4
 
-static int g_tune[8] = {-1, -1, 0, 0, 0, 0, 0, 0};   // [0] direct shape, [1] shares, [2] kernel (1 few, 2 many), [3] skinny MB*100+NB*10+U
-extern "C" void dn_gemm_tune(int i, int v) { g_tune[i] = v; }
-
 namespace skinny {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
@@ -482,6 +479,7 @@ struct NormIO {
   int blocks_in;             // K / 16
   const float* c1;           // NORM_IN: [N]  (c2 comes as the bias)
   float eps;
+  int no_mean;               // NORM_IN: the norm takes no mean off (x / sqrt(mean(x^2) + eps) * gamma): the row's mean counts as 0
   const float* gamma_out;    // NORM_OUT: [N] the next norm's weight
   bf16_t* copy_out;          // NORM_OUT: [M, ldcopy] the updated rows times gamma_out in bfloat16
   int ldcopy;
@@ -607,7 +605,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
 #pragma unroll
       for (int i = 0; i < SP; ++i)
         if (lane + 64 * i < nio.blocks_in) sm += st[t][i].x;
-      const float mean = wave_sum(sm) / blocks;
+      const float mean = nio.no_mean ? 0.f : wave_sum(sm) / blocks;      // (without it the squares are taken about 0)
       float sq = 0.f;
 #pragma unroll
       for (int i = 0; i < SP; ++i)
@@ -839,7 +837,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
 #pragma unroll
       for (int i = 0; i < SP; ++i)
         if (lane + 64 * i < nio.blocks_in) sm += st[t][i].x;
-      const float mean = wave_sum(sm) / blocks;
+      const float mean = nio.no_mean ? 0.f : wave_sum(sm) / blocks;      // (without it the squares are taken about 0)
       float sq = 0.f;
 #pragma unroll
       for (int i = 0; i < SP; ++i)
@@ -1007,18 +1005,10 @@ static void launch16(const Call& c, hipStream_t stream) {
 template <int WAVES>
 static void launch_mb(const Call& c, hipStream_t stream) {
   const int mb = (c.M + 15) / 16;
-  if (g_tune[3] > 0 && mb > 1) {
-    switch (g_tune[3]) {
-      case 424: return launch<4, 2, WAVES, 4>(c, stream);
-      case 444: return launch<4, 4, WAVES, 4>(c, stream);
-      case 442: return launch<4, 4, WAVES, 2>(c, stream);
-      case 418: return launch<4, 1, WAVES, 8>(c, stream);
-      case 224: return launch<2, 2, WAVES, 4>(c, stream);
-      case 244: return launch<2, 4, WAVES, 4>(c, stream);
-      case 822: return launch<8, 2, WAVES, 2>(c, stream);
-      default: break;
-    }
-  }
+  // 65 to 256 rows of a product with few columns and a short K (an output projection): four row blocks and two
+  // column blocks per workgroup, the rows shared out among workgroups (at 1,600 x 1,600: 6.7 us at 128 rows and 8.0
+  // at 256, where sixteen row blocks x one column block took 7.7 and 12.6: every workgroup read all rows)
+  if (mb > 4 && c.N < 2048 && c.K < 4096) return launch<4, 2, WAVES, 4>(c, stream);
   if (mb == 1 && !(c.packed & (PACKED_A | PACKED_C)) && c.M > 1) return launch16<WAVES>(c, stream);
   if (mb == 1) return launch<1, 1, WAVES, 8>(c, stream);
   if (mb > 4) {
@@ -1396,7 +1386,7 @@ __device__ __forceinline__ void wait_loads() {      // until at most N of this w
 }
 
 // WM x WN waves, each TM x TN blocks of 16 x 16: the tile is 16 WM TM rows x 16 WN TN columns
-template <typename TC, int WM, int WN, int TM, int TN, int STAGES, bool KV>
+template <typename TC, int WM, int WN, int TM, int TN, int STAGES, bool KV, int KB = 1>
 __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __restrict__ A, int lda,
                                                            const bf16_t* __restrict__ W, const float* __restrict__ bias,
                                                            TC* __restrict__ C, int ldc, float* __restrict__ resid, int ldr,
@@ -1405,9 +1395,10 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
                                                            int split_slabs) {
   constexpr int NW = WM * WN;
   constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
-  constexpr int AB = BM / 16, WB = BN / 16;              // 1 KB blocks per slab
-  constexpr int SLAB = (AB + WB) * 64;                   // in u32x4
-  constexpr int HI = (AB + WB + NW - 1) / NW, REM = (AB + WB) % NW;   // waves below REM load HI blocks, the others HI - 1
+  constexpr int AB = BM / 16, WB = BN / 16;              // 1 KB blocks per slab of 32 along K
+  constexpr int PER = (AB + WB) * KB;                    // blocks per stage: KB slabs travel and are multiplied together
+  constexpr int SLAB = PER * 64;                         // a stage, in u32x4
+  constexpr int HI = (PER + NW - 1) / NW, REM = PER % NW;   // waves below REM load HI blocks, the others HI - 1
   static_assert((STAGES - 2) * HI < 64, "vmcnt has six bits");
   extern __shared__ u32x4 lds[];
   const int total = tiles_m * tiles_n;
@@ -1420,9 +1411,10 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
   const int wmb = (wave / WN) * TM, wnb = (wave % WN) * TN;     // in blocks
   // part: K is shared out among the workgroups of blockIdx.y, split_slabs slabs each; a workgroup leaves
   // its sums in part[blockIdx.y][m][n] and a second kernel adds them in order and ends with the epilogue
+  // (stages of KB slabs: the host launches KB > 1 only where K is a multiple of 32 KB; split_slabs counts stages)
   const int kall = K / 32, nblocks = (N + 15) / 16;
   const int first = part ? blockIdx.y * split_slabs : 0;
-  const int ksteps = part ? min(split_slabs, kall - first) : kall;
+  const int ksteps = part ? min(split_slabs, kall / KB - first) : kall / KB;
   // where the 16 bytes of row lane % 16, columns 8 (lane / 16) .. of a block of A lie in its 1 KB
   // (see the loads below): any 8 and any 16 consecutive lanes read all banks once
   // (a packed A is in the operand's order already: lane l reads at 16 l)
@@ -1440,7 +1432,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
   int step[HI];
 #pragma unroll
   for (int u = 0; u < HI; ++u) {
-    const int b = min(wave + u * NW, AB + WB - 1);
+    const int q = min(wave + u * NW, PER - 1);
+    const int b = q % (AB + WB), kb = q / (AB + WB);      // block b of the stage's slab kb
     if (b < AB) {
       // 16 lanes in a row take 64 bytes from each of four rows (g, g + 4, g + 8, g + 12 of the block):
       // four cache lines, where a lane per row would touch sixteen
@@ -1456,14 +1449,15 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
       src[u] = W + static_cast<size_t>(min(n0 / 16 + b - AB, nblocks - 1)) * kall * 512 + lane * 8;
       step[u] = 512;
     }
-    src[u] += static_cast<size_t>(first) * step[u];
+    src[u] += (static_cast<size_t>(first) * KB + kb) * step[u];
+    step[u] *= KB;
   }
   auto issue = [&](int kt) {
     u32x4* slab = lds + (kt % STAGES) * SLAB;
 #pragma unroll
     for (int u = 0; u < HI; ++u) {
-      const int b = wave + u * NW;
-      if (u < HI - 1 || REM == 0 || wave < REM) load_to_lds(src[u] + static_cast<size_t>(kt) * step[u], slab + b * 64);
+      const int q = wave + u * NW;
+      if (u < HI - 1 || REM == 0 || wave < REM) load_to_lds(src[u] + static_cast<size_t>(kt) * step[u], slab + q * 64);
     }
   };
 #pragma unroll
@@ -1483,15 +1477,19 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const bf16_t* __rest
     __builtin_amdgcn_s_barrier();      // every wave's share of slab kt is there, and slab kt - 1 has been read
     if (kt + STAGES - 1 < ksteps) issue(kt + STAGES - 1);
     const u32x4* slab = lds + (kt % STAGES) * SLAB;
-    bf16x8 af[TM], wf[TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) af[i] = __builtin_bit_cast(bf16x8, slab[(wmb + i) * 64 + aslot]);
+    for (int kb = 0; kb < KB; ++kb) {
+      const u32x4* sl = slab + kb * (AB + WB) * 64;
+      bf16x8 af[TM], wf[TN];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) wf[j] = __builtin_bit_cast(bf16x8, slab[(AB + wnb + j) * 64 + lane]);
+      for (int i = 0; i < TM; ++i) af[i] = __builtin_bit_cast(bf16x8, sl[(wmb + i) * 64 + aslot]);
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+      for (int j = 0; j < TN; ++j) wf[j] = __builtin_bit_cast(bf16x8, sl[(AB + wnb + j) * 64 + lane]);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], af[i], acc[i][j], 0, 0, 0);
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], af[i], acc[i][j], 0, 0, 0);
+    }
   }
   // acc[i][j][r]: row m0 + 16 (wmb + i) + lane % 16, column n0 + 16 (wnb + j) + 4 (lane / 16) + r
   //
@@ -1629,31 +1627,32 @@ struct Args {
   float* part = nullptr; int splits = 1;       // part: K in `splits` shares, their sums in part[share][m][n]
 };
 
-template <typename TC, int WM, int WN, int TM, int TN, int STAGES, bool KV>
+template <typename TC, int WM, int WN, int TM, int TN, int STAGES, bool KV, int KB = 1>
 static int launch(const Args& a, hipStream_t stream) {
   constexpr int BM = WM * TM * 16, BN = WN * TN * 16;
   const int tiles_m = (a.M + BM - 1) / BM, tiles_n = (a.N + BN - 1) / BN;
-  constexpr size_t lds = static_cast<size_t>(STAGES) * (BM + BN) / 16 * 1024;
+  constexpr size_t lds = static_cast<size_t>(STAGES) * KB * (BM + BN) / 16 * 1024;
+  if (a.K % (32 * KB) != 0) return DN_ERR_SHAPE;
   static bool raised = false;      // more than 64 KB of LDS has to be asked for once per kernel
   if (lds > 65536 && !raised) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<TC, WM, WN, TM, TN, STAGES, KV>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<TC, WM, WN, TM, TN, STAGES, KV, KB>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     if (e != hipSuccess) return static_cast<int>(e);
     raised = true;
   }
-  const int split_slabs = (a.K / 32 + a.splits - 1) / a.splits;
-  hipLaunchKernelGGL((gemm_kernel<TC, WM, WN, TM, TN, STAGES, KV>), dim3(tiles_m * tiles_n, a.part ? a.splits : 1),
+  const int split_slabs = (a.K / (32 * KB) + a.splits - 1) / a.splits;
+  hipLaunchKernelGGL((gemm_kernel<TC, WM, WN, TM, TN, STAGES, KV, KB>), dim3(tiles_m * tiles_n, a.part ? a.splits : 1),
                      dim3(WM * WN * 64), lds, stream, static_cast<const bf16_t*>(a.A), a.lda,
                      static_cast<const bf16_t*>(a.W), a.bias, static_cast<TC*>(a.C), a.ldc, a.resid, a.ldr, a.M, a.N, a.K,
                      a.epi, a.packed, tiles_m, tiles_n, a.kv ? *a.kv : KVScatter{}, a.part, split_slabs);
   return 0;
 }
 
-template <int WM, int WN, int TM, int TN, int STAGES>
+template <int WM, int WN, int TM, int TN, int STAGES, int KB = 1>
 static int launch_as(const Args& a, hipStream_t stream) {
-  if (a.kv) return launch<bf16_t, WM, WN, TM, TN, STAGES, true>(a, stream);
-  if (a.out_dtype == DN_BF16 && !a.resid) return launch<bf16_t, WM, WN, TM, TN, STAGES, false>(a, stream);
-  return launch<float, WM, WN, TM, TN, STAGES, false>(a, stream);
+  if (a.kv) return launch<bf16_t, WM, WN, TM, TN, STAGES, true, KB>(a, stream);
+  if (a.out_dtype == DN_BF16 && !a.resid) return launch<bf16_t, WM, WN, TM, TN, STAGES, false, KB>(a, stream);
+  return launch<float, WM, WN, TM, TN, STAGES, false, KB>(a, stream);
 }
 
 // The tiles on offer: rows x columns, slabs in flight.  256 rows: 8 waves as 4 x 2, one workgroup
@@ -1661,8 +1660,9 @@ static int launch_as(const Args& a, hipStream_t stream) {
 // for products with few rows and a long K, whose larger tiles would leave most CUs idle.
 struct Shape { int bm, bn, stages; };
 constexpr Shape SHAPES[] = {{64, 128, 4}, {128, 128, 4}, {256, 128, 4}, {256, 160, 4}, {256, 192, 4},
-                            {256, 224, 4}, {256, 256, 4}, {256, 320, 3}, {64, 64, 4}, {32, 64, 4},
-                            {64, 64, 8}, {32, 64, 8}, {64, 128, 6}, {32, 128, 8}, {128, 64, 6}, {64, 32, 8}};
+                            {256, 224, 4}, {256, 256, 4}, {256, 320, 3}, {64, 64, 4}, {32, 64, 4}, {64, 64, 4}};
+constexpr int PICKED = 10;        // the shapes that `pick` chooses among
+constexpr int MID = 10;           // 64 x 64 with two slabs a stage: `mid_rows`
 
 static double model_us(const Shape& s, int M, int N, int K) {
   const double tiles = static_cast<double>((M + s.bm - 1) / s.bm) * ((N + s.bn - 1) / s.bn);
@@ -1675,37 +1675,49 @@ static double model_us(const Shape& s, int M, int N, int K) {
 }
 
 static int pick(int M, int N, int K) {
-  if (g_tune[0] >= 0) return g_tune[0];
   int best = 0;
   double best_us = 1e30;
-  for (int i = 0; i < 10; ++i) {
+  for (int i = 0; i < PICKED; ++i) {
     const double us = model_us(SHAPES[i], M, N, K);
     if (us < best_us) best_us = us, best = i;
   }
   return best;
 }
 
-// Up to 256 rows the few-rows kernel takes the product too (both read and write packed rows).
-// This one is the faster from 105 rows on where the product has 4,096 columns or more, and from 209 rows
-// on from 2,048 columns (both borders as measured); with fewer columns its tiles
-// leave most CUs idle and the few-rows kernel stays ahead, or level, at every size.
+// 65 to 512 rows.  A tile's walk along K costs a wave some dozens of instructions a slab beside its four matrix
+// instructions, and with one or two waves a SIMD nothing hides them: tiles of 64 x 64 take two slabs a stage
+// (SHAPES[MID]), which halves that and fills the chip from 65 rows on where the product is wide.  Measured on the
+// four products of a layer 1,600 wide (rows and weights that no cache holds; us, before -> now):
+//   128 rows: 4,800 columns 18.7 -> 15.7, 6,400 columns 15.3 -> 12.3, 1,600 columns from K = 6,400 19.4 -> 15.2
+//   256 rows: 25.6 -> 23.2, 19.3 -> 18.0, 25.6 -> 21.4;  512 rows, 1,600 columns: K = 1,600 12.6 -> 10.7, K = 6,400 38.7 -> 35.4
+// -> whether this kernel takes the product with SHAPES[MID] (else `pick` chooses, or the few-rows kernel runs)
+static bool mid_rows(int M, int N, int K) {
+  if (M <= 64 || M > 512 || K % 64 != 0) return false;
+  if (N < 2048) return K >= 4096 || M > 256;      // (few columns and a short K up to 256 rows: the few-rows kernel)
+  return M <= 256;
+}
+
+// Up to 256 rows the few-rows kernel takes the product too (both read and write packed rows): it stays ahead,
+// or level, where the product has few columns and a short K; everywhere else from 65 rows on this kernel is
+// the faster (`mid_rows`), and beyond 256 rows it is the only one.
 static bool beats_few_rows(int M, int N, int K) {
-  (void)K;
-  if (g_tune[2] > 0) return g_tune[2] == 2;
-  return (M > 104 && N >= 4096) || (M > 208 && N >= 2048);
+  return mid_rows(M, N, K) || (M > 104 && N >= 4096) || (M > 208 && N >= 2048);
 }
 
 // A long K beside few columns and few rows: the tiles are few and each walks all of K, a slab at a time,
 // so K is shared out among several workgroups per tile (whole, such a product takes the same time whatever
-// its rows up to 256, and a quarter of K less than a third of it).  The number of shares, 0 for none: 8
-// where the tiles of 32 x 64 are at most 96, else 4 (with more rows 8 shares gain nothing over 4).
+// its rows up to 256, and a quarter of K less than a third of it).  The number of shares, 0 for none.  With
+// fewer than 2,048 columns: 4 up to 128 rows, 2 up to 256, none beyond (1,600 columns, K = 6,400: 15.2, 21.4
+// and 35.4 us at 128, 256 and 512 rows; with 8, 4 and 4 shares of smaller tiles 19.4, 25.6, 38.7).  From 2,048 columns: 8
+// where the tiles of 32 x 64 are at most 96, else 4.
 static int shares_of_k(int M, int N, int K, int packed, bool kv) {
-  if (g_tune[1] >= 0) return (kv || (packed & PACKED_C)) ? 0 : g_tune[1];
   if (kv || (packed & PACKED_C) || M <= 64 || M > 512 || N >= 4096 || K < 4096) return 0;
+  if (N < 2048 && K % 64 == 0) return M <= 128 ? 4 : M <= 256 ? 2 : 0;
   return ((M + 31) / 32) * ((N + 63) / 64) <= 96 ? 8 : 4;
 }
 
 static int run(const Args& a, hipStream_t stream) {
+  if (mid_rows(a.M, a.N, a.K)) return launch_as<2, 2, 2, 2, 4, 2>(a, stream);
   switch (pick(a.M, a.N, a.part ? a.K / a.splits : a.K)) {
     case 0: return launch_as<2, 2, 2, 4, 4>(a, stream);
     case 1: return launch_as<4, 2, 2, 4, 4>(a, stream);
@@ -1716,20 +1728,14 @@ static int run(const Args& a, hipStream_t stream) {
     case 6: return launch_as<4, 2, 4, 8, 4>(a, stream);
     case 7: return launch_as<4, 2, 4, 10, 3>(a, stream);
     case 8: return launch_as<2, 2, 2, 2, 4>(a, stream);
-    case 9: return launch_as<2, 2, 1, 2, 4>(a, stream);
-    case 10: return launch_as<2, 2, 2, 2, 8>(a, stream);
-    case 11: return launch_as<2, 2, 1, 2, 8>(a, stream);
-    case 12: return launch_as<2, 2, 2, 4, 6>(a, stream);
-    case 13: return launch_as<2, 2, 1, 4, 8>(a, stream);
-    case 14: return launch_as<2, 2, 4, 2, 6>(a, stream);
-    default: return launch_as<2, 2, 2, 1, 8>(a, stream);
+    default: return launch_as<2, 2, 1, 2, 4>(a, stream);
   }
 }
 }  // namespace direct
 
 // the tile that a product of these sizes gets from the kernel above: rows * 1000 + columns
 extern "C" int dn_gemm_tile(int M, int N, int K) {
-  const direct::Shape& s = direct::SHAPES[direct::pick(M, N, K)];
+  const direct::Shape& s = direct::SHAPES[direct::mid_rows(M, N, K) ? direct::MID : direct::pick(M, N, K)];
   return s.bm * 1000 + s.bn;
 }
 
@@ -1850,7 +1856,7 @@ extern "C" int dn_gemm_norm_out(const void* A, int lda, const void* W, const flo
   const int packed = PACKED_W | (lda == 0 ? PACKED_A : 0);
   if (!skinny::takes(A, lda, W, M, K, packed)) return DN_ERR_SHAPE;
   skinny::Call c{A, lda, W, bias, nullptr, 0, resid, ldr, M, N, K, DN_F32, EPI_NONE, packed, nullptr};
-  skinny::NormIO nio{nullptr, 0, nullptr, 0.f, gamma, static_cast<bf16_t*>(copy), ldcopy, stats};
+  skinny::NormIO nio{nullptr, 0, nullptr, 0.f, 0, gamma, static_cast<bf16_t*>(copy), ldcopy, stats};
   if (M > 16)
     skinny::launch_mb_norm(c, nio, NORM_OUT, stream);
   else if (K >= 1024)
@@ -1863,13 +1869,14 @@ extern "C" int dn_gemm_norm_out(const void* A, int lda, const void* W, const flo
 // The product after such a norm: C [M, N] bfloat16 = act(LayerNorm(x) . W^T + b), where A is the
 // copy of x times gamma [M, K] (in rows, or lda == 0: packed rows) and stats [M][K / 16][2] what
 // dn_gemm_norm_out left, c1[n] = sum_k gamma[k] W[n,k] and c2[n] = sum_k beta[k] W[n,k] + b[n].
+// no_mean: the norm is x / sqrt(mean(x^2) + eps) * gamma (no mean taken off, no beta: c1 is not used).
 // Up to 16 rows (A in rows, K a multiple of 16 up to 4,096), or 17 to 64 rows (K from 1,024 to 2,048).
 // With slot_map, the key and value columns go to their pages as in dn_gemm_qkv; without, ldc == 0 asks
 // for C in packed rows (17 rows and more, N a multiple of 32).
 extern "C" int dn_gemm_norm_in(const void* A, int lda, const float* stats, const float* c1, const float* c2,
                                float eps, const void* W, void* C, int ldc, int M, int N, int K,
                                int epilogue, const int32_t* slot_map, void* k_pool, void* v_pool, int q_width,
-                               int Hkv, int dh, int page_size, int c_cols, hipStream_t stream) {
+                               int Hkv, int dh, int page_size, int c_cols, int no_mean, hipStream_t stream) {
   if (M < 1 || M > 64 || N < 1 || K < 16 || K % 16 != 0 || K > 4096 || (lda != 0 && lda < K) || !stats || !c1 || !c2 || !C)
     return DN_ERR_SHAPE;
   if (M <= 16 ? lda == 0 : (K < 1024 || K > 2048)) return DN_ERR_SHAPE;
@@ -1888,7 +1895,7 @@ extern "C" int dn_gemm_norm_in(const void* A, int lda, const float* stats, const
   }
   skinny::Call c{A, lda, W, c2, C, ldc, nullptr, 0, M, N, K, DN_BF16, epilogue, packed | (ldc == 0 ? PACKED_C : 0),
                  slot_map ? &kv : nullptr};
-  skinny::NormIO nio{stats, K / 16, c1, eps, nullptr, nullptr, 0, nullptr};
+  skinny::NormIO nio{stats, K / 16, c1, eps, no_mean ? 1 : 0, nullptr, nullptr, 0, nullptr};
   if (M > 16)
     skinny::launch_mb_norm(c, nio, NORM_IN, stream);
   else if (K >= 1024)

@@ -96,6 +96,7 @@ def _declare(name, lib):
     sigs = {
         "elementwise": {
             "dn_embed": [P, P, P, P, P, I, I, I, I, I, F, P],
+            "dn_embed_sum": [P, P, P, P, I, P, I, I, I, P],
             "dn_logits_post": [P, I, I, I, F, F, P],
             "dn_layernorm": [P, P, P, P, P, I, I, F, I, I, P],
             "dn_kv_write": [P, I, I, I, P, P, P, I, I, I, I, I, P],
@@ -107,7 +108,7 @@ def _declare(name, lib):
             "dn_gemm_plain_qkv": [P, I, P, P, P, I, I, I, I, I, P, P, P, I, I, I, I, P, c_longlong, P],
             "dn_pack_matrix": [P, P, I, I, P],
             "dn_gemm_norm_out": [P, I, P, P, P, I, I, I, I, P, P, I, P, P],
-            "dn_gemm_norm_in": [P, I, P, P, P, F, P, P, I, I, I, I, I, P, P, P, I, I, I, I, I, P],
+            "dn_gemm_norm_in": [P, I, P, P, P, F, P, P, I, I, I, I, I, P, P, P, I, I, I, I, I, I, P],
             "dn_gemm_qkv": [P, I, P, P, P, I, I, I, I, P, P, P, I, I, I, I, I, I, P],
         },
         "attention": {
@@ -209,6 +210,31 @@ def embed(tokens, positions, wte, wpe, out, token_scale=1.0):
     _ok(_lib("elementwise").dn_embed(tokens.data_ptr(), positions.data_ptr(), wte.data_ptr(), _ptr(wpe),
                                      out.data_ptr(), T, E, wte.shape[0], n_pos, _CODE[wte.dtype], float(token_scale),
                                      _stream()), "embed")
+    return out
+
+
+EMBED_TABLES_MAX = 4
+
+
+def embed_sum(parts, out):
+    """out[t,:] = sum over parts, in their order, of table[index[t],:] * scale.  parts: up to four
+    (table [rows, E], index int32 [T], scale); all tables of one dtype; out is 32-bit [T, E]."""
+    _need(1 <= len(parts) <= EMBED_TABLES_MAX, lambda: f"embed_sum: 1 to {EMBED_TABLES_MAX} tables, not {len(parts)}")
+    _dev(out, "out", (torch.float32,), 2)
+    T, E = out.shape
+    _need(out.is_contiguous(), "embed_sum: out")
+    dtype = parts[0][0].dtype
+    n = len(parts)
+    tables, indices = (c_void_p * n)(), (c_void_p * n)()
+    rows, scales = (c_int * n)(), (c_float * n)()
+    for i, (table, index, scale) in enumerate(parts):
+        _dev(table, "table", (dtype,), 2), _dev(index, "index", _I32, 1)
+        _need(dtype in _FLOATS, "embed_sum: table dtype")
+        _need(table.is_contiguous() and table.shape[1] == E, lambda: f"embed_sum: table {i} is {tuple(table.shape)}, rows are {E} wide")
+        _need(index.is_contiguous() and index.shape[0] == T, lambda: f"embed_sum: index {i}")
+        tables[i], indices[i], rows[i], scales[i] = table.data_ptr(), index.data_ptr(), table.shape[0], float(scale)
+    _ok(_lib("elementwise").dn_embed_sum(tables, indices, rows, scales, n, out.data_ptr(), T, E, _CODE[dtype], _stream()),
+        "embed")
     return out
 
 
@@ -499,6 +525,8 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
     _dev(block_tables, "block_tables", _I32, 2), _dev(tiles, "tiles", _I32, 2)
     n_pages, Hkv, ps, dh = k_pool.shape
     T = q.shape[0]
+    _need(v_pool.shape[2] == dh, lambda: f"attention: values of width {v_pool.shape[2]} beside keys of width {dh}: "
+                                         "these kernels take keys and values of one width")
     _need(k_pool.is_contiguous() and v_pool.is_contiguous() and tuple(v_pool.shape) == (n_pages, Hkv, dh, ps),
           "attention: pools")
     _need(q.shape[1] >= n_heads * dh and tuple(out.shape) == (T, n_heads * dh), "attention: q/out shapes")
@@ -706,13 +734,14 @@ def norm_stream_buffers(n_rows, width, device):
     return copy, torch.empty((n_rows, width // 16, 2), dtype=torch.float32, device=device)
 
 
-def norm_folded(w_rows, bias, gamma, beta):
+def norm_folded(w_rows, bias, gamma, beta, no_mean=False):
     """(c1, c2) for linear_norm_in: with y = (x - mean) / sqrt(var + eps) * gamma + beta,
     y @ w.T + bias = ((x * gamma) @ w.T - mean * c1) / sqrt(var + eps) + c2, where
     c1 = w @ gamma and c2 = w @ beta + bias, in 32-bit from the weight as the kernel holds it.
-    w_rows: [N, K] (any float dtype); made once per pair of norm and weight."""
+    w_rows: [N, K] (any float dtype); made once per pair of norm and weight.  no_mean: a norm that takes no
+    mean off (an RMS norm): c1 is zeros and is not used."""
     w = w_rows.float()
-    c1 = w @ gamma.float()
+    c1 = torch.zeros(w.shape[0], dtype=torch.float32, device=w.device) if no_mean else w @ gamma.float()
     c2 = torch.zeros_like(c1) if beta is None else w @ beta.float()
     if bias is not None:
         c2 = c2 + bias.float()
@@ -754,11 +783,12 @@ def linear_norm_out(a, w, bias, residual, gamma, copy, stats):
     return residual
 
 
-def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None):
+def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None, no_mean=False):
     """out = epilogue(LayerNorm(x) @ w.T + bias) where copy and stats are what linear_norm_out left
     of x (with this norm's gamma) and c1, c2 = norm_folded(w, bias, gamma, beta).  out: bfloat16
     [M, N]; kv = (slot_map, k_pool, v_pool, q_width): a fused projection whose key and value columns
-    go to the cache (out may then hold the queries alone); returns out, or the queries."""
+    go to the cache (out may then hold the queries alone); returns out, or the queries.
+    no_mean: the norm takes no mean off (x / sqrt(mean(x^2) + eps) * gamma); c1 is then not used."""
     M, K = copy.shape
     N = w.shape[0]
     _need(norm_stream_takes(M, K, w) and w.shape[1] == K, "linear_norm_in: sizes it does not take")
@@ -790,7 +820,7 @@ def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None):
         args = (slot_map.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), q_width, Hkv, dh, ps, out.shape[1])
     _ok(_lib("gemm").dn_gemm_norm_in(copy.data_ptr(), lda, stats.data_ptr(), c1.data_ptr(),
                                      c2.data_ptr(), float(eps), w.data_ptr(), out.data_ptr(), ldc,
-                                     M, N, K, EPILOGUES[epilogue], *args, _stream()),
+                                     M, N, K, EPILOGUES[epilogue], *args, int(bool(no_mean)), _stream()),
         "linear_norm_in" if _timed is None else
         f"norm + linear {K} -> {N}" + (", cache write" if kv is not None else "") + (f", {epilogue}" if epilogue != "none" else ""))
     return out if kv is None else out[:, :kv[3]]

@@ -31,11 +31,20 @@ from ..weights.spec import ParamSpec
 @dataclass(frozen=True)
 class PagedKV:
     """A mixer that keeps keys and values of `window` last positions (0: all) in pages.
-    dtype: what the pages hold ("bfloat16", "float32"); None: the engine's activation dtype."""
+    dtype: what the pages hold ("bfloat16", "float32"); None: the engine's activation dtype.
+    head_dim is the width of a key; value_dim that of a value (None: the same).  The pools are laid out for
+    both ([.., Hkv, page, head_dim] and [.., Hkv, value_dim, page]); the attention kernels of this package
+    take equal widths only and say so when they are asked for others (kernels.ops.attention), so a mixer whose
+    values are wider or narrower than its keys brings a kernel of its own for the same pools."""
     n_kv_heads: int
     head_dim: int
     window: int = 0
     dtype: Optional[str] = None
+    value_dim: Optional[int] = None
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)

@@ -16,21 +16,31 @@ from .base import LazyNorm
 
 class Linear:
     def __init__(self, in_features: int, out_features: int, weight_name: str, bias_name: Optional[str],
-                 stored_in_out: bool = False, init_std: float = 0.02):
+                 stored_in_out: bool = False, init_std: float = 0.02, weight_sources=None, bias_sources=None):
+        """weight_sources, bias_sources: ((file name, output columns), ...): the checkpoint stores the weight
+        (the bias) as several tensors, one per run of output columns (q, k and v of a fused projection; gate
+        and up); they are joined once, at load, and `weight_name` / `bias_name` then name only what is held."""
         self.in_features, self.out_features = in_features, out_features
         self.weight_name, self.bias_name = weight_name, bias_name
         self.stored_in_out = stored_in_out
         self.init_std = init_std
+        self.weight_sources = tuple((n, int(c)) for n, c in weight_sources) if weight_sources else None
+        self.bias_sources = tuple((n, int(c)) for n, c in bias_sources) if bias_sources else None
+        if self.bias_sources and not bias_name:
+            raise ValueError("Linear: bias_sources need a bias_name to hold them under")
         self.weight = None
         self.bias = None
         self._folded = {}      # id(norm) -> (c1, c2, eps): see fold_norm
 
     def param_specs(self):
         shape = (self.in_features, self.out_features) if self.stored_in_out else (self.out_features, self.in_features)
+        # (the output columns are the stored layout's first dimension, or its second where it is [in, out])
         specs = [ParamSpec(self.weight_name, shape, "matrix", ("normal", 0.0, self.init_std),
-                           transpose=self.stored_in_out)]
+                           transpose=self.stored_in_out, sources=self.weight_sources,
+                           concat_dim=1 if self.stored_in_out else 0)]
         if self.bias_name:
-            specs.append(ParamSpec(self.bias_name, (self.out_features,), "vector", ("normal", 0.0, 0.01)))
+            specs.append(ParamSpec(self.bias_name, (self.out_features,), "vector", ("normal", 0.0, 0.01),
+                                   sources=self.bias_sources))
         return specs
 
     def bind(self, tensors):
@@ -59,9 +69,13 @@ class Linear:
         if f is None or not (ops.norm_stream_takes(1, self.in_features, self.weight)
                              or ops.norm_stream_takes(17, self.in_features, self.weight)):
             return
+        # kinds: "layernorm" ((x - mean) / sqrt(var + eps) * gamma + beta) and "rmsnorm" (x / sqrt(mean(x^2) + eps)
+        # * gamma, beta None); a norm of another kind runs as its own kernel
         kind, gamma, beta, eps = f()
         if kind == "layernorm":
-            self._folded[id(norm)] = (*ops.norm_folded(self.weight.rows(), self.bias, gamma, beta), eps)
+            self._folded[id(norm)] = (*ops.norm_folded(self.weight.rows(), self.bias, gamma, beta), eps, False)
+        elif kind == "rmsnorm" and beta is None:
+            self._folded[id(norm)] = (*ops.norm_folded(self.weight.rows(), self.bias, gamma, None, no_mean=True), eps, True)
 
     def takes_lazy_norm(self, n_rows: int, norm) -> bool:
         """Whether a call with n_rows rows can run `norm` in its own kernel (fold_norm has been called)."""
@@ -72,7 +86,7 @@ class Linear:
         return ops.norm_stream_takes(n_rows, self.out_features, self.weight) and self.in_features % 8 == 0
 
     def _fusable(self, a, out_dtype):
-        """(c1, c2, eps) if `a` is a LazyNorm that this call can run in its own kernel."""
+        """(c1, c2, eps, no_mean) if `a` is a LazyNorm that this call can run in its own kernel."""
         if ((out_dtype or a.dtype) == torch.bfloat16 and a.stream is not None and a.stream.written
                 and a.stream.norm is a.norm and self.takes_lazy_norm(a.shape[0], a.norm)):
             return self._folded[id(a.norm)]
@@ -88,7 +102,8 @@ class Linear:
             if f is not None:
                 out = (ops.packed_rows(a.shape[0], self.out_features, a.device) if packed_out else
                        torch.empty((a.shape[0], self.out_features), dtype=torch.bfloat16, device=a.device))
-                return ops.linear_norm_in(a.stream.copy, a.stream.stats, f[0], f[1], f[2], self.weight, out, epilogue=epilogue)
+                return ops.linear_norm_in(a.stream.copy, a.stream.stats, f[0], f[1], f[2], self.weight, out, epilogue=epilogue,
+                                          no_mean=f[3])
             a = a.rows(packed=self.packed_input(a.shape[0]))
         if a.dtype != self.weight.dtype:
             a = ops.cast(a.contiguous(), torch.empty(a.shape, dtype=self.weight.dtype, device=a.device))
@@ -112,7 +127,7 @@ class Linear:
             if f is not None:
                 out = torch.empty((a.shape[0], q_width), dtype=torch.bfloat16, device=a.device)
                 return ops.linear_norm_in(a.stream.copy, a.stream.stats, f[0], f[1], f[2], self.weight, out,
-                                          kv=(slot_map, k_pool, v_pool, q_width))
+                                          kv=(slot_map, k_pool, v_pool, q_width), no_mean=f[3])
             a = a.rows(packed=self.packed_input(a.shape[0]))
         if a.dtype != self.weight.dtype:
             a = ops.cast(a.contiguous(), torch.empty(a.shape, dtype=self.weight.dtype, device=a.device))

@@ -18,12 +18,15 @@ class CausalSelfAttention(Part):
     window > 0: a query at position p reads keys p - window + 1 .. p only.
     scale multiplies the scores before the softmax.
     position: a position encoding of this layer's own, as (kind name, arguments), of the kind that
-    turns queries and keys; None: the model's."""
+    turns queries and keys; None: the model's.
+    qkv_weight_sources, qkv_bias_sources: ((file name, columns), ...) where the checkpoint stores the three
+    projections as tensors of their own; qkv_weight / qkv_bias then only name the joined tensors."""
     graph_safe = True
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                  qkv_weight: str, qkv_bias, out_weight: str, out_bias, stored_in_out: bool = False,
-                 window: int = 0, out_init_std: float = 0.02, position=None):
+                 window: int = 0, out_init_std: float = 0.02, position=None, qkv_weight_sources=None,
+                 qkv_bias_sources=None):
         self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
         self.scale, self.window = float(scale), int(window)
         if n_heads % n_kv_heads != 0:
@@ -32,7 +35,9 @@ class CausalSelfAttention(Part):
             raise ValueError(f"head size {head_dim}: the attention kernels take multiples of 16 up to 256")
         self.q_width = n_heads * head_dim
         self.kv_width = n_kv_heads * head_dim
-        self.qkv = Linear(width, self.q_width + 2 * self.kv_width, qkv_weight, qkv_bias, stored_in_out)
+        # (a checkpoint that stores q, k and v apart names them in qkv_*_sources: joined at load, one product here)
+        self.qkv = Linear(width, self.q_width + 2 * self.kv_width, qkv_weight, qkv_bias, stored_in_out,
+                          weight_sources=qkv_weight_sources, bias_sources=qkv_bias_sources)
         self.out = Linear(self.q_width, width, out_weight, out_bias, stored_in_out, out_init_std)
         self.position = POSITIONS.make(position) if position is not None else None
         if self.position is not None:

@@ -42,6 +42,16 @@ class LayerCall:
 
 
 @dataclass
+class EmbeddingTable:
+    """A further table [rows, width] whose rows are added to the token and position rows in the embedding kernel.
+    index: which per-row integers of the step pick its rows: "tokens" or "positions" (fields of StepContext)."""
+    name: str                     # checkpoint name
+    rows: int
+    index: str = "tokens"
+    scale: float = 1.0
+
+
+@dataclass
 class DecoderSpec:
     vocab: int
     width: int
@@ -56,6 +66,7 @@ class DecoderSpec:
     logit_scale: float = 1.0              # the logits times this
     logit_softcap: float = 0.0            # > 0: then cap * tanh(logit / cap)
     embedding_scale: float = 1.0          # the token table's rows times this, before the position table's
+    extra_embeddings: List[EmbeddingTable] = field(default_factory=list)   # added behind them, in this order
     eos_token_ids: Tuple[int, ...] = ()
     # how checkpoints of this architecture name things
     name_prefixes: Tuple[str, ...] = ("",)
@@ -84,6 +95,12 @@ class DecoderModel:
         self.spec = spec
         self.embedding = TokenEmbedding(spec.vocab, spec.width, spec.token_table)
         self.position = POSITIONS.make(spec.position)
+        for t in spec.extra_embeddings:
+            if t.index not in ("tokens", "positions"):
+                raise ValueError(f"embedding table {t.name!r}: rows are picked by 'tokens' or 'positions', not {t.index!r}")
+        if len(spec.extra_embeddings) > ops.EMBED_TABLES_MAX - 2:
+            raise ValueError(f"{len(spec.extra_embeddings)} further embedding tables; the kernel adds up {ops.EMBED_TABLES_MAX} in all")
+        self.extra_tables = {}
         self.blocks = []
         for i, ls in enumerate(spec.layers):
             if ls.arrangement not in ARRANGEMENTS:
@@ -146,6 +163,11 @@ class DecoderModel:
                     raise ValueError(f"two parts claim the tensor {s.name!r}")
                 seen.add(s.name)
                 specs.append(s)
+        for t in self.spec.extra_embeddings:
+            if t.name in seen:
+                raise ValueError(f"two parts claim the tensor {t.name!r}")
+            seen.add(t.name)
+            specs.append(ParamSpec(t.name, (t.rows, self.spec.width), "table", ("normal", 0.0, 0.02)))
         specs += [s for s in self.head.param_specs() if s.name not in seen]     # (a tied head's weight is the table's)
         return specs
 
@@ -156,6 +178,7 @@ class DecoderModel:
         for p in self.all_parts():
             p.bind(tensors, runtime)
         self.head.bind(tensors)
+        self.extra_tables = {t.name: tensors[t.name] for t in self.spec.extra_embeddings}
         for b in self.blocks:
             after = getattr(b, "after_bind", None)     # an arrangement may make its parts ready for each other
             if after is not None:
@@ -187,8 +210,15 @@ class DecoderModel:
         -> 32-bit logits [R, vocab] at ctx.logit_rows."""
         rt = self.runtime
         x = torch.empty((ctx.T, self.spec.width), dtype=torch.float32, device=rt.device)
-        ops.embed(ctx.tokens, ctx.positions, self.embedding.weight, self.position.table(), x,
-                  token_scale=self.spec.embedding_scale)
+        if not self.spec.extra_embeddings:
+            ops.embed(ctx.tokens, ctx.positions, self.embedding.weight, self.position.table(), x,
+                      token_scale=self.spec.embedding_scale)
+        else:
+            parts = [(self.embedding.weight, ctx.tokens, self.spec.embedding_scale)]
+            if self.position.table() is not None:
+                parts.append((self.position.table(), ctx.positions, 1.0))
+            parts += [(self.extra_tables[t.name], getattr(ctx, t.index), t.scale) for t in self.spec.extra_embeddings]
+            ops.embed_sum(parts, x)
         rt.stream_stats = None      # nobody has left anything for a norm of these rows yet
         order = self.spec.run_order
         for i, call in enumerate(order):

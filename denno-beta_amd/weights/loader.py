@@ -63,12 +63,18 @@ def load_checkpoint(model_dir: str, specs: Sequence[ParamSpec], *, engine_dtype:
     ignore:   regular expressions of file tensors that are buffers, not weights.
     tied:     {file name: spec name}: a file tensor that repeats another (a tied head);
               it must have that tensor's shape and is otherwise not read.
+    A spec with `sources` is read from those file tensors, joined along its `concat_dim` (in the stored layout,
+    before a transpose); missing pieces, unexpected tensors and wrong shapes are reported by the file's names.
     """
     where, files = open_checkpoint(model_dir)
     try:
         ignore_re = [re.compile(p) for p in ignore]
         tied = tied or {}
-        by_name = {s.name: s for s in specs}
+        # file name -> (spec, the piece's stored shape): a spec is one file tensor, or several joined at load
+        by_name, spec_of = {}, {s.name: s for s in specs}
+        for s in specs:
+            for fname, shape in s.pieces():
+                by_name[fname] = (s, shape)
         found, unexpected, wrong_shape, wrong_dtype = {}, [], [], []
         for fname in where:
             base = None
@@ -82,13 +88,13 @@ def load_checkpoint(model_dir: str, specs: Sequence[ParamSpec], *, engine_dtype:
                 continue
             stored, shape = where[fname].entries[fname]
             if base in tied:
-                want = by_name[tied[base]].shape
+                want = spec_of[tied[base]].shape
                 if tuple(shape) != tuple(want):
                     wrong_shape.append((fname, shape, want))
                 continue
-            spec = by_name[base]
-            if tuple(shape) != tuple(spec.shape):
-                wrong_shape.append((fname, shape, spec.shape))
+            spec, want = by_name[base]
+            if tuple(shape) != tuple(want):
+                wrong_shape.append((fname, shape, want))
             ok = _INT_STORED if spec.role == "int_table" else _FLOAT_STORED
             if stored not in ok:
                 wrong_dtype.append((fname, stored))
@@ -96,20 +102,26 @@ def load_checkpoint(model_dir: str, specs: Sequence[ParamSpec], *, engine_dtype:
                 unexpected.append(fname + " (a second copy of " + found[base] + ")")
             else:
                 found[base] = fname
-        missing = [s.name for s in specs if s.name not in found]
+        missing = [fname for s in specs for fname, _ in s.pieces() if fname not in found]
         if missing or unexpected or wrong_shape or wrong_dtype:
             raise CheckpointError(model_dir, missing, unexpected, wrong_shape, wrong_dtype)
 
         out, kept32 = {}, 0
         for spec in specs:
-            fname = found[spec.name]
-            sf = where[fname]
-            stored = sf.entries[fname][0]
+            names = [found[fname] for fname, _ in spec.pieces()]
+            kinds = [where[n].entries[n][0] for n in names]
+            # (pieces stored in different precisions: bfloat16 only if every piece is)
+            stored = kinds[0] if all(k == kinds[0] for k in kinds) else "F32"
             dt = held_dtype(spec, stored, engine_dtype, cast_matrices)
             if (engine_dtype == "bfloat16" and spec.role in ("matrix", "table")
                     and dt == torch.float32):
                 kept32 += 1
-            out[spec.name] = place(sf.tensor(fname), spec, dt, device)
+            if len(names) == 1:
+                t = where[names[0]].tensor(names[0])
+            else:
+                host_dt = torch.int64 if spec.role == "int_table" else (torch.float32 if stored != "BF16" else torch.bfloat16)
+                t = torch.cat([where[n].tensor(n).to(host_dt) for n in names], dim=spec.concat_dim)
+            out[spec.name] = place(t, spec, dt, device)
         if kept32 and notes is not None:
             notes.append(f"{kept32} matrices are stored in 32-bit and stay so; their products run "
                          "in 32-bit (cast_matrices rounds them to bfloat16 at load)")

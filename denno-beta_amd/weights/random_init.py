@@ -42,6 +42,20 @@ def draw(spec: ParamSpec, seed: int, device="cpu") -> torch.Tensor:
     raise ValueError(f"ParamSpec {spec.name}: unknown init {spec.init!r}")
 
 
+def _piece(spec: ParamSpec, fname: str, shape) -> ParamSpec:
+    """The spec of one file tensor of `spec`: itself, or one of its sources as a tensor of its own."""
+    if spec.sources is None:
+        return spec
+    return ParamSpec(fname, tuple(shape), spec.role, spec.init, dtype_hint=spec.dtype_hint)
+
+
+def draw_joined(spec: ParamSpec, seed: int, device="cpu") -> torch.Tensor:
+    """The tensor in its stored shape: drawn whole, or each source drawn under its own name and joined."""
+    if spec.sources is None:
+        return draw(spec, seed, device)
+    return torch.cat([draw(_piece(spec, fname, shape), seed, device) for fname, shape in spec.pieces()], dim=spec.concat_dim)
+
+
 def stored_dtype(spec: ParamSpec, dtype: str) -> torch.dtype:
     if spec.role == "int_table":
         return torch.int32
@@ -65,11 +79,12 @@ def write_model_folder(folder: str, config: dict, seed: int, dtype: str = "float
     out["torch_dtype"] = dtype
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(out, f, indent=1)
-    by_name = {name_prefix + s.name: s for s in specs}
-    layout = [(name_prefix + s.name, stored_dtype(s, dtype), tuple(s.shape)) for s in specs]
+    # (a tensor that a checkpoint stores in pieces is written in pieces, each drawn under its own name)
+    pieces = {name_prefix + fname: _piece(s, fname, shape) for s in specs for fname, shape in s.pieces()}
+    layout = [(n, stored_dtype(p, dtype), tuple(p.shape)) for n, p in pieces.items()]
     write_safetensors(
         os.path.join(folder, "model.safetensors"), layout,
-        lambda n: draw(by_name[n], seed).to(stored_dtype(by_name[n], dtype)),
+        lambda n: draw(pieces[n], seed).to(stored_dtype(pieces[n], dtype)),
         metadata={"format": "pt", "seed": seed})
     return folder
 
@@ -83,7 +98,7 @@ def draw_all(specs: Sequence[ParamSpec], seed: int, *, engine_dtype: str, device
     code = {"bfloat16": "BF16", "float32": "F32", "float16": "F16"}[stored]
     out = {}
     for s in specs:
-        t = draw(s, seed, device=device).to(stored_dtype(s, stored))
+        t = draw_joined(s, seed, device=device).to(stored_dtype(s, stored))
         dt = held_dtype(s, "I32" if s.role == "int_table" else code, engine_dtype, False)
         t = t.to(dt)
         out[s.name] = (t.t() if s.transpose else t).contiguous()

@@ -7,7 +7,7 @@ import contextlib
 import kernel_refs
 from denno_beta_amd.kernels import ops
 
-_NAMES = ["embed", "logits_post", "layernorm", "kv_write", "cast", "linear", "linear_qkv", "linear_norm_out", "linear_norm_in", "attention", "sample", "sample_top", "sample_full", "penalties", "history_append"]
+_NAMES = ["embed", "embed_sum", "logits_post", "layernorm", "kv_write", "cast", "linear", "linear_qkv", "linear_norm_out", "linear_norm_in", "attention", "sample", "sample_top", "sample_full", "penalties", "history_append"]
 
 
 @contextlib.contextmanager

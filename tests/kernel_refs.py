@@ -23,6 +23,17 @@ def embed(tokens, positions, wte, wpe, out, token_scale=1.0):
     return out
 
 
+def embed_sum(parts, out):
+    x = None
+    for table, index, scale in parts:
+        a = table[index.long()].float()
+        if scale != 1.0:
+            a = a * torch.tensor(scale, dtype=torch.float32)
+        x = a if x is None else x + a
+    out.copy_(x)
+    return out
+
+
 def logits_post(logits, scale=1.0, softcap=0.0):
     logits.mul_(torch.tensor(scale, dtype=torch.float32))
     if softcap > 0:
@@ -94,10 +105,12 @@ def linear_norm_out(a, w, bias, residual, gamma, copy, stats):
     return residual
 
 
-def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None):
+def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None, no_mean=False):
     """The kernel's own formula: the product of the rows that are not normalised, then the row's mean
-    and 1 / sqrt(var + eps), joined from the blocks' pairs, on the sums."""
+    and 1 / sqrt(var + eps), joined from the blocks' pairs, on the sums.  no_mean: the mean counts as 0."""
     mean = stats[:, :, 0].mean(dim=1, keepdim=True)
+    if no_mean:
+        mean = torch.zeros_like(mean)
     var = (stats[:, :, 1] + 16.0 * (stats[:, :, 0] - mean) ** 2).sum(dim=1, keepdim=True) / copy.shape[1]
     y = (copy.float() @ w.float().t() - mean * c1) / torch.sqrt(var + eps) + c2
     if epilogue == "gelu_tanh":

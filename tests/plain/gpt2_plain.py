@@ -180,12 +180,14 @@ class PlainGPT2:
         pre = f"h.{i}."
         return {k[len(pre):]: v for k, v in self.t.items() if k.startswith(pre)}
 
-    def logits(self, tokens, by_head=False) -> torch.Tensor:
+    def logits(self, tokens, by_head=False, input_table=None) -> torch.Tensor:
         """[len(tokens), vocab] logits of one whole sequence starting at position 0.
-        by_head: attention one head at a time as matrices (long sequences of deep models)."""
+        by_head: attention one head at a time as matrices (long sequences of deep models).
+        input_table: the token rows come from this table (the head stays the model's own token table)."""
         tok = torch.as_tensor(tokens, dtype=torch.long)
         pos = torch.arange(len(tok))
-        x = embed(tok, pos, self.t["wte.weight"], self.t["wpe.weight"])
+        x = embed(tok, pos, self.t["wte.weight"] if input_table is None else input_table.to(self.t["wte.weight"].dtype),
+                  self.t["wpe.weight"])
         dh = self.n_embd // self.n_head
         for i in range(self.n_layer):
             scale = attention_scale(dh, i, self.scale_w, self.scale_inv)

@@ -303,6 +303,39 @@ def test_a_norm_inside_products_of_17_to_64_rows(M, E, I, epilogue, layout):
     assert torch.allclose(few.float(), out_rows[:16].float(), atol=3e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("M,E,I", [(5, 96, 320), (16, 1600, 4800), (33, 1024, 4096), (64, 1600, 6400)])
+def test_a_norm_without_a_mean_inside_the_products(M, E, I):
+    """The same two kernels run a norm that takes no mean off, x / sqrt(mean(x^2) + eps) * gamma: the product after it
+    takes the squares about 0 and uses no c1.  Against that norm in 64-bit followed by the product, on rows whose mean
+    is as large as their spread (a mean taken off by mistake would show)."""
+    a = rnd(M, I, seed=1, dtype=torch.bfloat16)
+    x0 = rnd(M, E, seed=2, scale=2.0) + 2.0
+    w1, b1 = rnd(E, I, seed=3, dtype=torch.bfloat16, scale=0.05), rnd(E, seed=4)
+    w2, b2 = rnd(I, E, seed=5, dtype=torch.bfloat16, scale=0.1), rnd(I, seed=6)
+    gamma = 1 + rnd(E, seed=7, scale=0.1)
+    p1, p2 = ops().pack_matrix(w1), ops().pack_matrix(w2)
+    x = x0.clone()
+    copy, stats = ops().norm_stream_buffers(M, E, DEV)
+    ops().linear_norm_out(a, p1, b1, x, gamma, copy, stats)
+    c1, c2 = ops().norm_folded(p2.rows(), b2, gamma, None, no_mean=True)
+    assert not c1.any() and torch.allclose(c2, b2)
+    packed_out = M > 16
+    out = ops().packed_rows(M, I, DEV) if packed_out else torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
+    ops().linear_norm_in(copy, stats, c1, c2, 1e-6, p2, out, epilogue="gelu_tanh", no_mean=True)
+    got = (out.rows() if packed_out else out).float()
+    xd = x.double()
+    y = xd / torch.sqrt((xd * xd).mean(dim=1, keepdim=True) + 1e-6) * gamma.double()
+    want = torch.nn.functional.gelu(y @ w2.double().t() + b2.double(), approximate="tanh").float()
+    assert (got - want).norm() <= 1e-2 * want.norm(), (M, E, I, ((got - want).norm() / want.norm()).item())
+    # with the mean taken off the result is another one
+    wrong = torch.nn.functional.layer_norm(xd, (E,), gamma.double(), None, 1e-6)
+    wrong = torch.nn.functional.gelu(wrong @ w2.double().t() + b2.double(), approximate="tanh").float()
+    assert (got - wrong).norm() > 0.1 * want.norm()
+    plain = R.linear_norm_in(copy if not packed_out else copy.rows(), stats, c1, c2, 1e-6, w2, torch.empty(M, I, dtype=torch.bfloat16, device=DEV),
+                             epilogue="gelu_tanh", no_mean=True)
+    assert torch.allclose(got, plain.float(), atol=3e-2, rtol=2e-2)
+
+
 def test_a_norm_inside_a_fused_projection_writes_the_cache():
     H, Hkv, dh, ps, n_pages, E, M = 6, 2, 48, 16, 12, 160, 7
     N = (H + 2 * Hkv) * dh

@@ -1,6 +1,7 @@
 """The parts alone, and what the assembly allows: a layer named twice, a layer that reads
 another layer's cache, and a mixer with state of its own that is defined here, registered,
 built and stepped without a change to the framework's files."""
+import json
 import math
 
 import pytest
@@ -146,6 +147,63 @@ def test_a_cache_group_holds_the_dtype_that_its_mixers_ask_for():
     assert c.n_groups == 2 and c.k[0].dtype == torch.bfloat16 and c.k[1].dtype == torch.float32
     assert c.k[0].shape[0] == 2 and c.v[1].shape == (1, 4, 2, 16, 16)
     assert c.bytes_per_token() == 2 * 2 * 2 * 16 * 2 + 2 * 2 * 16 * 4
+
+
+def test_a_cache_group_may_hold_values_of_another_width_than_its_keys():
+    """PagedKV names a width for values where it is not the keys': the pools are laid out for both and are a
+    group of their own."""
+    from denno_beta_amd.cache import CacheStorage
+    from denno_beta_amd.parts import PagedKV
+    assert PagedKV(2, 32).v_dim == 32 and PagedKV(2, 32, value_dim=48).v_dim == 48
+    c = CacheStorage([PagedKV(2, 32), PagedKV(2, 32, value_dim=48)], kv_dtype=torch.float32, page_size=16,
+                     cache_tokens=64, max_live=2, device=torch.device("cpu"))
+    assert c.n_groups == 2 and c.k[1].shape == (1, 4, 2, 16, 32) and c.v[1].shape == (1, 4, 2, 48, 16)
+    assert c.bytes_per_token() == 2 * (32 + 32) * 4 + 2 * (32 + 48) * 4
+
+
+@pytest.mark.gpu
+def test_the_attention_kernels_refuse_values_of_another_width():
+    """The package's attention kernels take keys and values of one width; asked for others they say so."""
+    from denno_beta_amd.kernels import ops
+    dev = "cuda:0"
+    q = torch.zeros(4, 64, device=dev)
+    k = torch.zeros(2, 2, 16, 32, device=dev)
+    v = torch.zeros(2, 2, 48, 16, device=dev)
+    bt = torch.zeros(1, 2, dtype=torch.int32, device=dev)
+    tiles = torch.tensor([[0], [0], [4], [0]], dtype=torch.int32, device=dev)
+    with pytest.raises(ops.KernelError, match="one width"):
+        ops.attention(q, torch.empty(4, 64, device=dev), k, v, bt, tiles, 2, 0.5)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_further_embedding_tables_are_added_in_the_embedding_kernel(backend, dtype):
+    """A description may list further tables whose rows are added to the token and position rows: here a second
+    table over the tokens (times a half) and a second one over the positions.  Since every later part is linear
+    in nothing, the check is against the plain GPT-2 run on a token table and a position table that hold the
+    sums, which exist because each further table is indexed like one of the two."""
+    from denno_beta_amd.engine import ModelRunner
+    from denno_beta_amd.parts import EmbeddingTable
+    cfg, spec = gpt2_spec("A")
+    spec.extra_embeddings = [EmbeddingTable("tok2.weight", cfg["vocab_size"], "tokens", 0.5),
+                             EmbeddingTable("pos2.weight", cfg["n_positions"], "positions")]
+    assert [s.name for s in spec.param_specs() if s.role == "table"] == ["wte.weight", "wpe.weight", "tok2.weight", "pos2.weight"]
+    tensors = draw(spec, backend, dtype=dtype)
+    r = ModelRunner(spec, tensors, options(backend, dtype))
+    seq = seeded_tokens(2, 50, cfg["vocab_size"])
+    got = U.replay(r, U.chunk_trace([seq], sizes=(9, 2, 20)))["r0"]
+    st = stored(tensors, spec)
+    # the head is tied to the first token table alone: the plain model gets the summed table for its input rows
+    # and the first table for its head
+    plain = P.PlainGPT2(cfg, {**st, "wpe.weight": st["wpe.weight"] + st["pos2.weight"]})
+    want = plain.logits(seq, input_table=st["wte.weight"] + 0.5 * st["tok2.weight"])
+    U.assert_close(got, want, dtype, "further embedding tables")
+    # one table too many for the kernel, and an index that a step does not have
+    spec.extra_embeddings = [EmbeddingTable(f"t{i}", 8) for i in range(3)]
+    with pytest.raises(ValueError, match="in all"):
+        spec.instantiate()
+    spec.extra_embeddings = [EmbeddingTable("t", 8, "token_types")]
+    with pytest.raises(ValueError, match="token_types"):
+        spec.instantiate()
 
 
 # -- the order in which layers run is data -----------------------------------------------------
@@ -717,3 +775,166 @@ def test_norms_that_run_inside_the_products_beside_them(model_folders, name, row
     U.assert_close(got[True], got[False], "bfloat16", f"{name}: norms inside the products against norms as kernels")
     want = P.PlainGPT2.from_folder(folder).logits(seq)[40:]
     U.assert_close(got[True], want, "bfloat16", f"{name}: norms inside the products against the plain implementation")
+
+
+# -- a checkpoint that stores q, k and v apart still runs the fused projection ---------------------------
+def register_split_qkv_architecture():
+    """`ToySplitQKV`: GPT-2's own parts and configuration keys, but its checkpoints hold the three projections of
+    a layer as tensors of their own (`attn.q.weight`, `attn.k.weight`, `attn.v.weight` and their biases).  The
+    description names them as the sources of the attention mixer's one fused weight; nothing of the framework's
+    files changes."""
+    import copy
+    from denno_beta_amd.config import known_architectures, register_architecture
+    from denno_beta_amd.models.gpt2 import GPT2Config, build_gpt2
+    if "ToySplitQKV" in known_architectures():
+        return
+
+    def build(cfg):
+        spec = copy.deepcopy(build_gpt2(cfg))
+        E = cfg.n_embd
+        for i, layer in enumerate(spec.layers):
+            kind, args = layer.parts["mixer"]
+            p = f"h.{i}.attn."
+            args = dict(args, qkv_weight=p + "qkv_joined.weight", qkv_bias=p + "qkv_joined.bias",
+                        qkv_weight_sources=((p + "q.weight", E), (p + "k.weight", E), (p + "v.weight", E)),
+                        qkv_bias_sources=((p + "q.bias", E), (p + "k.bias", E), (p + "v.bias", E)))
+            layer.parts["mixer"] = (kind, args)
+        return spec
+    register_architecture(["ToySplitQKV"], GPT2Config, build)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_checkpoint_with_q_k_v_apart_feeds_the_fused_projection(backend, tmp_path, dtype):
+    """The folder holds q, k and v as tensors of their own and no fused one; the loader joins them once; the mixer
+    runs its one fused projection with the cache write (the same kernel as for a checkpoint that stores them
+    fused); the logits are those of the plain GPT-2 on the joined tensors, in every cutting."""
+    from safetensors.torch import load_file, save_file
+    from denno_beta_amd.engine import ModelRunner
+    from denno_beta_amd.kernels import ops
+    from denno_beta_amd.weights import write_model_folder
+    register_split_qkv_architecture()
+    cfg = dict(TINY["B"][0], architectures=["ToySplitQKV"])
+    folder = write_model_folder(str(tmp_path / "split"), cfg, seed=8, dtype=dtype)
+    t = load_file(folder + "/model.safetensors")
+    assert "h.0.attn.q.weight" in t and tuple(t["h.1.attn.k.weight"].shape) == (96, 96) and "h.2.attn.v.bias" in t
+    assert not any("qkv_joined" in n or "c_attn" in n for n in t)
+    assert not torch.equal(t["h.0.attn.q.weight"], t["h.0.attn.k.weight"])
+    # the same weights as a GPT-2 folder, for the plain implementation
+    joined = {n: x for n, x in t.items() if ".attn.q." not in n and ".attn.k." not in n and ".attn.v." not in n}
+    for i in range(cfg["n_layer"]):
+        p = f"h.{i}.attn."
+        joined[p + "c_attn.weight"] = torch.cat([t[p + f"{x}.weight"] for x in "qkv"], dim=1).contiguous()
+        joined[p + "c_attn.bias"] = torch.cat([t[p + f"{x}.bias"] for x in "qkv"]).contiguous()
+    plain_dir = tmp_path / "joined"
+    plain_dir.mkdir()
+    save_file(joined, str(plain_dir / "model.safetensors"))
+    (plain_dir / "config.json").write_text(json.dumps(dict(cfg, architectures=["GPT2LMHeadModel"])))
+    plain = P.PlainGPT2.from_folder(str(plain_dir))
+    seqs = [seeded_tokens(90 + i, n, cfg["vocab_size"]) for i, n in enumerate((40, 9, 70))]
+    want = [plain.logits(s) for s in seqs]
+    calls = {"fused": 0}
+    real = ops.linear_qkv
+
+    def counting(*a, **k):
+        calls["fused"] += 1
+        return real(*a, **k)
+    try:
+        ops.linear_qkv = counting
+        r = ModelRunner.from_folder(folder, options(backend, dtype, cache_tokens=256, use_graphs=False,
+                                                    norms_inside_products=False))
+        for kind, steps in (("whole", U.whole_trace(seqs)), ("tail", U.tail_decode_trace(seqs, 8)),
+                            ("portions", U.chunk_trace(seqs)), ("mixed", U.mixed_trace(seqs, seed=3))):
+            before = calls["fused"]
+            got = U.replay(r, steps)
+            assert calls["fused"] - before == cfg["n_layer"] * len(steps)
+            for i in range(len(seqs)):
+                U.assert_close(got[f"r{i}"], want[i], dtype, f"q, k, v apart, {dtype}, {kind}, request {i}")
+    finally:
+        ops.linear_qkv = real
+    r.cache.manager.check()
+
+
+# -- a norm without a mean, defined here, runs inside the products beside it -----------------------------
+def register_toy_rms_norm():
+    from denno_beta_amd.parts import NORMS, Part
+    from denno_beta_amd.weights import ParamSpec
+    if "toy_rms" in NORMS:
+        return
+
+    @NORMS.register("toy_rms")
+    class ToyRMSNorm(Part):
+        """x / sqrt(mean(x^2) + eps) * weight, with the library; `fused_params` says what a product's kernel needs to
+        run it itself."""
+        graph_safe = True
+
+        def __init__(self, width, eps, weight_name):
+            self.width, self.eps, self.weight_name = width, eps, weight_name
+
+        def param_specs(self):
+            return [ParamSpec(self.weight_name, (self.width,), "vector", ("normal", 1.0, 0.1))]
+
+        def bind(self, tensors, runtime):
+            super().bind(tensors, runtime)
+            self.weight = tensors[self.weight_name]
+
+        def fused_params(self):
+            return ("rmsnorm", self.weight, None, self.eps)
+
+        def forward(self, x, out_dtype, rows=None, packed=False):
+            src = x if rows is None else x[rows.long()]
+            y = src * torch.rsqrt((src * src).mean(dim=1, keepdim=True) + self.eps) * self.weight
+            return y.to(out_dtype)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows", [3, 16, 40])
+def test_a_norm_without_a_mean_runs_inside_the_products(rows):
+    """GPT-2's layers with a toy norm that takes no mean off in place of the layer norms: in steps of few rows the
+    products beside it run it (the calls are counted), and the logits are those of the same steps with the norm
+    run by its own forward, and of the plain formulas."""
+    import copy
+    from denno_beta_amd.engine import ModelRunner, StepEntry
+    from denno_beta_amd.kernels import ops
+    register_toy_rms_norm()
+    cfg, spec = gpt2_spec("F")
+    spec = copy.deepcopy(spec)
+    for i, layer in enumerate(spec.layers):
+        for slot in ("norm1", "norm2"):
+            layer.parts[slot] = ("toy_rms", dict(width=cfg["n_embd"], eps=1e-6, weight_name=f"h.{i}.{slot}.g"))
+    tensors = draw(spec, "cuda:0", dtype="bfloat16")
+    seq = seeded_tokens(6, 30 + rows, cfg["vocab_size"])
+    calls = {"in": 0}
+    real_in = ops.linear_norm_in
+
+    def count_in(*a, **k):
+        assert k.get("no_mean") is True
+        calls["in"] += 1
+        return real_in(*a, **k)
+    got = {}
+    try:
+        ops.linear_norm_in = count_in
+        for inside in (True, False):
+            r = ModelRunner(spec, dict(tensors), options("cuda:0", "bfloat16", use_graphs=False, norms_inside_products=inside))
+            r.start_request(0)
+            r.step([StepEntry(0, seq[:30], [])])
+            before = calls["in"]
+            got[inside] = r.step([StepEntry(0, seq[30:], list(range(rows)))]).float().cpu()
+            assert calls["in"] - before == (2 * cfg["n_layer"] - 1 if inside else 0)
+    finally:
+        ops.linear_norm_in = real_in
+    U.assert_close(got[True], got[False], "bfloat16", "a norm without a mean inside the products against its own forward")
+    # the plain formulas: GPT-2's functions with this norm in the two places
+    st = stored(tensors, spec)
+    x = P.embed(torch.tensor(seq), torch.arange(len(seq)), st["wte.weight"], st["wpe.weight"]).double()
+    rms = lambda v, g: v / torch.sqrt((v * v).mean(dim=1, keepdim=True) + 1e-6) * g.double()       # noqa: E731
+    dh = cfg["n_embd"] // cfg["n_head"]
+    for i in range(cfg["n_layer"]):
+        p = f"h.{i}."
+        qkv = rms(x, st[p + "norm1.g"]) @ st[p + "attn.c_attn.weight"].double() + st[p + "attn.c_attn.bias"].double()
+        q, k, v = qkv.split(cfg["n_embd"], dim=1)
+        o = P.causal_attention(q, k, v, cfg["n_head"], dh ** -0.5)
+        x = x + o @ st[p + "attn.c_proj.weight"].double() + st[p + "attn.c_proj.bias"].double()
+        f = torch.nn.functional.gelu(rms(x, st[p + "norm2.g"]) @ st[p + "mlp.c_fc.weight"].double() + st[p + "mlp.c_fc.bias"].double())
+        x = x + f @ st[p + "mlp.c_proj.weight"].double() + st[p + "mlp.c_proj.bias"].double()
+    want = P.head(x.float(), st["ln_f.weight"], st["ln_f.bias"], cfg["layer_norm_epsilon"], st["wte.weight"])[30:]
+    U.assert_close(got[True], want, "bfloat16", "a norm without a mean inside the products against the plain formulas")

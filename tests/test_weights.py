@@ -151,3 +151,51 @@ def test_streaming_writer_checks_its_layout(tmp_path):
     with pytest.raises(ValueError, match="layout says"):
         write_safetensors(str(tmp_path / "x.safetensors"), [("a", torch.float32, (2, 2))],
                           lambda n: torch.zeros(3))
+
+
+def test_a_tensor_stored_in_pieces_is_joined_at_load(tmp_path):
+    """A held tensor may be several file tensors joined along one dimension of the stored layout (a fused
+    projection whose q, k and v a checkpoint stores apart): the pieces are read by their own names, joined in
+    the spec's order, and everything wrong is reported by the file's names, all at once."""
+    from denno_beta_amd.weights import ParamSpec
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(n, 6, generator=g) for n in (8, 4, 4))           # stored [out, in]
+    qc, kc, vc = (torch.randn(6, n, generator=g) for n in (8, 4, 4))        # stored [in, out]
+    bq, bk, bv = (torch.randn(n, generator=g) for n in (8, 4, 4))
+    tensors = {"a.q": q, "a.k": k, "a.v": v, "c.q": qc, "c.k": kc, "c.v": vc, "a.bq": bq, "a.bk": bk, "a.bv": bv,
+               "n.w": torch.ones(6)}
+    specs = [ParamSpec("a.qkv", (16, 6), "matrix", sources=(("a.q", 8), ("a.k", 4), ("a.v", 4)), concat_dim=0),
+             ParamSpec("c.qkv", (6, 16), "matrix", transpose=True, sources=(("c.q", 8), ("c.k", 4), ("c.v", 4)), concat_dim=1),
+             ParamSpec("a.b", (16,), "vector", sources=(("a.bq", 8), ("a.bk", 4), ("a.bv", 4))),
+             ParamSpec("n.w", (6,), "vector")]
+
+    def write(d, t, dtype=torch.float32):
+        os.makedirs(d, exist_ok=True)
+        write_safetensors(os.path.join(d, "model.safetensors"),
+                          [(n, torch.float32 if x.dim() == 1 else dtype, tuple(x.shape)) for n, x in t.items()],
+                          lambda n: t[n].to(torch.float32 if t[n].dim() == 1 else dtype))
+        return d
+    d = write(str(tmp_path / "ok"), tensors)
+    got = load_checkpoint(d, specs, engine_dtype="float32", device="cpu")
+    assert set(got) == {"a.qkv", "c.qkv", "a.b", "n.w"}
+    assert torch.equal(got["a.qkv"], torch.cat([q, k, v], 0))
+    assert torch.equal(got["c.qkv"], torch.cat([qc, kc, vc], 1).t()) and got["c.qkv"].is_contiguous()
+    assert torch.equal(got["a.b"], torch.cat([bq, bk, bv]))
+    # bfloat16 pieces stay bfloat16 in a bfloat16 engine; one piece in 32-bit keeps the whole in 32-bit
+    d = write(str(tmp_path / "bf"), tensors, torch.bfloat16)
+    assert load_checkpoint(d, specs, engine_dtype="bfloat16", device="cpu")["a.qkv"].dtype == torch.bfloat16
+    rewrite(d, lambda t: t.__setitem__("a.k", t["a.k"].float()))
+    got = load_checkpoint(d, specs, engine_dtype="bfloat16", device="cpu")
+    assert got["a.qkv"].dtype == torch.float32 and got["c.qkv"].dtype == torch.bfloat16
+    # a missing piece, a piece of the wrong shape, the joined name itself in the file: one error
+    bad = dict(tensors)
+    del bad["a.k"]
+    bad["c.v"] = torch.zeros(6, 5)
+    bad["a.qkv"] = torch.zeros(16, 6)
+    with pytest.raises(CheckpointError) as e:
+        load_checkpoint(write(str(tmp_path / "bad"), bad), specs, engine_dtype="float32", device="cpu")
+    assert e.value.missing == ["a.k"] and e.value.unexpected == ["a.qkv"]
+    assert [(n, tuple(s), tuple(w)) for n, s, w in e.value.wrong_shape] == [("c.v", (6, 5), (6, 4))]
+    # sizes that do not add up are a fault of the description
+    with pytest.raises(ValueError, match="add up"):
+        ParamSpec("x", (16, 6), "matrix", sources=(("a", 8), ("b", 4)))

@@ -13,8 +13,8 @@ decode steps and prefill (`fp32`).  Peaks are the published ones of MI355X.
     python bench.py --only decode|prefill [--kernel-times]   one workload; with --kernel-times kernel by
                                                              kernel, each launch between two HIP events
     python bench.py --only serving [--dtype float32]         BASELINE.json's configs[3] through the scheduler
-    python bench.py --only replay [--sequences 8]            BASELINE.json's configs[4] against the plain
-                                                             implementation, in four ways of cutting
+    python bench.py --only replay [--sequences 8] [--shape xl]   BASELINE.json's configs[4] (or configs[2]'s sizes)
+                                                             against the plain implementation, in four ways of cutting
 """
 import argparse
 import json
@@ -170,8 +170,9 @@ def main():
     ap.add_argument("--top-k", type=int, default=None, help="--only decode, with --temperature")
     ap.add_argument("--top-p", type=float, default=None, help="--only decode, with --temperature")
     ap.add_argument("--repetition-penalty", type=float, default=None, help="--only decode: penalties over each request's tokens")
-    ap.add_argument("--shape", choices=["xl", "large", "medium"], default="xl",
-                    help="--only decode / prefill: the layer sizes of BASELINE.json's configs[2], [3] or [4]")
+    ap.add_argument("--shape", choices=["xl", "large", "medium"], default=None,
+                    help="--only decode / prefill / replay: the layer sizes of BASELINE.json's configs[2], [3] or [4] "
+                         "(default xl; for replay medium)")
     ap.add_argument("--only", choices=["decode", "prefill", "serving", "replay"], default=None,
                     help="run one workload and print a short line (decode, prefill: for profiling; serving: "
                          "BASELINE.json's configs[3], GPT-2 Large shape, 64 requests through the scheduler; replay: "
@@ -183,7 +184,9 @@ def main():
     if a.only == "serving":
         return serving(a)
     if a.only == "replay":
+        a.shape = a.shape or "medium"      # (configs[4] as written; --shape xl: the same replay at configs[2]'s sizes)
         return replay(a)
+    a.shape = a.shape or "xl"
 
     if a.only != "decode" and (a.temperature or a.top_k or a.top_p or a.repetition_penalty):
         print("bench.py: sampling options go with --only decode (the contract's line is greedy)")
@@ -248,7 +251,8 @@ def serving(a):
     """GPT-2 Large shape, random weights: 64 requests with prompt lengths uniform in [16, 768], 256
     generated tokens each, greedy, continuous batching with prompt portions of 512.  After the timed
     run four of the requests run again, each alone: their tokens must be the same (32-bit: exactly; in
-    bfloat16 a step's kernels depend on its rows, so the share of equal tokens is reported)."""
+    bfloat16 a step's kernels depend on its rows, so the count of equal tokens is reported, and the served
+    tokens are checked against the 32-bit engine wherever its lead is clear of bfloat16's rounding)."""
     import torch
     from denno_beta_amd.config import EngineOptions
     from denno_beta_amd.engine import Engine, SamplingParams
@@ -278,6 +282,31 @@ def serving(a):
     if a.dtype == "float32" and min(same) < 256:
         raise SystemExit(f"serving: a request's tokens differ from its run alone (equal tokens before the first "
                          f"difference, of 256: {same})")
+    clear_share = None
+    if a.dtype == "bfloat16":
+        # What can be asked of bfloat16: the 32-bit engine on the same weights, fed each request's prompt and the
+        # tokens that were served, says at every generated position which token leads and by how much; where the
+        # lead is clear of bfloat16's rounding (twice 0.04 of the row's spread, the bound of the replay tests) the
+        # served token must be that one.
+        from denno_beta_amd.engine import ModelRunner, StepEntry
+        del eng
+        r32 = ModelRunner.from_random(cfg, 0, EngineOptions(dtype="float32", page_size=16, cache_tokens=1024, max_live=1,
+                                                            use_graphs=False), stored="bfloat16")
+        clear = wrong = 0
+        for rid, i in enumerate((0, 21, 42, 63)):
+            seq = prompts[i] + out[i][:-1]
+            r32.start_request(rid)
+            logits = r32.step([StepEntry(rid, seq, list(range(len(prompts[i]) - 1, len(seq))))])
+            r32.end_request(rid)
+            top = logits.topk(2, dim=1)
+            sure = (top.values[:, 0] - top.values[:, 1]) > 2 * 0.04 * logits.std(dim=1)
+            served = torch.tensor(out[i], device=logits.device)
+            clear += int(sure.sum())
+            wrong += int((served != top.indices[:, 0])[sure].sum())
+        clear_share = clear / (4 * 256)
+        if wrong:
+            raise SystemExit(f"serving: {wrong} served tokens differ from the 32-bit engine's where its lead is clear "
+                             f"({clear} such positions of {4 * 256})")
     print(json.dumps({
         "workload": "GPT-2 Large shape, 64 requests, prompts U[16,768], 256 new tokens, prefill portions of 512",
         "seconds": dt, "generated_tokens": 64 * 256, "generated_tokens_per_s": 64 * 256 / dt,
@@ -285,12 +314,13 @@ def serving(a):
         "mean_rows_per_step": sum(r.rows for r in records) / steps,
         "mixed_steps": sum(1 for r in records if r.decode_rows and r.prefill_rows),
         "preemptions": sum(r.preempted for r in records), "dtype": a.dtype,
-        "tokens_equal_to_the_run_alone_before_the_first_difference": same}))
+        "tokens_equal_to_the_run_alone_before_the_first_difference": same,
+        "share_of_positions_where_the_32_bit_lead_is_clear_all_served_as_it_says": clear_share}))
 
 
 def replay(a):
-    """BASELINE.json's configs[4]: GPT-2 Medium shape, random weights stored in 32-bit, seeded sequences of
-    1,024 tokens replayed whole, token by token, in portions of 128 and mixed (four live requests, pages
+    """BASELINE.json's configs[4] (GPT-2 Medium shape; --shape xl: configs[2]'s sizes, all 48 layers): random
+    weights stored in 32-bit, seeded sequences of 1,024 tokens replayed whole, token by token, in portions of 128 and mixed (four live requests, pages
     used again), every logit compared with the plain implementation's; and the cuttings with each other."""
     import torch
     sys.path.insert(0, os.path.join(ROOT, "tests"))
@@ -301,7 +331,7 @@ def replay(a):
     from denno_beta_amd.engine.replay import TraceReplayer
     from denno_beta_amd.weights import write_model_folder
     import tempfile
-    cfg, _ = baseline_config(4, a.layers)
+    cfg, full = baseline_config({"xl": 2, "large": 3, "medium": 4}[a.shape], a.layers)
     V, n = cfg["vocab_size"], cfg["n_positions"]
     seqs = [torch.randint(0, V, (n,), generator=torch.Generator().manual_seed(100 + i)).tolist()
             for i in range(a.sequences)]
@@ -314,7 +344,7 @@ def replay(a):
     traces = {"whole": U.whole_trace(seqs), "token by token": token_by_token,
               "portions of 128": U.chunk_trace(seqs, sizes=(128,)),
               "mixed": U.mixed_trace(seqs, seed=3, sizes=(1, 1, 1, 2, 5, 17, 40, 128))}
-    result = {"workload": f"GPT-2 Medium shape, {cfg['n_layer']} layers, {len(seqs)} sequences of {n} tokens"}
+    result = {"workload": f"GPT-2 {a.shape} shape, {cfg['n_layer']} of {full} layers, {len(seqs)} sequences of {n} tokens"}
     with tempfile.TemporaryDirectory() as folder:
         print("replay: writing the model and running the plain implementation ...", file=sys.stderr, flush=True)
         write_model_folder(folder, cfg, 4, "float32")
@@ -343,8 +373,12 @@ def replay(a):
                         pos[e["id"]] = base + len(e["tokens"])
                 runner.cache.manager.check()
                 worst = max((g - wt).abs().max().item() for g, wt in zip(got, want))
+                # the same against what a row's logits differ by among themselves (their standard deviation)
+                rel = [(g - wt).abs() / wt.std(dim=1, keepdim=True) for g, wt in zip(got, want)]
                 agree = sum((g.argmax(1) == wt.argmax(1)).sum().item() for g, wt in zip(got, want)) / (len(seqs) * n)
                 entry = {"worst_difference_from_plain": worst, "greedy_token_agreement": agree,
+                         "worst_of_a_rows_spread": max(r.max().item() for r in rel),
+                         "mean_of_a_rows_spread": sum(r.mean().item() for r in rel) / len(rel),
                          "steps": len(steps), "pages_used_again": runner.cache.manager.reuse_count(0)}
                 if whole is None:
                     whole = got

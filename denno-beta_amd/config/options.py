@@ -24,6 +24,7 @@ class EngineOptions:
     kv_policy: str = "preempt"         # what happens when pages run out: see engine/scheduler.py
     device: str = "cuda:0"
     use_graphs: bool = True            # replay pure-decode steps from captured HIP graphs
+    graph_portions: bool = True        # steps of up to 512 rows that hold prompt portions are captured too, a bucket at its second step (engine/graphs.py)
     run_ahead: bool = True             # launch the next decode step before the host has read this one's tokens (engine/engine.py)
     seed: Optional[int] = None         # default seed of requests that bring none
     norms_inside_products: bool = True  # steps of few rows: a norm between two products runs inside them (parts/blocks.py)

@@ -121,8 +121,8 @@ __device__ __forceinline__ void join_tile(float& m, float& l, float* acc, float 
   m = m_new;
 }
 
-// the tile of BK keys from kt of one request and key head into LDS (keys beyond last_pos and pages
-// given back: zeros).  Where each key's dims and each key's values start in the pools is worked out
+// the tile of BK keys from kt of one request and key head into LDS, a key's dims and values ld floats apart
+// (keys beyond last_pos and pages given back: zeros).  Where each key's dims and each key's values start in the pools is worked out
 // first (Kb, Vb: BK entries each, -1 without a page), so that the loads of the keys and values
 // themselves wait for nothing, go out many at a time and need no division (BK is a power of two;
 // a thread's place in a key's dims moves on by carrying).  Every thread of the workgroup calls it; it
@@ -130,7 +130,7 @@ __device__ __forceinline__ void join_tile(float& m, float& l, float* acc, float 
 template <typename T>
 __device__ __forceinline__ void load_tile(float* Ks, float* Vs, long long* Kb, long long* Vb, const T* k_pool,
                                           const T* v_pool, const int32_t* bt, int kt, int last_pos, int BK, int dh,
-                                          int page_size, int Hkv, int hk) {
+                                          int page_size, int Hkv, int hk, int ld) {
   for (int j = threadIdx.x; j < BK; j += THREADS) {
     const int key = kt + j;
     const int page = key <= last_pos ? bt[key / page_size] : -1;
@@ -171,8 +171,8 @@ __device__ __forceinline__ void load_tile(float* Ks, float* Vs, long long* Kb, l
     for (int i = 0; i < PER; ++i) {
       const int e = threadIdx.x + i * THREADS;
       if (e < n) {
-        Ks[j * (dh + 1) + d] = kv[i];
-        Vs[(e & (BK - 1)) * (dh + 1) + (e >> shift)] = vv[i];
+        Ks[j * ld + d] = kv[i];
+        Vs[(e & (BK - 1)) * ld + (e >> shift)] = vv[i];
       }
       j += dj, d += dd;
       if (d >= dh) d -= dh, j += 1;
@@ -188,11 +188,15 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_row0,
     const int32_t* __restrict__ tile_nrows, const int32_t* __restrict__ tile_pos0, int H, int Hkv, int dh,
     int page_size, int BK, float scale, int window) {
+  // A head size that is no multiple of 16 lies in LDS padded to the next one (dhp): the dims beyond dh are
+  // zeros in the queries and the keys, add nothing to a score (a fused multiply-add of zeros leaves a sum as
+  // it is), and are not stored; the real dims keep their order of summation.
+  const int dhp = (dh + 15) / 16 * 16;
   extern __shared__ float smem[];
-  float* Qs = smem;                    // [BQ][dh]
-  float* Ks = Qs + BQ * dh;            // [BK][dh + 1]
-  float* Vs = Ks + BK * (dh + 1);      // [BK][dh + 1]
-  float* Ps = Vs + BK * (dh + 1);      // [BQ][BK]
+  float* Qs = smem;                    // [BQ][dhp]
+  float* Ks = Qs + BQ * dhp;           // [BK][dhp + 1]
+  float* Vs = Ks + BK * (dhp + 1);     // [BK][dhp + 1]
+  float* Ps = Vs + BK * (dhp + 1);     // [BQ][BK]
   long long* Kb = reinterpret_cast<long long*>(Ps + BQ * BK);   // [BK], [BK]
   long long* Vb = Kb + BK;
 
@@ -205,16 +209,20 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
   const int t = threadIdx.x, qi = t / 16, g = t % 16;
   const float NEG_INF = -INFINITY;
 
-  for (int e = t; e < BQ * dh; e += THREADS) {
-    int r = e / dh, d = e % dh;
-    Qs[e] = r < nrows ? to_float(q[static_cast<size_t>(row0 + r) * ldq + h * dh + d]) : 0.f;
+  for (int e = t; e < BQ * dhp; e += THREADS) {
+    int r = e / dhp, d = e % dhp;
+    Qs[e] = r < nrows && d < dh ? to_float(q[static_cast<size_t>(row0 + r) * ldq + h * dh + d]) : 0.f;
+  }
+  if (dhp != dh) {      // (load_tile writes the real dims only)
+    const int pad = dhp - dh;
+    for (int e = t; e < BK * pad; e += THREADS) Ks[(e / pad) * (dhp + 1) + dh + e % pad] = Vs[(e / pad) * (dhp + 1) + dh + e % pad] = 0.f;
   }
   const bool row_ok = qi < nrows;
   const int my_pos = pos0 + qi;
   const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
   const int last_pos = pos0 + nrows - 1;
   const int first_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
-  const int nd = dh / 16, nc = BK / 16;
+  const int nd = dhp / 16, nc = BK / 16;
 
   float m = NEG_INF, l = 0.f;
   float acc[16];
@@ -223,12 +231,12 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
 
   for (int kt = (first_lo / BK) * BK; kt <= last_pos; kt += BK) {
     __syncthreads();
-    load_tile(Ks, Vs, Kb, Vb, k_pool, v_pool, bt, kt, last_pos, BK, dh, page_size, Hkv, hk);
+    load_tile(Ks, Vs, Kb, Vb, k_pool, v_pool, bt, kt, last_pos, BK, dh, page_size, Hkv, hk, dhp + 1);
     float m_t, l_t, a_t[16];
-    tile_scores(Qs + qi * dh, Ks, Ps + qi * BK, g, nc, dh, kt, my_lo, my_pos, row_ok, scale, m_t, l_t);
+    tile_scores(Qs + qi * dhp, Ks, Ps + qi * BK, g, nc, dhp, kt, my_lo, my_pos, row_ok, scale, m_t, l_t);
     __syncthreads();
     if (m_t > NEG_INF) {                // the same for the 16 threads of a row
-      tile_values(Ps + qi * BK, Vs, g, nd, dh, BK, a_t);
+      tile_values(Ps + qi * BK, Vs, g, nd, dhp, BK, a_t);
       join_tile(m, l, acc, m_t, l_t, a_t, nd);
     }
   }
@@ -237,7 +245,7 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
     T* o = out + static_cast<size_t>(row0 + qi) * ldo + h * dh;
 #pragma unroll
     for (int i = 0; i < 16; ++i)
-      if (i < nd) o[g + 16 * i] = from_float<T>(acc[i] * inv);
+      if (i < nd && g + 16 * i < dh) o[g + 16 * i] = from_float<T>(acc[i] * inv);
   }
 }
 
@@ -273,7 +281,7 @@ __global__ __launch_bounds__(THREADS) void row_tiles_kernel(
   const int hk = h / (H / Hkv);
   const int32_t* bt = block_tables + static_cast<size_t>(seq) * max_blocks;
   for (int d = t; d < dh; d += THREADS) Qs[d] = to_float(q[static_cast<size_t>(tile) * ldq + h * dh + d]);
-  load_tile(Ks, Vs, Kb, Vb, k_pool, v_pool, bt, kt, pos, BK, dh, page_size, Hkv, hk);
+  load_tile(Ks, Vs, Kb, Vb, k_pool, v_pool, bt, kt, pos, BK, dh, page_size, Hkv, hk, dh + 1);
   // One row.  The same sums in the same order as 16 threads of the kernel above make them, spread wider:
   // a thread per key for the scores, 16 threads for the sum of p as there, a thread per dim for the values.
   const float NEG_INF = -INFINITY;
@@ -461,10 +469,11 @@ extern "C" int dn_attention(const void* q, int ldq, void* out, int ldo, const vo
                             int n_tiles, int H, int Hkv, int dh, int page_size, float scale, int window, int dtype,
                             hipStream_t stream) {
   if (n_tiles <= 0) return 0;
-  if (dh < 16 || dh > 256 || dh % 16 != 0 || Hkv < 1 || H % Hkv != 0 || page_size < 1 || max_blocks < 1)
-    return DN_ERR_SHAPE;
-  int BK = plain::tile_keys(dh);
-  size_t lds = sizeof(float) * (static_cast<size_t>(plain::BQ) * dh + 2 * static_cast<size_t>(BK) * (dh + 1) +
+  // (any head size up to 256: one that is no multiple of 16 is padded to the next inside the kernel)
+  if (dh < 1 || dh > 256 || Hkv < 1 || H % Hkv != 0 || page_size < 1 || max_blocks < 1) return DN_ERR_SHAPE;
+  const int dhp = (dh + 15) / 16 * 16;
+  int BK = plain::tile_keys(dhp);
+  size_t lds = sizeof(float) * (static_cast<size_t>(plain::BQ) * dhp + 2 * static_cast<size_t>(BK) * (dhp + 1) +
                                 static_cast<size_t>(plain::BQ) * BK + 4 * BK);
   dim3 grid(n_tiles, H), block(plain::THREADS);
   if (dtype == DN_F32)

@@ -169,7 +169,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const TI* __restrict__ A, int
       if (m < M && k < K) {
         const TI* p = A + static_cast<size_t>(m) * lda + k;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = to_float(p[i]);
+        for (int i = 0; i < 4; ++i)
+          if (k + i < K) v[i] = to_float(p[i]);       // (K need be no multiple of 4: zeros beyond it)
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) As[lk + i][lrow] = v[i];
@@ -178,7 +179,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const TI* __restrict__ A, int
       if (n < N && k < K) {
         const TI* p = W + static_cast<size_t>(n) * K + k;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) w[i] = to_float(p[i]);
+        for (int i = 0; i < 4; ++i)
+          if (k + i < K) w[i] = to_float(p[i]);
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) Ws[lk + i][lrow] = w[i];
@@ -936,9 +938,9 @@ static void launch_mb_norm(const Call& c, const NormIO& nio, int norm, hipStream
   const int mb = (c.M + 15) / 16;
   if (c.N >= 2560) {
     switch (mb) {
-      case 2: return launch_norm<2, 2, 8, 4>(c, nio, norm, stream);
-      case 3: return launch_norm<3, 2, 8, 4>(c, nio, norm, stream);
-      default: return launch_norm<4, 2, 8, 4>(c, nio, norm, stream);
+      case 2: return launch_norm<2, 2, 8, 6>(c, nio, norm, stream);
+      case 3: return launch_norm<3, 2, 8, 6>(c, nio, norm, stream);
+      default: return launch_norm<4, 2, 8, 6>(c, nio, norm, stream);
     }
   }
   // (few columns: the rows in two halves, so that there are workgroups for all CUs)
@@ -1028,10 +1030,12 @@ static void launch_mb(const Call& c, hipStream_t stream) {
     }
   }
   if (c.N >= 2560) {
+    // (six steps in flight a wave: with K = 1,600 a wave's seven steps are one round and a step, where four in
+    // flight made two rounds: 4,800 and 6,400 columns at 64 rows 10.3 -> 9.6 and 10.0 -> 9.1 us)
     switch (mb) {
-      case 2: return launch<2, 2, WAVES, 4>(c, stream);
-      case 3: return launch<3, 2, WAVES, 4>(c, stream);
-      default: return launch<4, 2, WAVES, 4>(c, stream);
+      case 2: return launch<2, 2, WAVES, 6>(c, stream);
+      case 3: return launch<3, 2, WAVES, 6>(c, stream);
+      default: return launch<4, 2, WAVES, 6>(c, stream);
     }
   }
   // (few columns: the rows in two halves, so that there are workgroups for all CUs)
@@ -1747,7 +1751,8 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
                        int ldr, int M, int N, int K, int in_dtype, int out_dtype, int epilogue, int packed,
                        float* work, long work_floats, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || K % 4 != 0 || (lda < K && !(packed & PACKED_A))) return DN_ERR_SHAPE;
+  if (K <= 0 || (lda < K && !(packed & PACKED_A))) return DN_ERR_SHAPE;
+  if ((packed & PACKED_W) && K % 8 != 0) return DN_ERR_SHAPE;      // (the plain kernels take any K)
   if (epilogue < EPI_NONE || epilogue > EPI_GELU_ERF) return DN_ERR_SHAPE;
   if (resid != nullptr && epilogue != EPI_NONE) return DN_ERR_SHAPE;
   if ((packed & (PACKED_A | PACKED_C)) && (!(packed & PACKED_W) || M > 256)) return DN_ERR_SHAPE;

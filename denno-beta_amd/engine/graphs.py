@@ -147,12 +147,143 @@ class DecodeGraph:
         return self.logits
 
 
+# -- steps that hold portions of prompts ---------------------------------------------------------------
+# Issued kernel by kernel, a step costs the host some 12 us a launch, seven launches a layer: at 48 layers more than
+# 4 ms, which a step of a few hundred rows does not keep the GPU busy for.  Such a step is captured too, over
+# buffers of a bucket's size: T rows, S requests, R wanted rows, and as many attention tiles as T rows of S
+# requests can make.  Rows, requests and tiles beyond the real ones are padding: a padding row has token 0,
+# position 0 and slot -1 (its keys and values go nowhere), belongs to no tile (attention leaves it alone) and is
+# wanted by nobody; rows never mix, so whatever a padding row holds stays in it.  A bucket is captured when a step
+# falls into it for the second time: a shape that comes once runs kernel by kernel.
+PORTION_ROWS = (16, 32, 48, 64, 96, 128, 192, 256, 384, 512)
+PORTION_REQUESTS = (1, 2, 4, 8, 16, 32, 64, 128, 256, 512)
+PORTION_GRAPHS_MAX = 48      # captured buckets per runner; steps of further shapes run kernel by kernel
+
+
+def _bucket(n, sizes):
+    for b in sizes:
+        if b >= n:
+            return b
+    return None
+
+
+class PortionGraph:
+    def __init__(self, runner, T: int, S: int, R: int):
+        from .batch import TILE_ROWS, WIDE_TILE_ROWS
+        self.manager, self.T, self.S, self.R = runner.cache.manager, T, S, R
+        cache, dev = runner.cache, runner.device
+        self.layouts = cache.layouts
+        self.vocab, self.max_positions = runner.spec.vocab, runner.spec.max_positions
+        self.max_blocks = [(-(-runner.spec.max_positions // l.page_size) if l.kind == 0 else 0) for l in self.layouts]
+        # (a request of n rows makes at most n / 16 + 1 tiles)
+        self.n_tiles, self.n_wide = T // TILE_ROWS + S, T // WIDE_TILE_ROWS + S
+        self.off, o = {}, 0
+        for name, n in (("tokens", T), ("positions", T), ("logit_rows", R), ("state_slots", S), ("row_start", S + 1),
+                        ("tiles", 4 * self.n_tiles), ("wide", 4 * self.n_wide)):
+            self.off[name] = (o, n)
+            o += n
+        for g, l in enumerate(self.layouts):
+            if l.kind == 0:
+                self.off[f"bt{g}"] = (o, S * self.max_blocks[g])
+                o += S * self.max_blocks[g]
+                self.off[f"sm{g}"] = (o, T)
+                o += T
+        self.host = [torch.empty(o, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self.copied = [None, None]
+        self.turn = 0
+        self.dev = torch.zeros(o, dtype=torch.int32, device=dev)
+        v = self._view
+        tiles, wide = v("tiles").view(4, self.n_tiles), v("wide").view(4, self.n_wide)
+        groups = []
+        for g, l in enumerate(self.layouts):
+            if l.kind != 0:
+                groups.append(GroupStep(0, 0, None, None, None))
+            else:
+                groups.append(GroupStep(l.page_size, l.window, v(f"sm{g}"), v(f"bt{g}").view(S, self.max_blocks[g]),
+                                        tiles, wide, False, 0))
+        self.ctx = StepContext(T=T, S=S, R=R, tokens=v("tokens"), positions=v("positions"),
+                               logit_rows=v("logit_rows"), state_slots=v("state_slots"), row_start=v("row_start"),
+                               groups=groups, host_row_start=[0] * (S + 1), host_first_pos=[0] * S,
+                               host_slots=[-1] * S, rids=[-1] * S)
+        self._fill(self.host[0].numpy(), [], np.empty(0, np.int64), np.empty(0, np.int32), np.empty(0, np.int32),
+                   np.empty(0, np.int32))
+        self.dev.copy_(self.host[0])
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            runner.model.forward(self.ctx, cache)
+        torch.cuda.current_stream(dev).wait_stream(side)
+        torch.cuda.synchronize(dev)
+        self.graph = torch.cuda.CUDAGraph()
+        collecting = gc.isenabled()       # (see DecodeGraph: no collection while the stream records)
+        gc.disable()
+        try:
+            with torch.cuda.graph(self.graph):
+                self.logits = runner.model.forward(self.ctx, cache)
+        finally:
+            if collecting:
+                gc.enable()
+
+    def _view(self, name):
+        b, n = self.off[name]
+        return self.dev[b:b + n]
+
+    def _fill(self, hv, entries, rids, starts, counts, slots):
+        """The step's tables into a host buffer; -> the number of wanted rows."""
+        from .batch import plan_rows
+        n = len(entries)
+        tokens, positions, logit_rows, row_start, tiles, wide = plan_rows(entries, starts.tolist(), self.vocab,
+                                                                          self.max_positions)
+        rows = len(tokens)
+
+        def put(name, vals, fill):
+            b, ln = self.off[name]
+            hv[b:b + ln] = fill
+            hv[b:b + len(vals)] = vals
+        put("tokens", tokens, 0), put("positions", positions, 0), put("logit_rows", logit_rows, 0)
+        put("state_slots", slots, -1), put("row_start", row_start, rows)
+        for name, table, width in (("tiles", tiles, self.n_tiles), ("wide", wide, self.n_wide)):
+            b, ln = self.off[name]
+            t = hv[b:b + ln].reshape(4, width)
+            t[0, :], t[1, :], t[2, :], t[3, :] = -1, 0, 1, 0
+            if table:
+                t[:, :len(table)] = np.asarray(table, dtype=np.int32).T
+        for g, l in enumerate(self.layouts):
+            if l.kind != 0:
+                continue
+            (b0, n0), (b1, n1) = self.off[f"bt{g}"], self.off[f"sm{g}"]
+            hv[b0:b0 + n0] = -1
+            hv[b1:b1 + n1] = -1
+            if n:
+                bad = self.manager.step_tables(g, rids, starts, counts,
+                                               hv[b0:b0 + n * self.max_blocks[g]].reshape(n, self.max_blocks[g]),
+                                               hv[b1:b1 + rows])
+                if bad >= 0:
+                    raise BatchError(f"request {int(rids[bad])}: a token's page was given back already")
+        return len(logit_rows)
+
+    def run(self, entries, rids, starts, counts, slots):
+        i = self.turn
+        self.turn ^= 1
+        if self.copied[i] is not None:
+            self.copied[i].synchronize()      # the copy that last read this host buffer has ended
+        wanted = self._fill(self.host[i].numpy(), entries, rids, starts, counts, slots)
+        self.dev.copy_(self.host[i], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self.copied[i] = ev
+        self.graph.replay()
+        return self.logits, wanted
+
+
 class DecodeGraphs:
     """The graphs of one runner, captured on demand."""
 
     def __init__(self, runner):
         self._runner = weakref.ref(runner)      # the runner owns these graphs; a reference back would be a cycle
         self.graphs: Dict[Tuple[int, int], DecodeGraph] = {}
+        self.portions: Dict[Tuple[int, int, int], PortionGraph] = {}
+        self.seen: Dict[Tuple[int, int, int], int] = {}      # bucket -> steps that fell into it so far
 
     @property
     def runner(self):
@@ -209,4 +340,48 @@ class DecodeGraphs:
         else:
             out = logits[torch.tensor(rows, dtype=torch.long, device=logits.device)] if rows else logits[:0].clone()
         mgr.commit_step(rids, new_lens)
+        return out
+
+    # -- steps that hold portions ---------------------------------------------------------------------
+    def portion_bucket(self, entries: Sequence[StepEntry]):
+        """(T, S, R) of the bucket that a step with portions falls into, or None if none takes it."""
+        runner = self.runner
+        if not runner.model.graph_safe or not runner.options.graph_portions:
+            return None
+        rows, wanted = sum(len(e.tokens) for e in entries), sum(len(e.want) for e in entries)
+        T, S = _bucket(rows, PORTION_ROWS), _bucket(len(entries), PORTION_REQUESTS)
+        if T is None or S is None or rows < 1:
+            return None
+        return (T, S, S if wanted <= S else T)
+
+    def takes_portions(self, entries: Sequence[StepEntry]) -> bool:
+        """Whether this step is replayed from a captured graph: its bucket has been met before (and is captured
+        now if it was not), and there is room for another graph."""
+        key = self.portion_bucket(entries)
+        if key is None:
+            return False
+        self.seen[key] = self.seen.get(key, 0) + 1
+        if key in self.portions:
+            return True
+        return self.seen[key] >= 2 and len(self.portions) < PORTION_GRAPHS_MAX
+
+    def step_portions(self, entries: Sequence[StepEntry], borrow=False) -> torch.Tensor:
+        """Runs a step of any mix from its bucket's graph; -> logits [R, vocab] at the wanted places (with `borrow`
+        a view of the graph's own buffer, which holds them until the same graph is replayed)."""
+        runner = self.runner
+        mgr = runner.cache.manager
+        key = self.portion_bucket(entries)
+        rids = np.asarray([e.rid for e in entries], dtype=np.int64)
+        counts = np.asarray([len(e.tokens) for e in entries], dtype=np.int32)
+        starts = mgr.lengths(rids)
+        # (what is wrong with the entries is found before pages are taken: plan_rows raises on them)
+        from .batch import plan_rows
+        plan_rows(entries, starts.tolist(), runner.spec.vocab, runner.spec.max_positions)
+        slots = mgr.reserve_step(rids, starts + counts)
+        g = self.portions.get(key)
+        if g is None:
+            g = self.portions[key] = PortionGraph(runner, *key)
+        logits, wanted = g.run(entries, rids, starts, counts, slots)
+        out = logits[:wanted] if borrow else logits[:wanted].clone()
+        mgr.commit_step(rids, starts + counts)
         return out

@@ -95,6 +95,9 @@ class ModelRunner:
             return self.graphs.step(entries, device_tokens, borrow)
         if device_tokens is not None:
             raise ValueError("device_tokens: only a step of single tokens that captured graphs run takes them")
+        if self.graphs is not None and self.graphs.takes_portions(entries):
+            self.steps_run += 1
+            return self.graphs.step_portions(entries, borrow)
         ctx = build_context(entries, self.cache, self.spec.vocab, self.spec.max_positions, self.device)
         logits = self.model.forward(ctx, self.cache)
         self.cache.manager.commit_step(

@@ -388,7 +388,7 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
     reference for bfloat16) or a PackedMatrix (the MFMA kernels); bias: 32-bit [N].  With a packed
     w and at most 256 rows, a and a bfloat16 out may be packed rows."""
     M, K = a.shape
-    _need(K % 8 == 0, lambda: f"linear: the inner size {K} must be a multiple of 8")
+    # (the plain kernels take any inner size; a packed matrix has one that is a multiple of 8: pack_matrix)
     lda, N, packed = _operands(a, w, "linear")
     wp = w.data_ptr()
     if bias is not None:
@@ -460,7 +460,6 @@ def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):
     if not isinstance(w, PackedMatrix) and not isinstance(a, PackedMatrix) and out.dtype == a.dtype and M <= 64:
         # few rows in the plain kernels: where K is shared out among workgroups, the kernel that adds their sums
         # writes the keys and values to the cache as well
-        _need(K % 8 == 0, lambda: f"linear_qkv: the inner size {K} must be a multiple of 8")
         lda, _, _ = _operands(a, w, "linear_qkv")
         _dev(out, "out", (a.dtype,), 2)
         if _lib_quiet("gemm").dn_gemm_plain_qkv_takes(a.data_ptr(), lda, w.data_ptr(), M, N, K, _CODE[a.dtype]):
@@ -531,7 +530,9 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
           "attention: pools")
     _need(q.shape[1] >= n_heads * dh and tuple(out.shape) == (T, n_heads * dh), "attention: q/out shapes")
     _need(block_tables.is_contiguous() and tiles.is_contiguous() and tiles.shape[0] == 4, "attention: tables")
-    _need(dh % 16 == 0 and 16 <= dh <= 256, lambda: f"attention: head size {dh} must be a multiple of 16 up to 256")
+    # (the plain kernel takes any head size up to 256; the bfloat16 kernels and the kernels for single rows take
+    # multiples of 16, and a head size that is none goes the plain kernel's way)
+    _need(1 <= dh <= 256, lambda: f"attention: head size {dh} must be at most 256")
     _need(n_heads % Hkv == 0, lambda: f"attention: {n_heads} heads over {Hkv} key heads")
     ldq, ldo = _rows(q, "q"), (0 if out_packed else _rows(out, "out"))
     lib = _lib("attention")
@@ -586,7 +587,7 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
         return out
     n_tiles = tiles.shape[1]
     base = tiles.data_ptr()
-    if single_rows and max_context > 0:
+    if single_rows and max_context > 0 and dh % 16 == 0:
         # a step of single rows in the plain kernels: every tile of keys a workgroup of its own, the
         # tiles' results joined in order by a second kernel; the same bits as the kernel below gives
         _need(max_context <= block_tables.shape[1] * ps, "attention: max_context exceeds the block tables")

@@ -18,8 +18,6 @@ class DenseMLP(Part):
                  down_bias, stored_in_out: bool = False, down_init_std: float = 0.02):
         if activation not in ACTIVATION_EPILOGUES:
             raise ValueError(f"activation {activation!r}; known: {sorted(ACTIVATION_EPILOGUES)}")
-        if inner % 8 != 0 or width % 8 != 0:
-            raise ValueError(f"feed-forward sizes {width} -> {inner}: the matrix kernels take multiples of 8")
         self.width, self.inner, self.activation = width, inner, activation
         self.up = Linear(width, inner, up_weight, up_bias, stored_in_out)
         self.down = Linear(inner, width, down_weight, down_bias, stored_in_out, down_init_std)

@@ -31,8 +31,8 @@ class CausalSelfAttention(Part):
         self.scale, self.window = float(scale), int(window)
         if n_heads % n_kv_heads != 0:
             raise ValueError(f"{n_heads} heads cannot share {n_kv_heads} key heads")
-        if head_dim % 16 != 0 or not 16 <= head_dim <= 256:
-            raise ValueError(f"head size {head_dim}: the attention kernels take multiples of 16 up to 256")
+        if not 1 <= head_dim <= 256:
+            raise ValueError(f"head size {head_dim}: the attention kernels take head sizes up to 256")
         self.q_width = n_heads * head_dim
         self.kv_width = n_kv_heads * head_dim
         # (a checkpoint that stores q, k and v apart names them in qkv_*_sources: joined at load, one product here)

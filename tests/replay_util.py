@@ -118,12 +118,28 @@ def collect_files(out_dir, steps, vocab):
     return {rid: torch.stack([r[p] for p in sorted(r)]) for rid, r in rows.items()}
 
 
-# Tolerances on logits of size about 1: 32-bit differs from the plain implementation by the
-# order of its sums; bfloat16 rounds every activation to 8 bits of mantissa.
-TOL = {"float32": dict(atol=2e-5, rtol=1e-5), "bfloat16": dict(atol=1.5e-2, rtol=1.5e-2)}
+# Tolerances.  32-bit differs from the plain implementation by the order of its sums: absolute and relative
+# bounds on logits of size about 1.  bfloat16 rounds every activation between kernels to 8 bits of mantissa, and
+# what that does to a logit is measured against what a row's logits differ by among themselves (their standard
+# deviation over the vocabulary, 0.14 to 0.8 with these random weights): over every bfloat16 comparison of these
+# tests the worst logit was off by 0.030 of its row's spread and a comparison's mean by 0.0035.  A lost key, a
+# wrong page or a neighbour's row move a logit by the spread itself.
+TOL = {"float32": dict(atol=2e-5, rtol=1e-5)}
+BF16_WORST, BF16_MEAN = 0.04, 0.007
 
 
 def assert_close(got, want, dtype, what):
+    got, want = got.float(), want.float()
+    if dtype == "bfloat16":
+        spread = want.std(dim=1, keepdim=True)
+        diff = (got - want).abs() / spread
+        worst, mean = diff.max().item(), diff.mean().item()
+        if not (worst <= BF16_WORST and mean <= BF16_MEAN):
+            at = (diff == diff.max()).nonzero()[0].tolist()
+            raise AssertionError(f"{what}: bfloat16 logits differ by {worst:.4f} of a row's spread at worst (position {at[0]}, "
+                                 f"token {at[1]}: got {got[at[0], at[1]].item()}, want {want[at[0], at[1]].item()}), "
+                                 f"{mean:.5f} on average; the bounds are {BF16_WORST} and {BF16_MEAN}")
+        return
     tol = TOL[dtype]
     diff = (got - want).abs()
     bound = tol["atol"] + tol["rtol"] * want.abs()

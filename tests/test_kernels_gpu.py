@@ -515,13 +515,40 @@ def test_plain_linear_has_one_order_of_summation_whatever_the_rows(N, K):
 def test_linear_refuses_what_it_cannot_take():
     o = ops()
     with pytest.raises(o.KernelError, match="multiple of 8"):
-        o.linear(rnd(2, 12), rnd(4, 12), None, out=torch.empty(2, 4, device=DEV))
+        o.pack_matrix(rnd(4, 12, dtype=torch.bfloat16))
     with pytest.raises(o.KernelError, match="does not fit"):
         o.linear(rnd(2, 16), rnd(4, 24), None, out=torch.empty(2, 4, device=DEV))
     with pytest.raises(o.KernelError):
         o.linear(rnd(2, 16), rnd(4, 16, dtype=torch.bfloat16), None, out=torch.empty(2, 4, device=DEV))
     with pytest.raises(o.KernelError, match="GPU"):
         o.linear(torch.zeros(2, 16), rnd(4, 16), None, out=torch.empty(2, 4, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(2, 4, 12), (5, 33, 7), (70, 50, 101), (64, 130, 1601), (300, 66, 30), (1, 9, 1)])
+def test_plain_linear_takes_any_inner_size(dtype, M, N, K):
+    """The plain product (all of 32-bit, and bfloat16 operands that the matrix-core kernels do not take) runs any
+    inner size, with every epilogue, against 64-bit sums; rows of a width that is no multiple of 4 included."""
+    o = ops()
+    a, w, bias = rnd(M, K, seed=1, dtype=dtype), rnd(N, K, seed=2, dtype=dtype, scale=0.3), rnd(N, seed=3)
+    exact = a.double() @ w.double().t() + bias.double()
+    tol = TOL[dtype]
+    for epi, f in (("none", lambda t: t), ("gelu_tanh", lambda t: torch.nn.functional.gelu(t, approximate="tanh")),
+                   ("gelu_erf", torch.nn.functional.gelu)):
+        out = torch.empty(M, N, dtype=dtype, device=DEV)
+        o.linear(a, w, bias, out=out, epilogue=epi)
+        assert torch.allclose(out.float(), f(exact).float(), **tol), (M, N, K, epi)
+    res = rnd(M, N, seed=4)
+    want = (res.double() + exact).float()
+    o.linear(a, w, bias, residual=res)
+    assert torch.allclose(res, want, **tol)
+    # a row's result does not depend on the rows beside it (one order of summation)
+    if dtype == torch.float32 and M > 1:
+        alone = torch.empty(1, N, device=DEV)
+        o.linear(a[M - 1:M].contiguous(), w, bias, out=alone)
+        both = torch.empty(M, N, device=DEV)
+        o.linear(a, w, bias, out=both)
+        assert torch.equal(alone[0], both[M - 1])
 
 
 def paged_case(seq_lens, new_rows, H, Hkv, dh, ps, dtype, seed=0, q_scale=1.0):
@@ -551,7 +578,8 @@ def paged_case(seq_lens, new_rows, H, Hkv, dh, ps, dtype, seed=0, q_scale=1.0):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,Hkv,dh,ps,window", [(4, 4, 16, 16, 0), (25, 25, 64, 16, 0), (6, 2, 48, 8, 0),
                                                 (2, 1, 128, 64, 0), (3, 3, 256, 16, 0), (4, 2, 32, 16, 20),
-                                                (5, 5, 80, 32, 7)])
+                                                (5, 5, 80, 32, 7), (4, 2, 15, 16, 0), (3, 3, 100, 8, 9), (2, 1, 250, 16, 0),
+                                                (5, 5, 1, 16, 0)])
 def test_attention(dtype, H, Hkv, dh, ps, window):
     # four requests: a decoded token far into a long context, a whole prompt, a portion, a first token
     seq_lens, new_rows = [300, 70, 133, 1], [1, 70, 21, 1]

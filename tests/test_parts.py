@@ -902,7 +902,7 @@ def test_a_norm_without_a_mean_runs_inside_the_products(rows):
         for slot in ("norm1", "norm2"):
             layer.parts[slot] = ("toy_rms", dict(width=cfg["n_embd"], eps=1e-6, weight_name=f"h.{i}.{slot}.g"))
     tensors = draw(spec, "cuda:0", dtype="bfloat16")
-    seq = seeded_tokens(6, 30 + rows, cfg["vocab_size"])
+    seq = seeded_tokens(6, 20 + rows, cfg["vocab_size"])
     calls = {"in": 0}
     real_in = ops.linear_norm_in
 
@@ -916,9 +916,9 @@ def test_a_norm_without_a_mean_runs_inside_the_products(rows):
         for inside in (True, False):
             r = ModelRunner(spec, dict(tensors), options("cuda:0", "bfloat16", use_graphs=False, norms_inside_products=inside))
             r.start_request(0)
-            r.step([StepEntry(0, seq[:30], [])])
+            r.step([StepEntry(0, seq[:20], [])])
             before = calls["in"]
-            got[inside] = r.step([StepEntry(0, seq[30:], list(range(rows)))]).float().cpu()
+            got[inside] = r.step([StepEntry(0, seq[20:], list(range(rows)))]).float().cpu()
             assert calls["in"] - before == (2 * cfg["n_layer"] - 1 if inside else 0)
     finally:
         ops.linear_norm_in = real_in
@@ -936,5 +936,5 @@ def test_a_norm_without_a_mean_runs_inside_the_products(rows):
         x = x + o @ st[p + "attn.c_proj.weight"].double() + st[p + "attn.c_proj.bias"].double()
         f = torch.nn.functional.gelu(rms(x, st[p + "norm2.g"]) @ st[p + "mlp.c_fc.weight"].double() + st[p + "mlp.c_fc.bias"].double())
         x = x + f @ st[p + "mlp.c_proj.weight"].double() + st[p + "mlp.c_proj.bias"].double()
-    want = P.head(x.float(), st["ln_f.weight"], st["ln_f.bias"], cfg["layer_norm_epsilon"], st["wte.weight"])[30:]
+    want = P.head(x.float(), st["ln_f.weight"], st["ln_f.bias"], cfg["layer_norm_epsilon"], st["wte.weight"])[20:]
     U.assert_close(got[True], want, "bfloat16", "a norm without a mean inside the products against the plain formulas")

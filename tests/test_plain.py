@@ -220,6 +220,33 @@ def test_score_scale_options_are_a_scaling_of_the_queries():
         assert not torch.allclose(got, P.PlainGPT2(off, m.t).logits(toks), atol=1e-5), option
 
 
+def test_the_first_layer_is_divided_by_one():
+    """`scale_attn_by_inverse_layer_idx` divides a layer's scores by its index counted so that the first layer
+    keeps its scores: a count from 0 as it stands would divide the first layer by zero, and any other start
+    changes a model of one layer.  So in a model of one layer the option changes nothing, to the last bit, and
+    in a model of two layers it changes the second layer alone: the first layer's output is the same with and
+    without it.  (What the option means is still this build's reading of the key's name: the reference has no
+    such option and no vector for it, and model code of installed packages is not consulted.)"""
+    cfg, m = tiny("B")
+    toks = seeded_tokens(7, 12, cfg["vocab_size"])
+    one = dict(cfg, n_layer=1)
+    on = P.PlainGPT2(dict(one, scale_attn_by_inverse_layer_idx=True), m.t).logits(toks)
+    off = P.PlainGPT2(dict(one, scale_attn_by_inverse_layer_idx=False), m.t).logits(toks)
+    assert torch.isfinite(on).all() and torch.equal(on, off)
+    assert P.attention_scale(48, 0, True, True) == P.attention_scale(48, 0, True, False) == 1 / math.sqrt(48)
+    assert P.attention_scale(48, 1, True, True) == 1 / math.sqrt(48) / 2 and P.attention_scale(48, 2, False, True) == 1 / 3
+    two = dict(cfg, n_layer=2)
+    assert not torch.equal(P.PlainGPT2(dict(two, scale_attn_by_inverse_layer_idx=True), m.t).logits(toks),
+                           P.PlainGPT2(dict(two, scale_attn_by_inverse_layer_idx=False), m.t).logits(toks))
+    # and the engine's own factor is the plain one's, layer by layer
+    from denno_beta_amd.models.gpt2 import GPT2Config, attention_scale
+    for inv in (False, True):
+        for sw in (False, True):
+            c = GPT2Config.from_dict(dict(cfg, scale_attn_by_inverse_layer_idx=inv, scale_attn_weights=sw))
+            for l in range(3):
+                assert attention_scale(c, l) == pytest.approx(P.attention_scale(c.head_dim, l, sw, inv), rel=1e-7)
+
+
 def test_float64_agrees_with_float32():
     cfg, m32 = tiny("B")
     _, m64 = tiny("B", torch.float64)

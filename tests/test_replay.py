@@ -114,6 +114,43 @@ def test_other_head_sizes_and_widths(tmp_path, name, dtype):
             U.assert_close(got[f"r{i}"], want[i], dtype, f"{name} {dtype} {kind} request {i}")
 
 
+ODD_SIZES = {
+    "four heads of 15": _cfg(2, 60, 4, 100, 301, 96),                       # nothing a multiple of 8
+    "three heads of 22": _cfg(3, 66, 3, 150, 77, 80, 1e-6, "gelu", True),   # an inner size that no 4 divides
+    "one head of 100": _cfg(1, 100, 1, 36, 129, 72),                        # padded to 112 in the kernel, a narrow feed-forward
+}
+
+
+@pytest.mark.parametrize("name", list(ODD_SIZES))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_that_are_multiples_of_nothing(backend, tmp_path, name, dtype):
+    """The architecture's forward runs any width, inner size and head size (gpt2.rs:138, the plain loops
+    :170-202): so do the plain kernels, which both engines fall to for sizes that the matrix-core kernels do
+    not take (a head size that is no multiple of 16, an inner size of a product that is no multiple of 8).
+    Four cuttings; 32-bit logits equal bit for bit across them."""
+    from denno_beta_amd.weights import write_model_folder
+    cfg = ODD_SIZES[name]
+    folder = str(tmp_path)
+    write_model_folder(folder, cfg, 9, dtype)
+    P = cfg["n_positions"]
+    seqs = [seeded_tokens(40 + i, n, cfg["vocab_size"]) for i, n in enumerate((5, 50, P - 2, 33))]
+    if backend == "cpu":
+        seqs = seqs[:3]
+    want = plain_logits(folder, seqs)
+    whole = None
+    for kind, steps in (("whole", U.whole_trace(seqs)), ("tail", U.tail_decode_trace(seqs, 32)),
+                        ("chunks", U.chunk_trace(seqs)), ("mixed", U.mixed_trace(seqs, seed=5))):
+        r = runner_for(folder, dtype, backend, cache_tokens=U.max_live_tokens(steps))
+        got = U.replay(r, steps)
+        r.cache.manager.check()
+        for i in range(len(seqs)):
+            U.assert_close(got[f"r{i}"], want[i], dtype, f"{name} {dtype} {kind} request {i}")
+            if dtype == "float32" and backend != "cpu" and whole is not None:
+                assert torch.equal(got[f"r{i}"], whole[f"r{i}"]), f"{name} {kind} request {i}: 32-bit logits depend on the cutting"
+        if whole is None:
+            whole = got
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_and_first_tokens(backend, model_folders, dtype):
     """A sequence decoded token by token from its first token on, across many pages."""

@@ -1,6 +1,6 @@
 """The four cuttings at the layer sizes that the measurements run, against the plain implementation:
 two layers of GPT-2 XL's sizes (1,600 wide, 25 heads, a feed-forward of 6,400, a vocabulary of 50,257,
-1,024 positions) and two of GPT-2 Medium's (1,024 wide, 16 heads).  The tiny models are too narrow for
+1,024 positions) and two of GPT-2 Medium's (1,024 wide, 16 heads, the same vocabulary).  The tiny models are too narrow for
 some of the kernels that serve these widths: steps of 17 to 64 rows whose norms run inside the products
 beside them, steps of 65 to 256 rows whose rows travel packed between kernels, the many-rows kernels
 beyond that.  A mixed trace here holds portions of prompts beside decoded tokens in steps of every one
@@ -22,7 +22,7 @@ def _cfg(L, E, H, V, P=1024):
 
 
 SHAPES = {"xl": (_cfg(2, 1600, 25, 50257), 21, (1024, 600, 257, 130, 64)),
-          "medium": (_cfg(2, 1024, 16, 12289), 22, (1024, 333, 600, 96, 150))}
+          "medium": (_cfg(2, 1024, 16, 50257), 22, (1024, 333, 600, 96, 150))}
 
 _made = {}
 

@@ -172,12 +172,23 @@ __device__ __forceinline__ float block_sum_256(float v, float* scratch) {
   return ((scratch[0] + scratch[1]) + scratch[2]) + scratch[3];
 }
 
-template <typename TO, int VPT>
+// What a product left for this norm to add into the rows before it norms them (JOIN): the sums of its shares
+// of K, part[share][row][e] (`stride` floats from one share to the next), and its bias.  The rows become
+// x + ((part[0] + part[1] + ...) + bias), shares in ascending order from zero, as the kernel that only adds
+// them makes it (gemm.hip, plain::join_kernel), and are stored back before they are normed.
+struct PendingSum {
+  const float* part;
+  const float* bias;
+  long long stride;
+  int shares;
+};
+
+template <typename TO, int VPT, bool JOIN = false>
 __global__ __launch_bounds__(256) void layernorm_row_kernel(const float* __restrict__ x,
                                                              const float* __restrict__ gamma,
                                                              const float* __restrict__ beta, TO* __restrict__ out,
                                                              const int32_t* __restrict__ rows, int E, float eps,
-                                                             int packed) {
+                                                             int packed, PendingSum pend, float* __restrict__ x_out) {
   __shared__ float scratch[4];
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
@@ -190,6 +201,28 @@ __global__ __launch_bounds__(256) void layernorm_row_kernel(const float* __restr
     v[i] = xr[e];
     gm[i] = gamma[e];
     bt[i] = beta ? beta[e] : 0.f;
+  }
+  if constexpr (JOIN) {
+    const float* pr = pend.part + static_cast<size_t>(src) * E;
+    float tot[VPT], pb[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      tot[i] = 0.f;
+      pb[i] = pend.bias ? pend.bias[min(static_cast<int>(threadIdx.x) + i * 256, E - 1)] : 0.f;
+    }
+    for (int sh = 0; sh < pend.shares; ++sh) {
+      float p[VPT];
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) p[i] = pr[sh * pend.stride + min(static_cast<int>(threadIdx.x) + i * 256, E - 1)];
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) tot[i] += p[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int e = threadIdx.x + i * 256;
+      v[i] = v[i] + (pend.bias ? tot[i] + pb[i] : tot[i]);
+      if (e < E) x_out[static_cast<size_t>(src) * E + e] = v[i];
+    }
   }
   float s = 0.f;
 #pragma unroll
@@ -220,18 +253,51 @@ __global__ __launch_bounds__(256) void layernorm_row_kernel(const float* __restr
 template <typename TO>
 static void launch_layernorm(const float* x, const float* gamma, const float* beta, TO* out, const int32_t* rows,
                              int R, int E, float eps, int packed, hipStream_t stream) {
+  const PendingSum none{};
   if (E <= 512)
-    hipLaunchKernelGGL((layernorm_row_kernel<TO, 2>), dim3(R), dim3(256), 0, stream, x, gamma, beta, out, rows, E, eps, packed);
+    hipLaunchKernelGGL((layernorm_row_kernel<TO, 2>), dim3(R), dim3(256), 0, stream, x, gamma, beta, out, rows, E, eps, packed, none, nullptr);
   else if (E <= 2048)
-    hipLaunchKernelGGL((layernorm_row_kernel<TO, 8>), dim3(R), dim3(256), 0, stream, x, gamma, beta, out, rows, E, eps, packed);
+    hipLaunchKernelGGL((layernorm_row_kernel<TO, 8>), dim3(R), dim3(256), 0, stream, x, gamma, beta, out, rows, E, eps, packed, none, nullptr);
   else if (E <= 8192)
     hipLaunchKernelGGL((layernorm_row_kernel<TO, 32>), dim3(R), dim3(256), 0, stream, x, gamma, beta, out, rows, E,
-                       eps, packed);
+                       eps, packed, none, nullptr);
   else {
     const int waves = 4;
     hipLaunchKernelGGL(layernorm_kernel<TO>, dim3((R + waves - 1) / waves), dim3(waves * DN_WAVE), 0, stream, x, gamma,
                        beta, out, rows, R, E, eps, packed);
   }
+}
+
+// LayerNorm of all R rows of x [R, E] after what a product left for them has been added (see PendingSum): x is
+// updated in place, out gets the normed rows.  E up to 8,192.
+extern "C" int dn_layernorm_join(float* x, const float* part, int shares, long long share_stride, const float* bias,
+                                 const float* gamma, const float* beta, void* out, int R, int E, float eps,
+                                 int out_dtype, int packed, hipStream_t stream) {
+  if (R <= 0) return 0;
+  if (!part || shares < 1 || share_stride < static_cast<long long>(R) * E || E > 8192) return DN_ERR_SHAPE;
+  if (packed && (out_dtype != DN_BF16 || E % 32 != 0)) return DN_ERR_SHAPE;
+  const PendingSum pend{part, bias, share_stride, shares};
+#define DN_LNJ(TO, VPT)                                                                                              \
+  hipLaunchKernelGGL((layernorm_row_kernel<TO, VPT, true>), dim3(R), dim3(256), 0, stream, x, gamma, beta,            \
+                     static_cast<TO*>(out), static_cast<const int32_t*>(nullptr), E, eps, packed, pend, x)
+#define DN_LNJ_E(TO)        \
+  do {                      \
+    if (E <= 512)           \
+      DN_LNJ(TO, 2);        \
+    else if (E <= 2048)     \
+      DN_LNJ(TO, 8);        \
+    else                    \
+      DN_LNJ(TO, 32);       \
+  } while (0)
+  if (out_dtype == DN_F32)
+    DN_LNJ_E(float);
+  else if (out_dtype == DN_BF16)
+    DN_LNJ_E(bf16_t);
+  else
+    return DN_ERR_DTYPE;
+#undef DN_LNJ_E
+#undef DN_LNJ
+  return dn_launch_status();
 }
 
 // packed: out is a packed matrix of ceil(R / 16) * 16 rows (bfloat16, E a multiple of 32)

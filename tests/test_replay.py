@@ -426,3 +426,44 @@ def test_sharp_attention_shows_a_wrong_key(backend, model_folders, tmp_path, dty
     changed = list(seqs[0])
     changed[3] = (changed[3] + 1) % 512
     assert (plain.logits(changed)[-1] - want[0][-1]).abs().max() > 1e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_with_portions_are_replayed_from_graphs(model_folders, dtype):
+    """A step that holds portions is captured as a graph when its bucket (rows, requests, wanted rows) comes a
+    second time, over buffers of the bucket's size with padding rows, requests and tiles.  The same traces with
+    and without: 32-bit logits equal bit for bit, bfloat16 within rounding (a bucket's rows may choose another
+    kernel than the real rows would); every graph replayed several times over other requests, other pages and
+    other positions, with steps that run kernel by kernel in between."""
+    from denno_beta_amd.config import EngineOptions
+    from denno_beta_amd.engine import ModelRunner
+    name = "B"
+    folder = model_folders(name, dtype)
+    seqs = sequences(name, (60, 200, 33, 120, 97, 250), seed=31)
+    want = plain_logits(folder, seqs)
+    traces = {"chunks": U.chunk_trace(seqs, sizes=(17, 2, 40, 17, 3, 64, 40, 2, 17)),
+              "mixed": U.mixed_trace(seqs, seed=8, sizes=(1, 1, 2, 17, 17, 40))}
+    for kind, steps in traces.items():
+        got = {}
+        for on in (True, False):
+            r = ModelRunner.from_folder(folder, EngineOptions(dtype=dtype, page_size=16, max_live=4, graph_portions=on,
+                                                              cache_tokens=U.max_live_tokens(steps)))
+            got[on] = U.replay(r, steps)
+            r.cache.manager.check()
+            assert r.cache.manager.live() == 0
+            if on:
+                assert len(r.graphs.portions) >= 3, sorted(r.graphs.portions)
+                replayed = sum(n - 1 for key, n in r.graphs.seen.items() if key in r.graphs.portions)
+                assert replayed >= len(r.graphs.portions) + 5
+                # (every bucket's first step ran kernel by kernel, between the replays of the buckets before it)
+                if kind == "mixed":
+                    assert r.cache.manager.reuse_count(0) > 0
+            else:
+                assert not r.graphs.portions
+        for i in range(len(seqs)):
+            U.assert_close(got[True][f"r{i}"], want[i], dtype, f"portions from graphs, {dtype}, {kind}, request {i}")
+            if dtype == "float32":
+                assert torch.equal(got[True][f"r{i}"], got[False][f"r{i}"]), (kind, i)
+            else:
+                U.assert_close(got[True][f"r{i}"], got[False][f"r{i}"], dtype, f"graphs against kernel by kernel, {kind}, request {i}")

@@ -59,7 +59,7 @@ class Workloads:
         live = max(64, a.batch)
         self.opts = EngineOptions(dtype=dtype, page_size=a.page_size, cache_tokens=live * P, max_live=live, max_batch_tokens=4096,
                                   prefill_chunk=1024, use_graphs=not (a.no_graphs or a.kernel_times), seed=0,
-                                  norms_inside_products=not a.norm_kernels)
+                                  norms_inside_products=not a.norm_kernels, deferred_sums=not a.no_deferred_sums)
         self.runner = ModelRunner.from_random(self.cfg, seed=0, options=self.opts, stored=dtype)
         self.gen = torch.Generator().manual_seed(0)
 
@@ -159,6 +159,8 @@ def main():
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--norm-kernels", action="store_true",
                     help="run every norm as a kernel of its own, also in steps of few rows (for comparisons)")
+    ap.add_argument("--no-deferred-sums", action="store_true",
+                    help="every product into the stream adds its own sum (steps of 65 to 256 rows; for comparison)")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64, the prefill and the 32-bit engine")
     ap.add_argument("--kernel-times", action="store_true",
                     help="with --only decode or prefill: every launch between two HIP events (no graphs), and a "
@@ -258,7 +260,7 @@ def serving(a):
     from denno_beta_amd.engine import Engine, SamplingParams
     cfg = large_config()
     opts = EngineOptions(dtype=a.dtype, page_size=16, cache_tokens=64 * 1024, max_live=64, max_batch_tokens=2048,
-                         prefill_chunk=512, use_graphs=not a.no_graphs, seed=0, norms_inside_products=not a.norm_kernels)
+                         prefill_chunk=512, use_graphs=not a.no_graphs, seed=0, norms_inside_products=not a.norm_kernels, deferred_sums=not a.no_deferred_sums)
     eng = Engine.from_random(cfg, 0, opts, stored=a.dtype)
     gen = torch.Generator().manual_seed(1)
     lengths = torch.randint(16, 769, (64,), generator=gen).tolist()

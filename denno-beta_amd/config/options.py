@@ -27,6 +27,7 @@ class EngineOptions:
     graph_portions: bool = True        # steps of up to 512 rows that hold prompt portions are captured too, a bucket at its second step (engine/graphs.py)
     run_ahead: bool = True             # launch the next decode step before the host has read this one's tokens (engine/engine.py)
     seed: Optional[int] = None         # default seed of requests that bring none
+    deferred_sums: bool = True         # steps of 65 to 256 rows: a product into the stream with few columns leaves its sum for the next norm's kernel (parts/blocks.py)
     norms_inside_products: bool = True  # steps of few rows: a norm between two products runs inside them (parts/blocks.py)
 
     def validate(self):

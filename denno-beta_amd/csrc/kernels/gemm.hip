@@ -1720,8 +1720,19 @@ static int shares_of_k(int M, int N, int K, int packed, bool kv) {
   return ((M + 31) / 32) * ((N + 63) / 64) <= 96 ? 8 : 4;
 }
 
+// A product into the residual stream whose sum a norm's kernel adds (dn_gemm_deferred): the shares of K that it
+// is cut into, 0 if it is not worth it.  Few columns and 65 to 256 rows: the tiles are too few to fill the chip,
+// and with the shares' sums left for the next kernel to add nothing has to join them here (1,600 x 1,600 at 128
+// and 256 rows: 4.8 and 6.2 us where the whole product takes 6.7 and 8.0; K = 6,400: the kernel that adds the
+// shares, 4.5 us, falls away).
+static int deferred_shares(int M, int N, int K) {
+  if (M <= 64 || M > 256 || N >= 2048 || K % 64 != 0) return 0;
+  if (K >= 4096) return M <= 128 ? 4 : 2;
+  return K / 64 >= 8 ? 2 : 0;
+}
+
 static int run(const Args& a, hipStream_t stream) {
-  if (mid_rows(a.M, a.N, a.K)) return launch_as<2, 2, 2, 2, 4, 2>(a, stream);
+  if (mid_rows(a.M, a.N, a.K) || (a.part && a.N < 2048 && a.K % 64 == 0)) return launch_as<2, 2, 2, 2, 4, 2>(a, stream);
   switch (pick(a.M, a.N, a.part ? a.K / a.splits : a.K)) {
     case 0: return launch_as<2, 2, 2, 4, 4>(a, stream);
     case 1: return launch_as<4, 2, 2, 4, 4>(a, stream);
@@ -1844,6 +1855,33 @@ extern "C" int dn_gemm_plain_qkv(const void* A, int lda, const void* W, const fl
 extern "C" long dn_gemm_work_floats(int M, int N, int K, int packed) {
   if (packed & PACKED_W) return static_cast<long>(direct::shares_of_k(M, N, K, packed, false)) * M * N;
   return plain::work_floats(M, N, K);
+}
+
+// A product whose sum somebody else adds into the residual stream: part[share][m][n] (32-bit) = the share's part of
+// A . W^T, for dn_gemm_deferred_shares(M, N, K) shares of K; no bias, no epilogue.  dn_layernorm_join (the norm
+// that reads the stream next) or dn_join adds them, in order.  A bfloat16 in rows or packed, W packed.
+extern "C" int dn_gemm_deferred_shares(int M, int N, int K) { return direct::deferred_shares(M, N, K); }
+
+extern "C" int dn_gemm_deferred(const void* A, int lda, const void* W, int M, int N, int K, int packed, float* part,
+                                long part_floats, hipStream_t stream) {
+  const int shares = direct::deferred_shares(M, N, K);
+  if (shares < 1 || !part || part_floats < static_cast<long>(shares) * M * N) return DN_ERR_SHAPE;
+  if (!(packed & PACKED_W) || (packed & PACKED_C) || ((packed & PACKED_A) && M > 256)) return DN_ERR_SHAPE;
+  if (!direct::takes(A, lda, W, nullptr, nullptr, 0, part, N, N, K, DN_F32, packed)) return DN_ERR_SHAPE;
+  direct::Args a{A, lda, W, nullptr, nullptr, 0, nullptr, 0, M, N, K, DN_F32, EPI_NONE, packed, nullptr};
+  a.part = part, a.splits = shares;
+  const int rc = direct::run(a, stream);
+  return rc != 0 ? rc : dn_launch_status();
+}
+
+// resid [M, N] += (part[0] + part[1] + ...) + bias: the shares' sums of a deferred product, where no norm adds them
+extern "C" int dn_join(const float* part, int shares, const float* bias, float* resid, int ldr, int M, int N,
+                       hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (!part || !resid || shares < 1 || ldr < N) return DN_ERR_SHAPE;
+  hipLaunchKernelGGL((plain::join_kernel<float>), dim3((N + 255) / 256, M), dim3(256), 0, stream, part, shares, bias,
+                     static_cast<float*>(nullptr), 0, resid, ldr, M, N, EPI_NONE, plain::KVRows<float>{});
+  return dn_launch_status();
 }
 
 // A product of few rows that adds into the residual stream and leaves what the norm after it needs:

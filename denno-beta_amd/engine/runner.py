@@ -26,7 +26,8 @@ class ModelRunner:
         self.spec, self.options, self.config = spec, options, config
         self.device = torch.device(options.device)
         self.runtime = Runtime(act_dtype=_ACT[options.dtype], device=self.device,
-                               norms_inside_products=options.norms_inside_products)
+                               norms_inside_products=options.norms_inside_products,
+                               deferred_sums=options.deferred_sums)
         self.model = spec.instantiate().bind(tensors, self.runtime)
         cache_tokens = options.cache_tokens or options.max_live * spec.max_positions
         self.cache = CacheStorage(self.model.cache_specs, kv_dtype=self.runtime.act_dtype,

@@ -99,6 +99,7 @@ def _declare(name, lib):
             "dn_embed_sum": [P, P, P, P, I, P, I, I, I, P],
             "dn_logits_post": [P, I, I, I, F, F, P],
             "dn_layernorm": [P, P, P, P, P, I, I, F, I, I, P],
+            "dn_layernorm_join": [P, P, I, c_longlong, P, P, P, P, I, I, F, I, I, P],
             "dn_kv_write": [P, I, I, I, P, P, P, I, I, I, I, I, P],
             "dn_cast": [P, P, c_longlong, I, I, P],
         },
@@ -110,6 +111,9 @@ def _declare(name, lib):
             "dn_gemm_norm_out": [P, I, P, P, P, I, I, I, I, P, P, I, P, P],
             "dn_gemm_norm_in": [P, I, P, P, P, F, P, P, I, I, I, I, I, P, P, P, I, I, I, I, I, I, P],
             "dn_gemm_qkv": [P, I, P, P, P, I, I, I, I, P, P, P, I, I, I, I, I, I, P],
+            "dn_gemm_deferred_shares": [I, I, I],
+            "dn_gemm_deferred": [P, I, P, I, I, I, I, P, c_longlong, P],
+            "dn_join": [P, I, P, P, I, I, I, P],
         },
         "attention": {
             "dn_attention": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, I, P],
@@ -331,6 +335,28 @@ def layernorm(x, gamma, beta, eps, out, rows=None):
     return out
 
 
+def layernorm_join(x, part, bias, gamma, beta, eps, out):
+    """x += (part[0] + part[1] + ...) + bias (in place: what `linear_deferred` left of a product into the stream),
+    then out = LayerNorm(x), all rows, in one kernel.  part: 32-bit [shares, R, E]; out: a tensor [R, E] or packed rows."""
+    packed = isinstance(out, PackedMatrix)
+    _dev(x, "x", (torch.float32,), 2), _dev(gamma, "gamma", (torch.float32,), 1), _dev(part, "part", (torch.float32,), 3)
+    if not packed:
+        _dev(out, "out", _FLOATS, 2)
+    R, E = x.shape
+    _need(x.is_contiguous() and part.is_contiguous() and tuple(part.shape[1:]) == (R, E) and part.shape[0] >= 1,
+          lambda: f"layernorm_join: shares of shape {tuple(part.shape)} for rows of shape {tuple(x.shape)}")
+    _need((packed or out.is_contiguous()) and tuple(out.shape) == (R, E) and gamma.is_contiguous() and gamma.shape[0] == E
+          and E <= 8192, "layernorm_join: shapes")
+    for v, name in ((beta, "beta"), (bias, "bias")):
+        if v is not None:
+            _dev(v, name, (torch.float32,), 1)
+            _need(v.is_contiguous() and v.shape[0] == E, lambda: f"layernorm_join: {name}")
+    _ok(_lib("elementwise").dn_layernorm_join(x.data_ptr(), part.data_ptr(), part.shape[0], R * E, _ptr(bias), gamma.data_ptr(),
+                                              _ptr(beta), out.data_ptr(), R, E, float(eps), _CODE[out.dtype], int(packed),
+                                              _stream()), "layernorm (adds a product's shares first)")
+    return out
+
+
 def kv_write(src, k_col, v_col, slot_map, k_pool, v_pool):
     """Rows of src ([T, ld]; keys at columns k_col.., values at v_col..) go to the slots
     slot_map[t] = page * page_size + offset; k_pool is [n_pages, Hkv, page_size, dh], v_pool
@@ -424,6 +450,41 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
                              _CODE[a.dtype], _CODE[out.dtype], epi, packed, _ptr(work), work_floats, _stream()),
         "linear" if _timed is None else f"linear {K} -> {N}" + (f", {epilogue}" if epi else ""))
     return out
+
+
+def linear_deferred_shares(n_rows, w):
+    """How many shares of K `linear_deferred` cuts the product of n_rows rows with w into; 0: it does not take it
+    (the product then adds into the stream itself)."""
+    if not isinstance(w, PackedMatrix):
+        return 0
+    return _lib_quiet("gemm").dn_gemm_deferred_shares(n_rows, w.shape[0], w.shape[1])
+
+
+def linear_deferred(a, w):
+    """-> part, 32-bit [shares, M, N]: the shares' parts of a @ w.T, for whoever adds them into the residual stream
+    with the bias (`layernorm_join`, the norm that reads the stream next, or `join`).  a: bfloat16 rows or packed
+    rows; w: a PackedMatrix."""
+    M, K = a.shape
+    lda, N, packed = _operands(a, w, "linear_deferred")
+    shares = linear_deferred_shares(M, w)
+    _need(shares > 0 and (packed & PACKED_W), lambda: f"linear_deferred: {M} rows x {tuple(w.shape)} is not deferred")
+    part = torch.empty((shares, M, N), dtype=torch.float32, device=a.device)
+    _ok(_lib("gemm").dn_gemm_deferred(a.data_ptr(), lda, w.data_ptr(), M, N, K, packed, part.data_ptr(), part.numel(), _stream()),
+        "linear_deferred" if _timed is None else f"linear {K} -> {N}, its shares left for the next norm")
+    return part
+
+
+def join(part, bias, residual):
+    """residual += (part[0] + part[1] + ...) + bias, in place: a deferred product's shares, where no norm adds them."""
+    _dev(part, "part", (torch.float32,), 3), _dev(residual, "residual", (torch.float32,), 2)
+    M, N = residual.shape
+    _need(part.is_contiguous() and tuple(part.shape[1:]) == (M, N), "join: shares of another shape than the rows")
+    if bias is not None:
+        _dev(bias, "bias", (torch.float32,), 1)
+        _need(bias.is_contiguous() and bias.shape[0] == N, "join: bias")
+    _ok(_lib("gemm").dn_join(part.data_ptr(), part.shape[0], _ptr(bias), residual.data_ptr(), _rows(residual, "residual"), M, N,
+                             _stream()), "join")
+    return residual
 
 
 def linear_qkv(a, w, bias, out, slot_map, k_pool, v_pool, q_width):

@@ -70,6 +70,10 @@ class Runtime:
     stream_stats: Optional["StreamStats"] = None
     # the norm that will read the stream first after the block that runs now (set by the model), or None
     next_norm: Optional["Part"] = None
+    next_takes_deferred: bool = False      # the block that runs next takes what is left in stream_deferred (set by the model)
+    deferred_sums: bool = True             # EngineOptions.deferred_sums
+    # a product's sum that is not in the stream yet (DeferredSum): the next norm's kernel adds it, or the model does
+    stream_deferred: Optional["DeferredSum"] = None
 
 
 class Part:
@@ -102,6 +106,12 @@ class Part:
         LazyNorm in place of the normed rows.  The default, normed rows, is always right."""
         return False
 
+    def defers_sum(self, n_rows: int) -> bool:
+        """A mixer or feed-forward whose last product, for a step of n_rows rows, can leave its sum for the norm
+        that reads the stream next to add (DeferredSum); its forward then takes `deferred=` (an empty DeferredSum
+        that it may fill instead of adding into the stream)."""
+        return False
+
     def writes_norm_stats(self, n_rows: int) -> bool:
         """A mixer or feed-forward whose last kernel, as it adds into the residual stream, can leave
         the statistics for the norm after it; its forward then takes `stats=` (a StreamStats)."""
@@ -121,6 +131,29 @@ class StreamStats:
     def __init__(self, copy, stats, norm):
         self.copy, self.stats, self.norm = copy, stats, norm
         self.written = False
+
+
+class DeferredSum:
+    """What a part's last product would have added into the residual stream, left for the kernel of the norm that
+    reads the stream next: the product's sums by shares of K, 32-bit [shares, rows, width], and its bias.  A norm
+    with `adds_deferred = True` takes it as `forward(..., deferred=)` and leaves the stream updated; anybody else
+    has it added first (`flush`)."""
+
+    def __init__(self):
+        self.part = self.bias = None
+
+    @property
+    def filled(self):
+        return self.part is not None
+
+    def fill(self, part, bias):
+        self.part, self.bias = part, bias
+
+    def flush(self, x):
+        from ..kernels import ops
+        if self.filled:
+            ops.join(self.part, self.bias, x)
+            self.part = self.bias = None
 
 
 class LazyNorm:

@@ -42,8 +42,11 @@ class DenseMLP(Part):
     def writes_norm_stats(self, n_rows):
         return self.down.writes_norm_stats(n_rows)
 
-    def forward(self, h, ctx, accumulate_into, stats=None):
+    def defers_sum(self, n_rows):
+        return self.down.defers(n_rows)
+
+    def forward(self, h, ctx, accumulate_into, stats=None, deferred=None):
         n = h.shape[0]
         f = self.up(h, out_dtype=self.runtime.act_dtype, epilogue=ACTIVATION_EPILOGUES[self.activation],
                     packed_out=self.up.few_rows(n) and self.down.packed_input(n))
-        self.down(f, residual=accumulate_into, stats=stats)
+        self.down(f, residual=accumulate_into, stats=stats, deferred=deferred)

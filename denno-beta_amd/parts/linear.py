@@ -85,6 +85,10 @@ class Linear:
         """Whether a call with n_rows rows that adds into the residual stream can leave what the norm after it needs."""
         return ops.norm_stream_takes(n_rows, self.out_features, self.weight) and self.in_features % 8 == 0
 
+    def defers(self, n_rows: int) -> bool:
+        """Whether a call with n_rows rows that adds into the residual stream can leave its sum for the next norm's kernel."""
+        return ops.linear_deferred_shares(n_rows, self.weight) > 0
+
     def _fusable(self, a, out_dtype):
         """(c1, c2, eps, no_mean) if `a` is a LazyNorm that this call can run in its own kernel."""
         if ((out_dtype or a.dtype) == torch.bfloat16 and a.stream is not None and a.stream.written
@@ -92,10 +96,11 @@ class Linear:
             return self._folded[id(a.norm)]
         return None
 
-    def __call__(self, a, out_dtype=None, epilogue="none", residual=None, packed_out=False, stats=None):
+    def __call__(self, a, out_dtype=None, epilogue="none", residual=None, packed_out=False, stats=None, deferred=None):
         """epilogue(a @ W^T + b) as a new [M, out] tensor of out_dtype (as packed rows if
         packed_out, for a Linear whose packed_input said so), or added into `residual` (32-bit) in
-        place.  An input in another precision than the weight is converted to the weight's (exact
+        place (or, with `deferred`, an empty parts.base.DeferredSum, left there for the next norm's kernel to add,
+        where `defers` says so).  An input in another precision than the weight is converted to the weight's (exact
         from bfloat16 to 32-bit)."""
         if isinstance(a, LazyNorm):
             f = self._fusable(a, out_dtype) if residual is None and not (packed_out and a.shape[0] <= 16) else None
@@ -108,6 +113,9 @@ class Linear:
         if a.dtype != self.weight.dtype:
             a = ops.cast(a.contiguous(), torch.empty(a.shape, dtype=self.weight.dtype, device=a.device))
         if residual is not None:
+            if deferred is not None and a.dtype == torch.bfloat16 and self.defers(a.shape[0]):
+                deferred.fill(ops.linear_deferred(a, self.weight), self.bias)       # (the stream itself stays as it is)
+                return residual
             if stats is not None and a.dtype == torch.bfloat16 and self.writes_norm_stats(a.shape[0]):
                 stats.written = True
                 return ops.linear_norm_out(a, self.weight, self.bias, residual, stats.norm.fused_params()[1],

@@ -69,7 +69,10 @@ class CausalSelfAttention(Part):
     def writes_norm_stats(self, n_rows):
         return self.out.writes_norm_stats(n_rows)
 
-    def forward(self, h, ctx, cache, accumulate_into, stats=None):
+    def defers_sum(self, n_rows):
+        return self.out.defers(n_rows)
+
+    def forward(self, h, ctx, cache, accumulate_into, stats=None, deferred=None):
         act = self.runtime.act_dtype
         g = ctx.groups[cache.group]
         position = self.position if self.position is not None else self.runtime.position
@@ -94,4 +97,4 @@ class CausalSelfAttention(Part):
         ops.attention(q, o, cache.k, cache.v, g.block_tables, g.tiles, self.n_heads,
                       self.scale, self.window, tiles_wide=g.tiles_wide, single_rows=g.single_rows,
                       max_context=g.max_context)
-        self.out(o, residual=accumulate_into, stats=stats)
+        self.out(o, residual=accumulate_into, stats=stats, deferred=deferred)

@@ -219,13 +219,21 @@ class DecoderModel:
                 parts.append((self.position.table(), ctx.positions, 1.0))
             parts += [(self.extra_tables[t.name], getattr(ctx, t.index), t.scale) for t in self.spec.extra_embeddings]
             ops.embed_sum(parts, x)
-        rt.stream_stats = None      # nobody has left anything for a norm of these rows yet
+        rt.stream_stats = rt.stream_deferred = None      # nobody has left anything for a norm of these rows yet
         order = self.spec.run_order
         for i, call in enumerate(order):
             nxt = self.blocks[order[i + 1].layer] if i + 1 < len(order) else None
             rt.next_norm = nxt.first_norm() if nxt is not None and hasattr(nxt, "first_norm") else None
-            self.blocks[call.layer].forward(x, ctx, [cache.view(c, call.writes_cache) for c in call.caches()], rt)
-        rt.stream_stats = rt.next_norm = None
+            rt.next_takes_deferred = nxt is not None and getattr(nxt, "takes_deferred", False)
+            block = self.blocks[call.layer]
+            if rt.stream_deferred is not None and not getattr(block, "takes_deferred", False):
+                rt.stream_deferred.flush(x)         # (an arrangement that knows nothing of sums left for its norm)
+                rt.stream_deferred = None
+            block.forward(x, ctx, [cache.view(c, call.writes_cache) for c in call.caches()], rt)
+        if rt.stream_deferred is not None:
+            rt.stream_deferred.flush(x)
+        rt.stream_stats = rt.next_norm = rt.stream_deferred = None
+        rt.next_takes_deferred = False
         if ctx.R == 0:
             return torch.empty((0, self.spec.vocab), dtype=torch.float32, device=rt.device)
         h = self.final_norm.forward(x, rt.act_dtype, rows=ctx.logit_rows, packed=self.head.packed_input(ctx.R))

@@ -33,10 +33,18 @@ class LayerNorm(Part):
         """What a kernel that runs this norm itself needs (parts.base.LazyNorm)."""
         return ("layernorm", self.weight, self.bias, self.eps)
 
-    def forward(self, x, out_dtype, rows=None, packed=False):
+    adds_deferred = True      # forward(..., deferred=): its kernel first adds a product's sum into the rows (parts.base.DeferredSum)
+
+    def forward(self, x, out_dtype, rows=None, packed=False, deferred=None):
         n = x.shape[0] if rows is None else rows.shape[0]
         if packed:
             out = ops.packed_rows(n, self.width, x.device)
         else:
             out = torch.empty((n, self.width), dtype=out_dtype, device=x.device)
+        if deferred is not None and deferred.filled:
+            if rows is None and self.width <= 8192:
+                part, bias = deferred.part, deferred.bias
+                deferred.part = deferred.bias = None
+                return ops.layernorm_join(x, part, bias, self.weight, self.bias, self.eps, out)
+            deferred.flush(x)
         return ops.layernorm(x, self.weight, self.bias, self.eps, out, rows)

@@ -993,3 +993,44 @@ def test_top_p_beyond_the_2048_largest_takes_the_whole_vocabulary():
     one = SamplingParams(temperature=1.0, top_p=1.0, seed=3)
     toks = Sampler(torch.device(DEV)).sample(logits[:4].clone(), [one] * 4, [3] * 4, [0, 1, 2, 3], [[]] * 4)
     assert toks == [SP.temperature_walk(row.tolist(), 1.0, uniform(3, i)) for i in range(4)]
+
+
+@pytest.mark.parametrize("M,N,K", [(65, 1600, 1600), (128, 1600, 6400), (200, 1280, 5120), (256, 1024, 1024), (100, 96, 4096)])
+@pytest.mark.parametrize("rows_in", ["packed", "rows"])
+def test_a_product_whose_sum_the_next_norm_adds(M, N, K, rows_in):
+    """A product into the stream may leave its shares' sums for the norm that reads the stream next: that norm's kernel
+    adds them (shares in order, then the bias) and norms the updated rows.  The stream and the normed rows are, bit
+    for bit, what the kernel that only adds the shares followed by the norm's own kernel give; the sum is right
+    against 64 bits; where the product that adds into the stream itself shares K out the same way, its bits too."""
+    o = ops()
+    a, w, bias = rnd(M, K, seed=1, dtype=torch.bfloat16), rnd(N, K, seed=2, dtype=torch.bfloat16, scale=0.05), rnd(N, seed=3)
+    gamma, beta = 1 + rnd(N, seed=4, scale=0.1), rnd(N, seed=5, scale=0.1)
+    x0 = rnd(M, N, seed=6)
+    wp = o.pack_matrix(w)
+    ain = o.pack_matrix(a) if rows_in == "packed" else a
+    assert o.linear_deferred_shares(M, wp) in (2, 4)
+    part = o.linear_deferred(ain, wp)
+    assert part.shape == (o.linear_deferred_shares(M, wp), M, N)
+    for b in (bias, None):
+        for packed_out in (False, True):
+            if packed_out and N % 32 != 0:
+                continue
+            x = x0.clone()
+            out = o.packed_rows(M, N, DEV) if packed_out else torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+            o.layernorm_join(x, part, b, gamma, beta, 1e-5, out)
+            x2 = o.join(part, b, x0.clone())
+            out2 = o.layernorm(x2, gamma, beta, 1e-5, o.packed_rows(M, N, DEV) if packed_out else torch.empty(M, N, dtype=torch.bfloat16, device=DEV))
+            assert torch.equal(x, x2)
+            assert torch.equal(out.rows() if packed_out else out, out2.rows() if packed_out else out2)
+    exact = (x0.double() + a.double() @ w.double().t() + bias.double()).float()
+    x = o.join(part, bias, x0.clone())
+    assert torch.allclose(x, exact, **TOL[torch.bfloat16])
+    if K >= 4096:       # the product that adds into the stream itself cuts K into the same shares
+        assert torch.equal(o.linear(ain, wp, bias, residual=x0.clone()), x)
+    # 32-bit out of the norm, and what is not deferred
+    out32 = torch.empty(M, N, device=DEV)
+    x = x0.clone()
+    o.layernorm_join(x, part, bias, gamma, None, 1e-5, out32)
+    assert torch.equal(out32, o.layernorm(x, gamma, None, 1e-5, torch.empty(M, N, device=DEV)))
+    assert o.linear_deferred_shares(64, wp) == 0 and o.linear_deferred_shares(300, wp) == 0
+    assert o.linear_deferred_shares(M, o.pack_matrix(rnd(4800, K, seed=7, dtype=torch.bfloat16))) == 0

@@ -938,3 +938,45 @@ def test_a_norm_without_a_mean_runs_inside_the_products(rows):
         x = x + f @ st[p + "mlp.c_proj.weight"].double() + st[p + "mlp.c_proj.bias"].double()
     want = P.head(x.float(), st["ln_f.weight"], st["ln_f.bias"], cfg["layer_norm_epsilon"], st["wte.weight"])[20:]
     U.assert_close(got[True], want, "bfloat16", "a norm without a mean inside the products against the plain formulas")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,rows", [("E", 40), ("F", 33)])
+def test_a_sum_left_for_the_next_norm(model_folders, name, rows):
+    """Steps of 65 to 256 rows: the attention's output projection and the feed-forward's second product leave their
+    sums for the norms behind them, whose kernels add them (the calls are counted: in a model of L layers every norm
+    but the first of the first layer; the last layer's feed-forward adds into the stream itself, since the final
+    norm reads chosen rows only).  The logits are those of the same steps with every product adding its own sum."""
+    from denno_beta_amd.engine import ModelRunner, StepEntry
+    from denno_beta_amd.kernels import ops
+    cfg = TINY[name][0]
+    folder = model_folders(name, "bfloat16")
+    seqs = [seeded_tokens(50 + i, rows, cfg["vocab_size"]) for i in range(3)]      # three requests: 99 to 120 rows a step
+    calls = {"join": 0, "flush": 0}
+    real_lj, real_j = ops.layernorm_join, ops.join
+
+    def count_lj(*a, **k):
+        calls["join"] += 1
+        return real_lj(*a, **k)
+
+    def count_j(*a, **k):
+        calls["flush"] += 1
+        return real_j(*a, **k)
+    got = {}
+    try:
+        ops.layernorm_join, ops.join = count_lj, count_j
+        for on in (True, False):
+            r = ModelRunner.from_folder(folder, options("cuda:0", "bfloat16", use_graphs=False, deferred_sums=on))
+            for i in range(3):
+                r.start_request(i)
+            before = dict(calls)
+            got[on] = r.step([StepEntry(i, s, list(range(rows))) for i, s in enumerate(seqs)]).float().cpu()
+            if on:
+                assert calls["join"] - before["join"] == 2 * cfg["n_layer"] - 1 and calls["flush"] == before["flush"]
+            else:
+                assert calls == before
+    finally:
+        ops.layernorm_join, ops.join = real_lj, real_j
+    U.assert_close(got[True], got[False], "bfloat16", f"{name}: sums left for the next norm against sums added at once")
+    want = torch.cat([P.PlainGPT2.from_folder(folder).logits(s) for s in seqs])
+    U.assert_close(got[True], want, "bfloat16", f"{name}: sums left for the next norm against the plain implementation")

@@ -584,6 +584,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
 
   // A in rows, or packed like W (PACKED_A): then a wave reads 1 KB in one piece per block
   const bf16_t* arow[MB];
+  const bf16_t* asafe[MB];
   bool a_ok[MB];
   const int astep = (packed & PACKED_A) ? 512 : 32;
 #pragma unroll
@@ -594,6 +595,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
     // rows end with the block that holds row M - 1)
     arow[mb] = (packed & PACKED_A) ? A + (static_cast<size_t>(min(static_cast<int>(blockIdx.y) * MB + mb, (M + 15) / 16 - 1)) * ksteps * 64 + lane) * 8
                                    : A + static_cast<size_t>(a_ok[mb] ? row : 0) * lda + g * 8;
+    // where a step's piece lies beyond K the load goes to an address that is surely inside A instead: the start
+    // of the row (with K < 32 the row's piece g itself may lie beyond the row, and the last row's beyond A)
+    asafe[mb] = (packed & PACKED_A) ? arow[mb] : A + static_cast<size_t>(a_ok[mb] ? row : 0) * lda;
   }
   // NORM_IN: the rows' means and 1 / sqrt(var + eps), joined while the first round of operands travels (a
   // wave does it in its first turn of the loop below, which every wave has: K >= 1024); the finishing
@@ -642,7 +646,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_kernel(const bf16_t* __restri
       }
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
-        a[u][mb] = *reinterpret_cast<const bf16x8*>(ok ? arow[mb] + ks * astep : arow[mb]);
+        a[u][mb] = *reinterpret_cast<const bf16x8*>(ok ? arow[mb] + ks * astep : asafe[mb]);
     }
     if constexpr (NORM == NORM_IN) {
       if (p0 == wave) join_stats();
@@ -777,6 +781,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
   const int lrow = lane / 8, lch = lane % 8;               // as loader: row and 16-byte chunk of the pair's 128 bytes
   const bf16_t* a0 = A + static_cast<size_t>(min(lrow, M - 1)) * lda + lch * 8;
   const bf16_t* a1 = A + static_cast<size_t>(min(lrow + 8, M - 1)) * lda + lch * 8;
+  // a chunk beyond K is not loaded; its load goes to the start of the row instead, which is surely inside A (a0
+  // itself is not where K < 64: chunk lch of a row of 32 elements lies in the next row, the last row's beyond A)
+  const bf16_t* asafe = A + static_cast<size_t>(min(lrow, M - 1)) * lda;
   bf16_t* mine = turn[wave][0];
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
   floatx4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -793,8 +800,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm16_kernel(const bf16_t* __rest
     for (int u = 0; u < U; ++u) {
       const int p = p0 + u * WAVES;
       const bool ok = p * 64 + lch * 8 < K;
-      al[u][0] = *reinterpret_cast<const u32x4*>(ok ? a0 + p * 64 : a0);
-      if constexpr (TWO) al[u][1] = *reinterpret_cast<const u32x4*>(ok ? a1 + p * 64 : a0);
+      al[u][0] = *reinterpret_cast<const u32x4*>(ok ? a0 + p * 64 : asafe);
+      if constexpr (TWO) al[u][1] = *reinterpret_cast<const u32x4*>(ok ? a1 + p * 64 : asafe);
     }
   };
   auto use = [&](int p0, const bf16x8 (*b)[2], const u32x4 (*al)[2]) {

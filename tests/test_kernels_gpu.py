@@ -1034,3 +1034,23 @@ def test_a_product_whose_sum_the_next_norm_adds(M, N, K, rows_in):
     assert torch.equal(out32, o.layernorm(x, gamma, None, 1e-5, torch.empty(M, N, device=DEV)))
     assert o.linear_deferred_shares(64, wp) == 0 and o.linear_deferred_shares(300, wp) == 0
     assert o.linear_deferred_shares(M, o.pack_matrix(rnd(4800, K, seed=7, dtype=torch.bfloat16))) == 0
+
+
+@pytest.mark.parametrize("M", [1, 5, 16, 40, 100])
+@pytest.mark.parametrize("K", [8, 16, 24, 32, 40, 56])
+def test_few_rows_product_with_an_inner_size_below_64(M, K):
+    """The few-rows kernels load A in pieces of 16 bytes at fixed places of a row (a row's share of a pair of steps
+    is 128 bytes); with an inner size below 64 some of those places lie beyond the row.  Such a piece is not loaded
+    (its load goes to the start of the row, which is inside A) and counts as zeros."""
+    o = ops()
+    for N in (16, 96):
+        a, w, bias = rnd(M, K, seed=1, dtype=torch.bfloat16), rnd(N, K, seed=2, dtype=torch.bfloat16, scale=0.3), rnd(N, seed=3)
+        wp = o.pack_matrix(w)
+        exact = (a.double() @ w.double().t() + bias.double()).float()
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        o.linear(a, wp, bias, out=out)
+        assert torch.allclose(out.float(), exact, **TOL[torch.bfloat16]), (M, N, K)
+        res = rnd(M, N, seed=4)
+        want = res + exact
+        o.linear(a, wp, bias, residual=res)
+        assert torch.allclose(res, want, **TOL[torch.bfloat16]), (M, N, K)

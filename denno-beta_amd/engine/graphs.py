@@ -329,7 +329,9 @@ class DecodeGraphs:
         new_lens = starts + 1
         slots = mgr.reserve_step(rids, new_lens)
         B = batch_bucket(n, runner.options.max_live)
-        ctx_bucket = min(-(-int(new_lens.max()) // DECODE_SPLIT) * DECODE_SPLIT, -(-spec.max_positions // 16) * 16)
+        # (contexts in buckets of 256, but no bucket beyond what a block table holds: whole pages up to the model's positions)
+        held = min(-(-spec.max_positions // l.page_size) * l.page_size for l in runner.cache.layouts if l.kind == 0)
+        ctx_bucket = min(-(-int(new_lens.max()) // DECODE_SPLIT) * DECODE_SPLIT, held)
         key = (B, ctx_bucket)
         g = self.graphs.get(key)
         if g is None:

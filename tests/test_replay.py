@@ -185,6 +185,27 @@ def test_page_sizes(backend, model_folders, page_size, dtype):
             U.assert_close(got[f"r{i}"], want[i], dtype, f"page size {page_size} {dtype} request {i}")
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page_size", [8, 48])
+def test_pages_that_do_not_divide_the_positions(tmp_path, page_size, dtype):
+    """130 positions in pages of 8 or 48 tokens: a request's block table holds whole pages (136 or 144 keys), and the
+    bucket of contexts that a captured decode step is made for stays within them.  Requests decoded to their last
+    position."""
+    from denno_beta_amd.weights import write_model_folder
+    cfg = _cfg(2, 64, 4, 128, 97, 130)
+    folder = write_model_folder(str(tmp_path), cfg, 3, dtype)
+    seqs = [seeded_tokens(60 + i, n, 97) for i, n in enumerate((130, 77, 129))]
+    want = plain_logits(folder, seqs)
+    for steps in (U.tail_decode_trace(seqs, 40), U.mixed_trace(seqs, seed=4)):
+        tokens = -(-U.max_live_tokens(steps) // page_size) * page_size
+        r = runner_for(folder, dtype, "cuda:0", cache_tokens=tokens + 2 * page_size, page_size=page_size)
+        got = U.replay(r, steps)
+        r.cache.manager.check()
+        for i in range(len(seqs)):
+            U.assert_close(got[f"r{i}"], want[i], dtype, f"page size {page_size} {dtype} request {i}")
+
+
 def test_step_refuses_what_it_cannot_run(backend, model_folders):
     from denno_beta_amd.cache import OutOfPages
     from denno_beta_amd.engine import BatchError, StepEntry

@@ -945,9 +945,11 @@ static void launch_mb_norm(const Call& c, const NormIO& nio, int norm, hipStream
   const int mb = (c.M + 15) / 16;
   if (c.N >= 2560) {
     switch (mb) {
-      case 2: return launch_norm<2, 2, 8, 6>(c, nio, norm, stream);
-      case 3: return launch_norm<3, 2, 8, 6>(c, nio, norm, stream);
-      default: return launch_norm<4, 2, 8, 6>(c, nio, norm, stream);
+      // (four steps in flight a wave: with six, the norm's sums beside them no longer fit the registers, and the
+      // product that also scatters keys and values took 24 us where it takes 13)
+      case 2: return launch_norm<2, 2, 8, 4>(c, nio, norm, stream);
+      case 3: return launch_norm<3, 2, 8, 4>(c, nio, norm, stream);
+      default: return launch_norm<4, 2, 8, 4>(c, nio, norm, stream);
     }
   }
   // (few columns: the rows in two halves, so that there are workgroups for all CUs)

@@ -145,7 +145,8 @@ __device__ __forceinline__ void finish(float v, int m, int n, const float* bias,
   }
 }
 
-template <typename TI, typename TC>
+// WHOLE: K is a multiple of 4, so a thread's four elements along K are all inside or all outside
+template <typename TI, typename TC, bool WHOLE>
 __global__ __launch_bounds__(256) void gemm_kernel(const TI* __restrict__ A, int lda, const TI* __restrict__ W,
                                                     const float* __restrict__ bias, TC* __restrict__ C, int ldc,
                                                     float* __restrict__ resid, int ldr, int M, int N, int K,
@@ -168,9 +169,14 @@ __global__ __launch_bounds__(256) void gemm_kernel(const TI* __restrict__ A, int
       float v[4] = {0.f, 0.f, 0.f, 0.f};
       if (m < M && k < K) {
         const TI* p = A + static_cast<size_t>(m) * lda + k;
+        if (WHOLE || k + 4 <= K) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (k + i < K) v[i] = to_float(p[i]);       // (K need be no multiple of 4: zeros beyond it)
+          for (int i = 0; i < 4; ++i) v[i] = to_float(p[i]);
+        } else {                                        // (K need be no multiple of 4: zeros beyond it)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (k + i < K) v[i] = to_float(p[i]);
+        }
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) As[lk + i][lrow] = v[i];
@@ -178,9 +184,14 @@ __global__ __launch_bounds__(256) void gemm_kernel(const TI* __restrict__ A, int
       float w[4] = {0.f, 0.f, 0.f, 0.f};
       if (n < N && k < K) {
         const TI* p = W + static_cast<size_t>(n) * K + k;
+        if (WHOLE || k + 4 <= K) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (k + i < K) w[i] = to_float(p[i]);
+          for (int i = 0; i < 4; ++i) w[i] = to_float(p[i]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (k + i < K) w[i] = to_float(p[i]);
+        }
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) Ws[lk + i][lrow] = w[i];
@@ -419,8 +430,12 @@ static int run(const void* A, int lda, const void* W, const float* bias, void* C
   if (!few_rows_take<TI>(A, lda, W, M, K)) {
     if (kv.slot_map) return DN_ERR_SHAPE;
     dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
-    hipLaunchKernelGGL((gemm_kernel<TI, TC>), grid, dim3(256), 0, stream, a, lda, w, bias, c, ldc, resid, ldr, M, N, K,
-                       epi);
+    if (K % 4 == 0)
+      hipLaunchKernelGGL((gemm_kernel<TI, TC, true>), grid, dim3(256), 0, stream, a, lda, w, bias, c, ldc, resid, ldr, M, N,
+                         K, epi);
+    else
+      hipLaunchKernelGGL((gemm_kernel<TI, TC, false>), grid, dim3(256), 0, stream, a, lda, w, bias, c, ldc, resid, ldr, M, N,
+                         K, epi);
     return 0;
   }
   const long need = work_floats(M, N, K);

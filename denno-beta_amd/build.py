@@ -192,6 +192,15 @@ def load_library(name) -> ctypes.CDLL:
         return lib
 
 
+def ensure_built(names, jobs=4):
+    """Compiles those of `names` that have no built file yet, side by side: a program's first call then waits for
+    the longest compilation, not for their sum."""
+    with _lock:
+        missing = [n for n in names if n not in _loaded and _find_built(n) is None]
+    if len(missing) > 1:
+        build_all(missing, jobs)
+
+
 def build_all(names=None, jobs=4):
     """Compiles every library (or `names`) anew, a few at a time."""
     names = list(names or LIBRARIES)

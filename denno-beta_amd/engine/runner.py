@@ -28,7 +28,15 @@ class ModelRunner:
         self.runtime = Runtime(act_dtype=_ACT[options.dtype], device=self.device,
                                norms_inside_products=options.norms_inside_products,
                                deferred_sums=options.deferred_sums)
-        self.model = spec.instantiate().bind(tensors, self.runtime)
+        model = spec.instantiate()
+        if self.device.type == "cuda":
+            # what this model needs is compiled now, side by side, if it is not built yet (else each library
+            # would be compiled at its first call, one after the other)
+            from ..build import ensure_built
+            from ..parts.base import PagedKV
+            paged = any(isinstance(cs, PagedKV) for cs in model.cache_specs)
+            ensure_built(["host", "elementwise", "gemm"] + (["attention"] if paged else []))
+        self.model = model.bind(tensors, self.runtime)
         cache_tokens = options.cache_tokens or options.max_live * spec.max_positions
         self.cache = CacheStorage(self.model.cache_specs, kv_dtype=self.runtime.act_dtype,
                                   page_size=options.page_size, cache_tokens=cache_tokens,

@@ -38,7 +38,8 @@ LIBRARIES = {
     "host": ("host", ["host/cache_manager.cpp", "host/scheduler.cpp", "host/c_api.cpp"],
              ["host/cache_manager.h", "host/scheduler.h"]),
     "elementwise": ("hip", ["kernels/elementwise.hip"], ["kernels/common.h"]),
-    "gemm": ("hip", ["kernels/gemm.hip"], ["kernels/common.h"]),
+    "gemm": ("hip", ["kernels/gemm.hip", "kernels/gemm_plain.hip", "kernels/gemm_skinny.hip", "kernels/gemm_tiled.hip",
+                     "kernels/gemm_direct.hip"], ["kernels/common.h", "kernels/gemm_common.h"]),
     "attention": ("hip", ["kernels/attention.hip"], ["kernels/common.h", "kernels/attention.h"]),
     "sampling": ("hip", ["kernels/sampling.hip"], ["kernels/common.h"]),
 }
@@ -139,14 +140,11 @@ def compile_library(name, quiet=False):
     out_dir = _lib_dir()
     final = os.path.join(out_dir, f"libdenno_{name}-{_digest(name)}.so")
     tmp = final + f".tmp{os.getpid()}"
-    cmd = [_compiler(kind)] + (HIP_FLAGS if kind == "hip" else HOST_FLAGS)
-    cmd += [os.path.join(_CSRC, s) for s in sources] + ["-I", os.path.join(_CSRC, "kernels"), "-o", tmp]
     if not quiet:
         _say(f"compiling {name} ({', '.join(sources)}) ...")
     t0 = time.time()
     env = dict(os.environ)
     env.setdefault("HOME", tempfile.gettempdir())   # hipcc wants a home for its caches
-    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
     # a line now and then while a long compilation runs
     done = threading.Event()
 
@@ -156,12 +154,48 @@ def compile_library(name, quiet=False):
     th = threading.Thread(target=tick, daemon=True)
     if not quiet:
         th.start()
-    out, _ = proc.communicate()
-    done.set()
-    if proc.returncode != 0:
+
+    def call(cmd):
+        proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
+        if proc.returncode != 0:
+            raise BuildError(f"building {name} failed ({' '.join(cmd)}):\n{proc.stdout}")
+        return proc.stdout
+
+    include = ["-I", os.path.join(_CSRC, "kernels")]
+    flags = HIP_FLAGS if kind == "hip" else HOST_FLAGS
+    objects = []
+    try:
+        if kind == "hip" and len(sources) > 1:
+            # a kernel library of several source files: each compiled to an object of its own, side by side,
+            # then linked (the files of the matrix products take a minute one after the other)
+            objects = [f"{tmp}.{i}.o" for i in range(len(sources))]
+            outs, errors = [None] * len(sources), []
+
+            def one(i):
+                try:
+                    outs[i] = call([_compiler(kind)] + [f for f in flags if f != "-shared"] +
+                                   ["-c", os.path.join(_CSRC, sources[i])] + include + ["-o", objects[i]])
+                except Exception as e:   # raised below, after every compilation has ended
+                    errors.append(e)
+            workers = [threading.Thread(target=one, args=(i,)) for i in range(len(sources))]
+            for w in workers:
+                w.start()
+            for w in workers:
+                w.join()
+            if errors:
+                raise errors[0]
+            out = "".join(outs) + call([_compiler(kind), "--offload-arch=" + HIP_ARCH, "-shared", "-fPIC"] + objects + ["-o", tmp])
+        else:
+            out = call([_compiler(kind)] + flags + [os.path.join(_CSRC, s) for s in sources] + include + ["-o", tmp])
+    except BaseException:
         if os.path.exists(tmp):
             os.remove(tmp)
-        raise BuildError(f"building {name} failed ({' '.join(cmd)}):\n{out}")
+        raise
+    finally:
+        done.set()
+        for o in objects:
+            if os.path.exists(o):
+                os.remove(o)
     os.replace(tmp, final)
     for f in os.listdir(out_dir):   # built files of older sources
         if f.startswith(f"libdenno_{name}-") and f.endswith(".so") and os.path.join(out_dir, f) != final:

@@ -27,6 +27,11 @@ class TraceReplayer:
         try:
             for e in record.get("entries", []):
                 name = str(e["id"])
+                if not e["tokens"]:
+                    # an entry that brings no tokens is a request left out of this step
+                    if e.get("want"):
+                        raise ValueError(f"step {record.get('step')}: request {name} wants logits of tokens it does not bring")
+                    continue
                 if name not in self._rid:
                     self.runner.start_request(self._next)
                     self._rid[name] = self._next

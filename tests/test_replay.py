@@ -250,6 +250,21 @@ def test_a_refused_step_leaves_nothing_of_the_requests_it_started(backend, model
     r.cache.manager.check()
 
 
+def test_an_entry_without_tokens_is_a_request_left_out(backend, model_folders):
+    from denno_beta_amd.engine.replay import TraceReplayer
+    r = runner_for(model_folders("A", "float32"), "float32", backend, cache_tokens=64, max_live=2)
+    rp = TraceReplayer(r)
+    a = rp.run_step({"step": 0, "entries": [{"id": "a", "tokens": [1, 2, 3], "want": [2]},
+                                            {"id": "b", "tokens": [], "want": []}], "end": []})
+    assert a.shape == (1, 512) and rp.live() == ["a"]          # "b" has not begun
+    assert rp.run_step({"step": 1, "entries": [{"id": "a", "tokens": [], "want": []}], "end": []}) is None
+    assert r.cache.manager.length(0) == 3
+    with pytest.raises(ValueError, match="does not bring"):
+        rp.run_step({"step": 2, "entries": [{"id": "a", "tokens": [], "want": [0]}], "end": []})
+    b = rp.run_step({"step": 3, "entries": [{"id": "a", "tokens": [4], "want": [0]}], "end": ["a"]})
+    assert b.shape == (1, 512) and rp.live() == [] and r.cache.manager.live() == 0
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decode_graphs_replay_what_eager_steps_compute(model_folders, dtype):

@@ -391,8 +391,20 @@ int deferred_shares(int M, int N, int K) {
   return K / 64 >= 8 ? 2 : 0;
 }
 
+static bool wide_mid(int M, int N) { return N >= 2048 && M <= 256; }
+static long mid_tiles_64(int M, int N) { return static_cast<long>((M + 63) / 64) * ((N + 63) / 64); }
+
 int run(const Args& a, hipStream_t stream) {
-  if (mid_rows(a.M, a.N, a.K) || (a.part && a.N < 2048 && a.K % 64 == 0)) return launch_as<2, 2, 2, 2, 4, 2>(a, stream);
+  if (mid_rows(a.M, a.N, a.K) || (a.part && a.N < 2048 && a.K % 64 == 0)) {
+    // Wide products: sixteen waves a workgroup, four a SIMD, each with one 16 x 16 block of a 64 x 64 tile (a wave
+    // of such a product waits on a counter for more than half of its life, and with one wave a SIMD nothing else
+    // runs meanwhile: 16.0 -> 13.9 and 12.8 -> 11.3 us for 4,800 and 6,400 columns at 128 rows); where those tiles
+    // are more than the chip has CUs, tiles of 128 x 64 with two blocks a wave (at 256 rows 23.3 -> 20.2 and
+    // 18.1 -> 15.2 us).  The narrow ones, whose K is shared out, take neither way faster: four waves as before.
+    if (wide_mid(a.M, a.N) && !a.part)
+      return mid_tiles_64(a.M, a.N) <= CUS ? launch_as<4, 4, 1, 1, 4, 2>(a, stream) : launch_as<4, 4, 2, 1, 4, 2>(a, stream);
+    return launch_as<2, 2, 2, 2, 4, 2>(a, stream);
+  }
   switch (pick(a.M, a.N, a.part ? a.K / a.splits : a.K)) {
     case 0: return launch_as<2, 2, 2, 4, 4>(a, stream);
     case 1: return launch_as<4, 2, 2, 4, 4>(a, stream);
@@ -409,7 +421,8 @@ int run(const Args& a, hipStream_t stream) {
 
 // the tile that a product of these sizes gets: rows * 1000 + columns
 int tile_of(int M, int N, int K) {
-  const Shape& s = SHAPES[mid_rows(M, N, K) ? MID : pick(M, N, K)];
+  if (mid_rows(M, N, K)) return wide_mid(M, N) && mid_tiles_64(M, N) > CUS ? 128064 : 64064;
+  const Shape& s = SHAPES[pick(M, N, K)];
   return s.bm * 1000 + s.bn;
 }
 }  // namespace direct

@@ -320,6 +320,13 @@ static int launch_as(const Args& a, hipStream_t stream) {
   return launch<float, WM, WN, TM, TN, STAGES, false, KB>(a, stream);
 }
 
+// (for tiles that never write the cache: the variant with the cache write is not built)
+template <int WM, int WN, int TM, int TN, int STAGES, int KB = 1>
+static int launch_without_kv(const Args& a, hipStream_t stream) {
+  if (a.out_dtype == DN_BF16 && !a.resid) return launch<bf16_t, WM, WN, TM, TN, STAGES, false, KB>(a, stream);
+  return launch<float, WM, WN, TM, TN, STAGES, false, KB>(a, stream);
+}
+
 // The tiles on offer: rows x columns, slabs in flight.  256 rows: 8 waves as 4 x 2, one workgroup
 // per CU; the small ones leave room for several workgroups per CU.  64 x 64 and 32 x 64 (4 waves) are
 // for products with few rows and a long K, whose larger tiles would leave most CUs idle.
@@ -405,14 +412,28 @@ int run(const Args& a, hipStream_t stream) {
       return mid_tiles_64(a.M, a.N) <= CUS ? launch_as<4, 4, 1, 1, 4, 2>(a, stream) : launch_as<4, 4, 2, 1, 4, 2>(a, stream);
     return launch_as<2, 2, 2, 2, 4, 2>(a, stream);
   }
+  // Tiles of 128 and 256 rows: sixteen waves a workgroup, four a SIMD, as 8 x 2 (a wave: 32 rows x a half of the
+  // tile's columns) or 4 x 4, where eight waves as 4 x 2 with twice the rows each left the SIMDs waiting (a wave
+  // waits on a counter for more than half of its life and the matrix cores were busy 30 % of the time).  At 2,048
+  // rows of the XL layer: 56.1 -> 41.0, 25.2 -> 21.3, 57.1 -> 46.6 and 71.8 -> 56.9 us.  Two slabs a stage where K
+  // allows it; a long K wants more stages in flight than a short one (with two, the MLP projection of 4,096 rows
+  // took 145 us for 125), and LDS decides how many fit.  The cache write's epilogue needs registers that sixteen
+  // waves do not leave beside seven column blocks and more a wave: those keep eight waves.
+  const bool sixteen = !a.part, two = a.K % 64 == 0, short_k = a.K < 4096;
   switch (pick(a.M, a.N, a.part ? a.K / a.splits : a.K)) {
     case 0: return launch_as<2, 2, 2, 4, 4>(a, stream);
-    case 1: return launch_as<4, 2, 2, 4, 4>(a, stream);
-    case 2: return launch_as<4, 2, 4, 4, 4>(a, stream);
-    case 3: return launch_as<4, 2, 4, 5, 4>(a, stream);
-    case 4: return launch_as<4, 2, 4, 6, 4>(a, stream);
-    case 5: return launch_as<4, 2, 4, 7, 4>(a, stream);
-    case 6: return launch_as<4, 2, 4, 8, 4>(a, stream);
+    case 1: return sixteen && two ? launch_as<4, 4, 2, 2, 3, 2>(a, stream) : launch_as<4, 2, 2, 4, 4>(a, stream);
+    case 2: return sixteen && two ? launch_as<8, 2, 2, 4, 3, 2>(a, stream) : launch_as<4, 2, 4, 4, 4>(a, stream);
+    case 3: return sixteen && two ? launch_as<8, 2, 2, 5, 3, 2>(a, stream) : launch_as<4, 2, 4, 5, 4>(a, stream);
+    case 4:
+      if (!sixteen) return launch_as<4, 2, 4, 6, 4>(a, stream);
+      return two && short_k ? launch_as<8, 2, 2, 6, 2, 2>(a, stream) : launch_as<8, 2, 2, 6, 3>(a, stream);
+    case 5:
+      if (a.kv || !sixteen) return launch_as<4, 2, 4, 7, 4>(a, stream);
+      return two && short_k ? launch_without_kv<8, 2, 2, 7, 2, 2>(a, stream) : launch_without_kv<8, 2, 2, 7, 5>(a, stream);
+    case 6:
+      if (a.kv || !sixteen) return launch_as<4, 2, 4, 8, 4>(a, stream);
+      return two && short_k ? launch_without_kv<8, 2, 2, 8, 2, 2>(a, stream) : launch_without_kv<8, 2, 2, 8, 3>(a, stream);
     case 7: return launch_as<4, 2, 4, 10, 3>(a, stream);
     case 8: return launch_as<2, 2, 2, 2, 4>(a, stream);
     default: return launch_as<2, 2, 1, 2, 4>(a, stream);

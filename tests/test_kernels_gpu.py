@@ -118,18 +118,20 @@ def test_linear(in_dtype, M, N, K):
 
 def test_linear_with_every_tile_of_the_many_rows_kernel():
     """Beyond 256 rows the tile is chosen per product from a list: every tile on the list, on sizes
-    that are no multiple of it, with a short K (fewer slabs than the kernel keeps in flight) and a
-    longer one, for each kind of output."""
+    that are no multiple of it, with a short K (fewer slabs than the kernel keeps in flight) and
+    longer ones (each picks another arrangement of waves and stages), for each kind of output."""
     o = ops()
     tile = o._lib("gemm").dn_gemm_tile
     cases = {}
-    for K in (64, 416):             # per tile the smallest product that gets it
+    # per tile and K the smallest product that gets it.  K = 64: one stage; 416: no multiple of 64, so a slab a
+    # stage; 448: two slabs a stage; 4,160: a long K, which takes more stages in flight
+    for K in (64, 416, 448, 4160):
         for M in range(260, 4200, 140):
             for N in range(136, 10000, 232):
                 t = tile(M, N, K)
-                if t not in cases or M * N < cases[t][0] * cases[t][1]:
-                    cases[t] = (M, N, K)
-    assert len(cases) == 10, sorted(cases)
+                if (t, K) not in cases or M * N < cases[(t, K)][0] * cases[(t, K)][1]:
+                    cases[(t, K)] = (M, N, K)
+    assert len({t for t, _ in cases}) == 10, sorted(cases)
     tol = dict(TOL[torch.bfloat16])
     for M, N, K in cases.values():
         a, w, bias = rnd(M, K, seed=1, dtype=torch.bfloat16), rnd(N, K, seed=2, dtype=torch.bfloat16, scale=0.2), rnd(N, seed=3)
@@ -381,15 +383,18 @@ def test_the_norm_inside_products_refuses_what_it_cannot_take():
         ops().linear_norm_out(rnd(17, 64, dtype=torch.bfloat16), wp, None, rnd(17, 32), c, *ops().norm_stream_buffers(17, 32, DEV))
 
 
-@pytest.mark.parametrize("M", [100, 129, 200, 256, 300])
+@pytest.mark.parametrize("M", [100, 129, 200, 256, 300, 1000, 2100, 4200])
 @pytest.mark.parametrize("rows_in", ["packed", "rows"])
-def test_linear_qkv_with_many_columns(M, rows_in):
+@pytest.mark.parametrize("K", [160, 192, 4160])
+def test_linear_qkv_with_many_columns(M, rows_in, K):
     """The fused projection where its columns are many (the many-rows kernel takes it from 129 rows on,
-    with packed rows too): heads of 48, a grouped cache, pages of 32, slots in runs that start anywhere."""
+    with packed rows too): heads of 48, a grouped cache, pages of 32, slots in runs that start anywhere.
+    An inner size that is a multiple of 64 goes two slabs a stage, a long one keeps more stages in flight,
+    and the rows decide the tile."""
     if rows_in == "packed" and M > 256:
         pytest.skip("packed rows end at 256")
     o = ops()
-    H, Hkv, dh, ps, K = 64, 16, 48, 32, 160
+    H, Hkv, dh, ps = 64, 16, 48, 32
     N = (H + 2 * Hkv) * dh
     assert N >= 4096
     n_pages = (M + 40) // ps + 2

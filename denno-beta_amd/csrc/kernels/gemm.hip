@@ -22,6 +22,8 @@
 
 // the tile that a product of these sizes gets from the kernel above: rows * 1000 + columns
 extern "C" int dn_gemm_tile(int M, int N, int K) { return direct::tile_of(M, N, K); }
+// the same for a fused projection that writes the cache (some tiles are not on offer to it)
+extern "C" int dn_gemm_tile_qkv(int M, int N, int K) { return direct::tile_of(M, N, K, true); }
 
 // packed: bit flags.  W in rows of K elements (the plain kernel, any dtype), or packed bfloat16
 // (PACKED_W 1: the MFMA kernels, which need A in bfloat16 and loadable 16 bytes at a time).  With

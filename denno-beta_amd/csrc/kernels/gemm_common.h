@@ -164,11 +164,11 @@ struct Args {
 struct Shape { int bm, bn, stages; };
 bool takes(const void* A, int lda, const void* W, const float* bias, const void* C, int ldc, const float* resid,
            int ldr, int N, int K, int out_dtype, int packed);
-int pick(int M, int N, int K);
+int pick(int M, int N, int K, bool kv = false);
 bool mid_rows(int M, int N, int K);
 bool beats_few_rows(int M, int N, int K);
 int shares_of_k(int M, int N, int K, int packed, bool kv);
 int deferred_shares(int M, int N, int K);
 int run(const Args& a, hipStream_t stream);
-int tile_of(int M, int N, int K);
+int tile_of(int M, int N, int K, bool kv = false);
 }  // namespace direct

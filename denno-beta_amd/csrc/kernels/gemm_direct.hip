@@ -327,13 +327,13 @@ static int launch_without_kv(const Args& a, hipStream_t stream) {
   return launch<float, WM, WN, TM, TN, STAGES, false, KB>(a, stream);
 }
 
-// The tiles on offer: rows x columns, slabs in flight.  256 rows: 8 waves as 4 x 2, one workgroup
-// per CU; the small ones leave room for several workgroups per CU.  64 x 64 and 32 x 64 (4 waves) are
-// for products with few rows and a long K, whose larger tiles would leave most CUs idle.
+// The tiles that `pick` chooses among: rows x columns, and the slabs in flight that its model counts LDS with.
+// 128 and 256 rows: one workgroup per CU; the small ones (four waves) leave room for several workgroups per CU and
+// are for products with few rows and a long K, whose larger tiles would leave most CUs idle.  (Tiles of 256 x 320
+// were on the list while the others ran with eight waves a workgroup; no product chooses them now.)
 constexpr Shape SHAPES[] = {{64, 128, 4}, {128, 128, 4}, {256, 128, 4}, {256, 160, 4}, {256, 192, 4},
-                            {256, 224, 4}, {256, 256, 4}, {256, 320, 3}, {64, 64, 4}, {32, 64, 4}, {64, 64, 4}};
-constexpr int PICKED = 10;        // the shapes that `pick` chooses among
-constexpr int MID = 10;           // 64 x 64 with two slabs a stage: `mid_rows`
+                            {256, 224, 4}, {256, 256, 4}, {64, 64, 4}, {32, 64, 4}};
+constexpr int PICKED = 9;
 
 static double model_us(const Shape& s, int M, int N, int K) {
   const double tiles = static_cast<double>((M + s.bm - 1) / s.bm) * ((N + s.bn - 1) / s.bn);
@@ -345,11 +345,15 @@ static double model_us(const Shape& s, int M, int N, int K) {
   return rounds * (K * (2.26e-7 * area + 3.07e-5 * (s.bm + s.bn)) + 1.9e-4 * area);
 }
 
-int pick(int M, int N, int K) {
+int pick(int M, int N, int K, bool kv) {
   int best = 0;
   double best_us = 1e30;
   for (int i = 0; i < PICKED; ++i) {
-    const double us = model_us(SHAPES[i], M, N, K);
+    double us = model_us(SHAPES[i], M, N, K);
+    // (the model is of eight waves a workgroup; the tiles that run with sixteen, see `run`, take about three
+    // quarters of its time, which moves the choice at 4,096 rows and more: the fused projection of 8,192 rows
+    // 185 -> 165 us)
+    if (i >= 1 && i <= 6 && !(kv && i >= 5)) us *= 0.75;
     if (us < best_us) best_us = us, best = i;
   }
   return best;
@@ -357,11 +361,11 @@ int pick(int M, int N, int K) {
 
 // 65 to 512 rows.  A tile's walk along K costs a wave some dozens of instructions a slab beside its four matrix
 // instructions, and with one or two waves a SIMD nothing hides them: tiles of 64 x 64 take two slabs a stage
-// (SHAPES[MID]), which halves that and fills the chip from 65 rows on where the product is wide.  Measured on the
+// which halves that and fills the chip from 65 rows on where the product is wide.  Measured on the
 // four products of a layer 1,600 wide (rows and weights that no cache holds; us, before -> now):
 //   128 rows: 4,800 columns 18.7 -> 15.7, 6,400 columns 15.3 -> 12.3, 1,600 columns from K = 6,400 19.4 -> 15.2
 //   256 rows: 25.6 -> 23.2, 19.3 -> 18.0, 25.6 -> 21.4;  512 rows, 1,600 columns: K = 1,600 12.6 -> 10.7, K = 6,400 38.7 -> 35.4
-// -> whether this kernel takes the product with SHAPES[MID] (else `pick` chooses, or the few-rows kernel runs)
+// -> whether this kernel takes the product with those tiles (else `pick` chooses, or the few-rows kernel runs)
 bool mid_rows(int M, int N, int K) {
   if (M <= 64 || M > 512 || K % 64 != 0) return false;
   if (N < 2048) return K >= 4096 || M > 256;      // (few columns and a short K up to 256 rows: the few-rows kernel)
@@ -399,7 +403,8 @@ int deferred_shares(int M, int N, int K) {
 }
 
 static bool wide_mid(int M, int N) { return N >= 2048 && M <= 256; }
-static long mid_tiles_64(int M, int N) { return static_cast<long>((M + 63) / 64) * ((N + 63) / 64); }
+static long tiles_of(int M, int N, int bm, int bn) { return static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn); }
+static long mid_tiles_64(int M, int N) { return tiles_of(M, N, 64, 64); }
 
 int run(const Args& a, hipStream_t stream) {
   if (mid_rows(a.M, a.N, a.K) || (a.part && a.N < 2048 && a.K % 64 == 0)) {
@@ -420,8 +425,11 @@ int run(const Args& a, hipStream_t stream) {
   // took 145 us for 125), and LDS decides how many fit.  The cache write's epilogue needs registers that sixteen
   // waves do not leave beside seven column blocks and more a wave: those keep eight waves.
   const bool sixteen = !a.part, two = a.K % 64 == 0, short_k = a.K < 4096;
-  switch (pick(a.M, a.N, a.part ? a.K / a.splits : a.K)) {
-    case 0: return launch_as<2, 2, 2, 4, 4>(a, stream);
+  switch (pick(a.M, a.N, a.part ? a.K / a.splits : a.K, a.kv != nullptr)) {
+    case 0:      // (the small tiles with sixteen waves too, where one round of them covers the product: several
+                 // workgroups of four waves share a CU, one of sixteen has it alone)
+      if (sixteen && two && tiles_of(a.M, a.N, 64, 128) <= CUS) return launch_as<4, 4, 1, 2, 4, 2>(a, stream);
+      return launch_as<2, 2, 2, 4, 4>(a, stream);
     case 1: return sixteen && two ? launch_as<4, 4, 2, 2, 3, 2>(a, stream) : launch_as<4, 2, 2, 4, 4>(a, stream);
     case 2: return sixteen && two ? launch_as<8, 2, 2, 4, 3, 2>(a, stream) : launch_as<4, 2, 4, 4, 4>(a, stream);
     case 3: return sixteen && two ? launch_as<8, 2, 2, 5, 3, 2>(a, stream) : launch_as<4, 2, 4, 5, 4>(a, stream);
@@ -434,16 +442,17 @@ int run(const Args& a, hipStream_t stream) {
     case 6:
       if (a.kv || !sixteen) return launch_as<4, 2, 4, 8, 4>(a, stream);
       return two && short_k ? launch_without_kv<8, 2, 2, 8, 2, 2>(a, stream) : launch_without_kv<8, 2, 2, 8, 3>(a, stream);
-    case 7: return launch_as<4, 2, 4, 10, 3>(a, stream);
-    case 8: return launch_as<2, 2, 2, 2, 4>(a, stream);
+    case 7:
+      if (sixteen && two && tiles_of(a.M, a.N, 64, 64) <= CUS) return launch_as<4, 4, 1, 1, 4, 2>(a, stream);
+      return launch_as<2, 2, 2, 2, 4>(a, stream);
     default: return launch_as<2, 2, 1, 2, 4>(a, stream);
   }
 }
 
 // the tile that a product of these sizes gets: rows * 1000 + columns
-int tile_of(int M, int N, int K) {
+int tile_of(int M, int N, int K, bool kv) {
   if (mid_rows(M, N, K)) return wide_mid(M, N) && mid_tiles_64(M, N) > CUS ? 128064 : 64064;
-  const Shape& s = SHAPES[pick(M, N, K)];
+  const Shape& s = SHAPES[pick(M, N, K, kv)];
   return s.bm * 1000 + s.bn;
 }
 }  // namespace direct

@@ -9,20 +9,22 @@
 // lanes, so 16 lanes take 64 bytes from each of four rows (four lines) and not 16 bytes from each of
 // sixteen (with a lane per row the lookups, 52 per load on average, kept the cache busy for three
 // quarters of the kernel's time), and the four 16-byte pieces of a row are exchanged by the row's
-// number so that the operand read (lane l wants row l % 16, piece l / 16) meets every bank once.  STAGES slabs are in flight (vmcnt counts a wave's
-// own loads; one barrier per slab publishes them and frees the slab read before).
+// number so that the operand read (lane l wants row l % 16, piece l / 16) meets every bank once.  STAGES
+// stages of KB slabs are in flight (vmcnt counts a wave's own loads; one barrier per stage publishes them and
+// frees the stage read before).
 //
 // The MFMA takes W as its first operand and A as its second: a lane then holds four consecutive
 // columns of one row of C, which it stores as 8 bytes (bfloat16) or adds as 16 (the 32-bit
 // residual) without a turn through LDS; for the fused QKV product they are one key's or one
 // value's four dims.
 //
-// What bounds these products here is the traffic from L2 into the CUs and the rounding of tiles to
-// 256 CUs, not the matrix cores: measured per tile and slab, time = 2.26e-7 us x BM x BN (matrix
-// cores at nine tenths of their peak) + 3.07e-5 us x (BM + BN) (loads), the two adding up rather
-// than overlapping, + 1.9e-4 us x BM x BN for the stores at the end.  So the tile is chosen per
-// product from a list, by that model: the largest that still fills the chip in whole rounds
-// (a tile count just above a multiple of 256 costs a whole further round).
+// What bounds these products here is not the matrix cores (busy 30 % of the time with eight waves a workgroup)
+// but a wave's chain of loads, waits and barriers, and the rounding of tiles to 256 CUs.  Measured per tile and
+// slab with eight waves: time = 2.26e-7 us x BM x BN (matrix cores at nine tenths of their peak) + 3.07e-5 us x
+// (BM + BN) (loads), the two adding up rather than overlapping, + 1.9e-4 us x BM x BN for the stores at the end.
+// The tile is chosen per product from a list, by that model: the largest that still fills the chip in whole
+// rounds (a tile count just above a multiple of 256 costs a whole further round); and the waves of a workgroup
+// are as many as give every SIMD four (see `run`), so that one of them can issue while the others wait.
 // ---------------------------------------------------------------------------------------
 namespace direct {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
